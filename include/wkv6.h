@@ -1,0 +1,143 @@
+/*
+ * wkv6.h -- C ABI of libwkv6_gfx950.so, the MI355X (gfx950) implementation of the WKV6
+ * time-mixing operator.  Plain pointers and sizes only; every pointer except `state_map`
+ * `workspace` arguments is a DEVICE pointer to a row-major contiguous array; all work is
+ * enqueued on `stream` (a hipStream_t, may be NULL = default stream) and the calls return
+ * without synchronising.  The library keeps no mutable global state: calls are re-entrant.
+ *
+ * Each entry point names the reference interface it replaces (paths relative to the
+ * reference tree infiy-quine/STAR-RWKV6).
+ *
+ * Tensors:  r,k,v,w,y,gy,gr,gk,gv,gw : (B,T,C), channel c = h*N + n, N = C/H (head size);
+ *           u : C elements (H,N);  gu : (B,C) per-batch partials (the caller sums over B,
+ *           as rwkv_kernel/torch_rwkv_kernel.py:73 and rwkv_kernel/jax_rwkv_kernel.py:166 do);
+ *           state s, ys : (n_state|B, H, N, N) indexed [key j][value i]
+ *           (rwkv_kernel/ops_rwkv_kernal.py:85-91);  state_map : (B,) int64 on the device.
+ *           w is the RAW decay input; the operator applies exp(-exp(w)) itself
+ *           (rwkv_kernel/jax_kernel/rwkv_kernels.cu:125).
+ * Element types (`dtype` = type of r,k,v,w,u): outputs, gy and states use the "output type":
+ *           F32 -> F32, BF16 -> BF16, F16 -> F32 (rwkv_kernel/torch_rwkv_kernel.py:35).
+ */
+#ifndef WKV6_H_
+#define WKV6_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Same numbering as `enum ElementType { BF16, F16, F32 }`, rwkv_kernel/jax_kernel/kernels.h:30. */
+enum { WKV6_BF16 = 0, WKV6_F16 = 1, WKV6_F32 = 2 };
+
+/* Return codes (the reference's natives return void and assert; this ABI never throws). */
+enum {
+    WKV6_OK = 0,
+    WKV6_ERR_ARG = 1,         /* null pointer, non-positive size, C != H*N, unknown dtype   */
+    WKV6_ERR_UNSUPPORTED = 2, /* head size the kernels are not built for                     */
+    WKV6_ERR_WORKSPACE = 3,   /* workspace missing or smaller than the query function says   */
+    WKV6_ERR_LAUNCH = 4       /* the HIP runtime refused a launch (see wkv6_last_hip_error)   */
+};
+
+/* Algorithm selector for the *_ex entry points. */
+enum {
+    WKV6_ALGO_AUTO = 0,  /* library picks: chunked MFMA path for bf16/f16 when T allows, else scan */
+    WKV6_ALGO_SCAN = 1,  /* per-timestep fp32 recurrence, state in VGPRs                       */
+    WKV6_ALGO_CHUNK = 2  /* chunk-parallel form, bf16 MFMA for the dense intra-chunk products   */
+};
+
+const char *wkv6_status_string(int status);
+int wkv6_version(void);
+/* Head sizes compiled into the library: returns 1 if N is supported. */
+int wkv6_supports_head_size(int64_t N);
+
+/* Stateless forward.
+ * Replaces forward_{bf16,fp16,fp32}(B,T,C,H,r,k,v,w,u,y), rwkv_kernel/torch_kernel/wkv6_op.cpp:22-30,
+ * i.e. cuda_forward<>, rwkv_kernel/torch_kernel/wkv6_cuda.cu:323-329 (kernel_forward). */
+int wkv6_forward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
+                 const void *r, const void *k, const void *v, const void *w, const void *u,
+                 void *y);
+
+/* Forward with optional initial state and final-state output.
+ * Replaces forward_with_state_{bf16,fp16,fp32}(B,T,C,H,S,map,r,k,v,w,u,s,y,ys),
+ * rwkv_kernel/torch_kernel/wkv6_op.cpp:44-52 (kernel_forward_state,
+ * rwkv_kernel/jax_kernel/rwkv_kernels.cu:165-190).  has_init_state==0: s and state_map ignored,
+ * zero initial state.  has_init_state!=0: S_0[b] = s[state_map[b]] (state_map NULL = identity);
+ * state_map values must lie in [0, rows of s) -- validated by the caller on the host.
+ * s and ys are in the output type.  ys may alias s only when state_map is the identity. */
+int wkv6_forward_with_state(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
+                            int has_init_state, const int64_t *state_map,
+                            const void *r, const void *k, const void *v, const void *w, const void *u,
+                            const void *s, void *y, void *ys);
+
+/* Same, with the state element type chosen separately (WKV6_F32 keeps a decode loop's carried
+ * state in fp32 while the activations stay bf16).  No counterpart in the reference, whose state
+ * type is always the output type (rwkv_kernel/torch_rwkv_kernel.py:126-131). */
+int wkv6_forward_with_state_ex(void *stream, int dtype, int state_dtype, int algo,
+                               int64_t B, int64_t T, int64_t C, int64_t H,
+                               int has_init_state, const int64_t *state_map,
+                               const void *r, const void *k, const void *v, const void *w, const void *u,
+                               const void *s, void *y, void *ys,
+                               void *workspace, size_t workspace_bytes);
+size_t wkv6_forward_workspace_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H);
+
+/* Backward of the stateless forward: gr,gk,gv,gw (B,T,C) and gu (B,C), all in the output type.
+ * Replaces backward_{bf16,fp16,fp32}(B,T,C,H,r,k,v,w,u,gy,gr,gk,gv,gw,gu),
+ * rwkv_kernel/torch_kernel/wkv6_op.cpp:33-41 (kernel_backward_101/102/103/201,
+ * rwkv_kernel/jax_kernel/rwkv_kernels.cu:205-407, launched by HostApplyGradient :436-444).
+ * `workspace` is device memory of at least wkv6_backward_workspace_bytes(...) bytes owned by the
+ * caller; its contents on entry and exit are meaningless. */
+int wkv6_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
+                  const void *r, const void *k, const void *v, const void *w, const void *u,
+                  const void *gy,
+                  void *gr, void *gk, void *gv, void *gw, void *gu,
+                  void *workspace, size_t workspace_bytes);
+size_t wkv6_backward_workspace_bytes(int dtype, int64_t B, int64_t T, int64_t C, int64_t H);
+
+/* Same two calls with the algorithm forced (tests and benchmarks compare the two paths). */
+int wkv6_forward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                    const void *r, const void *k, const void *v, const void *w, const void *u,
+                    void *y, void *workspace, size_t workspace_bytes);
+int wkv6_backward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                     const void *r, const void *k, const void *v, const void *w, const void *u,
+                     const void *gy,
+                     void *gr, void *gk, void *gv, void *gw, void *gu,
+                     void *workspace, size_t workspace_bytes);
+size_t wkv6_backward_workspace_bytes_ex(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H);
+
+/* ---- XLA custom-call surface (replaces the pybind module `gpu_ops`,
+ * rwkv_kernel/jax_kernel/gpu_ops.cpp:20-43) ---------------------------------------------- */
+
+/* 28-byte opaque descriptor, same field order as WKVDescriptor, rwkv_kernel/jax_kernel/kernels.h:32-42. */
+typedef struct wkv6_descriptor {
+    int32_t B, T, C, H;
+    uint8_t S;        /* has initial state */
+    uint8_t pad_[3];
+    int32_t x_type;   /* WKV6_BF16 | WKV6_F16 | WKV6_F32 */
+    int32_t y_type;
+} wkv6_descriptor;
+
+/* Replaces create_rwkv_descriptor (gpu_ops.cpp:33-36): fills out[0..28), returns 28. */
+size_t wkv6_create_descriptor(int B, int T, int C, int H, int S, int x_type, int y_type, void *out);
+
+/* XLA status-less custom-call targets, signature void(stream, buffers, opaque, opaque_len)
+ * (rwkv_kernel/jax_kernel/kernels.h:44-53).  Buffer order = operands then results:
+ *   wkv_forward            [r,k,v,w,u | y]                                (rwkv_kernels.cu:458-462)
+ *   wkv_backward           [r,k,v,w,u,gy | gr,gk,gv,gw,gu(B,C), workspace] (rwkv_kernels.cu:500-506,
+ *                          plus one trailing scratch result of wkv6_backward_workspace_bytes bytes)
+ *   wkv_forward_with_state S=1: [map,r,k,v,w,u,s | y,ys]   S=0: [r,k,v,w,u | y,ys]   (:474-488)
+ * A wrong opaque_len makes the call a no-op and records WKV6_ERR_ARG (wkv6_last_status);
+ * nothing is thrown across the boundary (the reference throws, kernel_helpers.h:56-58). */
+void wkv_forward(void *stream, void **buffers, const char *opaque, size_t opaque_len);
+void wkv_backward(void *stream, void **buffers, const char *opaque, size_t opaque_len);
+void wkv_forward_with_state(void *stream, void **buffers, const char *opaque, size_t opaque_len);
+/* Status of the calling thread's most recent custom-call target invocation. */
+int wkv6_last_status(void);
+/* hipError_t value of the calling thread's most recent failed launch (0 if none). */
+int wkv6_last_hip_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WKV6_H_ */

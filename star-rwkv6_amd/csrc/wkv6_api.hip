@@ -1,0 +1,173 @@
+// C ABI of libwkv6_gfx950.so: argument validation, algorithm choice, launch.  See include/wkv6.h.
+#include "wkv6.h"
+#include "wkv6_kernels.h"
+
+#include <string.h>
+
+namespace {
+
+thread_local int g_last_status = WKV6_OK;
+thread_local int g_last_hip_error = 0;
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+int check_shape(int dtype, int64_t B, int64_t T, int64_t C, int64_t H) {
+    if (dtype != WKV6_BF16 && dtype != WKV6_F16 && dtype != WKV6_F32) return WKV6_ERR_ARG;
+    if (B <= 0 || T <= 0 || C <= 0 || H <= 0 || C % H != 0) return WKV6_ERR_ARG;
+    if (B * H > 0x7fffffffLL || T > 0x7fffffffLL) return WKV6_ERR_ARG;
+    if (!wkv6_supports_head_size(C / H)) return WKV6_ERR_UNSUPPORTED;
+    return WKV6_OK;
+}
+
+int out_type(int dtype) { return dtype == WKV6_BF16 ? WKV6_BF16 : WKV6_F32; }
+
+int finish(hipError_t e) {
+    if (e != hipSuccess) { g_last_hip_error = (int)e; return WKV6_ERR_LAUNCH; }
+    return WKV6_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *wkv6_status_string(int s) {
+    switch (s) {
+    case WKV6_OK: return "ok";
+    case WKV6_ERR_ARG: return "invalid argument (null/misaligned pointer, bad size or dtype)";
+    case WKV6_ERR_UNSUPPORTED: return "unsupported head size (library is built for N = 64)";
+    case WKV6_ERR_WORKSPACE: return "workspace missing or too small";
+    case WKV6_ERR_LAUNCH: return "HIP launch failed";
+    default: return "unknown status";
+    }
+}
+
+int wkv6_version(void) { return 100; }
+int wkv6_supports_head_size(int64_t N) { return N == 64; }
+int wkv6_last_status(void) { return g_last_status; }
+int wkv6_last_hip_error(void) { return g_last_hip_error; }
+
+size_t wkv6_forward_workspace_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
+    (void)dtype; (void)algo; (void)B; (void)T; (void)C; (void)H;
+    return 0;
+}
+
+int wkv6_forward_with_state_ex(void *stream, int dtype, int state_dtype, int algo,
+                               int64_t B, int64_t T, int64_t C, int64_t H,
+                               int has_init_state, const int64_t *state_map,
+                               const void *r, const void *k, const void *v, const void *w, const void *u,
+                               const void *s, void *y, void *ys, void *workspace, size_t workspace_bytes) {
+    (void)workspace; (void)workspace_bytes;
+    int rc = check_shape(dtype, B, T, C, H);
+    if (rc != WKV6_OK) return rc;
+    if (!r || !k || !v || !w || !u || !y) return WKV6_ERR_ARG;
+    if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(y)) return WKV6_ERR_ARG;
+    if (has_init_state && !s) return WKV6_ERR_ARG;
+    if (state_dtype != out_type(dtype) && state_dtype != WKV6_F32) return WKV6_ERR_ARG;
+    if (algo != WKV6_ALGO_AUTO && algo != WKV6_ALGO_SCAN && algo != WKV6_ALGO_CHUNK) return WKV6_ERR_ARG;
+    hipStream_t st = (hipStream_t)stream;
+    return finish(wkv6::scan_forward(st, dtype, state_dtype, B, T, H, r, k, v, w, u,
+                                     has_init_state ? s : nullptr, has_init_state ? state_map : nullptr, y, ys));
+}
+
+int wkv6_forward_with_state(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
+                            int has_init_state, const int64_t *state_map,
+                            const void *r, const void *k, const void *v, const void *w, const void *u,
+                            const void *s, void *y, void *ys) {
+    if (!ys) return WKV6_ERR_ARG;
+    return wkv6_forward_with_state_ex(stream, dtype, out_type(dtype), WKV6_ALGO_AUTO, B, T, C, H, has_init_state,
+                                      state_map, r, k, v, w, u, s, y, ys, nullptr, 0);
+}
+
+int wkv6_forward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                    const void *r, const void *k, const void *v, const void *w, const void *u,
+                    void *y, void *workspace, size_t workspace_bytes) {
+    return wkv6_forward_with_state_ex(stream, dtype, out_type(dtype), algo, B, T, C, H, 0, nullptr,
+                                      r, k, v, w, u, nullptr, y, nullptr, workspace, workspace_bytes);
+}
+
+int wkv6_forward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
+                 const void *r, const void *k, const void *v, const void *w, const void *u, void *y) {
+    return wkv6_forward_ex(stream, dtype, WKV6_ALGO_AUTO, B, T, C, H, r, k, v, w, u, y, nullptr, 0);
+}
+
+size_t wkv6_backward_workspace_bytes_ex(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
+    (void)algo;
+    if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
+    return wkv6::scan_backward_workspace_bytes(B, T, C);
+}
+
+size_t wkv6_backward_workspace_bytes(int dtype, int64_t B, int64_t T, int64_t C, int64_t H) {
+    return wkv6_backward_workspace_bytes_ex(dtype, WKV6_ALGO_AUTO, B, T, C, H);
+}
+
+int wkv6_backward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                     const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                     void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, size_t workspace_bytes) {
+    int rc = check_shape(dtype, B, T, C, H);
+    if (rc != WKV6_OK) return rc;
+    if (!r || !k || !v || !w || !u || !gy || !gr || !gk || !gv || !gw || !gu) return WKV6_ERR_ARG;
+    if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(gy) || !aligned16(gr) ||
+        !aligned16(gk) || !aligned16(gv) || !aligned16(gw)) return WKV6_ERR_ARG;
+    if (algo != WKV6_ALGO_AUTO && algo != WKV6_ALGO_SCAN && algo != WKV6_ALGO_CHUNK) return WKV6_ERR_ARG;
+    const size_t need = wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H);
+    if (need > 0 && (!workspace || workspace_bytes < need || !aligned16(workspace))) return WKV6_ERR_WORKSPACE;
+    hipStream_t st = (hipStream_t)stream;
+    return finish(wkv6::scan_backward(st, dtype, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace));
+}
+
+int wkv6_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
+                  const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                  void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, size_t workspace_bytes) {
+    return wkv6_backward_ex(stream, dtype, WKV6_ALGO_AUTO, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu,
+                            workspace, workspace_bytes);
+}
+
+// ---- XLA custom-call surface ------------------------------------------------------------
+
+size_t wkv6_create_descriptor(int B, int T, int C, int H, int S, int x_type, int y_type, void *out) {
+    static_assert(sizeof(wkv6_descriptor) == 28, "descriptor must stay 28 bytes");
+    wkv6_descriptor d;
+    memset(&d, 0, sizeof d);
+    d.B = B; d.T = T; d.C = C; d.H = H; d.S = S ? 1 : 0; d.x_type = x_type; d.y_type = y_type;
+    if (out) memcpy(out, &d, sizeof d);
+    return sizeof d;
+}
+
+static bool unpack(const char *opaque, size_t len, wkv6_descriptor *d) {
+    if (!opaque || len != sizeof(wkv6_descriptor)) { g_last_status = WKV6_ERR_ARG; return false; }
+    memcpy(d, opaque, sizeof *d);
+    if (d->y_type != out_type(d->x_type)) { g_last_status = WKV6_ERR_ARG; return false; }
+    return true;
+}
+
+void wkv_forward(void *stream, void **buffers, const char *opaque, size_t opaque_len) {
+    wkv6_descriptor d;
+    if (!unpack(opaque, opaque_len, &d) || !buffers) { g_last_status = WKV6_ERR_ARG; return; }
+    g_last_status = wkv6_forward(stream, d.x_type, d.B, d.T, d.C, d.H, buffers[0], buffers[1], buffers[2],
+                                 buffers[3], buffers[4], buffers[5]);
+}
+
+void wkv_backward(void *stream, void **buffers, const char *opaque, size_t opaque_len) {
+    wkv6_descriptor d;
+    if (!unpack(opaque, opaque_len, &d) || !buffers) { g_last_status = WKV6_ERR_ARG; return; }
+    g_last_status = wkv6_backward(stream, d.x_type, d.B, d.T, d.C, d.H, buffers[0], buffers[1], buffers[2],
+                                  buffers[3], buffers[4], buffers[5], buffers[6], buffers[7], buffers[8],
+                                  buffers[9], buffers[10], buffers[11],
+                                  wkv6_backward_workspace_bytes(d.x_type, d.B, d.T, d.C, d.H));
+}
+
+void wkv_forward_with_state(void *stream, void **buffers, const char *opaque, size_t opaque_len) {
+    wkv6_descriptor d;
+    if (!unpack(opaque, opaque_len, &d) || !buffers) { g_last_status = WKV6_ERR_ARG; return; }
+    if (d.S) {
+        g_last_status = wkv6_forward_with_state(stream, d.x_type, d.B, d.T, d.C, d.H, 1,
+                                                (const int64_t *)buffers[0], buffers[1], buffers[2], buffers[3],
+                                                buffers[4], buffers[5], buffers[6], buffers[7], buffers[8]);
+    } else {
+        g_last_status = wkv6_forward_with_state(stream, d.x_type, d.B, d.T, d.C, d.H, 0, nullptr, buffers[0],
+                                                buffers[1], buffers[2], buffers[3], buffers[4], nullptr,
+                                                buffers[5], buffers[6]);
+    }
+}
+
+}  // extern "C"

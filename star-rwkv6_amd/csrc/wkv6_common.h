@@ -1,0 +1,80 @@
+// Shared device helpers for the WKV6 kernels (gfx950 only, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace wkv6 {
+
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+constexpr int kN = 64;  // head size the kernels are built for
+
+__device__ __forceinline__ float fast_exp(float x) { return __expf(x); }
+// decay d = exp(-exp(w)); w = -1e9 gives exactly 1, w >= ~5 gives exactly 0, never NaN for finite w.
+__device__ __forceinline__ float decay_from_raw(float w) { return __expf(-__expf(w)); }
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t hi16) { return __uint_as_float(hi16 << 16); }
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
+    uint32_t x = __float_as_uint(f);
+    if ((x & 0x7fffffffu) > 0x7f800000u) return (x >> 16) | 0x40u;  // NaN stays NaN
+    return (x + 0x7fffu + ((x >> 16) & 1u)) >> 16;                   // round to nearest even
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    return float_to_bf16_bits(lo) | (float_to_bf16_bits(hi) << 16);
+}
+
+// Eight consecutive elements as they sit in memory; converted to fp32 only when consumed, so a
+// prefetch held across a compute phase costs 4 VGPRs for 16-bit types.
+template <typename T> struct Raw8;
+template <> struct Raw8<float> {
+    float4 a, b;
+    __device__ __forceinline__ void load(const float *p) {
+        a = *reinterpret_cast<const float4 *>(p);
+        b = *reinterpret_cast<const float4 *>(p + 4);
+    }
+    __device__ __forceinline__ void zero() { a = make_float4(0, 0, 0, 0); b = a; }
+    __device__ __forceinline__ void to_float(float (&o)[8]) const {
+        o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+    }
+};
+template <> struct Raw8<bf16_t> {
+    uint4 a;
+    __device__ __forceinline__ void load(const bf16_t *p) { a = *reinterpret_cast<const uint4 *>(p); }
+    __device__ __forceinline__ void zero() { a = make_uint4(0, 0, 0, 0); }
+    __device__ __forceinline__ void to_float(float (&o)[8]) const {
+        o[0] = __uint_as_float(a.x << 16); o[1] = __uint_as_float(a.x & 0xffff0000u);
+        o[2] = __uint_as_float(a.y << 16); o[3] = __uint_as_float(a.y & 0xffff0000u);
+        o[4] = __uint_as_float(a.z << 16); o[5] = __uint_as_float(a.z & 0xffff0000u);
+        o[6] = __uint_as_float(a.w << 16); o[7] = __uint_as_float(a.w & 0xffff0000u);
+    }
+};
+template <> struct Raw8<f16_t> {
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    h8 a;
+    __device__ __forceinline__ void load(const f16_t *p) { a = *reinterpret_cast<const h8 *>(p); }
+    __device__ __forceinline__ void zero() { a = (h8)(0); }
+    __device__ __forceinline__ void to_float(float (&o)[8]) const {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = (float)a[i];
+    }
+};
+
+// Store n (4 or 8) consecutive fp32 values as the output type, one vector store.
+__device__ __forceinline__ void store4(float *p, float a, float b, float c, float d) {
+    *reinterpret_cast<float4 *>(p) = make_float4(a, b, c, d);
+}
+__device__ __forceinline__ void store4(bf16_t *p, float a, float b, float c, float d) {
+    *reinterpret_cast<uint2 *>(p) = make_uint2(pack_bf16x2(a, b), pack_bf16x2(c, d));
+}
+__device__ __forceinline__ void store1(float *p, float a) { *p = a; }
+__device__ __forceinline__ void store1(bf16_t *p, float a) {
+    *reinterpret_cast<uint16_t *>(p) = (uint16_t)float_to_bf16_bits(a);
+}
+__device__ __forceinline__ float load1(const float *p) { return *p; }
+__device__ __forceinline__ float load1(const bf16_t *p) {
+    return bf16_bits_to_float(*reinterpret_cast<const uint16_t *>(p));
+}
+__device__ __forceinline__ float load1(const f16_t *p) { return (float)*p; }
+
+}  // namespace wkv6

@@ -1,0 +1,20 @@
+// Host-side launchers of the WKV6 kernels (internal to the library; the public ABI is include/wkv6.h).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace wkv6 {
+
+enum { kBF16 = 0, kF16 = 1, kF32 = 2 };  // same numbering as the public header
+
+// --- per-timestep recurrence (wkv6_scan.hip) ---
+hipError_t scan_forward(hipStream_t st, int dtype, int state_dtype, int64_t B, int64_t T, int64_t H,
+                        const void *r, const void *k, const void *v, const void *w, const void *u,
+                        const void *s0, const int64_t *map, void *y, void *sT);
+size_t scan_backward_workspace_bytes(int64_t B, int64_t T, int64_t C);
+hipError_t scan_backward(hipStream_t st, int dtype, int64_t B, int64_t T, int64_t H,
+                         const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                         void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace);
+
+}  // namespace wkv6

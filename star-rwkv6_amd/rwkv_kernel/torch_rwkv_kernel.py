@@ -1,0 +1,171 @@
+"""torch flavour of the WKV6 operator: autograd.Function over libwkv6_gfx950.so.
+
+Mirrors rwkv_kernel/torch_rwkv_kernel.py of the reference (constructor, call signature, argument
+checks, 2-tuple return, dtype rules) but binds the library through its C ABI with ctypes instead
+of JIT-building a torch C++ extension, and launches on torch's CURRENT stream.
+
+Where the reference's torch flavour is broken as committed, the behaviour of its working
+flavours is implemented: the default state_map for a single shared state has length batch
+(ops_rwkv_kernal.py:54, against torch_rwkv_kernel.py:155), the stateful call actually runs
+(torch_rwkv_kernel.py:93 names a binding that does not exist), and state_map is moved to the
+device before the kernel reads it.
+"""
+import torch
+
+from . import _native
+
+_DTYPE_CODE = {torch.bfloat16: _native.BF16, torch.float16: _native.F16, torch.float32: _native.F32}
+
+
+def _out_dtype(dt):
+    # rwkv_kernel/torch_rwkv_kernel.py:35 -- float16 inputs produce float32 outputs
+    return torch.float32 if dt == torch.float16 else dt
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+class _WKV6(torch.autograd.Function):
+    """Stateless operator with gradients (rwkv_kernel/torch_rwkv_kernel.py:14-75)."""
+
+    @staticmethod
+    def forward(ctx, B, T, C, H, r, k, v, w, u, algo):
+        lib = _native.load()
+        with torch.no_grad():
+            assert r.dtype == k.dtype == v.dtype == w.dtype == u.dtype
+            assert r.dtype in _DTYPE_CODE
+            for x in (r, k, v, w, u):
+                assert x.is_contiguous()
+            ctx.dims = (B, T, C, H)
+            ctx.algo = algo
+            ctx.save_for_backward(r, k, v, w, u)
+            y = torch.empty((B, T, C), device=r.device, dtype=_out_dtype(r.dtype))
+            with torch.cuda.device(r.device):
+                ws_bytes = lib.wkv6_forward_workspace_bytes(_DTYPE_CODE[r.dtype], algo, B, T, C, H)
+                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=r.device) if ws_bytes else None
+                _native.check(lib.wkv6_forward_ex(_stream(), _DTYPE_CODE[r.dtype], algo, B, T, C, H,
+                                                  _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(y),
+                                                  _ptr(ws), ws_bytes))
+            return y
+
+    @staticmethod
+    def backward(ctx, gy):
+        lib = _native.load()
+        assert gy.is_cuda
+        with torch.no_grad():
+            B, T, C, H = ctx.dims
+            r, k, v, w, u = ctx.saved_tensors
+            odt = _out_dtype(r.dtype)
+            assert gy.dtype in (torch.bfloat16, torch.float32) and gy.dtype == odt
+            gy = gy.contiguous()
+            gr, gk, gv, gw = (torch.empty((B, T, C), device=gy.device, dtype=odt) for _ in range(4))
+            gu = torch.empty((B, C), device=gy.device, dtype=odt)
+            code = _DTYPE_CODE[r.dtype]
+            with torch.cuda.device(gy.device):
+                ws_bytes = lib.wkv6_backward_workspace_bytes_ex(code, ctx.algo, B, T, C, H)
+                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=gy.device) if ws_bytes else None
+                _native.check(lib.wkv6_backward_ex(_stream(), code, ctx.algo, B, T, C, H,
+                                                   _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(gy),
+                                                   _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu),
+                                                   _ptr(ws), ws_bytes))
+            # per-batch partials -> (H, N), rwkv_kernel/torch_rwkv_kernel.py:73
+            gu = torch.sum(gu, 0).reshape(u.shape)
+            return (None, None, None, None, gr, gk, gv, gw, gu, None)
+
+
+def _forward_with_state(B, T, C, H, state_map, r, k, v, w, u, init_state, algo=_native.ALGO_AUTO):
+    """Stateful forward, no gradient (rwkv_kernel/torch_rwkv_kernel.py:76-95)."""
+    lib = _native.load()
+    with torch.no_grad():
+        assert (init_state is None and state_map is None) or (init_state is not None and state_map is not None), \
+            "init_state and state_map go together"
+        assert state_map is None or state_map.dtype == torch.int64
+        odt = _out_dtype(r.dtype)
+        sdt = init_state.dtype if init_state is not None else odt
+        N = C // H
+        y = torch.empty((B, T, C), device=r.device, dtype=odt)
+        ys = torch.empty((B, H, N, N), device=r.device, dtype=sdt)
+        with torch.cuda.device(r.device):
+            _native.check(lib.wkv6_forward_with_state_ex(
+                _stream(), _DTYPE_CODE[r.dtype], _DTYPE_CODE[sdt], algo, B, T, C, H,
+                int(init_state is not None), _ptr(state_map),
+                _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(init_state), _ptr(y), _ptr(ys), None, 0))
+    return y, ys
+
+
+class RWKVKernelOperator:
+    def __init__(self, head_size, max_sequence_length):
+        lib = _native.load()
+        assert isinstance(head_size, int) and isinstance(max_sequence_length, int)
+        assert head_size > 0 and max_sequence_length > 0
+        assert head_size % 4 == 0, "head_size must be a multiple of 4"
+        if not lib.wkv6_supports_head_size(head_size):
+            raise _native.WKV6Error("libwkv6_gfx950 is built for head_size 64, got %d" % head_size)
+        self.head_size = head_size
+        # the reference bakes this into a per-thread array bound (-D_T_); nothing here is sized by
+        # it, so longer sequences simply work
+        self.max_sequence_length = max_sequence_length
+        self.algo = _native.ALGO_AUTO
+        self.normal_kernenl = _WKV6
+        self.kernel_with_state = _forward_with_state
+
+    def __call__(self, r, k, v, w, u, return_state=False, init_state=None, state_map=None):
+        B, T, C = r.shape
+        N = self.head_size
+        assert C % N == 0
+        H = C // N
+        if not isinstance(u, torch.Tensor):
+            u = u.value
+
+        for x in (r, k, v, w, u):
+            assert x.is_cuda
+        assert r.device == k.device == v.device == w.device == u.device
+        assert r.dtype == k.dtype == v.dtype == w.dtype == u.dtype
+        assert r.shape == k.shape == v.shape == w.shape
+        assert u.numel() == C, "u must hold one value per channel"
+
+        if init_state is not None:
+            assert init_state.dim() in (3, 4), \
+                "init_state must be (state_kinds <= batch, H, N, N) or (H, N, N)"
+            if init_state.dim() == 3:
+                init_state = init_state[None, :]
+            assert tuple(init_state.shape[1:]) == (H, N, N) and init_state.shape[0] <= B, \
+                "init_state must be (state_kinds <= batch, H, N, N) or (H, N, N)"
+            s_dtype = _out_dtype(r.dtype)
+            assert init_state.dtype in (s_dtype, torch.float32), "init_state dtype must be %s" % s_dtype
+            assert init_state.device == r.device
+
+        if state_map is not None:
+            if isinstance(state_map, (list, tuple)):
+                state_map = torch.tensor(state_map, dtype=torch.int64)
+            elif isinstance(state_map, torch.Tensor):
+                assert state_map.dtype in (torch.int32, torch.int64), "state_map must be int32/int64 of shape (batch,)"
+                state_map = state_map.to(torch.int64)
+            assert tuple(state_map.shape) == (B,), "state_map must have shape (batch,)"
+
+        if return_state:
+            if init_state is None:
+                assert state_map is None, "state_map needs init_state"
+            else:
+                n_state = init_state.shape[0]
+                if state_map is None:
+                    assert n_state == 1 or n_state == B, "cannot infer state_map; pass it explicitly"
+                    if n_state == 1:
+                        state_map = torch.zeros(B, dtype=torch.int64)
+                    else:
+                        state_map = torch.arange(B, dtype=torch.int64)
+                else:
+                    assert bool((state_map >= 0).all()) and bool((state_map < n_state).all()), \
+                        "state_map values must lie in [0, %d)" % n_state
+                state_map = state_map.to(r.device).contiguous()
+                init_state = init_state.contiguous()
+            for x in (r, k, v, w, u):
+                assert x.is_contiguous()
+            return _forward_with_state(B, T, C, H, state_map, r, k, v, w, u, init_state, self.algo)
+        o = _WKV6.apply(B, T, C, H, r, k, v, w, u, self.algo)
+        return o, None

@@ -1,0 +1,215 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the float64 CPU oracle on
+the same seeded (and identically rounded) inputs.  Run on the MI355X box with -m gpu."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from _util import cast_inputs, check_close, out_dtype, to_np
+
+pytestmark = pytest.mark.gpu
+
+SCAN, CHUNK = 1, 2
+DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+
+
+@pytest.fixture(scope="module")
+def op():
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    import rwkv_kernel
+
+    return rwkv_kernel.RWKVKernelOperator(64, 4096)
+
+
+def _run_fwd_bwd(op, dev, algo):
+    op.algo = algo
+    leaves = [x.clone().requires_grad_(True) for x in dev[:5]]
+    y, none = op(*leaves)
+    assert none is None
+    y.backward(dev[5])
+    torch.cuda.synchronize()
+    return y, [x.grad for x in leaves]
+
+
+def _case(op, oracle, B, T, H, seed, dtype, algo, strict=False):
+    N = 64
+    print("case B=%d T=%d H=%d seed=%d dtype=%s algo=%d" % (B, T, H, seed, dtype, algo), flush=True)
+    ins = oracle.make_inputs(B, T, H, N, seed)
+    odt = out_dtype(dtype)
+    dev, ref = cast_inputs(ins[:5], dtype)
+    gy_dev, gy_ref = cast_inputs(ins[5:6], odt)
+    y, grads = _run_fwd_bwd(op, dev + gy_dev, algo)
+    assert y.dtype == odt and all(g.dtype == dtype for g in grads)
+    y_ref, _ = oracle.forward_c(*ref, N)
+    g_ref = oracle.backward_c(*ref, gy_ref[0], N)
+    if strict:
+        assert np.abs(to_np(y) - y_ref).max() <= 1e-4
+    check_close("y", y, y_ref, odt)
+    for name, g, gr in zip("gr gk gv gw gu".split(), grads, g_ref):
+        check_close(name, to_np(g).reshape(gr.shape), gr, odt, is_grad=True)
+    return y, grads
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_config1_forward_fp32(op, oracle, seed):
+    # BASELINE config 1: fp32, B=2 T=128 H=4 N=64; max-abs(y) <= 1e-4
+    _case(op, oracle, 2, 128, 4, seed, torch.float32, SCAN, strict=True)
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("T", [1, 2, 15, 16, 17, 33, 100])
+def test_scan_fwd_bwd_ragged_T(op, oracle, dt, T):
+    _case(op, oracle, 2, T, 2, 10 + T, DTYPES[dt], SCAN)
+
+
+def test_scan_longer_sequence_bf16(op, oracle):
+    _case(op, oracle, 1, 1024, 2, 5, torch.bfloat16, SCAN)
+
+
+def test_scan_longer_sequence_f32(op, oracle):
+    _case(op, oracle, 1, 1024, 2, 6, torch.float32, SCAN)
+
+
+def test_constant_inputs_closed_form(op):
+    # reference test_jax.py:12-16: r=k=v=u=1, w=-4 -> y_t = 64*(1 + (1-d^t)/(1-d))
+    B, T, C = 4, 512, 512
+    one = torch.ones(B, T, C, device="cuda")
+    y, _ = op(one, one, one, one * 0 - 4, torch.ones(C, device="cuda"))
+    d = np.exp(-np.exp(-4.0))
+    expect = 64 * (1 + (1 - d ** np.arange(T)) / (1 - d))
+    got = to_np(y)
+    assert got[0, 0, 0] == 64.0 and got[0, 1, 0] == 128.0
+    np.testing.assert_allclose(got[2, :, 77], expect, rtol=2e-5)
+
+
+def test_padding_decay_value_is_finite(op, oracle):
+    # rwkv6_model.py:149-152 masks tokens with k=0, w=-1e9 (decay exactly 1)
+    B, T, H = 1, 40, 1
+    ins = oracle.make_inputs(B, T, H, 64, 3)
+    ins[3][:, 10:20] = -1e9
+    ins[1][:, 10:20] = 0
+    ins[3][:, 30] = 20.0  # decay exactly 0
+    dev, ref = cast_inputs(ins[:5], torch.float32)
+    gy_dev, gy_ref = cast_inputs(ins[5:6], torch.float32)
+    y, grads = _run_fwd_bwd(op, dev + gy_dev, SCAN)
+    check_close("y", y, oracle.forward_c(*ref, 64)[0], torch.float32)
+    for name, g, gr in zip("gr gk gv gw gu".split(), grads, oracle.backward_c(*ref, gy_ref[0], 64)):
+        check_close(name, to_np(g).reshape(gr.shape), gr, torch.float32, is_grad=True)
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
+def test_state_in_out(op, oracle, dt):
+    dtype = DTYPES[dt]
+    odt = out_dtype(dtype)
+    B, T, H, N = 3, 37, 2, 64
+    ins = oracle.make_inputs(B, T, H, N, 21, with_state=True)
+    dev, ref = cast_inputs(ins[:5], dtype)
+    s_dev, s_ref = cast_inputs([ins[6][:2]], odt)
+    smap = [1, 0, 1]
+    y, sT = op(*dev, return_state=True, init_state=s_dev[0], state_map=smap)
+    torch.cuda.synchronize()
+    assert sT.shape == (B, H, N, N) and sT.dtype == odt and y.dtype == odt
+    y_ref, sT_ref = oracle.forward_c(*ref, N, s_ref[0], smap)
+    check_close("y", y, y_ref, odt)
+    check_close("sT", sT, sT_ref, odt)
+    # zero-state stateful call equals the stateless call
+    y0, s0T = op(*dev, return_state=True)
+    y1, none = op(*dev)
+    assert none is None and torch.equal(y0, y1)
+    check_close("sT0", s0T, oracle.forward_c(*ref, N)[1], odt)
+    # shared single state: default map is all zeros; (H,N,N) accepted
+    y2, _ = op(*dev, return_state=True, init_state=s_dev[0][0])
+    check_close("y_shared", y2, oracle.forward_c(*ref, N, s_ref[0][:1], [0] * B)[0], odt)
+
+
+def test_state_split_consistency_fp32(op, oracle):
+    # op(T1+T2) == op(T1) -> op(T2, init_state): bit-identical in fp32 state
+    B, T, H, N = 2, 96, 2, 64
+    ins = oracle.make_inputs(B, T, H, N, 22)
+    dev, _ = cast_inputs(ins[:5], torch.float32)
+    y, sT = op(*dev, return_state=True)
+    cut = 41
+    a = [x[:, :cut].contiguous() for x in dev[:4]] + [dev[4]]
+    b = [x[:, cut:].contiguous() for x in dev[:4]] + [dev[4]]
+    ya, sa = op(*a, return_state=True)
+    yb, sb = op(*b, return_state=True, init_state=sa)
+    assert torch.equal(torch.cat([ya, yb], 1), y)
+    assert torch.equal(sb, sT)
+
+
+def test_bf16_activations_with_fp32_state(op, oracle):
+    B, T, H, N = 2, 20, 1, 64
+    ins = oracle.make_inputs(B, T, H, N, 23, with_state=True)
+    dev, ref = cast_inputs(ins[:5], torch.bfloat16)
+    s32 = ins[6].cuda()
+    y, sT = op(*dev, return_state=True, init_state=s32)
+    assert sT.dtype == torch.float32 and y.dtype == torch.bfloat16
+    y_ref, sT_ref = oracle.forward_c(*ref, N, to_np(s32))
+    check_close("y", y, y_ref, torch.bfloat16)
+    assert np.abs(to_np(sT) - sT_ref).max() <= 1e-4 * max(1, np.abs(sT_ref).max())
+
+
+def test_golden_fixture(op):
+    import os
+
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "wkv6_small.npz"))
+    t = {n: torch.from_numpy(z[n]).cuda() for n in "r k v w u gy s0".split()}
+    op.algo = SCAN
+    leaves = [t[n].clone().requires_grad_(True) for n in "r k v w u".split()]
+    y, _ = op(*leaves)
+    y.backward(t["gy"])
+    check_close("y", y, z["y"], torch.float32)
+    for n, leaf in zip("gr gk gv gw gu".split(), leaves):
+        check_close(n, leaf.grad, z[n], torch.float32, is_grad=True)
+    ys, sT = op(*[t[n] for n in "r k v w u".split()], return_state=True, init_state=t["s0"],
+                state_map=torch.from_numpy(z["state_map"]))
+    check_close("y_state", ys, z["y_state"], torch.float32)
+    check_close("sT", sT, z["sT"], torch.float32)
+
+
+def test_xla_custom_call_targets(op, oracle):
+    # the three status-less custom-call entry points with the 28-byte descriptor
+    from rwkv_kernel import _native
+
+    lib = _native.load()
+    B, T, H, N = 2, 19, 1, 64
+    C = H * N
+    ins = oracle.make_inputs(B, T, H, N, 31, with_state=True)
+    dev, ref = cast_inputs(ins[:5], torch.float32)
+    gy = ins[5].cuda()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def call(fn, bufs, desc):
+        arr = (ctypes.c_void_p * len(bufs))(*[b.data_ptr() for b in bufs])
+        fn(stream, arr, desc, len(desc))
+        torch.cuda.synchronize()
+        assert lib.wkv6_last_status() == 0
+
+    y = torch.empty(B, T, C, device="cuda")
+    call(lib.wkv_forward, dev + [y], _native.create_descriptor(B, T, C, H, False, _native.F32, _native.F32))
+    y_ref, _ = oracle.forward_c(*ref, N)
+    check_close("y", y, y_ref, torch.float32)
+
+    outs = [torch.empty(B, T, C, device="cuda") for _ in range(4)] + [torch.empty(B, C, device="cuda")]
+    ws = torch.empty(lib.wkv6_backward_workspace_bytes(_native.F32, B, T, C, H), dtype=torch.uint8, device="cuda")
+    call(lib.wkv_backward, dev + [gy] + outs + [ws], _native.create_descriptor(B, T, C, H, False, _native.F32, _native.F32))
+    g_ref = oracle.backward_c(*ref, to_np(gy), N)
+    for name, g, gr in zip("gr gk gv gw".split(), outs, g_ref):
+        check_close(name, g, gr, torch.float32, is_grad=True)
+    check_close("gu", to_np(outs[4]).sum(0).reshape(H, N), g_ref[4], torch.float32, is_grad=True)
+
+    s0 = ins[6].cuda()
+    smap = torch.tensor([1, 0], device="cuda")
+    ys = torch.empty(B, H, N, N, device="cuda")
+    call(lib.wkv_forward_with_state, [smap] + dev + [s0, y, ys],
+         _native.create_descriptor(B, T, C, H, True, _native.F32, _native.F32))
+    y_ref, s_ref = oracle.forward_c(*ref, N, to_np(s0), [1, 0])
+    check_close("y", y, y_ref, torch.float32)
+    check_close("ys", ys, s_ref, torch.float32)
+    call(lib.wkv_forward_with_state, dev + [y, ys], _native.create_descriptor(B, T, C, H, False, _native.F32, _native.F32))
+    check_close("ys0", ys, oracle.forward_c(*ref, N)[1], torch.float32)
+    # wrong opaque length: no-op + error status, nothing thrown
+    arr = (ctypes.c_void_p * 6)(*[b.data_ptr() for b in dev + [y]])
+    lib.wkv_forward(stream, arr, b"x" * 27, 27)
+    assert lib.wkv6_last_status() == 1
