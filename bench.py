@@ -1,0 +1,184 @@
+#!/usr/bin/env python3
+"""WKV6 forward+backward throughput on one MI355X, with roofline and CPU baseline.
+
+One "step" = one forward + one backward of the WKV6 operator over one batch of synthetic input
+at the RWKV6-1.6B layer shape (B=8, T=1024, C=2048, H=32, N=64, bf16 I/O, fp32 state), inputs
+resident in HBM, outputs and workspace pre-allocated, called through the C ABI of
+libwkv6_gfx950.so on torch's current stream, gu batch-sum included.
+
+Prints ONE JSON line.  `--gpus N` with N > 1 is refused: this operator has no cross-GPU part
+(every (batch, head) pair is independent), and this build measures a single GPU.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "star-rwkv6_amd"))
+os.environ.setdefault("KERAS_BACKEND", "torch")
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+WORKLOADS = {
+    # name: (B, T, H, dtype)
+    "c2": (8, 1024, 32, "bf16"),   # RWKV6-1.6B layer shape: the configuration the metric is quoted on
+    "c3": (4, 4096, 64, "bf16"),   # RWKV6-7B layer shape
+    "c1": (2, 128, 4, "f32"),
+}
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (separate runs), scaled
+# by the same counters' reading for a device-to-device copy of known size; see profiles/.
+# Keyed by (workload, algo, "fwd"|"bwd").  None = not measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--algo", default="auto", choices=["auto", "scan", "chunk"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-tokens", type=int, default=0, help="tokens in the CPU baseline sample (0 = default)")
+    ap.add_argument("--seed", type=int, default=0)
+    return ap.parse_args()
+
+
+def cpu_baseline(B, T_full, H, N, seed, tokens):
+    """The reference's python loop (restated in oracle/wkv6_ref.py) forward + autograd backward,
+    fp32, all host cores, on a bounded sample: same B, C and input distributions, fewer
+    timesteps (cost is linear in T)."""
+    import torch
+    from oracle import wkv6_ref
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    Ts = max(8, min(T_full, (tokens or 1024) // B))
+    r, k, v, w, u, gy = wkv6_ref.make_inputs(B, Ts, H, N, seed)
+    t0 = time.perf_counter()
+    leaves = [x.clone().requires_grad_(True) for x in (r, k, v, w, u)]
+    y, _ = wkv6_ref.loop_torch(*leaves, N)
+    y.backward(gy)
+    dt = time.perf_counter() - t0
+    return {
+        "value": B * Ts / dt / 1e6, "unit": "Mtokens/s", "cores": cores, "kind": "port",
+        "sample": "python-loop WKV6 fwd+bwd via torch.autograd, fp32, B=%d T=%d of %d C=%d (%.1f s)" % (
+            B, Ts, T_full, H * N, dt),
+    }
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py: this build measures ONE GPU; --gpus %d is not supported "
+              "(the operator needs no cross-GPU exchange; see DESIGN.md)" % a.gpus, file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from oracle import wkv6_ref
+    from rwkv_kernel import _native
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    lib = _native.load()
+    B, T, H, dt_name = WORKLOADS[a.workload]
+    N = 64
+    C = H * N
+    dtype = {"bf16": torch.bfloat16, "f32": torch.float32}[dt_name]
+    code = {"bf16": _native.BF16, "f32": _native.F32}[dt_name]
+    es = 2 if dt_name == "bf16" else 4
+    algo = {"auto": _native.ALGO_AUTO, "scan": _native.ALGO_SCAN, "chunk": _native.ALGO_CHUNK}[a.algo]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    r, k, v, w, u, gy = (x.to(dtype).to(dev).contiguous() for x in wkv6_ref.make_inputs(B, T, H, N, a.seed))
+    y = torch.empty(B, T, C, dtype=dtype, device=dev)
+    gr, gk, gv, gw = (torch.empty(B, T, C, dtype=dtype, device=dev) for _ in range(4))
+    gu_part = torch.empty(B, C, dtype=dtype, device=dev)
+    fws_bytes = lib.wkv6_forward_workspace_bytes(code, algo, B, T, C, H)
+    bws_bytes = lib.wkv6_backward_workspace_bytes_ex(code, algo, B, T, C, H)
+    fws = torch.empty(max(fws_bytes, 16), dtype=torch.uint8, device=dev)
+    bws = torch.empty(max(bws_bytes, 16), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    P = lambda t: t.data_ptr()
+
+    def fwd():
+        _native.check(lib.wkv6_forward_ex(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(y),
+                                          P(fws), fws_bytes))
+
+    def bwd():
+        _native.check(lib.wkv6_backward_ex(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy),
+                                           P(gr), P(gk), P(gv), P(gw), P(gu_part), P(bws), bws_bytes))
+        return torch.sum(gu_part, 0)
+
+    for _ in range(a.warmup):
+        fwd(); bwd()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        fwd(); bwd()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / a.steps * 1e3
+    tokens = B * T
+
+    # per-call GPU durations with events on the launch stream (torch's current stream)
+    def gpu_ms(fn, reps):
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
+        for s, e in ev:
+            s.record(); fn(); e.record()
+        torch.cuda.synchronize()
+        ts = sorted(s.elapsed_time(e) for s, e in ev)
+        return sum(ts) / len(ts), ts[len(ts) // 2]
+
+    reps = max(10, min(a.steps, 50))
+    f_avg, f_med = gpu_ms(fwd, reps)
+    b_avg, b_med = gpu_ms(bwd, reps)
+
+    # stream-copy bandwidth actually reachable on this box (read + write of a 1 GiB buffer)
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    c_avg, _ = gpu_ms(lambda: dst.copy_(src), 10)
+    copy_gbs = 2 * src.numel() / (c_avg * 1e-3) / 1e9
+    del src, dst
+
+    bytes_fwd = 5 * B * T * C * es + C * es
+    bytes_bwd = 9 * B * T * C * es + 2 * C * es
+    bytes_step = bytes_fwd + bytes_bwd
+    dom = "bwd" if b_avg >= f_avg else "fwd"
+    dom_bytes, dom_ms = (bytes_bwd, b_avg) if dom == "bwd" else (bytes_fwd, f_avg)
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    step_gbs = bytes_step / (ms_per_step * 1e-3) / 1e9
+    algo_used = a.algo
+
+    out = {
+        "metric": "WKV6 fwd+bwd Mtokens/s + % HBM roofline, B8 T1024 C2048 H32 bf16",
+        "value": tokens / (ms_per_step * 1e-3) / 1e6,
+        "unit": "Mtokens/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dt_name, "data": "synthetic",
+        "config": {"workload": "%s: WKV6 fwd+bwd B=%d T=%d C=%d H=%d N=%d %s I/O fp32 state" % (
+            a.workload, B, T, C, H, N, dt_name), "algo": algo_used, "tokens_per_step": tokens},
+        "roofline": {
+            "bound": "hbm", "kernel": "wkv6_%s (%s)" % ("backward" if dom == "bwd" else "forward", algo_used),
+            "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+            "traffic": MEASURED_TRAFFIC_BYTES.get((a.workload, algo_used, dom)),
+            "algorithmic_bytes": dom_bytes, "avg_ms": dom_ms,
+        },
+        "fwd_bwd": {
+            "algorithmic_bytes": bytes_step, "achieved_GBps": step_gbs, "frac_of_hbm_peak": step_gbs / HBM_PEAK_GBS,
+            "frac_of_measured_copy": step_gbs / copy_gbs, "measured_copy_GBps": copy_gbs,
+            "fwd_ms_avg": f_avg, "fwd_ms_median": f_med, "bwd_ms_avg": b_avg, "bwd_ms_median": b_med,
+            "fwd_GBps": bytes_fwd / (f_avg * 1e-3) / 1e9, "bwd_GBps": bytes_bwd / (b_avg * 1e-3) / 1e9,
+        },
+    }
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(B, T, H, N, a.seed, a.cpu_tokens)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

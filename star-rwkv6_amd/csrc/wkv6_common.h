@@ -20,8 +20,12 @@ __device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
     if ((x & 0x7fffffffu) > 0x7f800000u) return (x >> 16) | 0x40u;  // NaN stays NaN
     return (x + 0x7fffu + ((x >> 16) & 1u)) >> 16;                   // round to nearest even
 }
+// two fp32 -> packed bf16x2, round to nearest even (one v_cvt_pk_bf16_f32 on gfx950)
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-    return float_to_bf16_bits(lo) | (float_to_bf16_bits(hi) << 16);
+    typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+    const f32x2_t t = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(t, bf16x2_t));
 }
 
 // Eight consecutive elements as they sit in memory; converted to fp32 only when consumed, so a

@@ -41,12 +41,13 @@ __global__ __launch_bounds__(256) void scan_fwd_kernel(int T, int H,
         const Tin *__restrict__ r, const Tin *__restrict__ k, const Tin *__restrict__ v,
         const Tin *__restrict__ w, const Tin *__restrict__ u,
         const Ts *__restrict__ s0, const int64_t *__restrict__ map,
-        Tout *__restrict__ y, Ts *__restrict__ sT)
+        Tout *__restrict__ y, Ts *__restrict__ sT, Gate gate)
 {
     __shared__ __align__(16) float s_r[TC][kN], s_k[TC][kN], s_d[TC][kN], s_v[TC][kN];
     __shared__ __align__(16) float s_part[4][TC][kN];
     __shared__ float s_ruk[TC];
     __shared__ float s_u[kN];
+    if (gate.closed()) return;
 
     const int b = blockIdx.x / H, h = blockIdx.x % H;
     const int tid = threadIdx.x, lane = tid & 63, q = tid >> 6;
@@ -156,12 +157,13 @@ template <typename Tin, typename Tout>
 __global__ __launch_bounds__(256) void scan_bwd_a_kernel(int T, int H,
         const Tin *__restrict__ r, const Tin *__restrict__ k, const Tin *__restrict__ v,
         const Tin *__restrict__ w, const Tin *__restrict__ u, const Tout *__restrict__ gy,
-        Tout *__restrict__ gr, Tout *__restrict__ gu, float *__restrict__ wsP)
+        Tout *__restrict__ gr, Tout *__restrict__ gu, float *__restrict__ wsP, Gate gate)
 {
     __shared__ __align__(16) float s_r[TC][kN], s_k[TC][kN], s_d[TC][kN], s_v[TC][kN], s_g[TC][kN];
     __shared__ __align__(16) float s_part[4][TC][kN];
     __shared__ float s_vgy[TC];
     __shared__ float s_u[kN];
+    if (gate.closed()) return;
 
     const int b = blockIdx.x / H, h = blockIdx.x % H;
     const int tid = threadIdx.x, lane = tid & 63, q = tid >> 6;
@@ -297,8 +299,9 @@ __global__ __launch_bounds__(512) void scan_bwd_b_kernel(int T, int H,
         const Tin *__restrict__ r, const Tin *__restrict__ k, const Tin *__restrict__ v,
         const Tin *__restrict__ w, const Tin *__restrict__ u, const Tout *__restrict__ gy,
         const float *__restrict__ wsP,
-        Tout *__restrict__ gk, Tout *__restrict__ gv, Tout *__restrict__ gw)
+        Tout *__restrict__ gk, Tout *__restrict__ gv, Tout *__restrict__ gw, Gate gate)
 {
+    if (gate.closed()) return;
     __shared__ __align__(16) float s_r[TC][kN], s_k[TC][kN], s_d[TC][kN], s_v[TC][kN], s_g[TC][kN];
     __shared__ __align__(16) float s_pk[4][TC][kN], s_pv[4][TC][kN];
     __shared__ __align__(16) float s_e[TC][kN];
@@ -503,41 +506,41 @@ __global__ __launch_bounds__(512) void scan_bwd_b_kernel(int T, int H,
 template <typename Tin, typename Tout, typename Ts>
 static hipError_t launch_fwd(hipStream_t st, int64_t B, int64_t T, int64_t H, const void *r, const void *k,
                              const void *v, const void *w, const void *u, const void *s0, const int64_t *map,
-                             void *y, void *sT)
+                             void *y, void *sT, Gate gate)
 {
     hipLaunchKernelGGL((scan_fwd_kernel<Tin, Tout, Ts>), dim3((unsigned)(B * H)), dim3(256), 0, st, (int)T, (int)H,
                        (const Tin *)r, (const Tin *)k, (const Tin *)v, (const Tin *)w, (const Tin *)u,
-                       (const Ts *)s0, map, (Tout *)y, (Ts *)sT);
+                       (const Ts *)s0, map, (Tout *)y, (Ts *)sT, gate);
     return hipGetLastError();
 }
 
 hipError_t scan_forward(hipStream_t st, int dtype, int state_dtype, int64_t B, int64_t T, int64_t H,
                         const void *r, const void *k, const void *v, const void *w, const void *u,
-                        const void *s0, const int64_t *map, void *y, void *sT)
+                        const void *s0, const int64_t *map, void *y, void *sT, Gate gate)
 {
     const bool sf32 = (state_dtype == kF32);
     switch (dtype) {
-    case kF32: return launch_fwd<float, float, float>(st, B, T, H, r, k, v, w, u, s0, map, y, sT);
-    case kF16: return launch_fwd<f16_t, float, float>(st, B, T, H, r, k, v, w, u, s0, map, y, sT);
+    case kF32: return launch_fwd<float, float, float>(st, B, T, H, r, k, v, w, u, s0, map, y, sT, gate);
+    case kF16: return launch_fwd<f16_t, float, float>(st, B, T, H, r, k, v, w, u, s0, map, y, sT, gate);
     default:
-        return sf32 ? launch_fwd<bf16_t, bf16_t, float>(st, B, T, H, r, k, v, w, u, s0, map, y, sT)
-                    : launch_fwd<bf16_t, bf16_t, bf16_t>(st, B, T, H, r, k, v, w, u, s0, map, y, sT);
+        return sf32 ? launch_fwd<bf16_t, bf16_t, float>(st, B, T, H, r, k, v, w, u, s0, map, y, sT, gate)
+                    : launch_fwd<bf16_t, bf16_t, bf16_t>(st, B, T, H, r, k, v, w, u, s0, map, y, sT, gate);
     }
 }
 
 template <typename Tin, typename Tout>
 static hipError_t launch_bwd(hipStream_t st, int64_t B, int64_t T, int64_t H, const void *r, const void *k,
                              const void *v, const void *w, const void *u, const void *gy, void *gr, void *gk,
-                             void *gv, void *gw, void *gu, float *wsP)
+                             void *gv, void *gw, void *gu, float *wsP, Gate gate)
 {
     hipLaunchKernelGGL((scan_bwd_a_kernel<Tin, Tout>), dim3((unsigned)(B * H)), dim3(256), 0, st, (int)T, (int)H,
                        (const Tin *)r, (const Tin *)k, (const Tin *)v, (const Tin *)w, (const Tin *)u,
-                       (const Tout *)gy, (Tout *)gr, (Tout *)gu, wsP);
+                       (const Tout *)gy, (Tout *)gr, (Tout *)gu, wsP, gate);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((scan_bwd_b_kernel<Tin, Tout>), dim3((unsigned)(B * H)), dim3(512), 0, st, (int)T, (int)H,
                        (const Tin *)r, (const Tin *)k, (const Tin *)v, (const Tin *)w, (const Tin *)u,
-                       (const Tout *)gy, (const float *)wsP, (Tout *)gk, (Tout *)gv, (Tout *)gw);
+                       (const Tout *)gy, (const float *)wsP, (Tout *)gk, (Tout *)gv, (Tout *)gw, gate);
     return hipGetLastError();
 }
 
@@ -545,13 +548,13 @@ size_t scan_backward_workspace_bytes(int64_t B, int64_t T, int64_t C) { return (
 
 hipError_t scan_backward(hipStream_t st, int dtype, int64_t B, int64_t T, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
-                         void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace)
+                         void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, Gate gate)
 {
     float *wsP = (float *)workspace;
     switch (dtype) {
-    case kF32: return launch_bwd<float, float>(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, wsP);
-    case kF16: return launch_bwd<f16_t, float>(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, wsP);
-    default:   return launch_bwd<bf16_t, bf16_t>(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, wsP);
+    case kF32: return launch_bwd<float, float>(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, wsP, gate);
+    case kF16: return launch_bwd<f16_t, float>(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, wsP, gate);
+    default:   return launch_bwd<bf16_t, bf16_t>(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, wsP, gate);
     }
 }
 

@@ -213,3 +213,70 @@ def test_xla_custom_call_targets(op, oracle):
     arr = (ctypes.c_void_p * 6)(*[b.data_ptr() for b in dev + [y]])
     lib.wkv_forward(stream, arr, b"x" * 27, 27)
     assert lib.wkv6_last_status() == 1
+
+
+# ---------------------------------------------------------------------------------------------
+# chunk-parallel MFMA path (bf16 tensors)
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("B,T,H", [(1, 32, 1), (2, 64, 2), (2, 100, 1), (1, 129, 3), (2, 1000, 2), (1, 2048, 1)])
+def test_chunk_fwd_bwd_bf16(op, oracle, B, T, H):
+    _case(op, oracle, B, T, H, 40 + T, torch.bfloat16, CHUNK)
+
+
+def test_chunk_state_in_out(op, oracle):
+    B, T, H, N = 3, 150, 2, 64
+    ins = oracle.make_inputs(B, T, H, N, 51, with_state=True)
+    dev, ref = cast_inputs(ins[:5], torch.bfloat16)
+    op.algo = CHUNK
+    for sdt in (torch.bfloat16, torch.float32):
+        s_dev, s_ref = cast_inputs([ins[6][:2]], sdt)
+        smap = [1, 0, 1]
+        y, sT = op(*dev, return_state=True, init_state=s_dev[0], state_map=smap)
+        torch.cuda.synchronize()
+        assert sT.dtype == sdt
+        y_ref, sT_ref = oracle.forward_c(*ref, N, s_ref[0], smap)
+        check_close("y", y, y_ref, torch.bfloat16)
+        check_close("sT", sT, sT_ref, torch.bfloat16)
+
+
+def test_chunk_split_consistency(op, oracle):
+    # chunked prefill then continue from the returned fp32 state == one long call (to bf16 tolerance)
+    B, T, H, N = 2, 256, 2, 64
+    ins = oracle.make_inputs(B, T, H, N, 52, with_state=True)
+    dev, ref = cast_inputs(ins[:5], torch.bfloat16)
+    op.algo = CHUNK
+    s0 = ins[6].cuda()
+    cut = 96
+    a = [x[:, :cut].contiguous() for x in dev[:4]] + [dev[4]]
+    b = [x[:, cut:].contiguous() for x in dev[:4]] + [dev[4]]
+    ya, sa = op(*a, return_state=True, init_state=s0)
+    yb, sb = op(*b, return_state=True, init_state=sa)
+    y_ref, s_ref = oracle.forward_c(*ref, N, to_np(s0))
+    check_close("y", torch.cat([ya, yb], 1), y_ref, torch.bfloat16)
+    check_close("sT", sb, s_ref, torch.bfloat16)
+
+
+def test_chunk_falls_back_on_extreme_decay(op, oracle):
+    # a decay the tile scaling cannot represent raises the flag; the gated exact kernels redo the call
+    B, T, H, N = 2, 128, 2, 64
+    ins = oracle.make_inputs(B, T, H, N, 53)
+    ins[3][1, 40:60, 70:90] = 6.0     # exp(6) = 403 per step: far beyond the limit
+    ins[3][0, 5, 3] = 20.0            # decay exactly 0
+    ins[3][0, 90:100] = -1e9          # decay exactly 1
+    dev, ref = cast_inputs(ins[:5], torch.bfloat16)
+    gy_dev, gy_ref = cast_inputs(ins[5:6], torch.bfloat16)
+    y, grads = _run_fwd_bwd(op, dev + gy_dev, CHUNK)
+    check_close("y", y, oracle.forward_c(*ref, N)[0], torch.bfloat16)
+    for name, g, gr in zip("gr gk gv gw gu".split(), grads, oracle.backward_c(*ref, gy_ref[0], N)):
+        check_close(name, to_np(g).reshape(gr.shape), gr, torch.bfloat16, is_grad=True)
+
+
+def test_chunk_matches_scan_on_padding_mask(op, oracle):
+    B, T, H, N = 1, 96, 1, 64
+    ins = oracle.make_inputs(B, T, H, N, 54)
+    ins[3][:, 20:50] = -1e9
+    ins[1][:, 20:50] = 0
+    dev, ref = cast_inputs(ins[:5], torch.bfloat16)
+    op.algo = CHUNK
+    y, _ = op(*dev)
+    check_close("y", y, oracle.forward_c(*ref, N)[0], torch.bfloat16)
