@@ -44,7 +44,11 @@ enum {
 enum {
     WKV6_ALGO_AUTO = 0,  /* library picks: chunked MFMA path for bf16/f16 when T allows, else scan */
     WKV6_ALGO_SCAN = 1,  /* per-timestep fp32 recurrence, state in VGPRs                       */
-    WKV6_ALGO_CHUNK = 2  /* chunk-parallel form, bf16 MFMA for the dense intra-chunk products   */
+    WKV6_ALGO_CHUNK = 2, /* chunk-parallel form, bf16 MFMA for the dense intra-chunk products;
+                            bf16 tensors only.  An exact per-timestep pass is enqueued behind it
+                            and runs only if a tile's decay left the range the scaling can hold    */
+    WKV6_ALGO_CHUNK_ONLY = 3 /* the chunked kernels alone, without that guarded second pass: for
+                            tests and profiling; results are undefined for extreme decays          */
 };
 
 const char *wkv6_status_string(int status);

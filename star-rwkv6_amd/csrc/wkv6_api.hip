@@ -111,12 +111,13 @@ int wkv6_forward_with_state_ex(void *stream, int dtype, int state_dtype, int alg
     if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(y)) return WKV6_ERR_ARG;
     if (has_init_state && !s) return WKV6_ERR_ARG;
     if (state_dtype != out_type(dtype) && state_dtype != WKV6_F32) return WKV6_ERR_ARG;
-    if (algo != WKV6_ALGO_AUTO && algo != WKV6_ALGO_SCAN && algo != WKV6_ALGO_CHUNK) return WKV6_ERR_ARG;
+    if (algo < WKV6_ALGO_AUTO || algo > WKV6_ALGO_CHUNK_ONLY) return WKV6_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
     const void *s_in = has_init_state ? s : nullptr;
     const int64_t *map_in = has_init_state ? state_map : nullptr;
-    if (algo == WKV6_ALGO_CHUNK && dtype != WKV6_BF16) return WKV6_ERR_UNSUPPORTED;
-    const bool chunk = algo == WKV6_ALGO_CHUNK || (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T));
+    if ((algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY) && dtype != WKV6_BF16) return WKV6_ERR_UNSUPPORTED;
+    const bool chunk = algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY ||
+                       (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T));
     if (!chunk)
         return finish(wkv6::scan_forward(st, dtype, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys,
                                          wkv6::Gate{nullptr, 0}));
@@ -124,7 +125,7 @@ int wkv6_forward_with_state_ex(void *stream, int dtype, int state_dtype, int alg
     hipError_t e = take_flag_slot(&slot);
     if (e != hipSuccess) return finish(e);
     e = wkv6::chunk_forward(st, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys, slot.ptr, slot.epoch);
-    if (e != hipSuccess) return finish(e);
+    if (e != hipSuccess || algo == WKV6_ALGO_CHUNK_ONLY) return finish(e);
     // exact per-timestep kernel behind the gate: a no-op unless the chunked kernel raised the flag
     return finish(wkv6::scan_forward(st, dtype, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys,
                                      wkv6::Gate{slot.ptr, slot.epoch}));
@@ -152,9 +153,15 @@ int wkv6_forward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64
 }
 
 size_t wkv6_backward_workspace_bytes_ex(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
-    (void)algo;
     if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
-    return wkv6::scan_backward_workspace_bytes(B, T, C);
+    // The per-timestep path keeps one fp32 per element (P), the chunked path one fp32 state per
+    // 64-token chunk; the chunked call needs both because its gated fallback reuses the buffer.
+    size_t need = wkv6::scan_backward_workspace_bytes(B, T, C);
+    if (algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY || (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T))) {
+        const size_t c = wkv6::chunk_backward_workspace_bytes(B, T, H);
+        if (c > need) need = c;
+    }
+    return need;
 }
 
 size_t wkv6_backward_workspace_bytes(int dtype, int64_t B, int64_t T, int64_t C, int64_t H) {
@@ -169,13 +176,23 @@ int wkv6_backward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, in
     if (!r || !k || !v || !w || !u || !gy || !gr || !gk || !gv || !gw || !gu) return WKV6_ERR_ARG;
     if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(gy) || !aligned16(gr) ||
         !aligned16(gk) || !aligned16(gv) || !aligned16(gw)) return WKV6_ERR_ARG;
-    if (algo != WKV6_ALGO_AUTO && algo != WKV6_ALGO_SCAN && algo != WKV6_ALGO_CHUNK) return WKV6_ERR_ARG;
+    if (algo < WKV6_ALGO_AUTO || algo > WKV6_ALGO_CHUNK_ONLY) return WKV6_ERR_ARG;
     const size_t need = wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H);
     if (need > 0 && (!workspace || workspace_bytes < need || !aligned16(workspace))) return WKV6_ERR_WORKSPACE;
     hipStream_t st = (hipStream_t)stream;
-    if (algo == WKV6_ALGO_CHUNK && dtype != WKV6_BF16) return WKV6_ERR_UNSUPPORTED;
+    if ((algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY) && dtype != WKV6_BF16) return WKV6_ERR_UNSUPPORTED;
+    const bool chunk = algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY ||
+                       (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T));
+    if (!chunk)
+        return finish(wkv6::scan_backward(st, dtype, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace,
+                                          wkv6::Gate{nullptr, 0}));
+    FlagSlot slot;
+    hipError_t e = take_flag_slot(&slot);
+    if (e != hipSuccess) return finish(e);
+    e = wkv6::chunk_backward(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace, false, slot.ptr, slot.epoch);
+    if (e != hipSuccess || algo == WKV6_ALGO_CHUNK_ONLY) return finish(e);
     return finish(wkv6::scan_backward(st, dtype, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace,
-                                      wkv6::Gate{nullptr, 0}));
+                                      wkv6::Gate{slot.ptr, slot.epoch}));
 }
 
 int wkv6_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,

@@ -201,13 +201,13 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
         auto prefetch = [&](int c) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
+                // rows past the end are read from the last valid row and replaced by neutral values
+                // (r = k = v = 0, w = -inf: exp(w) = 0, decay 1) without a branch
                 const int t = c * CL + 16 * p + e;
-                if (t < T) {
-                    const int64_t o = (int64_t)t * C;
-                    qr[e] = r16[o]; qk[e] = k16[o]; qv[e] = v16[o]; qw[e] = w16[o];
-                } else {
-                    qr[e] = 0; qk[e] = 0; qv[e] = 0; qw[e] = 0xff80u;  // w = -inf: exp(w) = 0, decay 1
-                }
+                const bool ok = t < T;
+                const int64_t o = (int64_t)(ok ? t : T - 1) * C;
+                const uint32_t a = r16[o], bb = k16[o], cc = v16[o], dd = w16[o];
+                qr[e] = ok ? a : 0u; qk[e] = ok ? bb : 0u; qv[e] = ok ? cc : 0u; qw[e] = ok ? dd : 0xff80u;
             }
         };
         auto prepare = [&](int c) {   // consumes the prefetched registers, refills them for chunk c+1
@@ -260,6 +260,419 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
             if (c + 1 < nchunk) prepare(c + 1);
         }
     }
+}
+
+// ==========================================================================================
+// Backward.
+//
+// Same workgroup shape as the forward kernel.  Phase 1 sweeps the chunks in time order and writes
+// the state at every chunk start to the workspace (fp32, [b][h][chunk][j][i]); phase 2 sweeps them
+// in reverse order with the reverse state G in the accumulators.  G is kept twice, once with rows j
+// / columns i (for gv) and once transposed (for gk), so that it can be fed back to the MFMAs as an
+// operand without leaving the registers; the forward state at each of the 4 tile starts of a chunk
+// is recomputed from the checkpoint and held as packed bf16 operands.
+//
+// Per tile (16 tokens; t, s local token indices; c as in the forward kernel; G = reverse state
+// entering the tile from the future, S0 = forward state at the tile start):
+//   dA[t][s] = gy_t . v_s (s<t)                       A[t][s] = R~_t . K~_s (s<t),  A[t][t] = sum_j r u k
+//   X[t][j]  = sum_s dA[t][s] K~_s[j] + sum_i gy_t[i] S0[j][i]        gr'_t[j] = exp(-c_t) X,   P = R~ X
+//   W[s][j]  = sum_t dA[t][s] R~_t[j] + g_j sum_i v_s[i] G[j][i]      gk'_s[j] = exp(+c_{s+1}) W, Q = K~ W
+//   gv_s[i]  = sum_t A[t][s] gy_t[i] + sum_j K~_s[j] g_j G[j][i]
+//   G       <- diag(g) G + R~^T gY
+//   gr = gr' + u k <v,gy>,  gk = gk' + u r <v,gy>,  gu[j] = sum_t r k <v,gy>
+//   gw_t[j]  = -exp(w_t[j]) ( E[j] + sum_{m<t} (Q_m - P_m) - P_t ),  E[j] = sum_i S0[j][i] G_new[j][i]
+// (the last line is the flow balance across decay step t, anchored at the exact tile-boundary term E).
+// ==========================================================================================
+constexpr int LDFR = 80;  // floats per channel row of the decay-factor array: 4 tiles x (17 used + 3 pad)
+
+struct alignas(16) BwdBuf {
+    uint16_t rt[CL][LDA];    // R~[t][j]
+    uint16_t kt[CL][LDA];    // K~[t][j]
+    uint16_t rtT[kN][LDT];   // R~ stored [j][t]
+    uint16_t ktT[kN][LDT];   // K~ stored [j][t]
+    uint16_t vT[kN][LDT];    // V  stored [i][t]
+    uint16_t gyT[kN][LDT];   // gY stored [i][t]
+    float fr[kN][LDFR];      // fr[j][20p + t] = exp(-c_t) of tile p, t = 0..16
+    float g[4][kN];
+    float ruk[CL];
+    float vgy[CL];
+};
+
+// fragment of a global (B,T,C) bf16 tensor row for a 16x16x32 MFMA, same k-slot order as frag_tc
+__device__ __forceinline__ bf16x8 frag_global(const uint16_t *rowptr, bool valid, int h, int g) {
+    if (!valid) return make_bf16x8(0, 0, 0, 0);
+    const uint2 lo = *reinterpret_cast<const uint2 *>(rowptr + 32 * h + 4 * g);
+    const uint2 hi = *reinterpret_cast<const uint2 *>(rowptr + 32 * h + 16 + 4 * g);
+    return make_bf16x8(lo.x, lo.y, hi.x, hi.y);
+}
+__device__ __forceinline__ s16x4 pack4(const f32x4 &a) {
+    return make_s16x4(pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]));
+}
+__device__ __forceinline__ void unpack4(const s16x4 &a, float (&o)[4]) {
+    const u32x2 t = __builtin_bit_cast(u32x2, a);
+    o[0] = __uint_as_float(t[0] << 16); o[1] = __uint_as_float(t[0] & 0xffff0000u);
+    o[2] = __uint_as_float(t[1] << 16); o[3] = __uint_as_float(t[1] & 0xffff0000u);
+}
+__device__ __forceinline__ void unpack8(const bf16x8 &a, float (&o)[8]) {
+    const u32x4 t = __builtin_bit_cast(u32x4, a);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { o[2 * i] = __uint_as_float(t[i] << 16); o[2 * i + 1] = __uint_as_float(t[i] & 0xffff0000u); }
+}
+
+// operand number p of four, p uniform over the wave; dword-wise selects keep everything in registers
+__device__ __forceinline__ bf16x8 pick4(const bf16x8 &a0, const bf16x8 &a1, const bf16x8 &a2, const bf16x8 &a3, int p) {
+    const u32x4 x0 = __builtin_bit_cast(u32x4, a0), x1 = __builtin_bit_cast(u32x4, a1);
+    const u32x4 x2 = __builtin_bit_cast(u32x4, a2), x3 = __builtin_bit_cast(u32x4, a3);
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const uint32_t lo = (p == 1) ? x1[i] : x0[i];
+        const uint32_t hi = (p == 3) ? x3[i] : x2[i];
+        o[i] = (p >= 2) ? hi : lo;
+    }
+    return make_bf16x8(o[0], o[1], o[2], o[3]);
+}
+
+template <bool kSweepStates>
+__global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
+        const bf16_t *__restrict__ r, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v,
+        const bf16_t *__restrict__ w, const bf16_t *__restrict__ u, const bf16_t *__restrict__ gy,
+        bf16_t *__restrict__ gr, bf16_t *__restrict__ gk, bf16_t *__restrict__ gv, bf16_t *__restrict__ gw,
+        bf16_t *__restrict__ gu, float *__restrict__ ckpt,
+        unsigned long long *__restrict__ wild_flag, unsigned long long epoch)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    BwdBuf *buf = reinterpret_cast<BwdBuf *>(smem);
+
+    const int b = blockIdx.x / H, h = blockIdx.x % H;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t C = (int64_t)H * kN;
+    const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
+    const int nchunk = (T + CL - 1) / CL;
+    const int nitem = kSweepStates ? 2 * nchunk : nchunk;   // work items: [phase 1 chunks 0..n-1] then phase 2 chunks n-1..0
+    float *ck = ckpt + (int64_t)blockIdx.x * nchunk * (kN * kN);
+
+    if (wave < 4) {
+        // ------------------------------ consumer ------------------------------
+        const int q = wave, g = lane >> 4, l16 = lane & 15;
+        const int col = 16 * q + l16;   // the channel this lane's accumulator column holds (j for gr/gk/gw, i for gv)
+        int item = 0;
+        if (kSweepStates) {
+            // phase 1: S^T (rows i, column j = col), checkpoint at every chunk start
+            f32x4 S[4];
+#pragma unroll
+            for (int m = 0; m < 4; ++m) S[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            for (int c = 0; c < nchunk; ++c, ++item) {
+                __syncthreads();
+                const BwdBuf &B = buf[item & 1];
+                float *dst = ck + (int64_t)c * (kN * kN) + col * kN;
+#pragma unroll
+                for (int m = 0; m < 4; ++m)
+                    *reinterpret_cast<float4 *>(dst + 16 * m + 4 * g) = make_float4(S[m][0], S[m][1], S[m][2], S[m][3]);
+                if (c + 1 == nchunk) break;   // the state after the last chunk is never used
+#pragma unroll 1
+                for (int p = 0; p < 4; ++p) {
+                    const s16x4 kq = frag_ct(B.ktT, col, 16 * p + 4 * g);
+                    const float gq = B.g[p][col];
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) {
+                        S[m] = mfma16(frag_ct(B.vT, 16 * m + l16, 16 * p + 4 * g), kq, S[m]);
+                        S[m][0] *= gq; S[m][1] *= gq; S[m][2] *= gq; S[m][3] *= gq;
+                    }
+                }
+            }
+            if (nchunk >= 1) ++item;   // account for the `break` above skipping the increment
+        }
+        // phase 2
+        f32x4 Gi[4], Gj[4];   // Gi: rows j, column i = col.   Gj: rows i, column j = col.
+#pragma unroll
+        for (int m = 0; m < 4; ++m) { Gi[m] = (f32x4){0.f, 0.f, 0.f, 0.f}; Gj[m] = Gi[m]; }
+        const float uj = load1(u + h * kN + col);
+        float gu_acc = 0.f;
+        const uint16_t *r16 = reinterpret_cast<const uint16_t *>(r) + base;
+        const uint16_t *k16 = reinterpret_cast<const uint16_t *>(k) + base;
+        const uint16_t *v16 = reinterpret_cast<const uint16_t *>(v) + base;
+        const uint16_t *w16 = reinterpret_cast<const uint16_t *>(w) + base;
+        const uint16_t *g16 = reinterpret_cast<const uint16_t *>(gy) + base;
+        for (int c = nchunk - 1; c >= 0; --c, ++item) {
+            // forward state at the chunk start, straight from the checkpoint (written by this same lane)
+            f32x4 S[4];
+            {
+                const float *src = ck + (int64_t)c * (kN * kN) + col * kN;
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    const float4 x = *reinterpret_cast<const float4 *>(src + 16 * m + 4 * g);
+                    S[m] = (f32x4){x.x, x.y, x.z, x.w};
+                }
+            }
+            __syncthreads();
+            const BwdBuf &B = buf[item & 1];
+            const int t0 = c * CL;
+            // states at the four tile starts as packed bf16 operands
+            bf16x8 SopL[4], SopH[4];
+            SopL[0] = acc_as_operand(S[0], S[1]); SopH[0] = acc_as_operand(S[2], S[3]);
+#pragma unroll
+            for (int p = 0; p < 3; ++p) {
+                const s16x4 kq = frag_ct(B.ktT, col, 16 * p + 4 * g);
+                const float gq = B.g[p][col];
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    S[m] = mfma16(frag_ct(B.vT, 16 * m + l16, 16 * p + 4 * g), kq, S[m]);
+                    S[m][0] *= gq; S[m][1] *= gq; S[m][2] *= gq; S[m][3] *= gq;
+                }
+                SopL[p + 1] = acc_as_operand(S[0], S[1]); SopH[p + 1] = acc_as_operand(S[2], S[3]);
+            }
+#pragma unroll 1
+            for (int p = 3; p >= 0; --p) {
+                if (t0 + 16 * p >= T) continue;
+                const bf16x8 sL = pick4(SopL[0], SopL[1], SopL[2], SopL[3], p);
+                const bf16x8 sH = pick4(SopH[0], SopH[1], SopH[2], SopH[3], p);
+                const int row = 16 * p + l16;           // tile-local token l16 as a chunk row
+                const int trow = t0 + row;              // its global token index
+                const bool rowok = trow < T;
+                // operand fragments
+                const bf16x8 rf0 = frag_tc(B.rt, row, 0, g), rf1 = frag_tc(B.rt, row, 1, g);
+                const bf16x8 kf0 = frag_tc(B.kt, row, 0, g), kf1 = frag_tc(B.kt, row, 1, g);
+                const bf16x8 gf0 = frag_global(g16 + (int64_t)trow * C, rowok, 0, g);
+                const bf16x8 gf1 = frag_global(g16 + (int64_t)trow * C, rowok, 1, g);
+                const bf16x8 vf0 = frag_global(v16 + (int64_t)trow * C, rowok, 0, g);
+                const bf16x8 vf1 = frag_global(v16 + (int64_t)trow * C, rowok, 1, g);
+                const int tk = 16 * p + 4 * g;          // first of this lane group's 4 k-slot tokens
+                const s16x4 rtq = frag_ct(B.rtT, col, tk), ktq = frag_ct(B.ktT, col, tk), gyq = frag_ct(B.gyT, col, tk);
+                // raw r, k, w of the accumulator rows (tokens tk..tk+3, channel col)
+                float rraw[4], kraw[4], wraw[4];
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    const int t = t0 + tk + rr;
+                    if (t < T) {
+                        const int64_t o = (int64_t)t * C + col;
+                        rraw[rr] = bf16_bits_to_float(r16[o]); kraw[rr] = bf16_bits_to_float(k16[o]);
+                        wraw[rr] = bf16_bits_to_float(w16[o]);
+                    } else { rraw[rr] = 0.f; kraw[rr] = 0.f; wraw[rr] = -1e30f; }
+                }
+                // 16x16 intra-tile matrices
+                f32x4 dA = {0.f, 0.f, 0.f, 0.f}, dAT = dA, A = dA;
+                dA = mfma32(gf0, vf0, dA);   dA = mfma32(gf1, vf1, dA);     // rows t, col s
+                dAT = mfma32(vf0, gf0, dAT); dAT = mfma32(vf1, gf1, dAT);   // rows s, col t
+                A = mfma32(rf0, kf0, A);     A = mfma32(rf1, kf1, A);       // rows t, col s
+                const float rukv = B.ruk[row];
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    const int x = 4 * g + rr;
+                    dA[rr] = (x > l16) ? dA[rr] : 0.f;
+                    dAT[rr] = (l16 > x) ? dAT[rr] : 0.f;
+                    A[rr] = (x > l16) ? A[rr] : ((x == l16) ? rukv : 0.f);
+                }
+                // X (rows t, col j)
+                f32x4 X = {0.f, 0.f, 0.f, 0.f};
+                X = mfma16(pack4(dAT), ktq, X);
+                X = mfma32(gf0, sL, X);
+                X = mfma32(gf1, sH, X);
+                // W (rows s, col j); Gj is decayed first so that W picks up g_j G
+                const float gq = B.g[p][col];
+#pragma unroll
+                for (int m = 0; m < 4; ++m) { Gj[m][0] *= gq; Gj[m][1] *= gq; Gj[m][2] *= gq; Gj[m][3] *= gq; }
+                f32x4 W = {0.f, 0.f, 0.f, 0.f};
+                W = mfma16(pack4(dA), rtq, W);
+                W = mfma32(vf0, acc_as_operand(Gj[0], Gj[1]), W);
+                W = mfma32(vf1, acc_as_operand(Gj[2], Gj[3]), W);
+                // gv (rows s, col i); Gi decayed first
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    const float4 gg = *reinterpret_cast<const float4 *>(&B.g[p][16 * m + 4 * g]);
+                    Gi[m][0] *= gg.x; Gi[m][1] *= gg.y; Gi[m][2] *= gg.z; Gi[m][3] *= gg.w;
+                }
+                f32x4 GV = {0.f, 0.f, 0.f, 0.f};
+                GV = mfma16(pack4(A), gyq, GV);
+                GV = mfma32(kf0, acc_as_operand(Gi[0], Gi[1]), GV);
+                GV = mfma32(kf1, acc_as_operand(Gi[2], Gi[3]), GV);
+                // G <- diag(g) G + R~^T gY   (both copies)
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    Gi[m] = mfma16(frag_ct(B.rtT, 16 * m + l16, tk), gyq, Gi[m]);
+                    Gj[m] = mfma16(frag_ct(B.gyT, 16 * m + l16, tk), rtq, Gj[m]);
+                }
+                // tile-boundary term E[j] = sum_i S0[j][i] G_new[j][i]
+                float E = 0.f;
+                {
+                    float sl[8], sh[8];
+                    unpack8(sL, sl); unpack8(sH, sh);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        E = fmaf(sl[e], Gj[0][e], E); E = fmaf(sl[4 + e], Gj[1][e], E);
+                        E = fmaf(sh[e], Gj[2][e], E); E = fmaf(sh[4 + e], Gj[3][e], E);
+                    }
+                    E += __shfl_xor(E, 16);
+                    E += __shfl_xor(E, 32);
+                }
+                // epilogue on the accumulator rows (tokens tk..tk+3, channel col)
+                const float4 f4 = *reinterpret_cast<const float4 *>(&B.fr[col][20 * p + 4 * g]);
+                const float f5 = B.fr[col][20 * p + 4 * g + 4];
+                const float4 vg4 = *reinterpret_cast<const float4 *>(&B.vgy[tk]);
+                const float fr_[5] = {f4.x, f4.y, f4.z, f4.w, f5};
+                const float vg_[4] = {vg4.x, vg4.y, vg4.z, vg4.w};
+                float rt_[4], kt_[4], P[4], D[4], gro[4], gko[4];
+                unpack4(rtq, rt_); unpack4(ktq, kt_);
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    P[rr] = rt_[rr] * X[rr];
+                    D[rr] = kt_[rr] * W[rr] - P[rr];
+                    gro[rr] = fmaf(fr_[rr], X[rr], uj * kraw[rr] * vg_[rr]);
+                    gko[rr] = fmaf(__frcp_rn(fr_[rr + 1]), W[rr], uj * rraw[rr] * vg_[rr]);
+                    gu_acc = fmaf(rraw[rr] * kraw[rr], vg_[rr], gu_acc);
+                }
+                // exclusive prefix of D over the 16 tokens: 4 in this lane, the rest in the lane groups below
+                const float tot = D[0] + D[1] + D[2] + D[3];
+                const float o1 = __shfl_up(tot, 16), o2 = __shfl_up(tot, 32), o3 = __shfl_up(tot, 48);
+                float pre = E + ((g >= 1) ? o1 : 0.f) + ((g >= 2) ? o2 : 0.f) + ((g >= 3) ? o3 : 0.f);
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    const int t = t0 + tk + rr;
+                    const float ew = fast_exp(wraw[rr]);
+                    float gwv = (fast_exp(-ew) == 0.f) ? 0.f : -ew * (pre - P[rr]);
+                    if (t == 0 || t == T - 1) gwv = 0.f;
+                    pre += D[rr];
+                    if (t < T) {
+                        const int64_t o = base + (int64_t)t * C + col;
+                        store1(gr + o, gro[rr]); store1(gk + o, gko[rr]); store1(gw + o, gwv); store1(gv + o, GV[rr]);
+                    }
+                }
+            }
+        }
+        // gu: fold the four lane groups (different tokens, same channel) with wavefront shuffles
+        gu_acc += __shfl_xor(gu_acc, 16);
+        gu_acc += __shfl_xor(gu_acc, 32);
+        if (g == 0) store1(gu + (int64_t)b * C + h * kN + col, gu_acc);
+    } else {
+        // ------------------------------ producer ------------------------------
+        const int p = wave - 4, ch = lane;
+        const float uc = load1(u + h * kN + ch);
+        const uint16_t *r16 = reinterpret_cast<const uint16_t *>(r) + base + ch;
+        const uint16_t *k16 = reinterpret_cast<const uint16_t *>(k) + base + ch;
+        const uint16_t *v16 = reinterpret_cast<const uint16_t *>(v) + base + ch;
+        const uint16_t *w16 = reinterpret_cast<const uint16_t *>(w) + base + ch;
+        const uint16_t *g16 = reinterpret_cast<const uint16_t *>(gy) + base + ch;
+        uint32_t qr[16], qk[16], qv[16], qw[16], qg[16];
+        // item -> (chunk, full): phase 1 items need only k, v, w
+        auto item_chunk = [&](int it) { return kSweepStates ? (it < nchunk ? it : 2 * nchunk - 1 - it) : nchunk - 1 - it; };
+        auto item_full = [&](int it) { return kSweepStates ? it >= nchunk : true; };
+        auto prefetch = [&](int it) {
+            const int c = item_chunk(it);
+            const bool full = item_full(it);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int t = c * CL + 16 * p + e;
+                const bool ok = t < T;
+                const int64_t o = (int64_t)(ok ? t : T - 1) * C;
+                const uint32_t bb = k16[o], cc = v16[o], dd = w16[o];
+                qk[e] = ok ? bb : 0u; qv[e] = ok ? cc : 0u; qw[e] = ok ? dd : 0xff80u;
+            }
+            if (full) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int t = c * CL + 16 * p + e;
+                    const bool ok = t < T;
+                    const int64_t o = (int64_t)(ok ? t : T - 1) * C;
+                    const uint32_t a = r16[o], gg = g16[o];
+                    qr[e] = ok ? a : 0u; qg[e] = ok ? gg : 0u;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) { qr[e] = 0u; qg[e] = 0u; }
+            }
+        };
+        auto prepare = [&](int it) {
+            BwdBuf &B = buf[it & 1];
+            const bool full = item_full(it);
+            float fr[16], fk[16], fw[16], pv[16];
+            uint32_t vbits[8], gbits[8];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                fr[e] = bf16_bits_to_float(qr[e]); fk[e] = bf16_bits_to_float(qk[e]); fw[e] = bf16_bits_to_float(qw[e]);
+                pv[e] = bf16_bits_to_float(qv[e]) * bf16_bits_to_float(qg[e]);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                vbits[e] = qv[2 * e] | (qv[2 * e + 1] << 16);
+                gbits[e] = qg[2 * e] | (qg[2 * e + 1] << 16);
+            }
+            if (it + 1 < nitem) prefetch(it + 1);
+
+            float xr[16], xk[16], pr[16], fa[17];
+            float cs = 0.f, pa = 1.f;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const float ew = fast_exp(fw[e]);
+                fa[e] = pa;
+                xr[e] = fr[e] * pa;
+                cs += ew;
+                xk[e] = fk[e] * fast_exp(cs);
+                pa *= fast_exp(-ew);
+                pr[e] = fr[e] * uc * fk[e];
+            }
+            fa[16] = pa;
+            if (__builtin_amdgcn_ballot_w64(!(cs <= kWildLimit)) != 0ull) {
+                if (lane == 0 && wild_flag != nullptr) *wild_flag = epoch;
+            }
+            uint32_t pk[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pk[e] = pack_bf16x2(xk[2 * e], xk[2 * e + 1]);
+            *reinterpret_cast<uint4 *>(&B.ktT[ch][16 * p]) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+            *reinterpret_cast<uint4 *>(&B.ktT[ch][16 * p + 8]) = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+            *reinterpret_cast<uint4 *>(&B.vT[ch][16 * p]) = make_uint4(vbits[0], vbits[1], vbits[2], vbits[3]);
+            *reinterpret_cast<uint4 *>(&B.vT[ch][16 * p + 8]) = make_uint4(vbits[4], vbits[5], vbits[6], vbits[7]);
+            B.g[p][ch] = pa;
+            if (full) {
+                store_rows_paired(B.rt, 16 * p, lane, xr);
+                store_rows_paired(B.kt, 16 * p, lane, xk);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pk[e] = pack_bf16x2(xr[2 * e], xr[2 * e + 1]);
+                *reinterpret_cast<uint4 *>(&B.rtT[ch][16 * p]) = make_uint4(pk[0], pk[1], pk[2], pk[3]);
+                *reinterpret_cast<uint4 *>(&B.rtT[ch][16 * p + 8]) = make_uint4(pk[4], pk[5], pk[6], pk[7]);
+                *reinterpret_cast<uint4 *>(&B.gyT[ch][16 * p]) = make_uint4(gbits[0], gbits[1], gbits[2], gbits[3]);
+                *reinterpret_cast<uint4 *>(&B.gyT[ch][16 * p + 8]) = make_uint4(gbits[4], gbits[5], gbits[6], gbits[7]);
+#pragma unroll
+                for (int e = 0; e < 16; e += 4)
+                    *reinterpret_cast<float4 *>(&B.fr[ch][20 * p + e]) = make_float4(fa[e], fa[e + 1], fa[e + 2], fa[e + 3]);
+                B.fr[ch][20 * p + 16] = fa[16];
+                const float tr = transpose_reduce16(pr, lane);
+                const float tv = transpose_reduce16(pv, lane);
+                if ((lane & 3) == 0) {
+                    B.ruk[16 * p + ((lane >> 2) & 15)] = tr;
+                    B.vgy[16 * p + ((lane >> 2) & 15)] = tv;
+                }
+            }
+        };
+        prefetch(0);
+        prepare(0);
+        for (int it = 0; it < nitem; ++it) {
+            __syncthreads();
+            if (it + 1 < nitem) prepare(it + 1);
+        }
+    }
+}
+
+size_t chunk_backward_workspace_bytes(int64_t B, int64_t T, int64_t H) {
+    const int64_t nchunk = (T + CL - 1) / CL;
+    return (size_t)(B * H * nchunk) * kN * kN * sizeof(float);
+}
+
+hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                          const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, bool states_ready,
+                          unsigned long long *wild_flag, unsigned long long epoch)
+{
+    const size_t lds = 2 * sizeof(BwdBuf);
+    auto launch = [&](auto kern) -> hipError_t {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(512), lds, st, (int)T, (int)H,
+                           (const bf16_t *)r, (const bf16_t *)k, (const bf16_t *)v, (const bf16_t *)w, (const bf16_t *)u,
+                           (const bf16_t *)gy, (bf16_t *)gr, (bf16_t *)gk, (bf16_t *)gv, (bf16_t *)gw, (bf16_t *)gu,
+                           (float *)workspace, wild_flag, epoch);
+        return hipGetLastError();
+    };
+    return states_ready ? launch(chunk_bwd_kernel<false>) : launch(chunk_bwd_kernel<true>);
 }
 
 hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,

@@ -33,4 +33,11 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
                          const void *s0, const int64_t *map, void *y, void *sT,
                          unsigned long long *wild_flag, unsigned long long epoch);
 
+size_t chunk_backward_workspace_bytes(int64_t B, int64_t T, int64_t H);
+// states_ready: the workspace already holds the chunk-start states (written by a forward pass)
+hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                          const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, bool states_ready,
+                          unsigned long long *wild_flag, unsigned long long epoch);
+
 }  // namespace wkv6

@@ -10,7 +10,7 @@ from _util import cast_inputs, check_close, out_dtype, to_np
 
 pytestmark = pytest.mark.gpu
 
-SCAN, CHUNK = 1, 2
+SCAN, CHUNK, CHUNK_ONLY = 1, 2, 3
 DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
 
 
@@ -221,6 +221,12 @@ def test_xla_custom_call_targets(op, oracle):
 @pytest.mark.parametrize("B,T,H", [(1, 32, 1), (2, 64, 2), (2, 100, 1), (1, 129, 3), (2, 1000, 2), (1, 2048, 1)])
 def test_chunk_fwd_bwd_bf16(op, oracle, B, T, H):
     _case(op, oracle, B, T, H, 40 + T, torch.bfloat16, CHUNK)
+
+
+@pytest.mark.parametrize("B,T,H", [(1, 48, 1), (2, 64, 2), (2, 333, 2), (1, 1024, 4)])
+def test_chunk_kernels_alone_bf16(op, oracle, B, T, H):
+    # without the guarded exact second pass: the MFMA kernels themselves must meet the tolerance
+    _case(op, oracle, B, T, H, 60 + T, torch.bfloat16, CHUNK_ONLY)
 
 
 def test_chunk_state_in_out(op, oracle):
