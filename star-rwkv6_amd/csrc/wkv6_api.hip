@@ -52,7 +52,9 @@ hipError_t take_flag_slot(FlagSlot *out) {
 }
 
 // Shapes the chunked MFMA kernels take; everything else runs the per-timestep kernels.
-bool chunk_eligible(int dtype, int64_t T) { return dtype == WKV6_BF16 && T >= 32; }
+// (the chunked kernels index one batch row with 32-bit element offsets)
+bool chunk_possible(int dtype, int64_t T, int64_t C) { return dtype == WKV6_BF16 && T * C < (1LL << 31); }
+bool chunk_eligible(int dtype, int64_t T, int64_t C) { return chunk_possible(dtype, T, C) && T >= 32; }
 
 thread_local int g_last_status = WKV6_OK;
 thread_local int g_last_hip_error = 0;
@@ -115,9 +117,9 @@ int wkv6_forward_with_state_ex(void *stream, int dtype, int state_dtype, int alg
     hipStream_t st = (hipStream_t)stream;
     const void *s_in = has_init_state ? s : nullptr;
     const int64_t *map_in = has_init_state ? state_map : nullptr;
-    if ((algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY) && dtype != WKV6_BF16) return WKV6_ERR_UNSUPPORTED;
+    if ((algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY) && !chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;
     const bool chunk = algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY ||
-                       (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T));
+                       (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
     if (!chunk)
         return finish(wkv6::scan_forward(st, dtype, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys,
                                          wkv6::Gate{nullptr, 0}));
@@ -157,7 +159,7 @@ size_t wkv6_backward_workspace_bytes_ex(int dtype, int algo, int64_t B, int64_t 
     // The per-timestep path keeps one fp32 per element (P), the chunked path one fp32 state per
     // 64-token chunk; the chunked call needs both because its gated fallback reuses the buffer.
     size_t need = wkv6::scan_backward_workspace_bytes(B, T, C);
-    if (algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY || (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T))) {
+    if (algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY || (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C))) {
         const size_t c = wkv6::chunk_backward_workspace_bytes(B, T, H);
         if (c > need) need = c;
     }
@@ -180,9 +182,9 @@ int wkv6_backward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, in
     const size_t need = wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H);
     if (need > 0 && (!workspace || workspace_bytes < need || !aligned16(workspace))) return WKV6_ERR_WORKSPACE;
     hipStream_t st = (hipStream_t)stream;
-    if ((algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY) && dtype != WKV6_BF16) return WKV6_ERR_UNSUPPORTED;
+    if ((algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY) && !chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;
     const bool chunk = algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY ||
-                       (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T));
+                       (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
     if (!chunk)
         return finish(wkv6::scan_backward(st, dtype, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace,
                                           wkv6::Gate{nullptr, 0}));

@@ -49,6 +49,33 @@ __device__ __forceinline__ f32x4 mfma32(bf16x8 a, bf16x8 b, f32x4 c) {
 __device__ __forceinline__ f32x4 mfma16(s16x4 a, s16x4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
 }
+// Two software-inserted delays around the MFMAs.  Both pass the accumulators through an asm
+// statement, so neither the MFMAs that write them nor the code that reads them can move across.
+//
+// chain_gap(acc): 8 idle issue slots between two MFMAs of DIFFERENT shape (16x16x16 and 16x16x32)
+// that are chained through the same accumulator.  hipcc 7.2 schedules such a pair 0-3 slots apart,
+// and on gfx950 the second MFMA then reads a stale SrcC: the products came out wrong whenever the
+// scheduler happened to place the pair that close and right when it left 5 or more slots.
+// Same-shape accumulation chains are not affected.
+//
+// settle(acc...): 16 idle slots before VALU code (masks, scaling, bf16 conversion, stores) reads
+// MFMA results; belt and braces on top of the wait states the compiler inserts itself.
+#define WKV6_SETTLE_ASM "s_nop 15"
+__device__ __forceinline__ void chain_gap(f32x4 &a) { asm volatile("s_nop 7" : "+v"(a)); }
+__device__ __forceinline__ void settle(f32x4 &a) { asm volatile(WKV6_SETTLE_ASM : "+v"(a)); }
+__device__ __forceinline__ void settle(f32x4 &a, f32x4 &b, f32x4 &c) {
+    asm volatile(WKV6_SETTLE_ASM : "+v"(a), "+v"(b), "+v"(c));
+}
+__device__ __forceinline__ void settle(f32x4 &a, f32x4 &b, f32x4 &c, f32x4 &d) {
+    asm volatile(WKV6_SETTLE_ASM : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
+__device__ __forceinline__ void settle(f32x4 &a, f32x4 &b, f32x4 &c, f32x4 &d, f32x4 &e) {
+    asm volatile(WKV6_SETTLE_ASM : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e));
+}
+__device__ __forceinline__ void settle(f32x4 &a, f32x4 &b, f32x4 &c, f32x4 (&g1)[4], f32x4 (&g2)[4]) {
+    asm volatile(WKV6_SETTLE_ASM : "+v"(a), "+v"(b), "+v"(c), "+v"(g1[0]), "+v"(g1[1]), "+v"(g1[2]), "+v"(g1[3]),
+                 "+v"(g2[0]), "+v"(g2[1]), "+v"(g2[2]), "+v"(g2[3]));
+}
 __device__ __forceinline__ float xor1(float x) {   // value of the neighbouring lane (lane ^ 1)
     return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0xB1, 0xF, 0xF, true));
 }
@@ -141,6 +168,7 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
 #pragma unroll
             for (int m = 0; m < 4; ++m) S[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
         }
+        bf16_t *y_h = y + base;
         for (int c = 0; c < nchunk; ++c) {
             __syncthreads();
             const FwdBuf &B = buf[c & 1];
@@ -161,24 +189,27 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
                 f32x4 Y = {0.f, 0.f, 0.f, 0.f};
                 Y = mfma32(rf0, acc_as_operand(S[0], S[1]), Y);
                 Y = mfma32(rf1, acc_as_operand(S[2], S[3]), Y);
+                settle(AT);
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr) {
                     const int s = 4 * g + rr;
                     AT[rr] = (l16 > s) ? AT[rr] : ((l16 == s) ? rukv : 0.f);
                 }
                 // Y += A V : the masked A^T accumulator IS the A operand (row t = l16, k-slots s = 4g+r)
+                chain_gap(Y);
                 Y = mfma16(make_s16x4(pack_bf16x2(AT[0], AT[1]), pack_bf16x2(AT[2], AT[3])), vf, Y);
-#pragma unroll
-                for (int rr = 0; rr < 4; ++rr) {
-                    const int t = t0 + 16 * p + 4 * g + rr;
-                    if (t < T) store1(y + base + (int64_t)t * C + 16 * q + l16, Y[rr]);
-                }
                 // S <- diag(g) S + K^T V
 #pragma unroll
                 for (int m = 0; m < 4; ++m) {
                     const float4 gg = *reinterpret_cast<const float4 *>(&B.g[p][16 * m + 4 * g]);
                     S[m][0] *= gg.x; S[m][1] *= gg.y; S[m][2] *= gg.z; S[m][3] *= gg.w;
                     S[m] = mfma16(frag_ct(B.kbT, 16 * m + l16, 16 * p + 4 * g), vf, S[m]);
+                }
+                settle(Y, S[0], S[1], S[2], S[3]);   // Y is stored, S scaled and converted by VALU code from here on
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    const int t = t0 + 16 * p + 4 * g + rr;
+                    if (t < T) store1(y_h + (uint32_t)t * (uint32_t)C + (uint32_t)(16 * q + l16), Y[rr]);
                 }
             }
         }
@@ -299,8 +330,7 @@ struct alignas(16) BwdBuf {
 };
 
 // fragment of a global (B,T,C) bf16 tensor row for a 16x16x32 MFMA, same k-slot order as frag_tc
-__device__ __forceinline__ bf16x8 frag_global(const uint16_t *rowptr, bool valid, int h, int g) {
-    if (!valid) return make_bf16x8(0, 0, 0, 0);
+__device__ __forceinline__ bf16x8 frag_global(const uint16_t *rowptr, int h, int g) {
     const uint2 lo = *reinterpret_cast<const uint2 *>(rowptr + 32 * h + 4 * g);
     const uint2 hi = *reinterpret_cast<const uint2 *>(rowptr + 32 * h + 16 + 4 * g);
     return make_bf16x8(lo.x, lo.y, hi.x, hi.y);
@@ -375,10 +405,10 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                     const s16x4 kq = frag_ct(B.ktT, col, 16 * p + 4 * g);
                     const float gq = B.g[p][col];
 #pragma unroll
-                    for (int m = 0; m < 4; ++m) {
-                        S[m] = mfma16(frag_ct(B.vT, 16 * m + l16, 16 * p + 4 * g), kq, S[m]);
-                        S[m][0] *= gq; S[m][1] *= gq; S[m][2] *= gq; S[m][3] *= gq;
-                    }
+                    for (int m = 0; m < 4; ++m) S[m] = mfma16(frag_ct(B.vT, 16 * m + l16, 16 * p + 4 * g), kq, S[m]);
+                    settle(S[0], S[1], S[2], S[3]);
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) { S[m][0] *= gq; S[m][1] *= gq; S[m][2] *= gq; S[m][3] *= gq; }
                 }
             }
             if (nchunk >= 1) ++item;   // account for the `break` above skipping the increment
@@ -394,6 +424,7 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
         const uint16_t *v16 = reinterpret_cast<const uint16_t *>(v) + base;
         const uint16_t *w16 = reinterpret_cast<const uint16_t *>(w) + base;
         const uint16_t *g16 = reinterpret_cast<const uint16_t *>(gy) + base;
+        bf16_t *gr_h = gr + base, *gk_h = gk + base, *gv_h = gv + base, *gw_h = gw + base;
         for (int c = nchunk - 1; c >= 0; --c, ++item) {
             // forward state at the chunk start, straight from the checkpoint (written by this same lane)
             f32x4 S[4];
@@ -416,46 +447,54 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                 const s16x4 kq = frag_ct(B.ktT, col, 16 * p + 4 * g);
                 const float gq = B.g[p][col];
 #pragma unroll
-                for (int m = 0; m < 4; ++m) {
-                    S[m] = mfma16(frag_ct(B.vT, 16 * m + l16, 16 * p + 4 * g), kq, S[m]);
-                    S[m][0] *= gq; S[m][1] *= gq; S[m][2] *= gq; S[m][3] *= gq;
-                }
+                for (int m = 0; m < 4; ++m) S[m] = mfma16(frag_ct(B.vT, 16 * m + l16, 16 * p + 4 * g), kq, S[m]);
+                settle(S[0], S[1], S[2], S[3]);
+#pragma unroll
+                for (int m = 0; m < 4; ++m) { S[m][0] *= gq; S[m][1] *= gq; S[m][2] *= gq; S[m][3] *= gq; }
                 SopL[p + 1] = acc_as_operand(S[0], S[1]); SopH[p + 1] = acc_as_operand(S[2], S[3]);
             }
+            // Software pipeline over the tiles: the gY / V fragments of the next tile are requested
+            // as soon as the MFMAs of the current one have consumed them, so that the epilogue
+            // covers their latency; rows past T are read from row T-1 (they only ever meet zero
+            // operands) and never stored.
+            auto rowoff = [&](int t) { return (uint32_t)min(t, T - 1) * (uint32_t)C; };
+            // (the next tile's fragments land in their own registers and are moved over at the end of
+            // the iteration: loading straight into registers that MFMAs issued a few cycles earlier
+            // still name as sources gave wrong products on gfx950)
+            bf16x8 gf0, gf1, vf0, vf1, ngf0, ngf1, nvf0, nvf1;
+            auto load_frags = [&](int p) {
+                const uint32_t o = rowoff(t0 + 16 * p + l16);
+                ngf0 = frag_global(g16 + o, 0, g); ngf1 = frag_global(g16 + o, 1, g);
+                nvf0 = frag_global(v16 + o, 0, g); nvf1 = frag_global(v16 + o, 1, g);
+            };
+            int ptop = 3;
+            while (ptop > 0 && t0 + 16 * ptop >= T) --ptop;
+            load_frags(ptop);
 #pragma unroll 1
-            for (int p = 3; p >= 0; --p) {
-                if (t0 + 16 * p >= T) continue;
+            for (int p = ptop; p >= 0; --p) {
+                gf0 = ngf0; gf1 = ngf1; vf0 = nvf0; vf1 = nvf1;
                 const bf16x8 sL = pick4(SopL[0], SopL[1], SopL[2], SopL[3], p);
                 const bf16x8 sH = pick4(SopH[0], SopH[1], SopH[2], SopH[3], p);
                 const int row = 16 * p + l16;           // tile-local token l16 as a chunk row
-                const int trow = t0 + row;              // its global token index
-                const bool rowok = trow < T;
-                // operand fragments
-                const bf16x8 rf0 = frag_tc(B.rt, row, 0, g), rf1 = frag_tc(B.rt, row, 1, g);
-                const bf16x8 kf0 = frag_tc(B.kt, row, 0, g), kf1 = frag_tc(B.kt, row, 1, g);
-                const bf16x8 gf0 = frag_global(g16 + (int64_t)trow * C, rowok, 0, g);
-                const bf16x8 gf1 = frag_global(g16 + (int64_t)trow * C, rowok, 1, g);
-                const bf16x8 vf0 = frag_global(v16 + (int64_t)trow * C, rowok, 0, g);
-                const bf16x8 vf1 = frag_global(v16 + (int64_t)trow * C, rowok, 1, g);
-                const int tk = 16 * p + 4 * g;          // first of this lane group's 4 k-slot tokens
-                const s16x4 rtq = frag_ct(B.rtT, col, tk), ktq = frag_ct(B.ktT, col, tk), gyq = frag_ct(B.gyT, col, tk);
-                // raw r, k, w of the accumulator rows (tokens tk..tk+3, channel col)
+                const int tk = 16 * p + 4 * g;          // first of this lane group's 4 accumulator-row tokens
+                // raw r, k, w of the accumulator rows (tokens tk..tk+3, channel col): used by the epilogue only
                 float rraw[4], kraw[4], wraw[4];
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr) {
-                    const int t = t0 + tk + rr;
-                    if (t < T) {
-                        const int64_t o = (int64_t)t * C + col;
-                        rraw[rr] = bf16_bits_to_float(r16[o]); kraw[rr] = bf16_bits_to_float(k16[o]);
-                        wraw[rr] = bf16_bits_to_float(w16[o]);
-                    } else { rraw[rr] = 0.f; kraw[rr] = 0.f; wraw[rr] = -1e30f; }
+                    const uint32_t o = rowoff(t0 + tk + rr) + (uint32_t)col;
+                    rraw[rr] = bf16_bits_to_float(r16[o]); kraw[rr] = bf16_bits_to_float(k16[o]);
+                    wraw[rr] = bf16_bits_to_float(w16[o]);
                 }
+                const bf16x8 rf0 = frag_tc(B.rt, row, 0, g), rf1 = frag_tc(B.rt, row, 1, g);
+                const bf16x8 kf0 = frag_tc(B.kt, row, 0, g), kf1 = frag_tc(B.kt, row, 1, g);
+                const s16x4 rtq = frag_ct(B.rtT, col, tk), ktq = frag_ct(B.ktT, col, tk), gyq = frag_ct(B.gyT, col, tk);
                 // 16x16 intra-tile matrices
                 f32x4 dA = {0.f, 0.f, 0.f, 0.f}, dAT = dA, A = dA;
                 dA = mfma32(gf0, vf0, dA);   dA = mfma32(gf1, vf1, dA);     // rows t, col s
                 dAT = mfma32(vf0, gf0, dAT); dAT = mfma32(vf1, gf1, dAT);   // rows s, col t
                 A = mfma32(rf0, kf0, A);     A = mfma32(rf1, kf1, A);       // rows t, col s
                 const float rukv = B.ruk[row];
+                settle(dA, dAT, A);
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr) {
                     const int x = 4 * g + rr;
@@ -466,6 +505,7 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                 // X (rows t, col j)
                 f32x4 X = {0.f, 0.f, 0.f, 0.f};
                 X = mfma16(pack4(dAT), ktq, X);
+                chain_gap(X);
                 X = mfma32(gf0, sL, X);
                 X = mfma32(gf1, sH, X);
                 // W (rows s, col j); Gj is decayed first so that W picks up g_j G
@@ -474,8 +514,10 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                 for (int m = 0; m < 4; ++m) { Gj[m][0] *= gq; Gj[m][1] *= gq; Gj[m][2] *= gq; Gj[m][3] *= gq; }
                 f32x4 W = {0.f, 0.f, 0.f, 0.f};
                 W = mfma16(pack4(dA), rtq, W);
+                chain_gap(W);
                 W = mfma32(vf0, acc_as_operand(Gj[0], Gj[1]), W);
                 W = mfma32(vf1, acc_as_operand(Gj[2], Gj[3]), W);
+                if (p > 0) load_frags(p - 1);
                 // gv (rows s, col i); Gi decayed first
 #pragma unroll
                 for (int m = 0; m < 4; ++m) {
@@ -484,6 +526,7 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                 }
                 f32x4 GV = {0.f, 0.f, 0.f, 0.f};
                 GV = mfma16(pack4(A), gyq, GV);
+                chain_gap(GV);
                 GV = mfma32(kf0, acc_as_operand(Gi[0], Gi[1]), GV);
                 GV = mfma32(kf1, acc_as_operand(Gi[2], Gi[3]), GV);
                 // G <- diag(g) G + R~^T gY   (both copies)
@@ -492,6 +535,7 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                     Gi[m] = mfma16(frag_ct(B.rtT, 16 * m + l16, tk), gyq, Gi[m]);
                     Gj[m] = mfma16(frag_ct(B.gyT, 16 * m + l16, tk), rtq, Gj[m]);
                 }
+                settle(X, W, GV, Gi, Gj);   // all read by VALU code from here on
                 // tile-boundary term E[j] = sum_i S0[j][i] G_new[j][i]
                 float E = 0.f;
                 {
@@ -517,8 +561,9 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                 for (int rr = 0; rr < 4; ++rr) {
                     P[rr] = rt_[rr] * X[rr];
                     D[rr] = kt_[rr] * W[rr] - P[rr];
-                    gro[rr] = fmaf(fr_[rr], X[rr], uj * kraw[rr] * vg_[rr]);
-                    gko[rr] = fmaf(__frcp_rn(fr_[rr + 1]), W[rr], uj * rraw[rr] * vg_[rr]);
+                    const float uvg = uj * vg_[rr];
+                    gro[rr] = fmaf(fr_[rr], X[rr], uvg * kraw[rr]);
+                    gko[rr] = fmaf(__builtin_amdgcn_rcpf(fr_[rr + 1]), W[rr], uvg * rraw[rr]);
                     gu_acc = fmaf(rraw[rr] * kraw[rr], vg_[rr], gu_acc);
                 }
                 // exclusive prefix of D over the 16 tokens: 4 in this lane, the rest in the lane groups below
@@ -529,12 +574,13 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                 for (int rr = 0; rr < 4; ++rr) {
                     const int t = t0 + tk + rr;
                     const float ew = fast_exp(wraw[rr]);
-                    float gwv = (fast_exp(-ew) == 0.f) ? 0.f : -ew * (pre - P[rr]);
-                    if (t == 0 || t == T - 1) gwv = 0.f;
+                    // gw carries a factor exp(-ew): zero once that underflows (keeps exp(w) from
+                    // amplifying rounding residue); first and last token are zero by definition
+                    float gwv = (ew >= 88.f || t == 0 || t == T - 1) ? 0.f : -ew * (pre - P[rr]);
                     pre += D[rr];
                     if (t < T) {
-                        const int64_t o = base + (int64_t)t * C + col;
-                        store1(gr + o, gro[rr]); store1(gk + o, gko[rr]); store1(gw + o, gwv); store1(gv + o, GV[rr]);
+                        const uint32_t o = (uint32_t)t * (uint32_t)C + (uint32_t)col;
+                        store1(gr_h + o, gro[rr]); store1(gk_h + o, gko[rr]); store1(gw_h + o, gwv); store1(gv_h + o, GV[rr]);
                     }
                 }
             }

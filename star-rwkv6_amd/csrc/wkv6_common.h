@@ -73,7 +73,7 @@ __device__ __forceinline__ void store4(bf16_t *p, float a, float b, float c, flo
 }
 __device__ __forceinline__ void store1(float *p, float a) { *p = a; }
 __device__ __forceinline__ void store1(bf16_t *p, float a) {
-    *reinterpret_cast<uint16_t *>(p) = (uint16_t)float_to_bf16_bits(a);
+    *reinterpret_cast<uint16_t *>(p) = (uint16_t)pack_bf16x2(a, 0.f);
 }
 __device__ __forceinline__ float load1(const float *p) { return *p; }
 __device__ __forceinline__ float load1(const bf16_t *p) {
