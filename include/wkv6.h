@@ -1,9 +1,10 @@
 /*
  * wkv6.h -- C ABI of libwkv6_gfx950.so, the MI355X (gfx950) implementation of the WKV6
- * time-mixing operator.  Plain pointers and sizes only; every pointer except `state_map`
- * `workspace` arguments is a DEVICE pointer to a row-major contiguous array; all work is
+ * time-mixing operator.  Plain pointers and sizes only; every pointer (state_map and workspace
+ * included) is a DEVICE pointer to a row-major contiguous, 16-byte aligned array; all work is
  * enqueued on `stream` (a hipStream_t, may be NULL = default stream) and the calls return
- * without synchronising.  The library keeps no mutable global state: calls are re-entrant.
+ * without synchronising.  Calls are re-entrant: the only state the library keeps is a ring of
+ * flag words in its device image, one slot per call in flight (1024 slots).
  *
  * Each entry point names the reference interface it replaces (paths relative to the
  * reference tree infiy-quine/STAR-RWKV6).
