@@ -43,6 +43,7 @@ def parse():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
     ap.add_argument("--algo", default="auto", choices=["auto", "scan", "chunk", "chunk_only"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--plain-pair", action="store_true", help="time forward()+backward() without saved states")
     ap.add_argument("--cpu-tokens", type=int, default=0, help="tokens in the CPU baseline sample (0 = default)")
     ap.add_argument("--seed", type=int, default=0)
     return ap.parse_args()
@@ -105,13 +106,27 @@ def main():
     stream = torch.cuda.current_stream().cuda_stream
     P = lambda t: t.data_ptr()
 
+    # the pair a training step uses (the torch autograd.Function does the same): the forward saves the
+    # per-chunk states the backward would otherwise recompute; --plain-pair times the two calls the
+    # reference's binding corresponds to (forward(r..y), backward(r..gu)) instead
+    nsave = 0 if a.plain_pair else lib.wkv6_saved_bytes(code, algo, B, T, C, H)
+    saved = torch.empty(max(nsave, 16), dtype=torch.uint8, device=dev)
+
     def fwd():
-        _native.check(lib.wkv6_forward_ex(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(y),
-                                          P(fws), fws_bytes))
+        if nsave:
+            _native.check(lib.wkv6_forward_save(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(y),
+                                                P(saved), nsave))
+        else:
+            _native.check(lib.wkv6_forward_ex(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(y),
+                                              P(fws), fws_bytes))
 
     def bwd():
-        _native.check(lib.wkv6_backward_ex(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy),
-                                           P(gr), P(gk), P(gv), P(gw), P(gu_part), P(bws), bws_bytes))
+        if nsave:
+            _native.check(lib.wkv6_backward_saved(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy),
+                                                  P(gr), P(gk), P(gv), P(gw), P(gu_part), P(saved), nsave))
+        else:
+            _native.check(lib.wkv6_backward_ex(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy),
+                                               P(gr), P(gk), P(gv), P(gw), P(gu_part), P(bws), bws_bytes))
         return torch.sum(gu_part, 0)
 
     for _ in range(a.warmup):
@@ -162,7 +177,8 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dt_name, "data": "synthetic",
         "config": {"workload": "%s: WKV6 fwd+bwd B=%d T=%d C=%d H=%d N=%d %s I/O fp32 state" % (
-            a.workload, B, T, C, H, N, dt_name), "algo": algo_used, "tokens_per_step": tokens},
+            a.workload, B, T, C, H, N, dt_name), "algo": algo_used, "tokens_per_step": tokens,
+            "calls": "forward+backward" if (a.plain_pair or not nsave) else "forward_save+backward_saved"},
         "roofline": {
             "bound": "hbm", "kernel": "wkv6_%s (%s)" % ("backward" if dom == "bwd" else "forward", algo_used),
             "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,

@@ -111,6 +111,22 @@ int wkv6_backward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, in
                      void *workspace, size_t workspace_bytes);
 size_t wkv6_backward_workspace_bytes_ex(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H);
 
+/* Training pair: a forward that also saves what the backward can reuse (with the chunked kernels:
+ * the fp32 state at every 64-token chunk start), and the backward that consumes it and therefore
+ * skips its own forward state sweep.  `saved` is caller-owned device memory of wkv6_saved_bytes()
+ * bytes (0 = this path saves nothing; pass NULL), must be left untouched between the two calls,
+ * and serves the backward as its workspace too.  No counterpart in the reference, whose backward
+ * recomputes everything from the inputs (rwkv_kernel/torch_rwkv_kernel.py:33 saves only r,k,v,w,u). */
+size_t wkv6_saved_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H);
+int wkv6_forward_save(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                      const void *r, const void *k, const void *v, const void *w, const void *u,
+                      void *y, void *saved, size_t saved_bytes);
+int wkv6_backward_saved(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                        const void *r, const void *k, const void *v, const void *w, const void *u,
+                        const void *gy,
+                        void *gr, void *gk, void *gv, void *gw, void *gu,
+                        void *saved, size_t saved_bytes);
+
 /* ---- XLA custom-call surface (replaces the pybind module `gpu_ops`,
  * rwkv_kernel/jax_kernel/gpu_ops.cpp:20-43) ---------------------------------------------- */
 

@@ -101,12 +101,11 @@ size_t wkv6_forward_workspace_bytes(int dtype, int algo, int64_t B, int64_t T, i
     return 0;
 }
 
-int wkv6_forward_with_state_ex(void *stream, int dtype, int state_dtype, int algo,
-                               int64_t B, int64_t T, int64_t C, int64_t H,
-                               int has_init_state, const int64_t *state_map,
-                               const void *r, const void *k, const void *v, const void *w, const void *u,
-                               const void *s, void *y, void *ys, void *workspace, size_t workspace_bytes) {
-    (void)workspace; (void)workspace_bytes;
+static int forward_impl(void *stream, int dtype, int state_dtype, int algo,
+                        int64_t B, int64_t T, int64_t C, int64_t H,
+                        int has_init_state, const int64_t *state_map,
+                        const void *r, const void *k, const void *v, const void *w, const void *u,
+                        const void *s, void *y, void *ys, void *saved) {
     int rc = check_shape(dtype, B, T, C, H);
     if (rc != WKV6_OK) return rc;
     if (!r || !k || !v || !w || !u || !y) return WKV6_ERR_ARG;
@@ -126,11 +125,38 @@ int wkv6_forward_with_state_ex(void *stream, int dtype, int state_dtype, int alg
     FlagSlot slot;
     hipError_t e = take_flag_slot(&slot);
     if (e != hipSuccess) return finish(e);
-    e = wkv6::chunk_forward(st, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys, slot.ptr, slot.epoch);
+    e = wkv6::chunk_forward(st, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys, saved, slot.ptr, slot.epoch);
     if (e != hipSuccess || algo == WKV6_ALGO_CHUNK_ONLY) return finish(e);
     // exact per-timestep kernel behind the gate: a no-op unless the chunked kernel raised the flag
     return finish(wkv6::scan_forward(st, dtype, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys,
                                      wkv6::Gate{slot.ptr, slot.epoch}));
+}
+
+int wkv6_forward_with_state_ex(void *stream, int dtype, int state_dtype, int algo,
+                               int64_t B, int64_t T, int64_t C, int64_t H,
+                               int has_init_state, const int64_t *state_map,
+                               const void *r, const void *k, const void *v, const void *w, const void *u,
+                               const void *s, void *y, void *ys, void *workspace, size_t workspace_bytes) {
+    (void)workspace; (void)workspace_bytes;
+    return forward_impl(stream, dtype, state_dtype, algo, B, T, C, H, has_init_state, state_map, r, k, v, w, u, s, y, ys,
+                        nullptr);
+}
+
+size_t wkv6_saved_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
+    if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
+    const bool chunk = ((algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY) && chunk_possible(dtype, T, C)) ||
+                       (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
+    // sized so that the guarded per-timestep pass of the backward can use the same buffer
+    return chunk ? wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H) : 0;
+}
+
+int wkv6_forward_save(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                      const void *r, const void *k, const void *v, const void *w, const void *u,
+                      void *y, void *saved, size_t saved_bytes) {
+    const size_t need = wkv6_saved_bytes(dtype, algo, B, T, C, H);
+    if (need > 0 && (!saved || saved_bytes < need || !aligned16(saved))) return WKV6_ERR_WORKSPACE;
+    return forward_impl(stream, dtype, out_type(dtype), algo, B, T, C, H, 0, nullptr, r, k, v, w, u, nullptr, y, nullptr,
+                        need > 0 ? saved : nullptr);
 }
 
 int wkv6_forward_with_state(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
@@ -170,9 +196,10 @@ size_t wkv6_backward_workspace_bytes(int dtype, int64_t B, int64_t T, int64_t C,
     return wkv6_backward_workspace_bytes_ex(dtype, WKV6_ALGO_AUTO, B, T, C, H);
 }
 
-int wkv6_backward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
-                     const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
-                     void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, size_t workspace_bytes) {
+static int backward_impl(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                         const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                         void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, size_t workspace_bytes,
+                         bool states_ready) {
     int rc = check_shape(dtype, B, T, C, H);
     if (rc != WKV6_OK) return rc;
     if (!r || !k || !v || !w || !u || !gy || !gr || !gk || !gv || !gw || !gu) return WKV6_ERR_ARG;
@@ -191,10 +218,26 @@ int wkv6_backward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, in
     FlagSlot slot;
     hipError_t e = take_flag_slot(&slot);
     if (e != hipSuccess) return finish(e);
-    e = wkv6::chunk_backward(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace, false, slot.ptr, slot.epoch);
+    e = wkv6::chunk_backward(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace, states_ready, slot.ptr, slot.epoch);
     if (e != hipSuccess || algo == WKV6_ALGO_CHUNK_ONLY) return finish(e);
     return finish(wkv6::scan_backward(st, dtype, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace,
                                       wkv6::Gate{slot.ptr, slot.epoch}));
+}
+
+int wkv6_backward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                     const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                     void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, size_t workspace_bytes) {
+    return backward_impl(stream, dtype, algo, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace,
+                         workspace_bytes, false);
+}
+
+int wkv6_backward_saved(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                        const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                        void *gr, void *gk, void *gv, void *gw, void *gu, void *saved, size_t saved_bytes) {
+    // `saved` doubles as the workspace: the guarded per-timestep pass only runs when the chunked
+    // results (and with them the saved states) are discarded anyway
+    return backward_impl(stream, dtype, algo, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, saved, saved_bytes,
+                         wkv6_saved_bytes(dtype, algo, B, T, C, H) > 0);
 }
 
 int wkv6_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,

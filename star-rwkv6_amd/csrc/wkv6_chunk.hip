@@ -22,6 +22,8 @@
 #include "wkv6_common.h"
 #include "wkv6_kernels.h"
 
+#include <type_traits>
+
 namespace wkv6 {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -34,6 +36,8 @@ constexpr int CL = 64;   // tokens per chunk
 constexpr int LDA = 68;  // row pitch (elements) of [token][channel] operand arrays: 136 B, conflict-free 8-byte fragment reads
 constexpr int LDT = 72;  // row pitch (elements) of [channel][token] operand arrays: 144 B, 16-byte aligned rows
 constexpr float kWildLimit = 64.f;
+constexpr float kLog2e = 1.4426950408889634f;
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }   // v_exp_f32
 
 __device__ __forceinline__ bf16x8 make_bf16x8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
     const u32x4 t = {a, b, c, d};
@@ -63,6 +67,13 @@ __device__ __forceinline__ f32x4 mfma16(s16x4 a, s16x4 b, f32x4 c) {
 #define WKV6_SETTLE_ASM "s_nop 15"
 __device__ __forceinline__ void chain_gap(f32x4 &a) { asm volatile("s_nop 7" : "+v"(a)); }
 __device__ __forceinline__ void settle(f32x4 &a) { asm volatile(WKV6_SETTLE_ASM : "+v"(a)); }
+__device__ __forceinline__ void settle(f32x4 &a, f32x4 &b) { asm volatile(WKV6_SETTLE_ASM : "+v"(a), "+v"(b)); }
+__device__ __forceinline__ void settle(f32x4 &a, f32x4 &b, f32x4 (&g1)[4]) {
+    asm volatile(WKV6_SETTLE_ASM : "+v"(a), "+v"(b), "+v"(g1[0]), "+v"(g1[1]), "+v"(g1[2]), "+v"(g1[3]));
+}
+__device__ __forceinline__ void settle(f32x4 &a, f32x4 (&g1)[4]) {
+    asm volatile(WKV6_SETTLE_ASM : "+v"(a), "+v"(g1[0]), "+v"(g1[1]), "+v"(g1[2]), "+v"(g1[3]));
+}
 __device__ __forceinline__ void settle(f32x4 &a, f32x4 &b, f32x4 &c) {
     asm volatile(WKV6_SETTLE_ASM : "+v"(a), "+v"(b), "+v"(c));
 }
@@ -136,12 +147,14 @@ struct alignas(16) FwdBuf {
     float ruk[CL];          // sum_j r u k per token
 };
 
-template <typename Ts>
+// kSave: also write the state at every chunk start to `ckpt` (fp32, [b][h][chunk][j][i]) for the
+// backward pass, which then skips its own forward sweep.
+template <typename Ts, bool kSave>
 __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
         const bf16_t *__restrict__ r, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v,
         const bf16_t *__restrict__ w, const bf16_t *__restrict__ u,
         const Ts *__restrict__ s0, const int64_t *__restrict__ map,
-        bf16_t *__restrict__ y, Ts *__restrict__ sT,
+        bf16_t *__restrict__ y, Ts *__restrict__ sT, float *__restrict__ ckpt,
         unsigned long long *__restrict__ wild_flag, unsigned long long epoch)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -170,6 +183,13 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
         }
         bf16_t *y_h = y + base;
         for (int c = 0; c < nchunk; ++c) {
+            if (kSave) {
+                float *dst = ckpt + ((int64_t)blockIdx.x * nchunk + c) * (kN * kN) + 16 * q + l16;
+#pragma unroll
+                for (int m = 0; m < 4; ++m)
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) dst[(16 * m + 4 * g + rr) * kN] = S[m][rr];
+            }
             __syncthreads();
             const FwdBuf &B = buf[c & 1];
             const int t0 = c * CL;
@@ -326,7 +346,7 @@ struct alignas(16) BwdBuf {
     float fr[kN][LDFR];      // fr[j][20p + t] = exp(-c_t) of tile p, t = 0..16
     float g[4][kN];
     float ruk[CL];
-    float vgy[CL];
+    float vgyw[4][16];       // <v_t, gy_t> of the tile in flight, one private copy per consumer wave
 };
 
 // fragment of a global (B,T,C) bf16 tensor row for a 16x16x32 MFMA, same k-slot order as frag_tc
@@ -363,7 +383,18 @@ __device__ __forceinline__ bf16x8 pick4(const bf16x8 &a0, const bf16x8 &a1, cons
     return make_bf16x8(o[0], o[1], o[2], o[3]);
 }
 
-template <bool kSweepStates>
+// kRagged: T is not a multiple of 16, so the last tile has rows past the end.  The common
+// kRagged = false build has no per-lane predicates in the tile loops at all: with them every tile
+// body splits into several basic blocks, the compiler sinks the early-issued loads back next to
+// their uses and, since vmcnt is a single in-order counter, makes each tile wait for the previous
+// tile's stores to be acknowledged.
+#ifdef WKV6_TIMING
+#define WKV6_STAMP() do { if (blockIdx.x == 0 && lane == 0 && dbg_n < 250) dbg[wave * 256 + dbg_n++] = __builtin_readcyclecounter(); } while (0)
+#else
+#define WKV6_STAMP() do { } while (0)
+#endif
+
+template <bool kSweepStates, bool kRagged>
 __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
         const bf16_t *__restrict__ r, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v,
         const bf16_t *__restrict__ w, const bf16_t *__restrict__ u, const bf16_t *__restrict__ gy,
@@ -381,6 +412,10 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
     const int nchunk = (T + CL - 1) / CL;
     const int nitem = kSweepStates ? 2 * nchunk : nchunk;   // work items: [phase 1 chunks 0..n-1] then phase 2 chunks n-1..0
     float *ck = ckpt + (int64_t)blockIdx.x * nchunk * (kN * kN);
+#ifdef WKV6_TIMING
+    long long *dbg = reinterpret_cast<long long *>(ckpt + (int64_t)gridDim.x * nchunk * (kN * kN));
+    int dbg_n = 0;
+#endif
 
     if (wave < 4) {
         // ------------------------------ consumer ------------------------------
@@ -414,9 +449,10 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
             if (nchunk >= 1) ++item;   // account for the `break` above skipping the increment
         }
         // phase 2
-        f32x4 Gi[4], Gj[4];   // Gi: rows j, column i = col.   Gj: rows i, column j = col.
+        float (*vgyw)[16] = buf[0].vgyw;
+        f32x4 Gj[4];   // reverse state, rows i, column j = col (the copy with rows j lives in waves 4..7)
 #pragma unroll
-        for (int m = 0; m < 4; ++m) { Gi[m] = (f32x4){0.f, 0.f, 0.f, 0.f}; Gj[m] = Gi[m]; }
+        for (int m = 0; m < 4; ++m) Gj[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
         const float uj = load1(u + h * kN + col);
         float gu_acc = 0.f;
         const uint16_t *r16 = reinterpret_cast<const uint16_t *>(r) + base;
@@ -424,7 +460,19 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
         const uint16_t *v16 = reinterpret_cast<const uint16_t *>(v) + base;
         const uint16_t *w16 = reinterpret_cast<const uint16_t *>(w) + base;
         const uint16_t *g16 = reinterpret_cast<const uint16_t *>(gy) + base;
-        bf16_t *gr_h = gr + base, *gk_h = gk + base, *gv_h = gv + base, *gw_h = gw + base;
+        bf16_t *gr_h = gr + base, *gk_h = gk + base, *gw_h = gw + base;
+        // Software pipeline over the tiles: the gY / V fragments of the NEXT tile (possibly the top
+        // tile of the next chunk) are requested as soon as the MFMAs of the current one have consumed
+        // theirs, so that the epilogue covers their latency.  They land in their own registers and are
+        // moved over at the top of the next iteration.  Rows past T are read from row T-1: they only
+        // ever meet zero operands and are never stored.
+        auto rowoff = [&](int t) { return (uint32_t)(kRagged ? min(t, T - 1) : t) * (uint32_t)C; };
+        bf16x8 gf0, gf1, vf0, vf1, ngf0, ngf1, nvf0, nvf1;
+        auto load_frags = [&](int tile_t0) {
+            const uint32_t o = rowoff(tile_t0 + l16);
+            ngf0 = frag_global(g16 + o, 0, g); ngf1 = frag_global(g16 + o, 1, g);
+            nvf0 = frag_global(v16 + o, 0, g); nvf1 = frag_global(v16 + o, 1, g);
+        };
         for (int c = nchunk - 1; c >= 0; --c, ++item) {
             // forward state at the chunk start, straight from the checkpoint (written by this same lane)
             f32x4 S[4];
@@ -436,7 +484,9 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                     S[m] = (f32x4){x.x, x.y, x.z, x.w};
                 }
             }
+            WKV6_STAMP();
             __syncthreads();
+            WKV6_STAMP();
             const BwdBuf &B = buf[item & 1];
             const int t0 = c * CL;
             // states at the four tile starts as packed bf16 operands
@@ -453,23 +503,10 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                 for (int m = 0; m < 4; ++m) { S[m][0] *= gq; S[m][1] *= gq; S[m][2] *= gq; S[m][3] *= gq; }
                 SopL[p + 1] = acc_as_operand(S[0], S[1]); SopH[p + 1] = acc_as_operand(S[2], S[3]);
             }
-            // Software pipeline over the tiles: the gY / V fragments of the next tile are requested
-            // as soon as the MFMAs of the current one have consumed them, so that the epilogue
-            // covers their latency; rows past T are read from row T-1 (they only ever meet zero
-            // operands) and never stored.
-            auto rowoff = [&](int t) { return (uint32_t)min(t, T - 1) * (uint32_t)C; };
-            // (the next tile's fragments land in their own registers and are moved over at the end of
-            // the iteration: loading straight into registers that MFMAs issued a few cycles earlier
-            // still name as sources gave wrong products on gfx950)
-            bf16x8 gf0, gf1, vf0, vf1, ngf0, ngf1, nvf0, nvf1;
-            auto load_frags = [&](int p) {
-                const uint32_t o = rowoff(t0 + 16 * p + l16);
-                ngf0 = frag_global(g16 + o, 0, g); ngf1 = frag_global(g16 + o, 1, g);
-                nvf0 = frag_global(v16 + o, 0, g); nvf1 = frag_global(v16 + o, 1, g);
-            };
             int ptop = 3;
             while (ptop > 0 && t0 + 16 * ptop >= T) --ptop;
-            load_frags(ptop);
+            if (c == nchunk - 1) load_frags(t0 + 16 * ptop);   // later chunks: requested by the previous chunk's last tile
+            WKV6_STAMP();
 #pragma unroll 1
             for (int p = ptop; p >= 0; --p) {
                 gf0 = ngf0; gf1 = ngf1; vf0 = nvf0; vf1 = nvf1;
@@ -485,22 +522,22 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                     rraw[rr] = bf16_bits_to_float(r16[o]); kraw[rr] = bf16_bits_to_float(k16[o]);
                     wraw[rr] = bf16_bits_to_float(w16[o]);
                 }
-                const bf16x8 rf0 = frag_tc(B.rt, row, 0, g), rf1 = frag_tc(B.rt, row, 1, g);
-                const bf16x8 kf0 = frag_tc(B.kt, row, 0, g), kf1 = frag_tc(B.kt, row, 1, g);
-                const s16x4 rtq = frag_ct(B.rtT, col, tk), ktq = frag_ct(B.ktT, col, tk), gyq = frag_ct(B.gyT, col, tk);
+                const s16x4 rtq = frag_ct(B.rtT, col, tk), ktq = frag_ct(B.ktT, col, tk);
                 // 16x16 intra-tile matrices
-                f32x4 dA = {0.f, 0.f, 0.f, 0.f}, dAT = dA, A = dA;
+                f32x4 dA = {0.f, 0.f, 0.f, 0.f}, dAT = dA;
                 dA = mfma32(gf0, vf0, dA);   dA = mfma32(gf1, vf1, dA);     // rows t, col s
                 dAT = mfma32(vf0, gf0, dAT); dAT = mfma32(vf1, gf1, dAT);   // rows s, col t
-                A = mfma32(rf0, kf0, A);     A = mfma32(rf1, kf1, A);       // rows t, col s
-                const float rukv = B.ruk[row];
-                settle(dA, dAT, A);
+                settle(dA, dAT);
+                // the diagonal of dA is <v_t, gy_t>: lanes holding it publish it to this wave's LDS slot
+                if ((l16 >> 2) == g) {
+                    const int rs = l16 & 3;
+                    vgyw[q][l16] = (rs == 0) ? dA[0] : (rs == 1) ? dA[1] : (rs == 2) ? dA[2] : dA[3];
+                }
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr) {
                     const int x = 4 * g + rr;
                     dA[rr] = (x > l16) ? dA[rr] : 0.f;
                     dAT[rr] = (l16 > x) ? dAT[rr] : 0.f;
-                    A[rr] = (x > l16) ? A[rr] : ((x == l16) ? rukv : 0.f);
                 }
                 // X (rows t, col j)
                 f32x4 X = {0.f, 0.f, 0.f, 0.f};
@@ -517,44 +554,37 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                 chain_gap(W);
                 W = mfma32(vf0, acc_as_operand(Gj[0], Gj[1]), W);
                 W = mfma32(vf1, acc_as_operand(Gj[2], Gj[3]), W);
-                if (p > 0) load_frags(p - 1);
-                // gv (rows s, col i); Gi decayed first
+                // next tile: p-1 of this chunk, else the top tile of the chunk before (always full),
+                // else (very last tile of the sweep) this one again, unused
+                load_frags(p > 0 ? t0 + 16 * (p - 1) : (c > 0 ? t0 - 16 : t0));
+                // G <- diag(g) G + R~^T gY   (this wave's copy)
 #pragma unroll
-                for (int m = 0; m < 4; ++m) {
-                    const float4 gg = *reinterpret_cast<const float4 *>(&B.g[p][16 * m + 4 * g]);
-                    Gi[m][0] *= gg.x; Gi[m][1] *= gg.y; Gi[m][2] *= gg.z; Gi[m][3] *= gg.w;
-                }
-                f32x4 GV = {0.f, 0.f, 0.f, 0.f};
-                GV = mfma16(pack4(A), gyq, GV);
-                chain_gap(GV);
-                GV = mfma32(kf0, acc_as_operand(Gi[0], Gi[1]), GV);
-                GV = mfma32(kf1, acc_as_operand(Gi[2], Gi[3]), GV);
-                // G <- diag(g) G + R~^T gY   (both copies)
-#pragma unroll
-                for (int m = 0; m < 4; ++m) {
-                    Gi[m] = mfma16(frag_ct(B.rtT, 16 * m + l16, tk), gyq, Gi[m]);
-                    Gj[m] = mfma16(frag_ct(B.gyT, 16 * m + l16, tk), rtq, Gj[m]);
-                }
-                settle(X, W, GV, Gi, Gj);   // all read by VALU code from here on
+                for (int m = 0; m < 4; ++m) Gj[m] = mfma16(frag_ct(B.gyT, 16 * m + l16, tk), rtq, Gj[m]);
+                settle(X, W, Gj);   // all read by VALU code from here on
                 // tile-boundary term E[j] = sum_i S0[j][i] G_new[j][i]
-                float E = 0.f;
+                float E;
                 {
-                    float sl[8], sh[8];
+                    float sl[8], sh[8], e0 = 0.f, e1 = 0.f, e2 = 0.f, e3 = 0.f;
                     unpack8(sL, sl); unpack8(sH, sh);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        E = fmaf(sl[e], Gj[0][e], E); E = fmaf(sl[4 + e], Gj[1][e], E);
-                        E = fmaf(sh[e], Gj[2][e], E); E = fmaf(sh[4 + e], Gj[3][e], E);
+                        e0 = fmaf(sl[e], Gj[0][e], e0); e1 = fmaf(sl[4 + e], Gj[1][e], e1);
+                        e2 = fmaf(sh[e], Gj[2][e], e2); e3 = fmaf(sh[4 + e], Gj[3][e], e3);
                     }
+                    E = (e0 + e1) + (e2 + e3);
                     E += __shfl_xor(E, 16);
                     E += __shfl_xor(E, 32);
                 }
                 // epilogue on the accumulator rows (tokens tk..tk+3, channel col)
                 const float4 f4 = *reinterpret_cast<const float4 *>(&B.fr[col][20 * p + 4 * g]);
                 const float f5 = B.fr[col][20 * p + 4 * g + 4];
-                const float4 vg4 = *reinterpret_cast<const float4 *>(&B.vgy[tk]);
+                const float4 vg4 = *reinterpret_cast<const float4 *>(&vgyw[q][4 * g]);
                 const float fr_[5] = {f4.x, f4.y, f4.z, f4.w, f5};
-                const float vg_[4] = {vg4.x, vg4.y, vg4.z, vg4.w};
+                float vg_[4] = {vg4.x, vg4.y, vg4.z, vg4.w};
+                if (kRagged) {
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) vg_[rr] = (t0 + tk + rr < T) ? vg_[rr] : 0.f;
+                }
                 float rt_[4], kt_[4], P[4], D[4], gro[4], gko[4];
                 unpack4(rtq, rt_); unpack4(ktq, kt_);
 #pragma unroll
@@ -578,11 +608,12 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                     // amplifying rounding residue); first and last token are zero by definition
                     float gwv = (ew >= 88.f || t == 0 || t == T - 1) ? 0.f : -ew * (pre - P[rr]);
                     pre += D[rr];
-                    if (t < T) {
+                    if (!kRagged || t < T) {
                         const uint32_t o = (uint32_t)t * (uint32_t)C + (uint32_t)col;
-                        store1(gr_h + o, gro[rr]); store1(gk_h + o, gko[rr]); store1(gw_h + o, gwv); store1(gv_h + o, GV[rr]);
+                        store1(gr_h + o, gro[rr]); store1(gk_h + o, gko[rr]); store1(gw_h + o, gwv);
                     }
                 }
+                WKV6_STAMP();
             }
         }
         // gu: fold the four lane groups (different tokens, same channel) with wavefront shuffles
@@ -593,32 +624,39 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
         // ------------------------------ producer ------------------------------
         const int p = wave - 4, ch = lane;
         const float uc = load1(u + h * kN + ch);
-        const uint16_t *r16 = reinterpret_cast<const uint16_t *>(r) + base + ch;
-        const uint16_t *k16 = reinterpret_cast<const uint16_t *>(k) + base + ch;
-        const uint16_t *v16 = reinterpret_cast<const uint16_t *>(v) + base + ch;
-        const uint16_t *w16 = reinterpret_cast<const uint16_t *>(w) + base + ch;
-        const uint16_t *g16 = reinterpret_cast<const uint16_t *>(gy) + base + ch;
+        const uint16_t *r16 = reinterpret_cast<const uint16_t *>(r) + base;   // uniform bases, 32-bit lane offsets
+        const uint16_t *k16 = reinterpret_cast<const uint16_t *>(k) + base;
+        const uint16_t *v16 = reinterpret_cast<const uint16_t *>(v) + base;
+        const uint16_t *w16 = reinterpret_cast<const uint16_t *>(w) + base;
+        const uint16_t *g16 = reinterpret_cast<const uint16_t *>(gy) + base;
         uint32_t qr[16], qk[16], qv[16], qw[16], qg[16];
         // item -> (chunk, full): phase 1 items need only k, v, w
         auto item_chunk = [&](int it) { return kSweepStates ? (it < nchunk ? it : 2 * nchunk - 1 - it) : nchunk - 1 - it; };
         auto item_full = [&](int it) { return kSweepStates ? it >= nchunk : true; };
+        // Tokens past the end read as r = k = v = gy = 0, w = -inf (exp(w) = 0, decay 1).  Without
+        // kRagged a tile is either entirely inside the sequence or entirely outside.
         auto prefetch = [&](int it) {
-            const int c = item_chunk(it);
+            const int tb = item_chunk(it) * CL + 16 * p;
             const bool full = item_full(it);
+            if (!kRagged && tb >= T) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) { qr[e] = 0u; qk[e] = 0u; qv[e] = 0u; qg[e] = 0u; qw[e] = 0xff80u; }
+                return;
+            }
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const int t = c * CL + 16 * p + e;
-                const bool ok = t < T;
-                const int64_t o = (int64_t)(ok ? t : T - 1) * C;
+                const int t = tb + e;
+                const bool ok = !kRagged || t < T;
+                const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * (uint32_t)C + (uint32_t)ch;
                 const uint32_t bb = k16[o], cc = v16[o], dd = w16[o];
                 qk[e] = ok ? bb : 0u; qv[e] = ok ? cc : 0u; qw[e] = ok ? dd : 0xff80u;
             }
             if (full) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    const int t = c * CL + 16 * p + e;
-                    const bool ok = t < T;
-                    const int64_t o = (int64_t)(ok ? t : T - 1) * C;
+                    const int t = tb + e;
+                    const bool ok = !kRagged || t < T;
+                    const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * (uint32_t)C + (uint32_t)ch;
                     const uint32_t a = r16[o], gg = g16[o];
                     qr[e] = ok ? a : 0u; qg[e] = ok ? gg : 0u;
                 }
@@ -630,12 +668,11 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
         auto prepare = [&](int it) {
             BwdBuf &B = buf[it & 1];
             const bool full = item_full(it);
-            float fr[16], fk[16], fw[16], pv[16];
+            float fr[16], fk[16], fw[16];
             uint32_t vbits[8], gbits[8];
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 fr[e] = bf16_bits_to_float(qr[e]); fk[e] = bf16_bits_to_float(qk[e]); fw[e] = bf16_bits_to_float(qw[e]);
-                pv[e] = bf16_bits_to_float(qv[e]) * bf16_bits_to_float(qg[e]);
             }
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
@@ -644,20 +681,21 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
             }
             if (it + 1 < nitem) prefetch(it + 1);
 
+            // exponents are kept in base 2 (one v_exp_f32 each, no extra scaling multiply)
             float xr[16], xk[16], pr[16], fa[17];
-            float cs = 0.f, pa = 1.f;
+            float cs2 = 0.f, pa = 1.f;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const float ew = fast_exp(fw[e]);
+                const float ew2 = exp2_fast(fw[e] * kLog2e) * kLog2e;   // exp(w) * log2(e)
                 fa[e] = pa;
                 xr[e] = fr[e] * pa;
-                cs += ew;
-                xk[e] = fk[e] * fast_exp(cs);
-                pa *= fast_exp(-ew);
+                cs2 += ew2;
+                xk[e] = fk[e] * exp2_fast(cs2);
+                pa *= exp2_fast(-ew2);
                 pr[e] = fr[e] * uc * fk[e];
             }
             fa[16] = pa;
-            if (__builtin_amdgcn_ballot_w64(!(cs <= kWildLimit)) != 0ull) {
+            if (__builtin_amdgcn_ballot_w64(!(cs2 <= kWildLimit * kLog2e)) != 0ull) {
                 if (lane == 0 && wild_flag != nullptr) *wild_flag = epoch;
             }
             uint32_t pk[8];
@@ -682,18 +720,66 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                     *reinterpret_cast<float4 *>(&B.fr[ch][20 * p + e]) = make_float4(fa[e], fa[e + 1], fa[e + 2], fa[e + 3]);
                 B.fr[ch][20 * p + 16] = fa[16];
                 const float tr = transpose_reduce16(pr, lane);
-                const float tv = transpose_reduce16(pv, lane);
-                if ((lane & 3) == 0) {
-                    B.ruk[16 * p + ((lane >> 2) & 15)] = tr;
-                    B.vgy[16 * p + ((lane >> 2) & 15)] = tv;
+                if ((lane & 3) == 0) B.ruk[16 * p + ((lane >> 2) & 15)] = tr;
+            }
+        };
+        // gv role (second half of the consumer work, on the waves the operand preparation leaves
+        // mostly idle): wave 4+q owns value columns i = 16q..16q+15 of the reverse state Gi (rows j).
+        const int g = lane >> 4, l16 = lane & 15;
+        const int col = 16 * p + l16;
+        f32x4 Gi[4];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) Gi[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        bf16_t *gv_h = gv + base;
+        auto gv_tiles = [&](int it) {
+            const BwdBuf &B = buf[it & 1];
+            const int t0 = item_chunk(it) * CL;
+            int ptop = 3;
+            while (ptop > 0 && t0 + 16 * ptop >= T) --ptop;
+#pragma unroll 1
+            for (int pp = ptop; pp >= 0; --pp) {
+                const int row = 16 * pp + l16, tk = 16 * pp + 4 * g;
+                const bf16x8 rf0 = frag_tc(B.rt, row, 0, g), rf1 = frag_tc(B.rt, row, 1, g);
+                const bf16x8 kf0 = frag_tc(B.kt, row, 0, g), kf1 = frag_tc(B.kt, row, 1, g);
+                const s16x4 gyq = frag_ct(B.gyT, col, tk);
+                const float rukv = B.ruk[row];
+                f32x4 A = {0.f, 0.f, 0.f, 0.f};
+                A = mfma32(rf0, kf0, A); A = mfma32(rf1, kf1, A);   // rows t, col s
+                settle(A);
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    const int x = 4 * g + rr;
+                    A[rr] = (x > l16) ? A[rr] : ((x == l16) ? rukv : 0.f);
+                }
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    const float4 gg = *reinterpret_cast<const float4 *>(&B.g[pp][16 * m + 4 * g]);
+                    Gi[m][0] *= gg.x; Gi[m][1] *= gg.y; Gi[m][2] *= gg.z; Gi[m][3] *= gg.w;
+                }
+                f32x4 GV = {0.f, 0.f, 0.f, 0.f};
+                GV = mfma16(pack4(A), gyq, GV);
+                chain_gap(GV);
+                GV = mfma32(kf0, acc_as_operand(Gi[0], Gi[1]), GV);
+                GV = mfma32(kf1, acc_as_operand(Gi[2], Gi[3]), GV);
+#pragma unroll
+                for (int m = 0; m < 4; ++m) Gi[m] = mfma16(frag_ct(B.rtT, 16 * m + l16, tk), gyq, Gi[m]);
+                settle(GV, Gi);
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    const int t = t0 + tk + rr;
+                    if (!kRagged || t < T) store1(gv_h + (uint32_t)t * (uint32_t)C + (uint32_t)col, GV[rr]);
                 }
             }
         };
         prefetch(0);
         prepare(0);
         for (int it = 0; it < nitem; ++it) {
+            WKV6_STAMP();
             __syncthreads();
+            WKV6_STAMP();
             if (it + 1 < nitem) prepare(it + 1);
+            WKV6_STAMP();
+            if (item_full(it)) gv_tiles(it);
         }
     }
 }
@@ -718,32 +804,30 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
                            (float *)workspace, wild_flag, epoch);
         return hipGetLastError();
     };
-    return states_ready ? launch(chunk_bwd_kernel<false>) : launch(chunk_bwd_kernel<true>);
+    const bool ragged = (T % 16) != 0;
+    if (states_ready) return ragged ? launch(chunk_bwd_kernel<false, true>) : launch(chunk_bwd_kernel<false, false>);
+    return ragged ? launch(chunk_bwd_kernel<true, true>) : launch(chunk_bwd_kernel<true, false>);
 }
 
 hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u,
-                         const void *s0, const int64_t *map, void *y, void *sT,
+                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states,
                          unsigned long long *wild_flag, unsigned long long epoch)
 {
     const size_t lds = 2 * sizeof(FwdBuf);
-    hipError_t e;
-    if (state_dtype == kF32) {
-        auto kern = chunk_fwd_kernel<float>;
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    auto launch = [&](auto kern, auto *state_tag) -> hipError_t {
+        typedef std::remove_pointer_t<decltype(state_tag)> Ts;
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(512), lds, st, (int)T, (int)H,
                            (const bf16_t *)r, (const bf16_t *)k, (const bf16_t *)v, (const bf16_t *)w, (const bf16_t *)u,
-                           (const float *)s0, map, (bf16_t *)y, (float *)sT, wild_flag, epoch);
-    } else {
-        auto kern = chunk_fwd_kernel<bf16_t>;
-        e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(512), lds, st, (int)T, (int)H,
-                           (const bf16_t *)r, (const bf16_t *)k, (const bf16_t *)v, (const bf16_t *)w, (const bf16_t *)u,
-                           (const bf16_t *)s0, map, (bf16_t *)y, (bf16_t *)sT, wild_flag, epoch);
-    }
-    return hipGetLastError();
+                           (const Ts *)s0, map, (bf16_t *)y, (Ts *)sT, (float *)saved_states, wild_flag, epoch);
+        return hipGetLastError();
+    };
+    const bool save = saved_states != nullptr;
+    if (state_dtype == kF32)
+        return save ? launch(chunk_fwd_kernel<float, true>, (float *)nullptr) : launch(chunk_fwd_kernel<float, false>, (float *)nullptr);
+    return save ? launch(chunk_fwd_kernel<bf16_t, true>, (bf16_t *)nullptr) : launch(chunk_fwd_kernel<bf16_t, false>, (bf16_t *)nullptr);
 }
 
 }  // namespace wkv6

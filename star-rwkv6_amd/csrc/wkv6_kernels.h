@@ -30,7 +30,7 @@ hipError_t scan_backward(hipStream_t st, int dtype, int64_t B, int64_t T, int64_
 // --- chunk-parallel MFMA form, bf16 tensors only (wkv6_chunk.hip) ---
 hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u,
-                         const void *s0, const int64_t *map, void *y, void *sT,
+                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states,
                          unsigned long long *wild_flag, unsigned long long epoch);
 
 size_t chunk_backward_workspace_bytes(int64_t B, int64_t T, int64_t H);

@@ -31,7 +31,11 @@ def _ptr(t):
 
 
 class _WKV6(torch.autograd.Function):
-    """Stateless operator with gradients (rwkv_kernel/torch_rwkv_kernel.py:14-75)."""
+    """Stateless operator with gradients (rwkv_kernel/torch_rwkv_kernel.py:14-75).
+
+    When a gradient will be needed and the library has something worth keeping for it (the chunked
+    kernels' per-chunk states), the forward runs as wkv6_forward_save and the backward as
+    wkv6_backward_saved; otherwise the plain pair the reference's binding corresponds to."""
 
     @staticmethod
     def forward(ctx, B, T, C, H, r, k, v, w, u, algo):
@@ -43,14 +47,22 @@ class _WKV6(torch.autograd.Function):
                 assert x.is_contiguous()
             ctx.dims = (B, T, C, H)
             ctx.algo = algo
-            ctx.save_for_backward(r, k, v, w, u)
+            code = _DTYPE_CODE[r.dtype]
             y = torch.empty((B, T, C), device=r.device, dtype=_out_dtype(r.dtype))
+            saved = None
             with torch.cuda.device(r.device):
-                ws_bytes = lib.wkv6_forward_workspace_bytes(_DTYPE_CODE[r.dtype], algo, B, T, C, H)
-                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=r.device) if ws_bytes else None
-                _native.check(lib.wkv6_forward_ex(_stream(), _DTYPE_CODE[r.dtype], algo, B, T, C, H,
-                                                  _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(y),
-                                                  _ptr(ws), ws_bytes))
+                need_grad = any(ctx.needs_input_grad[4:9])
+                nsave = lib.wkv6_saved_bytes(code, algo, B, T, C, H) if need_grad else 0
+                if nsave:
+                    saved = torch.empty(nsave, dtype=torch.uint8, device=r.device)
+                    _native.check(lib.wkv6_forward_save(_stream(), code, algo, B, T, C, H,
+                                                        _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(y),
+                                                        _ptr(saved), nsave))
+                else:
+                    _native.check(lib.wkv6_forward_ex(_stream(), code, algo, B, T, C, H,
+                                                      _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(y), None, 0))
+            ctx.saved_states = saved
+            ctx.save_for_backward(r, k, v, w, u)
             return y
 
     @staticmethod
@@ -66,14 +78,18 @@ class _WKV6(torch.autograd.Function):
             gr, gk, gv, gw = (torch.empty((B, T, C), device=gy.device, dtype=odt) for _ in range(4))
             gu = torch.empty((B, C), device=gy.device, dtype=odt)
             code = _DTYPE_CODE[r.dtype]
+            args = (_ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(gy), _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu))
             with torch.cuda.device(gy.device):
-                ws_bytes = lib.wkv6_backward_workspace_bytes_ex(code, ctx.algo, B, T, C, H)
-                ws = torch.empty(ws_bytes, dtype=torch.uint8, device=gy.device) if ws_bytes else None
-                _native.check(lib.wkv6_backward_ex(_stream(), code, ctx.algo, B, T, C, H,
-                                                   _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(gy),
-                                                   _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu),
-                                                   _ptr(ws), ws_bytes))
-            # per-batch partials -> (H, N), rwkv_kernel/torch_rwkv_kernel.py:73
+                saved = ctx.saved_states
+                if saved is not None:
+                    ctx.saved_states = None
+                    _native.check(lib.wkv6_backward_saved(_stream(), code, ctx.algo, B, T, C, H, *args,
+                                                          _ptr(saved), saved.numel()))
+                else:
+                    ws_bytes = lib.wkv6_backward_workspace_bytes_ex(code, ctx.algo, B, T, C, H)
+                    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=gy.device) if ws_bytes else None
+                    _native.check(lib.wkv6_backward_ex(_stream(), code, ctx.algo, B, T, C, H, *args, _ptr(ws), ws_bytes))
+            # per-batch partials -> shape of u, rwkv_kernel/torch_rwkv_kernel.py:73
             gu = torch.sum(gu, 0).reshape(u.shape)
             return (None, None, None, None, gr, gk, gv, gw, gu, None)
 

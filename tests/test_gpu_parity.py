@@ -286,3 +286,46 @@ def test_chunk_matches_scan_on_padding_mask(op, oracle):
     op.algo = CHUNK
     y, _ = op(*dev)
     check_close("y", y, oracle.forward_c(*ref, N)[0], torch.bfloat16)
+
+
+def test_plain_backward_equals_saved_backward(op, oracle):
+    # wkv6_backward (recomputes the chunk states) and wkv6_backward_saved (takes them from the
+    # forward) agree to rounding (the two sweeps scale k differently before the bf16 rounding),
+    # and both meet the tolerance against the oracle
+    from rwkv_kernel import _native
+
+    lib = _native.load()
+    B, T, H, N = 2, 320, 2, 64
+    C = H * N
+    ins = oracle.make_inputs(B, T, H, N, 77)
+    dev, _ = cast_inputs(ins[:6], torch.bfloat16)
+    r, k, v, w, u, gy = dev
+    st = torch.cuda.current_stream().cuda_stream
+    P = lambda t: t.data_ptr()
+    res = []
+    for mode in ("plain", "saved"):
+        y = torch.empty_like(r)
+        outs = [torch.empty_like(r) for _ in range(4)] + [torch.empty(B, C, dtype=r.dtype, device="cuda")]
+        n = lib.wkv6_saved_bytes(_native.BF16, CHUNK, B, T, C, H)
+        assert n == lib.wkv6_backward_workspace_bytes_ex(_native.BF16, CHUNK, B, T, C, H) > 0
+        buf = torch.empty(n, dtype=torch.uint8, device="cuda")
+        if mode == "plain":
+            _native.check(lib.wkv6_forward_ex(st, _native.BF16, CHUNK, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(y), None, 0))
+            _native.check(lib.wkv6_backward_ex(st, _native.BF16, CHUNK, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy),
+                                               *[P(o) for o in outs], P(buf), n))
+        else:
+            _native.check(lib.wkv6_forward_save(st, _native.BF16, CHUNK, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(y), P(buf), n))
+            _native.check(lib.wkv6_backward_saved(st, _native.BF16, CHUNK, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy),
+                                                  *[P(o) for o in outs], P(buf), n))
+        torch.cuda.synchronize()
+        res.append([y] + outs)
+    assert torch.equal(res[0][0], res[1][0])
+    _, ref = cast_inputs(ins[:6], torch.bfloat16)
+    g_ref = oracle.backward_c(*ref[:5], ref[5], N)
+    for which in res:
+        for name, g, gr in zip("gr gk gv gw".split(), which[1:5], g_ref):
+            check_close(name, g, gr, torch.bfloat16, is_grad=True)
+        check_close("gu", to_np(which[5]).sum(0).reshape(H, N), g_ref[4], torch.bfloat16, is_grad=True)
+    for a, b in zip(res[0][1:5], res[1][1:5]):
+        assert (a.float() - b.float()).abs().max() <= 5e-3 * b.float().abs().max()
+    assert lib.wkv6_saved_bytes(_native.F32, SCAN, B, T, C, H) == 0
