@@ -91,6 +91,12 @@ __device__ __forceinline__ float xor1(float x) {   // value of the neighbouring 
     return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0xB1, 0xF, 0xF, true));
 }
 
+// 16-bit load at a uniform base + 32-bit per-lane byte offset (lets the compiler use the
+// scalar-base addressing form instead of 64-bit per-lane address arithmetic)
+__device__ __forceinline__ uint32_t ld16(const void *base, uint32_t byteoff) {
+    return *reinterpret_cast<const uint16_t *>(reinterpret_cast<const char *>(base) + byteoff);
+}
+
 // A/B fragment of a [token][channel] array for one 16x16x32 MFMA covering channels [32h, 32h+32).
 // Lane group g = lane/16 takes the k-slots {32h+4g+e, 32h+16+4g+e : e<4}: the same channels its
 // accumulator registers hold when a 64x16 fp32 tile stack (rows 16m+4g+r) is reused as an operand.
@@ -141,7 +147,7 @@ __device__ __forceinline__ void store_rows_paired(uint16_t (*a)[LDA], int row0, 
 struct alignas(16) FwdBuf {
     uint16_t rt[CL][LDA];   // R~[t][j]
     uint16_t kt[CL][LDA];   // K~[t][j]
-    uint16_t kbT[kN][LDT];  // K^[t][j] stored [j][t]
+    uint16_t ktT[kN][LDT];  // K~[t][j] stored [j][t]  (K^ = g K~ is never formed: S <- g (S + K~^T V))
     uint16_t vT[kN][LDT];   // V[t][i]  stored [i][t]
     float g[4][kN];         // per-tile decay exp(-c_16)
     float ruk[CL];          // sum_j r u k per token
@@ -149,7 +155,7 @@ struct alignas(16) FwdBuf {
 
 // kSave: also write the state at every chunk start to `ckpt` (fp32, [b][h][chunk][j][i]) for the
 // backward pass, which then skips its own forward sweep.
-template <typename Ts, bool kSave>
+template <typename Ts, bool kSave, bool kRagged>
 __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
         const bf16_t *__restrict__ r, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v,
         const bf16_t *__restrict__ w, const bf16_t *__restrict__ u,
@@ -218,18 +224,19 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
                 // Y += A V : the masked A^T accumulator IS the A operand (row t = l16, k-slots s = 4g+r)
                 chain_gap(Y);
                 Y = mfma16(make_s16x4(pack_bf16x2(AT[0], AT[1]), pack_bf16x2(AT[2], AT[3])), vf, Y);
-                // S <- diag(g) S + K^T V
+                // S <- diag(g) (S + K~^T V)
+#pragma unroll
+                for (int m = 0; m < 4; ++m) S[m] = mfma16(frag_ct(B.ktT, 16 * m + l16, 16 * p + 4 * g), vf, S[m]);
+                settle(Y, S[0], S[1], S[2], S[3]);   // Y is stored, S scaled and converted by VALU code from here on
 #pragma unroll
                 for (int m = 0; m < 4; ++m) {
                     const float4 gg = *reinterpret_cast<const float4 *>(&B.g[p][16 * m + 4 * g]);
                     S[m][0] *= gg.x; S[m][1] *= gg.y; S[m][2] *= gg.z; S[m][3] *= gg.w;
-                    S[m] = mfma16(frag_ct(B.kbT, 16 * m + l16, 16 * p + 4 * g), vf, S[m]);
                 }
-                settle(Y, S[0], S[1], S[2], S[3]);   // Y is stored, S scaled and converted by VALU code from here on
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr) {
                     const int t = t0 + 16 * p + 4 * g + rr;
-                    if (t < T) store1(y_h + (uint32_t)t * (uint32_t)C + (uint32_t)(16 * q + l16), Y[rr]);
+                    if (!kRagged || t < T) store1(y_h + (uint32_t)t * (uint32_t)C + (uint32_t)(16 * q + l16), Y[rr]);
                 }
             }
         }
@@ -244,20 +251,24 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
         // ------------------------------ producer: operand preparation ------------------------------
         const int p = wave - 4, ch = lane;
         const float uc = load1(u + h * kN + ch);
-        const uint16_t *r16 = reinterpret_cast<const uint16_t *>(r) + base + ch;
-        const uint16_t *k16 = reinterpret_cast<const uint16_t *>(k) + base + ch;
-        const uint16_t *v16 = reinterpret_cast<const uint16_t *>(v) + base + ch;
-        const uint16_t *w16 = reinterpret_cast<const uint16_t *>(w) + base + ch;
+        const bf16_t *rb = r + base, *kb_ = k + base, *vb = v + base, *wb = w + base;   // uniform
+        const uint32_t rowbytes = (uint32_t)C * 2u;
         uint32_t qr[16], qk[16], qv[16], qw[16];
+        // Tokens past the end read as r = k = v = 0, w = -inf (exp(w) = 0, decay 1).  Without kRagged
+        // a tile is either entirely inside the sequence or entirely outside.
         auto prefetch = [&](int c) {
+            const int tb = c * CL + 16 * p;
+            if (!kRagged && tb >= T) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) { qr[e] = 0u; qk[e] = 0u; qv[e] = 0u; qw[e] = 0xff80u; }
+                return;
+            }
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                // rows past the end are read from the last valid row and replaced by neutral values
-                // (r = k = v = 0, w = -inf: exp(w) = 0, decay 1) without a branch
-                const int t = c * CL + 16 * p + e;
-                const bool ok = t < T;
-                const int64_t o = (int64_t)(ok ? t : T - 1) * C;
-                const uint32_t a = r16[o], bb = k16[o], cc = v16[o], dd = w16[o];
+                const int t = tb + e;
+                const bool ok = !kRagged || t < T;
+                const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes + 2u * (uint32_t)ch;
+                const uint32_t a = ld16(rb, o), bb = ld16(kb_, o), cc = ld16(vb, o), dd = ld16(wb, o);
                 qr[e] = ok ? a : 0u; qk[e] = ok ? bb : 0u; qv[e] = ok ? cc : 0u; qw[e] = ok ? dd : 0xff80u;
             }
         };
@@ -273,31 +284,28 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
             for (int e = 0; e < 8; ++e) vbits[e] = qv[2 * e] | (qv[2 * e + 1] << 16);
             if (c + 1 < nchunk) prefetch(c + 1);
 
-            float d[16], xr[16], xk[16], pr[16];
-            float cs = 0.f, pa = 1.f;
+            // exponents are kept in base 2 (one v_exp_f32 each, no extra scaling multiply)
+            float xr[16], xk[16], pr[16];
+            float cs2 = 0.f, pa = 1.f;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-                const float ew = fast_exp(fw[e]);
-                d[e] = fast_exp(-ew);
-                xr[e] = fr[e] * pa;          // r exp(-c_t)
-                cs += ew;
-                xk[e] = fk[e] * fast_exp(cs);  // k exp(+c_{t+1})
-                pa *= d[e];
+                const float ew2 = exp2_fast(fw[e] * kLog2e) * kLog2e;   // exp(w) * log2(e)
+                xr[e] = fr[e] * pa;               // r exp(-c_t)
+                cs2 += ew2;
+                xk[e] = fk[e] * exp2_fast(cs2);   // k exp(+c_{t+1})
+                pa *= exp2_fast(-ew2);
                 pr[e] = fr[e] * uc * fk[e];
             }
-            if (__builtin_amdgcn_ballot_w64(!(cs <= kWildLimit)) != 0ull) {
+            if (__builtin_amdgcn_ballot_w64(!(cs2 <= kWildLimit * kLog2e)) != 0ull) {
                 if (lane == 0 && wild_flag != nullptr) *wild_flag = epoch;
             }
             store_rows_paired(B.rt, 16 * p, lane, xr);
             store_rows_paired(B.kt, 16 * p, lane, xk);
-            float pb = 1.f;
-#pragma unroll
-            for (int e = 15; e >= 0; --e) { xk[e] = fk[e] * pb; pb *= d[e]; }   // k exp(-(c_16 - c_{t+1}))
             uint32_t kb[8];
 #pragma unroll
             for (int e = 0; e < 8; ++e) kb[e] = pack_bf16x2(xk[2 * e], xk[2 * e + 1]);
-            *reinterpret_cast<uint4 *>(&B.kbT[ch][16 * p]) = make_uint4(kb[0], kb[1], kb[2], kb[3]);
-            *reinterpret_cast<uint4 *>(&B.kbT[ch][16 * p + 8]) = make_uint4(kb[4], kb[5], kb[6], kb[7]);
+            *reinterpret_cast<uint4 *>(&B.ktT[ch][16 * p]) = make_uint4(kb[0], kb[1], kb[2], kb[3]);
+            *reinterpret_cast<uint4 *>(&B.ktT[ch][16 * p + 8]) = make_uint4(kb[4], kb[5], kb[6], kb[7]);
             *reinterpret_cast<uint4 *>(&B.vT[ch][16 * p]) = make_uint4(vbits[0], vbits[1], vbits[2], vbits[3]);
             *reinterpret_cast<uint4 *>(&B.vT[ch][16 * p + 8]) = make_uint4(vbits[4], vbits[5], vbits[6], vbits[7]);
             B.g[p][ch] = pa;
@@ -624,11 +632,8 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
         // ------------------------------ producer ------------------------------
         const int p = wave - 4, ch = lane;
         const float uc = load1(u + h * kN + ch);
-        const uint16_t *r16 = reinterpret_cast<const uint16_t *>(r) + base;   // uniform bases, 32-bit lane offsets
-        const uint16_t *k16 = reinterpret_cast<const uint16_t *>(k) + base;
-        const uint16_t *v16 = reinterpret_cast<const uint16_t *>(v) + base;
-        const uint16_t *w16 = reinterpret_cast<const uint16_t *>(w) + base;
-        const uint16_t *g16 = reinterpret_cast<const uint16_t *>(gy) + base;
+        const bf16_t *rb = r + base, *kb_ = k + base, *vb = v + base, *wb = w + base, *gb = gy + base;   // uniform
+        const uint32_t rowbytes = (uint32_t)C * 2u;
         uint32_t qr[16], qk[16], qv[16], qw[16], qg[16];
         // item -> (chunk, full): phase 1 items need only k, v, w
         auto item_chunk = [&](int it) { return kSweepStates ? (it < nchunk ? it : 2 * nchunk - 1 - it) : nchunk - 1 - it; };
@@ -647,8 +652,8 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
             for (int e = 0; e < 16; ++e) {
                 const int t = tb + e;
                 const bool ok = !kRagged || t < T;
-                const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * (uint32_t)C + (uint32_t)ch;
-                const uint32_t bb = k16[o], cc = v16[o], dd = w16[o];
+                const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes + 2u * (uint32_t)ch;
+                const uint32_t bb = ld16(kb_, o), cc = ld16(vb, o), dd = ld16(wb, o);
                 qk[e] = ok ? bb : 0u; qv[e] = ok ? cc : 0u; qw[e] = ok ? dd : 0xff80u;
             }
             if (full) {
@@ -656,8 +661,8 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                 for (int e = 0; e < 16; ++e) {
                     const int t = tb + e;
                     const bool ok = !kRagged || t < T;
-                    const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * (uint32_t)C + (uint32_t)ch;
-                    const uint32_t a = r16[o], gg = g16[o];
+                    const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes + 2u * (uint32_t)ch;
+                    const uint32_t a = ld16(rb, o), gg = ld16(gb, o);
                     qr[e] = ok ? a : 0u; qg[e] = ok ? gg : 0u;
                 }
             } else {
@@ -824,10 +829,15 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
                            (const Ts *)s0, map, (bf16_t *)y, (Ts *)sT, (float *)saved_states, wild_flag, epoch);
         return hipGetLastError();
     };
-    const bool save = saved_states != nullptr;
-    if (state_dtype == kF32)
-        return save ? launch(chunk_fwd_kernel<float, true>, (float *)nullptr) : launch(chunk_fwd_kernel<float, false>, (float *)nullptr);
-    return save ? launch(chunk_fwd_kernel<bf16_t, true>, (bf16_t *)nullptr) : launch(chunk_fwd_kernel<bf16_t, false>, (bf16_t *)nullptr);
+    const bool save = saved_states != nullptr, ragged = (T % 16) != 0;
+    float *f32tag = nullptr;
+    bf16_t *bf16tag = nullptr;
+    if (state_dtype == kF32) {
+        if (ragged) return save ? launch(chunk_fwd_kernel<float, true, true>, f32tag) : launch(chunk_fwd_kernel<float, false, true>, f32tag);
+        return save ? launch(chunk_fwd_kernel<float, true, false>, f32tag) : launch(chunk_fwd_kernel<float, false, false>, f32tag);
+    }
+    if (ragged) return save ? launch(chunk_fwd_kernel<bf16_t, true, true>, bf16tag) : launch(chunk_fwd_kernel<bf16_t, false, true>, bf16tag);
+    return save ? launch(chunk_fwd_kernel<bf16_t, true, false>, bf16tag) : launch(chunk_fwd_kernel<bf16_t, false, false>, bf16tag);
 }
 
 }  // namespace wkv6
