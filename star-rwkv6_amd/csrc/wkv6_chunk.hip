@@ -97,6 +97,10 @@ __device__ __forceinline__ uint32_t ld16(const void *base, uint32_t byteoff) {
     return *reinterpret_cast<const uint16_t *>(reinterpret_cast<const char *>(base) + byteoff);
 }
 
+__device__ __forceinline__ void st16(void *base, uint32_t byteoff, float x) {
+    *reinterpret_cast<uint16_t *>(reinterpret_cast<char *>(base) + byteoff) = (uint16_t)pack_bf16x2(x, 0.f);
+}
+
 // A/B fragment of a [token][channel] array for one 16x16x32 MFMA covering channels [32h, 32h+32).
 // Lane group g = lane/16 takes the k-slots {32h+4g+e, 32h+16+4g+e : e<4}: the same channels its
 // accumulator registers hold when a 64x16 fp32 tile stack (rows 16m+4g+r) is reused as an operand.
@@ -236,7 +240,7 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr) {
                     const int t = t0 + 16 * p + 4 * g + rr;
-                    if (!kRagged || t < T) store1(y_h + (uint32_t)t * (uint32_t)C + (uint32_t)(16 * q + l16), Y[rr]);
+                    if (!kRagged || t < T) st16(y_h, (uint32_t)t * (uint32_t)C * 2u + 2u * (uint32_t)(16 * q + l16), Y[rr]);
                 }
             }
         }
@@ -357,10 +361,12 @@ struct alignas(16) BwdBuf {
     float vgyw[4][16];       // <v_t, gy_t> of the tile in flight, one private copy per consumer wave
 };
 
-// fragment of a global (B,T,C) bf16 tensor row for a 16x16x32 MFMA, same k-slot order as frag_tc
-__device__ __forceinline__ bf16x8 frag_global(const uint16_t *rowptr, int h, int g) {
-    const uint2 lo = *reinterpret_cast<const uint2 *>(rowptr + 32 * h + 4 * g);
-    const uint2 hi = *reinterpret_cast<const uint2 *>(rowptr + 32 * h + 16 + 4 * g);
+// fragment of a global (B,T,C) bf16 tensor row (uniform base + 32-bit byte offset of the row) for a
+// 16x16x32 MFMA, same k-slot order as frag_tc
+__device__ __forceinline__ bf16x8 frag_global(const void *base, uint32_t rowbyte, int h, int g) {
+    const char *b = reinterpret_cast<const char *>(base);
+    const uint2 lo = *reinterpret_cast<const uint2 *>(b + (rowbyte + 2u * (uint32_t)(32 * h + 4 * g)));
+    const uint2 hi = *reinterpret_cast<const uint2 *>(b + (rowbyte + 2u * (uint32_t)(32 * h + 16 + 4 * g)));
     return make_bf16x8(lo.x, lo.y, hi.x, hi.y);
 }
 __device__ __forceinline__ s16x4 pack4(const f32x4 &a) {
@@ -463,23 +469,20 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
         for (int m = 0; m < 4; ++m) Gj[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
         const float uj = load1(u + h * kN + col);
         float gu_acc = 0.f;
-        const uint16_t *r16 = reinterpret_cast<const uint16_t *>(r) + base;
-        const uint16_t *k16 = reinterpret_cast<const uint16_t *>(k) + base;
-        const uint16_t *v16 = reinterpret_cast<const uint16_t *>(v) + base;
-        const uint16_t *w16 = reinterpret_cast<const uint16_t *>(w) + base;
-        const uint16_t *g16 = reinterpret_cast<const uint16_t *>(gy) + base;
+        const bf16_t *rb = r + base, *kb_ = k + base, *vb = v + base, *wb = w + base, *gb = gy + base;   // uniform
         bf16_t *gr_h = gr + base, *gk_h = gk + base, *gw_h = gw + base;
+        const uint32_t rowbytes = (uint32_t)C * 2u;
         // Software pipeline over the tiles: the gY / V fragments of the NEXT tile (possibly the top
         // tile of the next chunk) are requested as soon as the MFMAs of the current one have consumed
         // theirs, so that the epilogue covers their latency.  They land in their own registers and are
         // moved over at the top of the next iteration.  Rows past T are read from row T-1: they only
         // ever meet zero operands and are never stored.
-        auto rowoff = [&](int t) { return (uint32_t)(kRagged ? min(t, T - 1) : t) * (uint32_t)C; };
+        auto rowoff = [&](int t) { return (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes; };
         bf16x8 gf0, gf1, vf0, vf1, ngf0, ngf1, nvf0, nvf1;
         auto load_frags = [&](int tile_t0) {
             const uint32_t o = rowoff(tile_t0 + l16);
-            ngf0 = frag_global(g16 + o, 0, g); ngf1 = frag_global(g16 + o, 1, g);
-            nvf0 = frag_global(v16 + o, 0, g); nvf1 = frag_global(v16 + o, 1, g);
+            ngf0 = frag_global(gb, o, 0, g); ngf1 = frag_global(gb, o, 1, g);
+            nvf0 = frag_global(vb, o, 0, g); nvf1 = frag_global(vb, o, 1, g);
         };
         for (int c = nchunk - 1; c >= 0; --c, ++item) {
             // forward state at the chunk start, straight from the checkpoint (written by this same lane)
@@ -515,20 +518,20 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
             while (ptop > 0 && t0 + 16 * ptop >= T) --ptop;
             if (c == nchunk - 1) load_frags(t0 + 16 * ptop);   // later chunks: requested by the previous chunk's last tile
             WKV6_STAMP();
-#pragma unroll 1
-            for (int p = ptop; p >= 0; --p) {
+#pragma unroll
+            for (int p = 3; p >= 0; --p) {
+                if (p > ptop) continue;   // uniform: tiles past the end of the sequence
                 gf0 = ngf0; gf1 = ngf1; vf0 = nvf0; vf1 = nvf1;
-                const bf16x8 sL = pick4(SopL[0], SopL[1], SopL[2], SopL[3], p);
-                const bf16x8 sH = pick4(SopH[0], SopH[1], SopH[2], SopH[3], p);
+                const bf16x8 sL = SopL[p], sH = SopH[p];
                 const int row = 16 * p + l16;           // tile-local token l16 as a chunk row
                 const int tk = 16 * p + 4 * g;          // first of this lane group's 4 accumulator-row tokens
                 // raw r, k, w of the accumulator rows (tokens tk..tk+3, channel col): used by the epilogue only
                 float rraw[4], kraw[4], wraw[4];
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr) {
-                    const uint32_t o = rowoff(t0 + tk + rr) + (uint32_t)col;
-                    rraw[rr] = bf16_bits_to_float(r16[o]); kraw[rr] = bf16_bits_to_float(k16[o]);
-                    wraw[rr] = bf16_bits_to_float(w16[o]);
+                    const uint32_t o = rowoff(t0 + tk + rr) + 2u * (uint32_t)col;
+                    rraw[rr] = bf16_bits_to_float(ld16(rb, o)); kraw[rr] = bf16_bits_to_float(ld16(kb_, o));
+                    wraw[rr] = bf16_bits_to_float(ld16(wb, o));
                 }
                 const s16x4 rtq = frag_ct(B.rtT, col, tk), ktq = frag_ct(B.ktT, col, tk);
                 // 16x16 intra-tile matrices
@@ -617,8 +620,8 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                     float gwv = (ew >= 88.f || t == 0 || t == T - 1) ? 0.f : -ew * (pre - P[rr]);
                     pre += D[rr];
                     if (!kRagged || t < T) {
-                        const uint32_t o = (uint32_t)t * (uint32_t)C + (uint32_t)col;
-                        store1(gr_h + o, gro[rr]); store1(gk_h + o, gko[rr]); store1(gw_h + o, gwv);
+                        const uint32_t o = (uint32_t)t * rowbytes + 2u * (uint32_t)col;
+                        st16(gr_h, o, gro[rr]); st16(gk_h, o, gko[rr]); st16(gw_h, o, gwv);
                     }
                 }
                 WKV6_STAMP();
@@ -772,7 +775,7 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr) {
                     const int t = t0 + tk + rr;
-                    if (!kRagged || t < T) store1(gv_h + (uint32_t)t * (uint32_t)C + (uint32_t)col, GV[rr]);
+                    if (!kRagged || t < T) st16(gv_h, (uint32_t)t * rowbytes + 2u * (uint32_t)col, GV[rr]);
                 }
             }
         };
