@@ -51,20 +51,26 @@ def parse():
 
 def cpu_baseline(B, T_full, H, N, seed, tokens):
     """The reference's python loop (restated in oracle/wkv6_ref.py) forward + autograd backward,
-    fp32, all host cores, on a bounded sample: same B, C and input distributions, fewer
-    timesteps (cost is linear in T)."""
+    fp32, all host cores, on a bounded sample of the same workload: same B, C and input
+    distributions, fewer timesteps (cost is linear in T).  The sample doubles until it has taken
+    about 10 s (or reaches the full T)."""
     import torch
     from oracle import wkv6_ref
 
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
-    Ts = max(8, min(T_full, (tokens or 1024) // B))
-    r, k, v, w, u, gy = wkv6_ref.make_inputs(B, Ts, H, N, seed)
-    t0 = time.perf_counter()
-    leaves = [x.clone().requires_grad_(True) for x in (r, k, v, w, u)]
-    y, _ = wkv6_ref.loop_torch(*leaves, N)
-    y.backward(gy)
-    dt = time.perf_counter() - t0
+    Ts = max(8, min(T_full, (tokens or 512) // B))
+    while True:
+        r, k, v, w, u, gy = wkv6_ref.make_inputs(B, Ts, H, N, seed)
+        t0 = time.perf_counter()
+        leaves = [x.clone().requires_grad_(True) for x in (r, k, v, w, u)]
+        y, _ = wkv6_ref.loop_torch(*leaves, N)
+        y.backward(gy)
+        dt = time.perf_counter() - t0
+        del leaves, y
+        if tokens or dt >= 8.0 or Ts >= T_full:
+            break
+        Ts = min(T_full, Ts * (2 if dt > 2.0 else 4))
     return {
         "value": B * Ts / dt / 1e6, "unit": "Mtokens/s", "cores": cores, "kind": "port",
         "sample": "python-loop WKV6 fwd+bwd via torch.autograd, fp32, B=%d T=%d of %d C=%d (%.1f s)" % (
