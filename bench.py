@@ -32,7 +32,11 @@ WORKLOADS = {
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (separate runs), scaled
 # by the same counters' reading for a device-to-device copy of known size; see profiles/.
 # Keyed by (workload, algo, "fwd"|"bwd").  None = not measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {
+    # profiles/c2_fwd_bwd_hbm_traffic_pmc.md: backward_saved 398.3 MB read + 144.8 MB written
+    ("c2", "auto", "bwd"): 543.1e6, ("c2", "chunk", "bwd"): 543.1e6,
+    ("c2", "auto", "fwd"): 235.1e6, ("c2", "chunk", "fwd"): 235.1e6,
+}
 
 
 def parse():
