@@ -44,7 +44,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c5"])
     ap.add_argument("--algo", default="auto", choices=["auto", "scan", "chunk", "chunk_only"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--plain-pair", action="store_true", help="time forward()+backward() without saved states")
@@ -82,6 +82,59 @@ def cpu_baseline(B, T_full, H, N, seed, tokens):
     }
 
 
+def bench_stateful(a):
+    """Config 5: B=64 sequences at C=2048, chunked prefill of T=512 from h0 then 256 single-token
+    steps carrying the fp32 state, through the C ABI with pre-allocated buffers.  Prints its own JSON
+    line (prefill Mtokens/s, decode steps/s and the state bandwidth of a decode step)."""
+    import torch
+    from oracle import wkv6_ref
+    from rwkv_kernel import _native
+
+    lib = _native.load()
+    B, H, N, Tp, Td = 64, 32, 64, 512, 256
+    C = H * N
+    dev = torch.device("cuda:0")
+    ins = wkv6_ref.make_inputs(B, Tp + 1, H, N, a.seed, with_state=True)
+    r, k, v, w, u = (x.to(torch.bfloat16).to(dev) for x in ins[:5])
+    h0 = ins[6].to(dev)
+    pre = [x[:, :Tp].contiguous() for x in (r, k, v, w)]
+    one = [x[:, Tp:].contiguous() for x in (r, k, v, w)]
+    yp = torch.empty(B, Tp, C, dtype=torch.bfloat16, device=dev)
+    y1 = torch.empty(B, 1, C, dtype=torch.bfloat16, device=dev)
+    sa, sb = torch.empty_like(h0), torch.empty_like(h0)
+    st = torch.cuda.current_stream().cuda_stream
+    P = lambda t: t.data_ptr()
+
+    def call(x, T, y, si, so):
+        _native.check(lib.wkv6_forward_with_state_ex(st, _native.BF16, _native.F32, _native.ALGO_AUTO, B, T, C, H, 1, None,
+                                                     P(x[0]), P(x[1]), P(x[2]), P(x[3]), P(u), P(si), P(y), P(so), None, 0))
+
+    def timed(fn, reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        fn(); torch.cuda.synchronize()
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record(); torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    pre_ms = timed(lambda: call(pre, Tp, yp, h0, sa), 20)
+
+    def two_steps():
+        call(one, 1, y1, sa, sb); call(one, 1, y1, sb, sa)
+
+    dec_ms = timed(two_steps, Td // 2) / 2
+    state_bytes = 2 * B * H * N * N * 4
+    print(json.dumps({
+        "metric": "WKV6 stateful forward, B64 C2048 H32 bf16 activations, fp32 state", "n_gpus": 1,
+        "config": {"workload": "c5: prefill T=512 then T=1 decode steps with carried state"},
+        "prefill_Mtokens_per_s": B * Tp / (pre_ms * 1e-3) / 1e6, "prefill_ms": pre_ms,
+        "decode_steps_per_s": 1.0 / (dec_ms * 1e-3), "decode_us_per_step": dec_ms * 1e3,
+        "decode_state_GBps": state_bytes / (dec_ms * 1e-3) / 1e9,
+        "decode_frac_of_hbm_peak": state_bytes / (dec_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "dtype": "bf16", "data": "synthetic"}))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -93,6 +146,9 @@ def main():
     from rwkv_kernel import _native
 
     assert torch.cuda.is_available(), "bench.py needs the GPU"
+    if a.workload == "c5":
+        torch.cuda.set_device(0)
+        return bench_stateful(a)
     lib = _native.load()
     B, T, H, dt_name = WORKLOADS[a.workload]
     N = 64

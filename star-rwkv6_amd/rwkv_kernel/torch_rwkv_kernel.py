@@ -98,8 +98,8 @@ def _forward_with_state(B, T, C, H, state_map, r, k, v, w, u, init_state, algo=_
     """Stateful forward, no gradient (rwkv_kernel/torch_rwkv_kernel.py:76-95)."""
     lib = _native.load()
     with torch.no_grad():
-        assert (init_state is None and state_map is None) or (init_state is not None and state_map is not None), \
-            "init_state and state_map go together"
+        # state_map None with an init_state means the identity map (row b starts from init_state[b])
+        assert init_state is not None or state_map is None, "state_map needs init_state"
         assert state_map is None or state_map.dtype == torch.int64
         odt = _out_dtype(r.dtype)
         sdt = init_state.dtype if init_state is not None else odt
@@ -127,6 +127,7 @@ class RWKVKernelOperator:
         # it, so longer sequences simply work
         self.max_sequence_length = max_sequence_length
         self.algo = _native.ALGO_AUTO
+        self._zero_maps = {}
         self.normal_kernenl = _WKV6
         self.kernel_with_state = _forward_with_state
 
@@ -171,14 +172,17 @@ class RWKVKernelOperator:
                 n_state = init_state.shape[0]
                 if state_map is None:
                     assert n_state == 1 or n_state == B, "cannot infer state_map; pass it explicitly"
-                    if n_state == 1:
-                        state_map = torch.zeros(B, dtype=torch.int64)
-                    else:
-                        state_map = torch.arange(B, dtype=torch.int64)
+                    if n_state == 1 and B > 1:
+                        key = (B, r.device)
+                        if key not in self._zero_maps:
+                            self._zero_maps[key] = torch.zeros(B, dtype=torch.int64, device=r.device)
+                        state_map = self._zero_maps[key]
+                    # n_state == B: identity, expressed as "no map" so that a decode loop pays
+                    # neither a host-to-device copy nor a range check per step
                 else:
                     assert bool((state_map >= 0).all()) and bool((state_map < n_state).all()), \
                         "state_map values must lie in [0, %d)" % n_state
-                state_map = state_map.to(r.device).contiguous()
+                    state_map = state_map.to(r.device).contiguous()
                 init_state = init_state.contiguous()
             for x in (r, k, v, w, u):
                 assert x.is_contiguous()
