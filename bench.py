@@ -45,7 +45,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c5"])
-    ap.add_argument("--algo", default="auto", choices=["auto", "scan", "chunk", "chunk_only"])
+    ap.add_argument("--algo", default="auto", choices=["auto", "scan", "chunk"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--plain-pair", action="store_true", help="time forward()+backward() without saved states")
     ap.add_argument("--cpu-tokens", type=int, default=0, help="tokens in the CPU baseline sample (0 = default)")
@@ -156,8 +156,7 @@ def main():
     dtype = {"bf16": torch.bfloat16, "f32": torch.float32}[dt_name]
     code = {"bf16": _native.BF16, "f32": _native.F32}[dt_name]
     es = 2 if dt_name == "bf16" else 4
-    algo = {"auto": _native.ALGO_AUTO, "scan": _native.ALGO_SCAN, "chunk": _native.ALGO_CHUNK,
-            "chunk_only": _native.ALGO_CHUNK_ONLY}[a.algo]
+    algo = {"auto": _native.ALGO_AUTO, "scan": _native.ALGO_SCAN, "chunk": _native.ALGO_CHUNK}[a.algo]
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 

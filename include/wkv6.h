@@ -3,8 +3,7 @@
  * time-mixing operator.  Plain pointers and sizes only; every pointer (state_map and workspace
  * included) is a DEVICE pointer to a row-major contiguous, 16-byte aligned array; all work is
  * enqueued on `stream` (a hipStream_t, may be NULL = default stream) and the calls return
- * without synchronising.  Calls are re-entrant: the only state the library keeps is a ring of
- * flag words in its device image, one slot per call in flight (1024 slots).
+ * without synchronising.  The library keeps no mutable state: calls are re-entrant.
  *
  * Each entry point names the reference interface it replaces (paths relative to the
  * reference tree infiy-quine/STAR-RWKV6).
@@ -45,11 +44,10 @@ enum {
 enum {
     WKV6_ALGO_AUTO = 0,  /* library picks: chunked MFMA path for bf16/f16 when T allows, else scan */
     WKV6_ALGO_SCAN = 1,  /* per-timestep fp32 recurrence, state in VGPRs                       */
-    WKV6_ALGO_CHUNK = 2, /* chunk-parallel form, bf16 MFMA for the dense intra-chunk products;
-                            bf16 tensors only.  An exact per-timestep pass is enqueued behind it
-                            and runs only if a tile's decay left the range the scaling can hold    */
-    WKV6_ALGO_CHUNK_ONLY = 3 /* the chunked kernels alone, without that guarded second pass: for
-                            tests and profiling; results are undefined for extreme decays          */
+    WKV6_ALGO_CHUNK = 2  /* chunk-parallel form, bf16 MFMA for the dense intra-chunk products; bf16
+                            tensors only.  A workgroup whose (batch, head) pair has a 16-token tile
+                            with decay beyond what the operand scaling can hold redoes that pair
+                            with the exact per-timestep code inside the same launch                */
 };
 
 const char *wkv6_status_string(int status);

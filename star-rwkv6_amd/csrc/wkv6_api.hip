@@ -4,52 +4,7 @@
 
 #include <string.h>
 
-#include <atomic>
-#include <chrono>
-#include <mutex>
-
 namespace {
-
-// Flag words the chunked kernels raise when they meet a decay range they cannot scale (see Gate in
-// wkv6_kernels.h).  Each call takes the next slot and a process-unique epoch; a slot is reused
-// only after kRing further calls.  Living in device memory of the library image, the ring needs no
-// allocation and exists once per GPU.
-constexpr int kRing = 1024;
-__device__ __align__(256) unsigned long long g_wild_ring[kRing];
-
-std::atomic<unsigned long long> g_call_counter{0};
-unsigned long long g_salt = 0;
-std::once_flag g_salt_once;
-std::mutex g_ring_mutex;
-unsigned long long *g_ring_ptr[64] = {nullptr};
-
-struct FlagSlot { unsigned long long *ptr; unsigned long long epoch; };
-
-hipError_t take_flag_slot(FlagSlot *out) {
-    std::call_once(g_salt_once, [] {
-        const unsigned long long t = (unsigned long long)std::chrono::steady_clock::now().time_since_epoch().count();
-        g_salt = (t * 0x9E3779B97F4A7C15ull) | (1ull << 62);
-    });
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    if (dev < 0 || dev >= 64) return hipErrorInvalidDevice;
-    unsigned long long *base;
-    {
-        std::lock_guard<std::mutex> lock(g_ring_mutex);
-        if (g_ring_ptr[dev] == nullptr) {
-            void *p = nullptr;
-            e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_wild_ring));
-            if (e != hipSuccess) return e;
-            g_ring_ptr[dev] = static_cast<unsigned long long *>(p);
-        }
-        base = g_ring_ptr[dev];
-    }
-    const unsigned long long n = g_call_counter.fetch_add(1) + 1;
-    out->ptr = base + (n % kRing);
-    out->epoch = g_salt + n;
-    return hipSuccess;
-}
 
 // Shapes the chunked MFMA kernels take; everything else runs the per-timestep kernels.
 // (the chunked kernels index one batch row with 32-bit element offsets)
@@ -112,24 +67,16 @@ static int forward_impl(void *stream, int dtype, int state_dtype, int algo,
     if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(y)) return WKV6_ERR_ARG;
     if (has_init_state && !s) return WKV6_ERR_ARG;
     if (state_dtype != out_type(dtype) && state_dtype != WKV6_F32) return WKV6_ERR_ARG;
-    if (algo < WKV6_ALGO_AUTO || algo > WKV6_ALGO_CHUNK_ONLY) return WKV6_ERR_ARG;
+    if (algo < WKV6_ALGO_AUTO || algo > WKV6_ALGO_CHUNK) return WKV6_ERR_ARG;
     hipStream_t st = (hipStream_t)stream;
     const void *s_in = has_init_state ? s : nullptr;
     const int64_t *map_in = has_init_state ? state_map : nullptr;
-    if ((algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY) && !chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;
-    const bool chunk = algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY ||
+    if (algo == WKV6_ALGO_CHUNK && !chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;
+    const bool chunk = algo == WKV6_ALGO_CHUNK ||
                        (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
     if (!chunk)
-        return finish(wkv6::scan_forward(st, dtype, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys,
-                                         wkv6::Gate{nullptr, 0}));
-    FlagSlot slot;
-    hipError_t e = take_flag_slot(&slot);
-    if (e != hipSuccess) return finish(e);
-    e = wkv6::chunk_forward(st, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys, saved, slot.ptr, slot.epoch);
-    if (e != hipSuccess || algo == WKV6_ALGO_CHUNK_ONLY) return finish(e);
-    // exact per-timestep kernel behind the gate: a no-op unless the chunked kernel raised the flag
-    return finish(wkv6::scan_forward(st, dtype, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys,
-                                     wkv6::Gate{slot.ptr, slot.epoch}));
+        return finish(wkv6::scan_forward(st, dtype, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys));
+    return finish(wkv6::chunk_forward(st, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys, saved));
 }
 
 int wkv6_forward_with_state_ex(void *stream, int dtype, int state_dtype, int algo,
@@ -144,7 +91,7 @@ int wkv6_forward_with_state_ex(void *stream, int dtype, int state_dtype, int alg
 
 size_t wkv6_saved_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
     if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
-    const bool chunk = ((algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY) && chunk_possible(dtype, T, C)) ||
+    const bool chunk = (algo == WKV6_ALGO_CHUNK && chunk_possible(dtype, T, C)) ||
                        (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
     // sized so that the guarded per-timestep pass of the backward can use the same buffer
     return chunk ? wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H) : 0;
@@ -183,9 +130,9 @@ int wkv6_forward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64
 size_t wkv6_backward_workspace_bytes_ex(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
     if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
     // The per-timestep path keeps one fp32 per element (P), the chunked path one fp32 state per
-    // 64-token chunk; the chunked call needs both because its gated fallback reuses the buffer.
+    // 64-token chunk (which a workgroup's exact second pass reuses for its own P).
     size_t need = wkv6::scan_backward_workspace_bytes(B, T, C);
-    if (algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY || (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C))) {
+    if (algo == WKV6_ALGO_CHUNK || (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C))) {
         const size_t c = wkv6::chunk_backward_workspace_bytes(B, T, H);
         if (c > need) need = c;
     }
@@ -205,23 +152,16 @@ static int backward_impl(void *stream, int dtype, int algo, int64_t B, int64_t T
     if (!r || !k || !v || !w || !u || !gy || !gr || !gk || !gv || !gw || !gu) return WKV6_ERR_ARG;
     if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(gy) || !aligned16(gr) ||
         !aligned16(gk) || !aligned16(gv) || !aligned16(gw)) return WKV6_ERR_ARG;
-    if (algo < WKV6_ALGO_AUTO || algo > WKV6_ALGO_CHUNK_ONLY) return WKV6_ERR_ARG;
+    if (algo < WKV6_ALGO_AUTO || algo > WKV6_ALGO_CHUNK) return WKV6_ERR_ARG;
     const size_t need = wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H);
     if (need > 0 && (!workspace || workspace_bytes < need || !aligned16(workspace))) return WKV6_ERR_WORKSPACE;
     hipStream_t st = (hipStream_t)stream;
-    if ((algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY) && !chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;
-    const bool chunk = algo == WKV6_ALGO_CHUNK || algo == WKV6_ALGO_CHUNK_ONLY ||
+    if (algo == WKV6_ALGO_CHUNK && !chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;
+    const bool chunk = algo == WKV6_ALGO_CHUNK ||
                        (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
     if (!chunk)
-        return finish(wkv6::scan_backward(st, dtype, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace,
-                                          wkv6::Gate{nullptr, 0}));
-    FlagSlot slot;
-    hipError_t e = take_flag_slot(&slot);
-    if (e != hipSuccess) return finish(e);
-    e = wkv6::chunk_backward(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace, states_ready, slot.ptr, slot.epoch);
-    if (e != hipSuccess || algo == WKV6_ALGO_CHUNK_ONLY) return finish(e);
-    return finish(wkv6::scan_backward(st, dtype, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace,
-                                      wkv6::Gate{slot.ptr, slot.epoch}));
+        return finish(wkv6::scan_backward(st, dtype, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace));
+    return finish(wkv6::chunk_backward(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace, states_ready));
 }
 
 int wkv6_backward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,

@@ -16,11 +16,13 @@
 // buffers are double-buffered and the two roles meet at one barrier per chunk.  HBM traffic is
 // exactly the algorithmic minimum (r,k,v,w read once, y written once).
 //
-// exp(+c) needs the decay accumulated inside one 16-token tile to stay in range.  A tile whose
-// summed exp(w) exceeds kWildLimit in any channel raises a flag; the launcher always enqueues the
-// exact per-timestep kernel behind this one, and that kernel runs only if the flag was raised.
+// exp(+c) needs the decay accumulated inside one 16-token tile to stay in range.  A producer wave
+// that meets a tile whose summed exp(w) exceeds kWildLimit in any channel raises a flag in LDS, and
+// the workgroup then redoes ITS (batch, head) pair with the exact per-timestep code
+// (wkv6_scan_body.h) before the kernel ends; other workgroups are unaffected.
 #include "wkv6_common.h"
 #include "wkv6_kernels.h"
+#include "wkv6_scan_body.h"
 
 #include <type_traits>
 
@@ -164,11 +166,14 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
         const bf16_t *__restrict__ r, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v,
         const bf16_t *__restrict__ w, const bf16_t *__restrict__ u,
         const Ts *__restrict__ s0, const int64_t *__restrict__ map,
-        bf16_t *__restrict__ y, Ts *__restrict__ sT, float *__restrict__ ckpt,
-        unsigned long long *__restrict__ wild_flag, unsigned long long epoch)
+        bf16_t *__restrict__ y, Ts *__restrict__ sT, float *__restrict__ ckpt)
 {
     extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ int s_wild;
     FwdBuf *buf = reinterpret_cast<FwdBuf *>(smem);
+    static_assert(sizeof(ScanFwdLds) <= 2 * sizeof(FwdBuf), "the exact second pass reuses the operand buffers");
+    if (threadIdx.x == 0) s_wild = 0;
+    __syncthreads();
 
     const int b = blockIdx.x / H, h = blockIdx.x % H;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -262,31 +267,32 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
         // a tile is either entirely inside the sequence or entirely outside.
         auto prefetch = [&](int c) {
             const int tb = c * CL + 16 * p;
-            if (!kRagged && tb >= T) {
+            if (tb < T) {   // uniform: a tile entirely past the end is neither loaded, prepared nor consumed
 #pragma unroll
-                for (int e = 0; e < 16; ++e) { qr[e] = 0u; qk[e] = 0u; qv[e] = 0u; qw[e] = 0xff80u; }
-                return;
-            }
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int t = tb + e;
-                const bool ok = !kRagged || t < T;
-                const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes + 2u * (uint32_t)ch;
-                const uint32_t a = ld16(rb, o), bb = ld16(kb_, o), cc = ld16(vb, o), dd = ld16(wb, o);
-                qr[e] = ok ? a : 0u; qk[e] = ok ? bb : 0u; qv[e] = ok ? cc : 0u; qw[e] = ok ? dd : 0xff80u;
+                for (int e = 0; e < 16; ++e) {
+                    const int t = tb + e;
+                    const bool ok = !kRagged || t < T;
+                    const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes + 2u * (uint32_t)ch;
+                    const uint32_t a = ld16(rb, o), bb = ld16(kb_, o), cc = ld16(vb, o), dd = ld16(wb, o);
+                    qr[e] = ok ? a : 0u; qk[e] = ok ? bb : 0u; qv[e] = ok ? cc : 0u; qw[e] = ok ? dd : 0xff80u;
+                }
             }
         };
         auto prepare = [&](int c) {   // consumes the prefetched registers, refills them for chunk c+1
             FwdBuf &B = buf[c & 1];
+            const bool tile_in = c * CL + 16 * p < T;
             float fr[16], fk[16], fw[16];
             uint32_t vbits[8];
+            if (tile_in) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                fr[e] = bf16_bits_to_float(qr[e]); fk[e] = bf16_bits_to_float(qk[e]); fw[e] = bf16_bits_to_float(qw[e]);
+                for (int e = 0; e < 16; ++e) {
+                    fr[e] = bf16_bits_to_float(qr[e]); fk[e] = bf16_bits_to_float(qk[e]); fw[e] = bf16_bits_to_float(qw[e]);
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) vbits[e] = qv[2 * e] | (qv[2 * e + 1] << 16);
             }
-#pragma unroll
-            for (int e = 0; e < 8; ++e) vbits[e] = qv[2 * e] | (qv[2 * e + 1] << 16);
             if (c + 1 < nchunk) prefetch(c + 1);
+            if (tile_in) {
 
             // exponents are kept in base 2 (one v_exp_f32 each, no extra scaling multiply)
             float xr[16], xk[16], pr[16];
@@ -301,7 +307,7 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
                 pr[e] = fr[e] * uc * fk[e];
             }
             if (__builtin_amdgcn_ballot_w64(!(cs2 <= kWildLimit * kLog2e)) != 0ull) {
-                if (lane == 0 && wild_flag != nullptr) *wild_flag = epoch;
+                if (lane == 0) s_wild = 1;
             }
             store_rows_paired(B.rt, 16 * p, lane, xr);
             store_rows_paired(B.kt, 16 * p, lane, xk);
@@ -315,6 +321,7 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
             B.g[p][ch] = pa;
             const float tot = transpose_reduce16(pr, lane);
             if ((lane & 3) == 0) B.ruk[16 * p + ((lane >> 2) & 15)] = tot;
+            }
         };
         prefetch(0);
         prepare(0);
@@ -323,6 +330,11 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
             if (c + 1 < nchunk) prepare(c + 1);
         }
     }
+    // exact second pass for this (b, h) if any of its tiles left the representable range
+    __threadfence_block();   // workgroup scope is enough (and a device-scope fence would write back the L2)
+    __syncthreads();
+    if (s_wild)
+        scan_fwd_body<bf16_t, bf16_t, Ts>(*reinterpret_cast<ScanFwdLds *>(smem), b, h, T, H, r, k, v, w, u, s0, map, y, sT);
 }
 
 // ==========================================================================================
@@ -413,11 +425,15 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
         const bf16_t *__restrict__ r, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v,
         const bf16_t *__restrict__ w, const bf16_t *__restrict__ u, const bf16_t *__restrict__ gy,
         bf16_t *__restrict__ gr, bf16_t *__restrict__ gk, bf16_t *__restrict__ gv, bf16_t *__restrict__ gw,
-        bf16_t *__restrict__ gu, float *__restrict__ ckpt,
-        unsigned long long *__restrict__ wild_flag, unsigned long long epoch)
+        bf16_t *__restrict__ gu, float *__restrict__ ckpt)
 {
     extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ int s_wild;
     BwdBuf *buf = reinterpret_cast<BwdBuf *>(smem);
+    static_assert(sizeof(ScanBwdALds) <= 2 * sizeof(BwdBuf) && sizeof(ScanBwdBLds) <= 2 * sizeof(BwdBuf),
+                  "the exact second pass reuses the operand buffers");
+    if (threadIdx.x == 0) s_wild = 0;
+    __syncthreads();
 
     const int b = blockIdx.x / H, h = blockIdx.x % H;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -451,6 +467,7 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                 if (c + 1 == nchunk) break;   // the state after the last chunk is never used
 #pragma unroll 1
                 for (int p = 0; p < 4; ++p) {
+                    if (c * CL + 16 * p >= T) break;
                     const s16x4 kq = frag_ct(B.ktT, col, 16 * p + 4 * g);
                     const float gq = B.g[p][col];
 #pragma unroll
@@ -505,6 +522,7 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
             SopL[0] = acc_as_operand(S[0], S[1]); SopH[0] = acc_as_operand(S[2], S[3]);
 #pragma unroll
             for (int p = 0; p < 3; ++p) {
+                if (t0 + 16 * (p + 1) >= T) continue;   // uniform: no tile starts there
                 const s16x4 kq = frag_ct(B.ktT, col, 16 * p + 4 * g);
                 const float gq = B.g[p][col];
 #pragma unroll
@@ -646,48 +664,49 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
         auto prefetch = [&](int it) {
             const int tb = item_chunk(it) * CL + 16 * p;
             const bool full = item_full(it);
-            if (!kRagged && tb >= T) {
-#pragma unroll
-                for (int e = 0; e < 16; ++e) { qr[e] = 0u; qk[e] = 0u; qv[e] = 0u; qg[e] = 0u; qw[e] = 0xff80u; }
-                return;
-            }
-#pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                const int t = tb + e;
-                const bool ok = !kRagged || t < T;
-                const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes + 2u * (uint32_t)ch;
-                const uint32_t bb = ld16(kb_, o), cc = ld16(vb, o), dd = ld16(wb, o);
-                qk[e] = ok ? bb : 0u; qv[e] = ok ? cc : 0u; qw[e] = ok ? dd : 0xff80u;
-            }
-            if (full) {
+            if (tb < T) {   // uniform: a tile entirely past the end is neither loaded, prepared nor consumed
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
                     const int t = tb + e;
                     const bool ok = !kRagged || t < T;
                     const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes + 2u * (uint32_t)ch;
-                    const uint32_t a = ld16(rb, o), gg = ld16(gb, o);
-                    qr[e] = ok ? a : 0u; qg[e] = ok ? gg : 0u;
+                    const uint32_t bb = ld16(kb_, o), cc = ld16(vb, o), dd = ld16(wb, o);
+                    qk[e] = ok ? bb : 0u; qv[e] = ok ? cc : 0u; qw[e] = ok ? dd : 0xff80u;
                 }
-            } else {
+                if (full) {
 #pragma unroll
-                for (int e = 0; e < 16; ++e) { qr[e] = 0u; qg[e] = 0u; }
+                    for (int e = 0; e < 16; ++e) {
+                        const int t = tb + e;
+                        const bool ok = !kRagged || t < T;
+                        const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes + 2u * (uint32_t)ch;
+                        const uint32_t a = ld16(rb, o), gg = ld16(gb, o);
+                        qr[e] = ok ? a : 0u; qg[e] = ok ? gg : 0u;
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) { qr[e] = 0u; qg[e] = 0u; }
+                }
             }
         };
         auto prepare = [&](int it) {
             BwdBuf &B = buf[it & 1];
             const bool full = item_full(it);
+            const bool tile_in = item_chunk(it) * CL + 16 * p < T;
             float fr[16], fk[16], fw[16];
             uint32_t vbits[8], gbits[8];
+            if (tile_in) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                fr[e] = bf16_bits_to_float(qr[e]); fk[e] = bf16_bits_to_float(qk[e]); fw[e] = bf16_bits_to_float(qw[e]);
-            }
+                for (int e = 0; e < 16; ++e) {
+                    fr[e] = bf16_bits_to_float(qr[e]); fk[e] = bf16_bits_to_float(qk[e]); fw[e] = bf16_bits_to_float(qw[e]);
+                }
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                vbits[e] = qv[2 * e] | (qv[2 * e + 1] << 16);
-                gbits[e] = qg[2 * e] | (qg[2 * e + 1] << 16);
+                for (int e = 0; e < 8; ++e) {
+                    vbits[e] = qv[2 * e] | (qv[2 * e + 1] << 16);
+                    gbits[e] = qg[2 * e] | (qg[2 * e + 1] << 16);
+                }
             }
             if (it + 1 < nitem) prefetch(it + 1);
+            if (tile_in) {
 
             // exponents are kept in base 2 (one v_exp_f32 each, no extra scaling multiply)
             float xr[16], xk[16], pr[16], fa[17];
@@ -704,7 +723,7 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
             }
             fa[16] = pa;
             if (__builtin_amdgcn_ballot_w64(!(cs2 <= kWildLimit * kLog2e)) != 0ull) {
-                if (lane == 0 && wild_flag != nullptr) *wild_flag = epoch;
+                if (lane == 0) s_wild = 1;
             }
             uint32_t pk[8];
 #pragma unroll
@@ -729,6 +748,7 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
                 B.fr[ch][20 * p + 16] = fa[16];
                 const float tr = transpose_reduce16(pr, lane);
                 if ((lane & 3) == 0) B.ruk[16 * p + ((lane >> 2) & 15)] = tr;
+            }
             }
         };
         // gv role (second half of the consumer work, on the waves the operand preparation leaves
@@ -790,6 +810,16 @@ __global__ __launch_bounds__(512) void chunk_bwd_kernel(int T, int H,
             if (item_full(it)) gv_tiles(it);
         }
     }
+    // exact second pass for this (b, h) if any of its tiles left the representable range; the
+    // workgroup's own slice of the state workspace (nchunk x 64 x 64 floats = T' x 64) holds P
+    __threadfence_block();   // workgroup scope is enough (and a device-scope fence would write back the L2)
+    __syncthreads();
+    if (s_wild) {
+        scan_bwd_a_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdALds *>(smem), b, h, T, H, r, k, v, w, u, gy, gr, gu, ck, kN);
+        __threadfence_block();
+        __syncthreads();
+        scan_bwd_b_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdBLds *>(smem), b, h, T, H, r, k, v, w, u, gy, ck, kN, gk, gv, gw);
+    }
 }
 
 size_t chunk_backward_workspace_bytes(int64_t B, int64_t T, int64_t H) {
@@ -799,8 +829,7 @@ size_t chunk_backward_workspace_bytes(int64_t B, int64_t T, int64_t H) {
 
 hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
                           const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
-                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, bool states_ready,
-                          unsigned long long *wild_flag, unsigned long long epoch)
+                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, bool states_ready)
 {
     const size_t lds = 2 * sizeof(BwdBuf);
     auto launch = [&](auto kern) -> hipError_t {
@@ -809,7 +838,7 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
         hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(512), lds, st, (int)T, (int)H,
                            (const bf16_t *)r, (const bf16_t *)k, (const bf16_t *)v, (const bf16_t *)w, (const bf16_t *)u,
                            (const bf16_t *)gy, (bf16_t *)gr, (bf16_t *)gk, (bf16_t *)gv, (bf16_t *)gw, (bf16_t *)gu,
-                           (float *)workspace, wild_flag, epoch);
+                           (float *)workspace);
         return hipGetLastError();
     };
     const bool ragged = (T % 16) != 0;
@@ -819,8 +848,7 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
 
 hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u,
-                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states,
-                         unsigned long long *wild_flag, unsigned long long epoch)
+                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states)
 {
     const size_t lds = 2 * sizeof(FwdBuf);
     auto launch = [&](auto kern, auto *state_tag) -> hipError_t {
@@ -829,7 +857,7 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(512), lds, st, (int)T, (int)H,
                            (const bf16_t *)r, (const bf16_t *)k, (const bf16_t *)v, (const bf16_t *)w, (const bf16_t *)u,
-                           (const Ts *)s0, map, (bf16_t *)y, (Ts *)sT, (float *)saved_states, wild_flag, epoch);
+                           (const Ts *)s0, map, (bf16_t *)y, (Ts *)sT, (float *)saved_states);
         return hipGetLastError();
     };
     const bool save = saved_states != nullptr, ragged = (T % 16) != 0;

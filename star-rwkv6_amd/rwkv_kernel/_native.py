@@ -10,7 +10,7 @@ _PKG = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(_PKG, "lib", "libwkv6_gfx950.so")
 
 BF16, F16, F32 = 0, 1, 2
-ALGO_AUTO, ALGO_SCAN, ALGO_CHUNK, ALGO_CHUNK_ONLY = 0, 1, 2, 3
+ALGO_AUTO, ALGO_SCAN, ALGO_CHUNK = 0, 1, 2
 
 _i64, _int, _p, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
 
