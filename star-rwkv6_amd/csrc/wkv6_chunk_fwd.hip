@@ -1,0 +1,247 @@
+// WKV6 in chunk-parallel form for gfx950: bf16 MFMA for the dense products, fp32 state.
+//
+// One workgroup (8 waves) per (batch, head).  Time is cut into chunks of 64 tokens, each chunk
+// into 4 tiles of 16 tokens.  The fp32 state S[j][i] lives in the MFMA accumulators of the four
+// "consumer" waves (wave q owns value columns 16q..16q+15) and is advanced one tile at a time:
+//
+//   c_t = sum_{s<t} exp(w_s) inside the tile (so exp(-c_t) is the decay from the tile start to t)
+//   R~[t][j] = r_t[j] exp(-c_t[j])            K~[t][j] = k_t[j] exp(+c_{t+1}[j])
+//   K^[t][j] = k_t[j] exp(-(c_16[j] - c_{t+1}[j]))         g[j] = exp(-c_16[j])
+//   A[t][s]  = R~_t . K~_s  (s < t),  A[t][t] = sum_j r_t[j] u[j] k_t[j]
+//   Y        = R~ S + A V          (16x64x64 and 16x16x16 MFMA, K index j resp. s)
+//   S       <- diag(g) S + K^T V   (64x16x16 MFMA, K index s)
+//
+// The four "producer" waves (wave 4+p prepares tile p, lane = channel) compute these operands in
+// fp32 for the NEXT chunk while the consumers run the MFMAs of the current one; LDS operand
+// buffers are double-buffered and the two roles meet at one barrier per chunk.  HBM traffic is
+// exactly the algorithmic minimum (r,k,v,w read once, y written once).
+//
+// exp(+c) needs the decay accumulated inside one 16-token tile to stay in range.  A producer wave
+// that meets a tile whose summed exp(w) exceeds kWildLimit in any channel raises a flag in LDS, and
+// the workgroup then redoes ITS (batch, head) pair with the exact per-timestep code
+// (wkv6_scan_body.h) before the kernel ends; other workgroups are unaffected.
+#include "wkv6_mfma.h"
+#include "wkv6_kernels.h"
+#include "wkv6_scan_body.h"
+
+#include <type_traits>
+
+namespace wkv6 {
+
+constexpr int CL = 64;   // tokens per chunk
+constexpr int LDT = 72;  // row pitch (elements) of [channel][token] operand arrays: 144 B, 16-byte aligned rows
+
+struct alignas(16) FwdBuf {
+    uint16_t rt[CL][LDA];   // R~[t][j]
+    uint16_t kt[CL][LDA];   // K~[t][j]
+    uint16_t ktT[kN][LDT];  // K~[t][j] stored [j][t]  (K^ = g K~ is never formed: S <- g (S + K~^T V))
+    uint16_t vT[kN][LDT];   // V[t][i]  stored [i][t]
+    float g[4][kN];         // per-tile decay exp(-c_16)
+    float ruk[CL];          // sum_j r u k per token
+};
+
+// kSave: also write the state at every chunk start to `ckpt` (fp32, [b][h][chunk][j][i]) for the
+// backward pass, which then skips its own forward sweep.
+template <typename Ts, bool kSave, bool kRagged>
+__global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
+        const bf16_t *__restrict__ r, const bf16_t *__restrict__ k, const bf16_t *__restrict__ v,
+        const bf16_t *__restrict__ w, const bf16_t *__restrict__ u,
+        const Ts *__restrict__ s0, const int64_t *__restrict__ map,
+        bf16_t *__restrict__ y, Ts *__restrict__ sT, float *__restrict__ ckpt)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ int s_wild;
+    FwdBuf *buf = reinterpret_cast<FwdBuf *>(smem);
+    static_assert(sizeof(ScanFwdLds) <= 2 * sizeof(FwdBuf), "the exact second pass reuses the operand buffers");
+    if (threadIdx.x == 0) s_wild = 0;
+    __syncthreads();
+
+    const int b = blockIdx.x / H, h = blockIdx.x % H;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t C = (int64_t)H * kN;
+    const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
+    const int nchunk = (T + CL - 1) / CL;
+
+    if (wave < 4) {
+        // ------------------------------ consumer: MFMA ------------------------------
+        const int q = wave, g = lane >> 4, l16 = lane & 15;
+        f32x4 S[4];
+        if (s0 != nullptr) {
+            const int64_t row = map ? map[b] : (int64_t)b;
+            const Ts *p = s0 + (row * H + h) * kN * kN + 16 * q + l16;
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) S[m][rr] = load1(p + (16 * m + 4 * g + rr) * kN);
+        } else {
+#pragma unroll
+            for (int m = 0; m < 4; ++m) S[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        }
+        bf16_t *y_h = y + base;
+        for (int c = 0; c < nchunk; ++c) {
+            if (kSave) {
+                float *dst = ckpt + ((int64_t)blockIdx.x * nchunk + c) * (kN * kN) + 16 * q + l16;
+#pragma unroll
+                for (int m = 0; m < 4; ++m)
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) dst[(16 * m + 4 * g + rr) * kN] = S[m][rr];
+            }
+            __syncthreads();
+            const FwdBuf &B = buf[c & 1];
+            const int t0 = c * CL;
+#pragma unroll 1
+            for (int p = 0; p < 4; ++p) {
+                if (t0 + 16 * p >= T) break;
+                const int row = 16 * p + l16;
+                const bf16x8 rf0 = frag_tc(B.rt, row, 0, g), rf1 = frag_tc(B.rt, row, 1, g);
+                const bf16x8 kf0 = frag_tc(B.kt, row, 0, g), kf1 = frag_tc(B.kt, row, 1, g);
+                const s16x4 vf = frag_ct(B.vT, 16 * q + l16, 16 * p + 4 * g);
+                const float rukv = B.ruk[row];
+                // A^T[s][t] = K~_s . R~_t  (accumulator rows s = 4g+r, column t = l16)
+                f32x4 AT = {0.f, 0.f, 0.f, 0.f};
+                AT = mfma32(kf0, rf0, AT);
+                AT = mfma32(kf1, rf1, AT);
+                // Y = R~ S
+                f32x4 Y = {0.f, 0.f, 0.f, 0.f};
+                Y = mfma32(rf0, acc_as_operand(S[0], S[1]), Y);
+                Y = mfma32(rf1, acc_as_operand(S[2], S[3]), Y);
+                settle(AT);
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    const int s = 4 * g + rr;
+                    AT[rr] = (l16 > s) ? AT[rr] : ((l16 == s) ? rukv : 0.f);
+                }
+                // Y += A V : the masked A^T accumulator IS the A operand (row t = l16, k-slots s = 4g+r)
+                chain_gap(Y);
+                Y = mfma16(make_s16x4(pack_bf16x2(AT[0], AT[1]), pack_bf16x2(AT[2], AT[3])), vf, Y);
+                // S <- diag(g) (S + K~^T V)
+#pragma unroll
+                for (int m = 0; m < 4; ++m) S[m] = mfma16(frag_ct(B.ktT, 16 * m + l16, 16 * p + 4 * g), vf, S[m]);
+                settle(Y, S[0], S[1], S[2], S[3]);   // Y is stored, S scaled and converted by VALU code from here on
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    const float4 gg = *reinterpret_cast<const float4 *>(&B.g[p][16 * m + 4 * g]);
+                    S[m][0] *= gg.x; S[m][1] *= gg.y; S[m][2] *= gg.z; S[m][3] *= gg.w;
+                }
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    const int t = t0 + 16 * p + 4 * g + rr;
+                    if (!kRagged || t < T) st16(y_h, (uint32_t)t * (uint32_t)C * 2u + 2u * (uint32_t)(16 * q + l16), Y[rr]);
+                }
+            }
+        }
+        if (sT != nullptr) {
+            Ts *p = sT + ((int64_t)b * H + h) * kN * kN + 16 * q + l16;
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) store1(p + (16 * m + 4 * g + rr) * kN, S[m][rr]);
+        }
+    } else {
+        // ------------------------------ producer: operand preparation ------------------------------
+        const int p = wave - 4, ch = lane;
+        const float uc = load1(u + h * kN + ch);
+        const bf16_t *rb = r + base, *kb_ = k + base, *vb = v + base, *wb = w + base;   // uniform
+        const uint32_t rowbytes = (uint32_t)C * 2u;
+        uint32_t qr[16], qk[16], qv[16], qw[16];
+        // Tokens past the end read as r = k = v = 0, w = -inf (exp(w) = 0, decay 1).  Without kRagged
+        // a tile is either entirely inside the sequence or entirely outside.
+        auto prefetch = [&](int c) {
+            const int tb = c * CL + 16 * p;
+            if (tb < T) {   // uniform: a tile entirely past the end is neither loaded, prepared nor consumed
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int t = tb + e;
+                    const bool ok = !kRagged || t < T;
+                    const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes + 2u * (uint32_t)ch;
+                    const uint32_t a = ld16(rb, o), bb = ld16(kb_, o), cc = ld16(vb, o), dd = ld16(wb, o);
+                    qr[e] = ok ? a : 0u; qk[e] = ok ? bb : 0u; qv[e] = ok ? cc : 0u; qw[e] = ok ? dd : 0xff80u;
+                }
+            }
+        };
+        auto prepare = [&](int c) {   // consumes the prefetched registers, refills them for chunk c+1
+            FwdBuf &B = buf[c & 1];
+            const bool tile_in = c * CL + 16 * p < T;
+            float fr[16], fk[16], fw[16];
+            uint32_t vbits[8];
+            if (tile_in) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    fr[e] = bf16_bits_to_float(qr[e]); fk[e] = bf16_bits_to_float(qk[e]); fw[e] = bf16_bits_to_float(qw[e]);
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) vbits[e] = qv[2 * e] | (qv[2 * e + 1] << 16);
+            }
+            if (c + 1 < nchunk) prefetch(c + 1);
+            if (tile_in) {
+
+            // exponents are kept in base 2 (one v_exp_f32 each, no extra scaling multiply)
+            float xr[16], xk[16], pr[16];
+            float cs2 = 0.f, pa = 1.f;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const float ew2 = exp2_fast(fw[e] * kLog2e) * kLog2e;   // exp(w) * log2(e)
+                xr[e] = fr[e] * pa;               // r exp(-c_t)
+                cs2 += ew2;
+                xk[e] = fk[e] * exp2_fast(cs2);   // k exp(+c_{t+1})
+                pa *= exp2_fast(-ew2);
+                pr[e] = fr[e] * uc * fk[e];
+            }
+            if (__builtin_amdgcn_ballot_w64(!(cs2 <= kWildLimit * kLog2e)) != 0ull) {
+                if (lane == 0) s_wild = 1;
+            }
+            store_rows_paired(B.rt, 16 * p, lane, xr);
+            store_rows_paired(B.kt, 16 * p, lane, xk);
+            uint32_t kb[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) kb[e] = pack_bf16x2(xk[2 * e], xk[2 * e + 1]);
+            *reinterpret_cast<uint4 *>(&B.ktT[ch][16 * p]) = make_uint4(kb[0], kb[1], kb[2], kb[3]);
+            *reinterpret_cast<uint4 *>(&B.ktT[ch][16 * p + 8]) = make_uint4(kb[4], kb[5], kb[6], kb[7]);
+            *reinterpret_cast<uint4 *>(&B.vT[ch][16 * p]) = make_uint4(vbits[0], vbits[1], vbits[2], vbits[3]);
+            *reinterpret_cast<uint4 *>(&B.vT[ch][16 * p + 8]) = make_uint4(vbits[4], vbits[5], vbits[6], vbits[7]);
+            B.g[p][ch] = pa;
+            const float tot = transpose_reduce16(pr, lane);
+            if ((lane & 3) == 0) B.ruk[16 * p + ((lane >> 2) & 15)] = tot;
+            }
+        };
+        prefetch(0);
+        prepare(0);
+        for (int c = 0; c < nchunk; ++c) {
+            __syncthreads();
+            if (c + 1 < nchunk) prepare(c + 1);
+        }
+    }
+    // exact second pass for this (b, h) if any of its tiles left the representable range
+    __threadfence_block();   // workgroup scope is enough (and a device-scope fence would write back the L2)
+    __syncthreads();
+    if (s_wild)
+        scan_fwd_body<bf16_t, bf16_t, Ts>(*reinterpret_cast<ScanFwdLds *>(smem), b, h, T, H, r, k, v, w, u, s0, map, y, sT);
+}
+
+hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
+                         const void *r, const void *k, const void *v, const void *w, const void *u,
+                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states)
+{
+    const size_t lds = 2 * sizeof(FwdBuf);
+    auto launch = [&](auto kern, auto *state_tag) -> hipError_t {
+        typedef std::remove_pointer_t<decltype(state_tag)> Ts;
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(512), lds, st, (int)T, (int)H,
+                           (const bf16_t *)r, (const bf16_t *)k, (const bf16_t *)v, (const bf16_t *)w, (const bf16_t *)u,
+                           (const Ts *)s0, map, (bf16_t *)y, (Ts *)sT, (float *)saved_states);
+        return hipGetLastError();
+    };
+    const bool save = saved_states != nullptr, ragged = (T % 16) != 0;
+    float *f32tag = nullptr;
+    bf16_t *bf16tag = nullptr;
+    if (state_dtype == kF32) {
+        if (ragged) return save ? launch(chunk_fwd_kernel<float, true, true>, f32tag) : launch(chunk_fwd_kernel<float, false, true>, f32tag);
+        return save ? launch(chunk_fwd_kernel<float, true, false>, f32tag) : launch(chunk_fwd_kernel<float, false, false>, f32tag);
+    }
+    if (ragged) return save ? launch(chunk_fwd_kernel<bf16_t, true, true>, bf16tag) : launch(chunk_fwd_kernel<bf16_t, false, true>, bf16tag);
+    return save ? launch(chunk_fwd_kernel<bf16_t, true, false>, bf16tag) : launch(chunk_fwd_kernel<bf16_t, false, false>, bf16tag);
+}
+
+}  // namespace wkv6
+

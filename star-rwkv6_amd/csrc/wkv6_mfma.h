@@ -1,0 +1,169 @@
+// MFMA fragment helpers shared by the chunked WKV6 kernels (gfx950, wave64).
+#pragma once
+#include "wkv6_common.h"
+
+namespace wkv6 {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+constexpr int LDA = 68;  // row pitch (elements) of [token][channel] operand arrays: 136 B, conflict-free 8-byte fragment reads
+constexpr float kWildLimit = 64.f;
+constexpr float kLog2e = 1.4426950408889634f;
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }   // v_exp_f32
+
+__device__ __forceinline__ bf16x8 make_bf16x8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
+    const u32x4 t = {a, b, c, d};
+    return __builtin_bit_cast(bf16x8, t);
+}
+__device__ __forceinline__ s16x4 make_s16x4(uint32_t a, uint32_t b) {
+    const u32x2 t = {a, b};
+    return __builtin_bit_cast(s16x4, t);
+}
+__device__ __forceinline__ f32x4 mfma32(bf16x8 a, bf16x8 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mfma16(s16x4 a, s16x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
+}
+// Two software-inserted delays around the MFMAs.  Both pass the accumulators through an asm
+// statement, so neither the MFMAs that write them nor the code that reads them can move across.
+//
+// chain_gap(acc): 8 idle issue slots between two MFMAs of DIFFERENT shape (16x16x16 and 16x16x32)
+// that are chained through the same accumulator.  hipcc 7.2 schedules such a pair 0-3 slots apart,
+// and on gfx950 the second MFMA then reads a stale SrcC: the products came out wrong whenever the
+// scheduler happened to place the pair that close and right when it left 5 or more slots.
+// Same-shape accumulation chains are not affected.
+//
+// settle(acc...): 16 idle slots before VALU code (masks, scaling, bf16 conversion, stores) reads
+// MFMA results; belt and braces on top of the wait states the compiler inserts itself.
+#define WKV6_SETTLE_ASM "s_nop 15"
+__device__ __forceinline__ void chain_gap(f32x4 &a) { asm volatile("s_nop 7" : "+v"(a)); }
+__device__ __forceinline__ void settle(f32x4 &a) { asm volatile(WKV6_SETTLE_ASM : "+v"(a)); }
+__device__ __forceinline__ void settle(f32x4 &a, f32x4 &b) { asm volatile(WKV6_SETTLE_ASM : "+v"(a), "+v"(b)); }
+__device__ __forceinline__ void settle(f32x4 &a, f32x4 &b, f32x4 (&g1)[4]) {
+    asm volatile(WKV6_SETTLE_ASM : "+v"(a), "+v"(b), "+v"(g1[0]), "+v"(g1[1]), "+v"(g1[2]), "+v"(g1[3]));
+}
+__device__ __forceinline__ void settle(f32x4 &a, f32x4 (&g1)[4]) {
+    asm volatile(WKV6_SETTLE_ASM : "+v"(a), "+v"(g1[0]), "+v"(g1[1]), "+v"(g1[2]), "+v"(g1[3]));
+}
+__device__ __forceinline__ void settle(f32x4 &a, f32x4 &b, f32x4 &c) {
+    asm volatile(WKV6_SETTLE_ASM : "+v"(a), "+v"(b), "+v"(c));
+}
+__device__ __forceinline__ void settle(f32x4 &a, f32x4 &b, f32x4 &c, f32x4 &d) {
+    asm volatile(WKV6_SETTLE_ASM : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
+__device__ __forceinline__ void settle(f32x4 &a, f32x4 &b, f32x4 &c, f32x4 &d, f32x4 &e) {
+    asm volatile(WKV6_SETTLE_ASM : "+v"(a), "+v"(b), "+v"(c), "+v"(d), "+v"(e));
+}
+__device__ __forceinline__ void settle(f32x4 &a, f32x4 &b, f32x4 &c, f32x4 (&g1)[4], f32x4 (&g2)[4]) {
+    asm volatile(WKV6_SETTLE_ASM : "+v"(a), "+v"(b), "+v"(c), "+v"(g1[0]), "+v"(g1[1]), "+v"(g1[2]), "+v"(g1[3]),
+                 "+v"(g2[0]), "+v"(g2[1]), "+v"(g2[2]), "+v"(g2[3]));
+}
+__device__ __forceinline__ float xor1(float x) {   // value of the neighbouring lane (lane ^ 1)
+    return __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0xB1, 0xF, 0xF, true));
+}
+
+// Sum over the four 16-lane rows of the wave (lanes l, l^16, l^32, l^48), result in every lane,
+// with the gfx950 row-swap instructions instead of LDS permutes.
+__device__ __forceinline__ float sum_rows(float x) {
+    const uint32_t xi = __float_as_uint(x);
+    const u32x2 a = __builtin_amdgcn_permlane16_swap(xi, xi, false, false);   // rows (0,0,2,2) and (1,1,3,3)
+    const uint32_t si = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
+    const u32x2 b = __builtin_amdgcn_permlane32_swap(si, si, false, false);   // rows (0,1,0,1) and (2,3,2,3)
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+// Exclusive prefix over the four rows: row g receives the sum of x over rows 0..g-1.
+__device__ __forceinline__ float prefix_rows(float x, int g) {
+    const uint32_t xi = __float_as_uint(x);
+    const u32x2 a = __builtin_amdgcn_permlane16_swap(xi, xi, false, false);   // a[0] = rows (0,0,2,2), a[1] = rows (1,1,3,3)
+    const float below = __uint_as_float(a[0]);                                 // in odd rows: the row just below
+    const uint32_t si = __float_as_uint(__uint_as_float(a[0]) + __uint_as_float(a[1]));
+    const u32x2 b = __builtin_amdgcn_permlane32_swap(si, si, false, false);   // b[0] = rows 0+1 everywhere
+    return ((g & 1) ? below : 0.f) + ((g & 2) ? __uint_as_float(b[0]) : 0.f);
+}
+
+// 16-bit load at a uniform base + 32-bit per-lane byte offset (lets the compiler use the
+// scalar-base addressing form instead of 64-bit per-lane address arithmetic)
+__device__ __forceinline__ uint32_t ld16(const void *base, uint32_t byteoff) {
+    return *reinterpret_cast<const uint16_t *>(reinterpret_cast<const char *>(base) + byteoff);
+}
+
+__device__ __forceinline__ void st16(void *base, uint32_t byteoff, float x) {
+    *reinterpret_cast<uint16_t *>(reinterpret_cast<char *>(base) + byteoff) = (uint16_t)pack_bf16x2(x, 0.f);
+}
+
+// A/B fragment of a [token][channel] array for one 16x16x32 MFMA covering channels [32h, 32h+32).
+// Lane group g = lane/16 takes the k-slots {32h+4g+e, 32h+16+4g+e : e<4}: the same channels its
+// accumulator registers hold when a 64x16 fp32 tile stack (rows 16m+4g+r) is reused as an operand.
+__device__ __forceinline__ bf16x8 frag_tc(const uint16_t (*a)[LDA], int row, int h, int g) {
+    const uint2 lo = *reinterpret_cast<const uint2 *>(&a[row][32 * h + 4 * g]);
+    const uint2 hi = *reinterpret_cast<const uint2 *>(&a[row][32 * h + 16 + 4 * g]);
+    return make_bf16x8(lo.x, lo.y, hi.x, hi.y);
+}
+// A/B fragment of a [channel][token] array for one 16x16x16 MFMA: 4 consecutive tokens.
+template <int LD>
+__device__ __forceinline__ s16x4 frag_ct(const uint16_t (*a)[LD], int ch, int tok) {
+    const uint2 x = *reinterpret_cast<const uint2 *>(&a[ch][tok]);
+    return make_s16x4(x.x, x.y);
+}
+// two accumulator tiles (rows 16m+4g+r and 16(m+1)+4g+r) as the bf16 operand of a 16x16x32 MFMA
+__device__ __forceinline__ bf16x8 acc_as_operand(const f32x4 &a, const f32x4 &b) {
+    return make_bf16x8(pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]), pack_bf16x2(b[0], b[1]), pack_bf16x2(b[2], b[3]));
+}
+
+// sum over the 64 lanes of 16 per-lane values; lane l receives the total of value (l>>2)&15
+__device__ __forceinline__ float transpose_reduce16(const float (&p)[16], int lane) {
+    float x8[8], x4[4], x2[2];
+    const bool b5 = lane & 32, b4 = lane & 16, b3 = lane & 8, b2 = lane & 4;
+#pragma unroll
+    for (int a = 0; a < 8; ++a) x8[a] = (b5 ? p[a + 8] : p[a]) + __shfl_xor(b5 ? p[a] : p[a + 8], 32);
+#pragma unroll
+    for (int a = 0; a < 4; ++a) x4[a] = (b4 ? x8[a + 4] : x8[a]) + __shfl_xor(b4 ? x8[a] : x8[a + 4], 16);
+#pragma unroll
+    for (int a = 0; a < 2; ++a) x2[a] = (b3 ? x4[a + 2] : x4[a]) + __shfl_xor(b3 ? x4[a] : x4[a + 2], 8);
+    float x = (b2 ? x2[1] : x2[0]) + __shfl_xor(b2 ? x2[0] : x2[1], 4);
+    x += __shfl_xor(x, 2);
+    x += __shfl_xor(x, 1);
+    return x;
+}
+
+// Writes row-major [token][channel] bf16 with 4-byte stores: lanes 2c and 2c+1 swap one value so
+// that the even lane stores (x[c], x[c+1]) of an even token row and the odd lane those of the
+// next row.
+__device__ __forceinline__ void store_rows_paired(uint16_t (*a)[LDA], int row0, int lane, const float (&x)[16]) {
+    const bool odd = lane & 1;
+#pragma unroll
+    for (int e = 0; e < 16; e += 2) {
+        const float got = xor1(odd ? x[e] : x[e + 1]);
+        const uint32_t pk = odd ? pack_bf16x2(got, x[e + 1]) : pack_bf16x2(x[e], got);
+        *reinterpret_cast<uint32_t *>(&a[row0 + e + (odd ? 1 : 0)][lane & ~1]) = pk;
+    }
+}
+
+// fragment of a global (B,T,C) bf16 tensor row (uniform base + 32-bit byte offset of the row) for a
+// 16x16x32 MFMA, same k-slot order as frag_tc
+__device__ __forceinline__ bf16x8 frag_global(const void *base, uint32_t rowbyte, int h, int g) {
+    const char *b = reinterpret_cast<const char *>(base);
+    const uint2 lo = *reinterpret_cast<const uint2 *>(b + (rowbyte + 2u * (uint32_t)(32 * h + 4 * g)));
+    const uint2 hi = *reinterpret_cast<const uint2 *>(b + (rowbyte + 2u * (uint32_t)(32 * h + 16 + 4 * g)));
+    return make_bf16x8(lo.x, lo.y, hi.x, hi.y);
+}
+__device__ __forceinline__ s16x4 pack4(const f32x4 &a) {
+    return make_s16x4(pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]));
+}
+__device__ __forceinline__ void unpack4(const s16x4 &a, float (&o)[4]) {
+    const u32x2 t = __builtin_bit_cast(u32x2, a);
+    o[0] = __uint_as_float(t[0] << 16); o[1] = __uint_as_float(t[0] & 0xffff0000u);
+    o[2] = __uint_as_float(t[1] << 16); o[3] = __uint_as_float(t[1] & 0xffff0000u);
+}
+__device__ __forceinline__ void unpack8(const bf16x8 &a, float (&o)[8]) {
+    const u32x4 t = __builtin_bit_cast(u32x4, a);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { o[2 * i] = __uint_as_float(t[i] << 16); o[2 * i + 1] = __uint_as_float(t[i] & 0xffff0000u); }
+}
+
+}  // namespace wkv6
