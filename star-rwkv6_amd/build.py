@@ -17,7 +17,7 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17", "-fno-gpu-rdc",
     # packed-fp32 VALU forms are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option", "-Wno-unknown-attributes",
+    "-Wno-unused-command-line-argument", "-Wno-inline-asm", "-Wno-unknown-warning-option", "-Wno-unknown-attributes",
     "-I" + INCLUDE, "-I" + CSRC,
 ]
 

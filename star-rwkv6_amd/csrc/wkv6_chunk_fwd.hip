@@ -6,15 +6,19 @@
 //
 //   c_t = sum_{s<t} exp(w_s) inside the tile (so exp(-c_t) is the decay from the tile start to t)
 //   R~[t][j] = r_t[j] exp(-c_t[j])            K~[t][j] = k_t[j] exp(+c_{t+1}[j])
-//   K^[t][j] = k_t[j] exp(-(c_16[j] - c_{t+1}[j]))         g[j] = exp(-c_16[j])
+//   g[j] = exp(-c_16[j])
 //   A[t][s]  = R~_t . K~_s  (s < t),  A[t][t] = sum_j r_t[j] u[j] k_t[j]
 //   Y        = R~ S + A V          (16x64x64 and 16x16x16 MFMA, K index j resp. s)
-//   S       <- diag(g) S + K^T V   (64x16x16 MFMA, K index s)
+//   S       <- diag(g) (S + K~^T V)   (64x16x16 MFMA, K index s)
 //
-// The four "producer" waves (wave 4+p prepares tile p, lane = channel) compute these operands in
-// fp32 for the NEXT chunk while the consumers run the MFMAs of the current one; LDS operand
-// buffers are double-buffered and the two roles meet at one barrier per chunk.  HBM traffic is
-// exactly the algorithmic minimum (r,k,v,w read once, y written once).
+// Data path.  The raw r, k, w, v rows of a chunk go from global memory straight into LDS tiles
+// (16-byte pieces, no registers), two chunks ahead of their use.  The four "producer" waves (wave
+// 4+p prepares tile p, lane = channel) read r, k, w from there, compute R~, K~, g and the diagonal
+// in fp32 for the NEXT chunk and write them back as bf16 tiles while the consumers run the MFMAs of
+// the current one; the consumers take V directly from its raw tile.  Every tile is stored once,
+// [token][channel]; fragments with the k-slots along the tokens come from the transposing LDS read.
+// The two roles meet at one barrier per chunk.  HBM traffic is exactly the algorithmic minimum
+// (r,k,v,w read once, y written once).
 //
 // exp(+c) needs the decay accumulated inside one 16-token tile to stay in range.  A producer wave
 // that meets a tile whose summed exp(w) exceeds kWildLimit in any channel raises a flag in LDS, and
@@ -29,15 +33,15 @@
 namespace wkv6 {
 
 constexpr int CL = 64;   // tokens per chunk
-constexpr int LDT = 72;  // row pitch (elements) of [channel][token] operand arrays: 144 B, 16-byte aligned rows
 
-struct alignas(16) FwdBuf {
-    uint16_t rt[CL][LDA];   // R~[t][j]
-    uint16_t kt[CL][LDA];   // K~[t][j]
-    uint16_t ktT[kN][LDT];  // K~[t][j] stored [j][t]  (K^ = g K~ is never formed: S <- g (S + K~^T V))
-    uint16_t vT[kN][LDT];   // V[t][i]  stored [i][t]
-    float g[4][kN];         // per-tile decay exp(-c_16)
-    float ruk[CL];          // sum_j r u k per token
+// LDS map of the forward kernel (byte offsets into the dynamic block)
+struct FwdLds {
+    static constexpr int kRawRKW = 0;                                   // [2 chunk parities][r,k,w] raw tiles
+    static constexpr int kRawV = kRawRKW + 2 * 3 * kTileBytes;          // [3] raw v tiles (chunk % 3)
+    static constexpr int kOp = kRawV + 3 * kTileBytes;                  // [2] operand blocks
+    static constexpr int kOpRt = 0, kOpKt = kTileBytes, kOpG = 2 * kTileBytes, kOpRuk = kOpG + 4 * kN * 4;
+    static constexpr int kOpBytes = kOpRuk + CL * 4;
+    static constexpr int kBytes = kOp + 2 * kOpBytes;
 };
 
 // kSave: also write the state at every chunk start to `ckpt` (fp32, [b][h][chunk][j][i]) for the
@@ -51,8 +55,7 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
 {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_wild;
-    FwdBuf *buf = reinterpret_cast<FwdBuf *>(smem);
-    static_assert(sizeof(ScanFwdLds) <= 2 * sizeof(FwdBuf), "the exact second pass reuses the operand buffers");
+    static_assert(sizeof(ScanFwdLds) <= FwdLds::kBytes, "the exact second pass reuses the LDS block");
     if (threadIdx.x == 0) s_wild = 0;
     __syncthreads();
 
@@ -87,16 +90,20 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
                     for (int rr = 0; rr < 4; ++rr) dst[(16 * m + 4 * g + rr) * kN] = S[m][rr];
             }
             __syncthreads();
-            const FwdBuf &B = buf[c & 1];
+            const unsigned char *op = smem + FwdLds::kOp + (c & 1) * FwdLds::kOpBytes;
+            const unsigned char *rt = op + FwdLds::kOpRt, *kt = op + FwdLds::kOpKt;
+            const float *gv_ = reinterpret_cast<const float *>(op + FwdLds::kOpG);
+            const float *ruk = reinterpret_cast<const float *>(op + FwdLds::kOpRuk);
+            const unsigned char *vt = smem + FwdLds::kRawV + (c % 3) * kTileBytes;
             const int t0 = c * CL;
 #pragma unroll 1
             for (int p = 0; p < 4; ++p) {
                 if (t0 + 16 * p >= T) break;
                 const int row = 16 * p + l16;
-                const bf16x8 rf0 = frag_tc(B.rt, row, 0, g), rf1 = frag_tc(B.rt, row, 1, g);
-                const bf16x8 kf0 = frag_tc(B.kt, row, 0, g), kf1 = frag_tc(B.kt, row, 1, g);
-                const s16x4 vf = frag_ct(B.vT, 16 * q + l16, 16 * p + 4 * g);
-                const float rukv = B.ruk[row];
+                const bf16x8 rf0 = tile_frag_ch(rt, row, 0, g), rf1 = tile_frag_ch(rt, row, 1, g);
+                const bf16x8 kf0 = tile_frag_ch(kt, row, 0, g), kf1 = tile_frag_ch(kt, row, 1, g);
+                const s16x4 vf = tile_frag_tok(vt, 16 * q, 16 * p, l16, g);
+                const float rukv = ruk[row];
                 // A^T[s][t] = K~_s . R~_t  (accumulator rows s = 4g+r, column t = l16)
                 f32x4 AT = {0.f, 0.f, 0.f, 0.f};
                 AT = mfma32(kf0, rf0, AT);
@@ -116,11 +123,11 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
                 Y = mfma16(make_s16x4(pack_bf16x2(AT[0], AT[1]), pack_bf16x2(AT[2], AT[3])), vf, Y);
                 // S <- diag(g) (S + K~^T V)
 #pragma unroll
-                for (int m = 0; m < 4; ++m) S[m] = mfma16(frag_ct(B.ktT, 16 * m + l16, 16 * p + 4 * g), vf, S[m]);
+                for (int m = 0; m < 4; ++m) S[m] = mfma16(tile_frag_tok(kt, 16 * m, 16 * p, l16, g), vf, S[m]);
                 settle(Y, S[0], S[1], S[2], S[3]);   // Y is stored, S scaled and converted by VALU code from here on
 #pragma unroll
                 for (int m = 0; m < 4; ++m) {
-                    const float4 gg = *reinterpret_cast<const float4 *>(&B.g[p][16 * m + 4 * g]);
+                    const float4 gg = *reinterpret_cast<const float4 *>(&gv_[p * kN + 16 * m + 4 * g]);
                     S[m][0] *= gg.x; S[m][1] *= gg.y; S[m][2] *= gg.z; S[m][3] *= gg.w;
                 }
 #pragma unroll
@@ -138,43 +145,52 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
                 for (int rr = 0; rr < 4; ++rr) store1(p + (16 * m + 4 * g + rr) * kN, S[m][rr]);
         }
     } else {
-        // ------------------------------ producer: operand preparation ------------------------------
+        // ------------------------------ producer: loads and operand preparation ------------------------------
         const int p = wave - 4, ch = lane;
         const float uc = load1(u + h * kN + ch);
         const bf16_t *rb = r + base, *kb_ = k + base, *vb = v + base, *wb = w + base;   // uniform
         const uint32_t rowbytes = (uint32_t)C * 2u;
-        uint32_t qr[16], qk[16], qv[16], qw[16];
-        // Tokens past the end read as r = k = v = 0, w = -inf (exp(w) = 0, decay 1).  Without kRagged
-        // a tile is either entirely inside the sequence or entirely outside.
-        auto prefetch = [&](int c) {
+        const uint32_t lds0 = lds_address(smem);
+        // this lane's part of an 8-row block load: row (lane >> 3), 16-byte piece swizzled with the row
+        const int lrow = lane >> 3;
+        const uint32_t lpiece = (uint32_t)(((lane & 7) ^ lrow) << 4);
+        // Rows past the end of the sequence are fetched from row T-1 (valid memory); the operand
+        // preparation turns them into r = k = 0, w = -inf, and v rows that only ever meet zero
+        // operands.  A tile entirely past the end is neither loaded, prepared nor consumed.
+        auto issue_loads = [&](int c) -> bool {
             const int tb = c * CL + 16 * p;
-            if (tb < T) {   // uniform: a tile entirely past the end is neither loaded, prepared nor consumed
+            if (tb >= T) return false;
+            const uint32_t rkw = lds0 + FwdLds::kRawRKW + (c & 1) * 3 * kTileBytes + 16 * p * kTileRow;
+            const uint32_t vv = lds0 + FwdLds::kRawV + (c % 3) * kTileBytes + 16 * p * kTileRow;
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    const int t = tb + e;
-                    const bool ok = !kRagged || t < T;
-                    const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes + 2u * (uint32_t)ch;
-                    const uint32_t a = ld16(rb, o), bb = ld16(kb_, o), cc = ld16(vb, o), dd = ld16(wb, o);
-                    qr[e] = ok ? a : 0u; qk[e] = ok ? bb : 0u; qv[e] = ok ? cc : 0u; qw[e] = ok ? dd : 0xff80u;
-                }
+            for (int hf = 0; hf < 2; ++hf) {
+                const int t = tb + 8 * hf + lrow;
+                const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes + lpiece;
+                load_rows8_to_lds(rb, o, rkw + 8 * hf * kTileRow);
+                load_rows8_to_lds(kb_, o, rkw + kTileBytes + 8 * hf * kTileRow);
+                load_rows8_to_lds(wb, o, rkw + 2 * kTileBytes + 8 * hf * kTileRow);
+                load_rows8_to_lds(vb, o, vv + 8 * hf * kTileRow);
             }
+            return true;
         };
-        auto prepare = [&](int c) {   // consumes the prefetched registers, refills them for chunk c+1
-            FwdBuf &B = buf[c & 1];
-            const bool tile_in = c * CL + 16 * p < T;
+        // per-lane byte offsets of channel `ch` inside a tile row, for the 8 swizzle phases
+        uint32_t choff[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) choff[s] = (uint32_t)((((ch >> 3) ^ s) << 4) + ((ch & 7) << 1)) + (uint32_t)(16 * p * kTileRow);
+        auto prepare = [&](int c) {
+            if (c * CL + 16 * p >= T) return;
+            const unsigned char *raw = smem + FwdLds::kRawRKW + (c & 1) * 3 * kTileBytes;
+            unsigned char *op = smem + FwdLds::kOp + (c & 1) * FwdLds::kOpBytes;
             float fr[16], fk[16], fw[16];
-            uint32_t vbits[8];
-            if (tile_in) {
 #pragma unroll
-                for (int e = 0; e < 16; ++e) {
-                    fr[e] = bf16_bits_to_float(qr[e]); fk[e] = bf16_bits_to_float(qk[e]); fw[e] = bf16_bits_to_float(qw[e]);
-                }
-#pragma unroll
-                for (int e = 0; e < 8; ++e) vbits[e] = qv[2 * e] | (qv[2 * e + 1] << 16);
+            for (int e = 0; e < 16; ++e) {
+                const uint32_t o = choff[e & 7] + e * kTileRow;
+                uint32_t a = *reinterpret_cast<const uint16_t *>(raw + o);
+                uint32_t bb = *reinterpret_cast<const uint16_t *>(raw + kTileBytes + o);
+                uint32_t dd = *reinterpret_cast<const uint16_t *>(raw + 2 * kTileBytes + o);
+                if (kRagged && c * CL + 16 * p + e >= T) { a = 0u; bb = 0u; dd = 0xff80u; }
+                fr[e] = bf16_bits_to_float(a); fk[e] = bf16_bits_to_float(bb); fw[e] = bf16_bits_to_float(dd);
             }
-            if (c + 1 < nchunk) prefetch(c + 1);
-            if (tile_in) {
-
             // exponents are kept in base 2 (one v_exp_f32 each, no extra scaling multiply)
             float xr[16], xk[16], pr[16];
             float cs2 = 0.f, pa = 1.f;
@@ -190,26 +206,35 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
             if (__builtin_amdgcn_ballot_w64(!(cs2 <= kWildLimit * kLog2e)) != 0ull) {
                 if (lane == 0) s_wild = 1;
             }
-            store_rows_paired(B.rt, 16 * p, lane, xr);
-            store_rows_paired(B.kt, 16 * p, lane, xk);
-            uint32_t kb[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) kb[e] = pack_bf16x2(xk[2 * e], xk[2 * e + 1]);
-            *reinterpret_cast<uint4 *>(&B.ktT[ch][16 * p]) = make_uint4(kb[0], kb[1], kb[2], kb[3]);
-            *reinterpret_cast<uint4 *>(&B.ktT[ch][16 * p + 8]) = make_uint4(kb[4], kb[5], kb[6], kb[7]);
-            *reinterpret_cast<uint4 *>(&B.vT[ch][16 * p]) = make_uint4(vbits[0], vbits[1], vbits[2], vbits[3]);
-            *reinterpret_cast<uint4 *>(&B.vT[ch][16 * p + 8]) = make_uint4(vbits[4], vbits[5], vbits[6], vbits[7]);
-            B.g[p][ch] = pa;
-            const float tot = transpose_reduce16(pr, lane);
-            if ((lane & 3) == 0) B.ruk[16 * p + ((lane >> 2) & 15)] = tot;
+            for (int e = 0; e < 16; e += 2) {
+                const uint32_t pr2 = pack_bf16x2(xr[e], xr[e + 1]), pk2 = pack_bf16x2(xk[e], xk[e + 1]);
+                const uint32_t o0 = choff[e & 7] + e * kTileRow, o1 = choff[(e + 1) & 7] + (e + 1) * kTileRow;
+                *reinterpret_cast<uint16_t *>(op + FwdLds::kOpRt + o0) = (uint16_t)pr2;
+                *reinterpret_cast<uint16_t *>(op + FwdLds::kOpRt + o1) = (uint16_t)(pr2 >> 16);
+                *reinterpret_cast<uint16_t *>(op + FwdLds::kOpKt + o0) = (uint16_t)pk2;
+                *reinterpret_cast<uint16_t *>(op + FwdLds::kOpKt + o1) = (uint16_t)(pk2 >> 16);
             }
+            reinterpret_cast<float *>(op + FwdLds::kOpG)[p * kN + ch] = pa;
+            const float tot = transpose_reduce16(pr, lane);
+            if ((lane & 3) == 0) reinterpret_cast<float *>(op + FwdLds::kOpRuk)[16 * p + ((lane >> 2) & 15)] = tot;
         };
-        prefetch(0);
+        // chunk c is loaded during iteration c-2 (or the prologue), prepared during iteration c-1
+        issue_loads(0);
+        bool next_in_flight = nchunk > 1 && issue_loads(1);
+        if (next_in_flight) wait_loads<8>(); else wait_loads<0>();
         prepare(0);
         for (int c = 0; c < nchunk; ++c) {
             __syncthreads();
-            if (c + 1 < nchunk) prepare(c + 1);
+            // the raw r, k, w block of chunk c (read by this wave's prepare(c) before the barrier) and the
+            // raw v block of chunk c-1 (read by the consumers before the barrier) are free again
+            const bool far_in_flight = c + 2 < nchunk && issue_loads(c + 2);
+            if (c + 1 < nchunk) {
+                if (far_in_flight) wait_loads<8>(); else wait_loads<0>();
+                prepare(c + 1);
+            }
         }
+        wait_loads<0>();
     }
     // exact second pass for this (b, h) if any of its tiles left the representable range
     __threadfence_block();   // workgroup scope is enough (and a device-scope fence would write back the L2)
@@ -222,7 +247,7 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
                          const void *r, const void *k, const void *v, const void *w, const void *u,
                          const void *s0, const int64_t *map, void *y, void *sT, void *saved_states)
 {
-    const size_t lds = 2 * sizeof(FwdBuf);
+    const size_t lds = FwdLds::kBytes;
     auto launch = [&](auto kern, auto *state_tag) -> hipError_t {
         typedef std::remove_pointer_t<decltype(state_tag)> Ts;
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -244,4 +269,3 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
 }
 
 }  // namespace wkv6
-

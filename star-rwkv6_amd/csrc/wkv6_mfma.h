@@ -166,4 +166,50 @@ __device__ __forceinline__ void unpack8(const bf16x8 &a, float (&o)[8]) {
     for (int i = 0; i < 4; ++i) { o[2 * i] = __uint_as_float(t[i] << 16); o[2 * i + 1] = __uint_as_float(t[i] & 0xffff0000u); }
 }
 
+
+// ------------------------------------------------------------------------------------------
+// LDS tiles: bf16 [token][64 channels], 128-byte rows, no padding; the eight 16-byte pieces of a
+// row are XOR-swizzled with (token & 7).  One layout serves the loads that fill a tile straight
+// from global memory, the lane = channel accesses of the operand preparation, and both MFMA
+// fragment orientations (the second through the transposing LDS read of gfx950).
+// ------------------------------------------------------------------------------------------
+constexpr int kTileRow = 128;                 // bytes per token row
+constexpr int kTileBytes = 64 * kTileRow;     // one 64-token chunk of one tensor
+
+__device__ __forceinline__ uint32_t tile_off(int t, int ch) {
+    return ((uint32_t)t << 7) + (((((uint32_t)ch >> 3) ^ (uint32_t)t) & 7u) << 4) + (((uint32_t)ch & 7u) << 1);
+}
+
+// Eight token rows (t0 .. t0+7 of the tile, t0 a multiple of 8) of one head's 128-byte row
+// segments, global -> LDS without passing through registers: lane L brings the 16-byte piece that
+// belongs at LDS position 16 L of the block.  `voff` is the lane's byte offset from the uniform
+// `gbase` (row (L >> 3), piece ((L & 7) ^ (L >> 3))); `lds_addr` the uniform LDS byte address of
+// row t0.  Completion is counted by vmcnt; the compiler does not know about these loads, so the
+// caller waits with wait_loads<N>() (N = number of younger loads allowed to stay in flight).
+__device__ __forceinline__ void load_rows8_to_lds(const void *gbase, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(gbase) : "memory", "m0");
+}
+template <int N> __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
+
+__device__ __forceinline__ uint32_t lds_address(const void *p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const unsigned char *)p;
+}
+
+// A/B fragment with the k-slots along the CHANNELS of token `row`, for one 16x16x32 MFMA over
+// channels [32h, 32h+32): k-slots {32h+4g+e, 32h+16+4g+e : e<4} (the order acc_as_operand produces).
+__device__ __forceinline__ bf16x8 tile_frag_ch(const unsigned char *tile, int row, int h, int g) {
+    const uint2 lo = *reinterpret_cast<const uint2 *>(tile + tile_off(row, 32 * h + 4 * g));
+    const uint2 hi = *reinterpret_cast<const uint2 *>(tile + tile_off(row, 32 * h + 16 + 4 * g));
+    return make_bf16x8(lo.x, lo.y, hi.x, hi.y);
+}
+// A/B fragment with the k-slots along the TOKENS, for one 16x16x16 MFMA: the lane (l16, g) of the
+// result holds tile[tk0 + 4g + e][n0 + l16], e < 4.  (The transposing read hands lane l16 of a
+// 16-lane group the l16-th element of each of four 16-element rows; row e is assembled from the
+// 8-byte pieces that lanes 4e..4e+3 of the group point at.)
+__device__ __forceinline__ s16x4 tile_frag_tok(const unsigned char *tile, int n0, int tk0, int l16, int g) {
+    const unsigned char *p = tile + tile_off(tk0 + 4 * g + (l16 >> 2), n0 + 4 * (l16 & 3));
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p);
+}
+
 }  // namespace wkv6
