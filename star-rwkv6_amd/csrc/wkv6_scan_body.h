@@ -313,7 +313,7 @@ struct alignas(16) ScanBwdBLds {
     float s_u[kN];
 };
 
-// All 512 threads of the workgroup work.  P addressed as in sweep A.
+// Threads 0..511 of the workgroup work.  P addressed as in sweep A.
 template <typename Tin, typename Tout>
 __device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLds &L, int b, int h, int T, int H,
         const Tin *__restrict__ r, const Tin *__restrict__ k, const Tin *__restrict__ v,
@@ -325,6 +325,11 @@ __device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLds &L, int b, int h, in
     auto &s_pk = L.s_pk; auto &s_pv = L.s_pv; auto &s_e = L.s_e;
     auto &s_vgy = L.s_vgy; auto &s_ruk = L.s_ruk; auto &s_u = L.s_u;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid >= 512) {   // a larger workgroup: same barrier sequence as below, no work
+        __syncthreads();
+        for (int t0 = ((T - 1) / TC) * TC; t0 >= 0; t0 -= TC) { __syncthreads(); __syncthreads(); __syncthreads(); }
+        return;
+    }
     const int q = wave & 3;
     const bool role_k = wave < 4;
     const int64_t C = (int64_t)H * kN;
