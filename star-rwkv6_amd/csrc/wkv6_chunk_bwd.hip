@@ -33,6 +33,7 @@
 #include "wkv6_kernels.h"
 #include "wkv6_scan_body.h"
 
+#include <stdlib.h>
 #include <type_traits>
 
 namespace wkv6 {
@@ -54,7 +55,17 @@ struct BwdLds {
 };
 static_assert(BwdLds::kBytes <= 160 * 1024, "LDS block of the backward kernel");
 
+// development aid (-DWKV6_TIMING): cycle stamps of workgroup 0, 256 slots per wave, behind the workspace
+#ifdef WKV6_TIMING
+#define WKV6_STAMP() do { if (blockIdx.x == 0 && lane == 0 && dbg_n < 250) a.dbg[(threadIdx.x >> 6) * 256 + dbg_n++] = __builtin_readcyclecounter(); } while (0)
+#define WKV6_STAMP_DECL int dbg_n = 0
+#else
+#define WKV6_STAMP() do { } while (0)
+#define WKV6_STAMP_DECL do { } while (0)
+#endif
+
 struct BwdArgs {
+    long long *dbg;
     int T, H;
     const bf16_t *r, *k, *v, *w, *u, *gy;
     bf16_t *gr, *gk, *gv, *gw, *gu;
@@ -73,9 +84,11 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     const int64_t C = (int64_t)H * kN;
     const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
     const int nchunk = (T + CL - 1) / CL;
-    float *ck = a.ckpt + (int64_t)blockIdx.x * nchunk * (kN * kN);
+    // chunk states: bf16 [chunk][j][i] in the first half of this workgroup's workspace slice
+    bf16_t *ck = reinterpret_cast<bf16_t *>(a.ckpt + (int64_t)blockIdx.x * nchunk * (kN * kN));
     auto mine = [](int p) { return NG == 1 || (p & 1) == (GRP ^ 1); };   // group 0: tiles 3, 1; group 1: tiles 2, 0
     int item = 0;
+    WKV6_STAMP_DECL;
     if (kSweepStates) {
         // phase 1: S^T (rows i, column j = col), checkpoint at every chunk start; group 0 only
         f32x4 S[4];
@@ -88,14 +101,13 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
             const unsigned char *kt = op + BwdLds::kOpKt;
             const float *gg = reinterpret_cast<const float *>(op + BwdLds::kOpG);
             const unsigned char *vt = smem + BwdLds::kRawVG + (item % 3) * 2 * kTileBytes;
-            float *dst = ck + (int64_t)c * (kN * kN) + col * kN;
+            bf16_t *dst = ck + (int64_t)c * (kN * kN) + col * kN;
 #pragma unroll
             for (int m = 0; m < 4; ++m)
-                *reinterpret_cast<float4 *>(dst + 16 * m + 4 * g) = make_float4(S[m][0], S[m][1], S[m][2], S[m][3]);
+                *reinterpret_cast<uint2 *>(dst + 16 * m + 4 * g) = make_uint2(pack_bf16x2(S[m][0], S[m][1]), pack_bf16x2(S[m][2], S[m][3]));
             if (c + 1 == nchunk) continue;   // the state after the last chunk is never used
 #pragma unroll 1
             for (int p = 0; p < 4; ++p) {
-                if (c * CL + 16 * p >= T) break;
                 const s16x4 kq = tile_frag_tok(kt, 16 * q, 16 * p, l16, g);
                 const float gq = gg[p * kN + col];
 #pragma unroll
@@ -117,37 +129,56 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     float gu_acc = 0.f;
     bf16_t *gr_h = a.gr + base, *gk_h = a.gk + base, *gw_h = a.gw + base;
     const uint32_t rowbytes = (uint32_t)C * 2u;
-    // checkpointed forward state of a chunk
-    f32x4 S[4];
+    // checkpointed forward state of a chunk, as loaded (packed bf16)
+    uint2 Sraw[4];
     auto load_state = [&](int c) {
-        const float *src = ck + (int64_t)c * (kN * kN) + col * kN;
+        const bf16_t *src = ck + (int64_t)c * (kN * kN) + col * kN;
 #pragma unroll
-        for (int m = 0; m < 4; ++m) {
-            const float4 x = *reinterpret_cast<const float4 *>(src + 16 * m + 4 * g);
-            S[m] = (f32x4){x.x, x.y, x.z, x.w};
-        }
+        for (int m = 0; m < 4; ++m) Sraw[m] = *reinterpret_cast<const uint2 *>(src + 16 * m + 4 * g);
     };
+    // One chunk visit.  All four tiles are always processed (tokens past the end were prepared as
+    // r = k = 0, decay 1, so they leave both states alone and contribute nothing), which keeps the
+    // body free of branches that change the number of memory operations: the wait for the
+    // prefetched next state (the fake use at the end) is then counted exactly instead of draining
+    // this wave's stores every chunk.
     if (!kSweepStates && nchunk > 0) load_state(nchunk - 1);
     for (int c = nchunk - 1; c >= 0; --c, ++item) {
+        WKV6_STAMP();
         __syncthreads();
+        WKV6_STAMP();
         // with kSweepStates the checkpoints were written by this kernel a moment ago: read them
         // here; otherwise the load was issued during the previous chunk
         if (kSweepStates) load_state(c);
-        const unsigned char *op = smem + BwdLds::kOp + (item & 1) * BwdLds::kOpBytes;
-        const unsigned char *rt = op + BwdLds::kOpRt, *kt = op + BwdLds::kOpKt, *fr = op + BwdLds::kOpFr;
-        const float *gg = reinterpret_cast<const float *>(op + BwdLds::kOpG);
-        const unsigned char *vt = smem + BwdLds::kRawVG + (item % 3) * 2 * kTileBytes, *gyt = vt + kTileBytes;
-        const unsigned char *wt = smem + BwdLds::kRawW + (item % 3) * kTileBytes;
+        // Uniform block offsets of this item.  They pass through fresh_s() before every tile, which
+        // keeps the compiler from forming (block + lane offset) for all tiles at once and holding
+        // two dozen address registers across the chunk.
+        int op_off = BwdLds::kOp + (item & 1) * BwdLds::kOpBytes;
+        int vg_off = BwdLds::kRawVG + (item % 3) * 2 * kTileBytes;
+        int w_off = BwdLds::kRawW + (item % 3) * kTileBytes;
+        const unsigned char *rt, *kt, *fr, *vt, *gyt, *wt;
+        const float *gg;
+        auto fresh_pointers = [&]() {
+            op_off = fresh_s(op_off); vg_off = fresh_s(vg_off); w_off = fresh_s(w_off);
+            rt = smem + op_off + BwdLds::kOpRt; kt = smem + op_off + BwdLds::kOpKt; fr = smem + op_off + BwdLds::kOpFr;
+            gg = reinterpret_cast<const float *>(smem + op_off + BwdLds::kOpG);
+            vt = smem + vg_off; gyt = vt + kTileBytes; wt = smem + w_off;
+        };
+        fresh_pointers();
         const int t0 = c * CL;
-        int ptop = 3;
-        while (ptop > 0 && t0 + 16 * ptop >= T) --ptop;
         // states at the tile starts this group works on, as packed bf16 operands
         bf16x8 SopL[4], SopH[4];
-        if (mine(0)) { SopL[0] = acc_as_operand(S[0], S[1]); SopH[0] = acc_as_operand(S[2], S[3]); }
+        f32x4 S[4];
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+            S[m] = (f32x4){__uint_as_float(Sraw[m].x << 16), __uint_as_float(Sraw[m].x & 0xffff0000u),
+                           __uint_as_float(Sraw[m].y << 16), __uint_as_float(Sraw[m].y & 0xffff0000u)};
+        if (mine(0)) {
+            SopL[0] = make_bf16x8(Sraw[0].x, Sraw[0].y, Sraw[1].x, Sraw[1].y);
+            SopH[0] = make_bf16x8(Sraw[2].x, Sraw[2].y, Sraw[3].x, Sraw[3].y);
+        }
 #pragma unroll
         for (int p = 0; p < 3; ++p) {
             if (NG == 2 && GRP == 1 && p == 2) continue;   // group 1 needs the states of tiles 0 and 2 only
-            if (p + 1 > ptop) continue;                    // uniform: no tile starts there
             const s16x4 kq = tile_frag_tok(kt, 16 * q, 16 * p, l16, g);
             const float gq = gg[p * kN + col];
 #pragma unroll
@@ -157,10 +188,13 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
             for (int m = 0; m < 4; ++m) { S[m][0] *= gq; S[m][1] *= gq; S[m][2] *= gq; S[m][3] *= gq; }
             if (mine(p + 1)) { SopL[p + 1] = acc_as_operand(S[0], S[1]); SopH[p + 1] = acc_as_operand(S[2], S[3]); }
         }
-        if (!kSweepStates && c > 0) load_state(c - 1);   // S is free again: fetch the next chunk's state under this chunk's work
+        // S is free again: fetch the next chunk's state under this chunk's work (chunk 0 fetches itself again, unused)
+        if (!kSweepStates) load_state(c > 0 ? c - 1 : 0);
+        WKV6_STAMP();
+        __builtin_amdgcn_sched_barrier(0);   // keep the scheduler from interleaving the tiles (register pressure)
 #pragma unroll
         for (int p = 3; p >= 0; --p) {
-            if (p > ptop) continue;   // uniform: tiles past the end of the sequence
+            fresh_pointers();
             const float gq = gg[p * kN + col];
             const s16x4 rtq = tile_frag_tok(rt, 16 * q, 16 * p, l16, g);
             if (!mine(p)) {
@@ -170,6 +204,8 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
 #pragma unroll
                 for (int m = 0; m < 4; ++m) Gj[m] = mfma16(tile_frag_tok(gyt, 16 * m, 16 * p, l16, g), rtq, Gj[m]);
                 settle(Gj[0], Gj[1], Gj[2], Gj[3]);
+                WKV6_STAMP();
+                __builtin_amdgcn_sched_barrier(0);
                 continue;
             }
             const bf16x8 sL = SopL[p], sH = SopH[p];
@@ -213,6 +249,8 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
 #pragma unroll
             for (int m = 0; m < 4; ++m) Gj[m] = mfma16(tile_frag_tok(gyt, 16 * m, 16 * p, l16, g), rtq, Gj[m]);
             settle(X, W, Gj);   // all read by VALU code from here on
+            WKV6_STAMP();
+            __builtin_amdgcn_sched_barrier(0);
             // tile-boundary term E[j] = sum_i S0[j][i] G_new[j][i]
             float E;
             {
@@ -270,7 +308,12 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
                     st16(gr_h, o, gro[rr]); st16(gk_h, o, gko[rr]); st16(gw_h, o, gwv);
                 }
             }
+            WKV6_STAMP();
+            __builtin_amdgcn_sched_barrier(0);
         }
+        // fake use of the prefetched state: the wait for its loads lands here, after this chunk's
+        // stores in program order and with their number known
+        if (!kSweepStates) asm volatile("" : "+v"(Sraw[0]), "+v"(Sraw[1]), "+v"(Sraw[2]), "+v"(Sraw[3]));
     }
     // gu: fold the four lane groups (different tokens, same channel), then the consumer groups
     gu_acc = sum_rows(gu_acc);
@@ -308,10 +351,8 @@ __device__ __forceinline__ void bwd_gv_chunk(GvState &st, const BwdArgs &a, cons
     const float *ruk = reinterpret_cast<const float *>(op + BwdLds::kOpRuk);
     const unsigned char *gyt = smem + BwdLds::kRawVG + (item % 3) * 2 * kTileBytes + kTileBytes;
     const int t0 = c * CL;
-    int ptop = 3;
-    while (ptop > 0 && t0 + 16 * ptop >= T) --ptop;
 #pragma unroll 1
-    for (int pp = ptop; pp >= 0; --pp) {
+    for (int pp = 3; pp >= 0; --pp) {
         const int row = 16 * pp + l16, tk = 16 * pp + 4 * g;
         const bf16x8 rf0 = tile_frag_ch(rt, row, 0, g), rf1 = tile_frag_ch(rt, row, 1, g);
         const bf16x8 kf0 = tile_frag_ch(kt, row, 0, g), kf1 = tile_frag_ch(kt, row, 1, g);
@@ -389,11 +430,10 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     const int lrow = lane >> 3;
     const uint32_t lpiece = (uint32_t)(((lane & 7) ^ lrow) << 4);
     // Rows past the end of the sequence are fetched from row T-1 (valid memory); the preparation
-    // turns them into r = k = 0, w = -inf, and the v, gy rows only ever meet zero operands.  A tile
-    // entirely past the end is neither loaded, prepared nor consumed.  Returns the number of loads.
+    // turns them into r = k = 0, w = -inf (decay 1), and the v, gy rows only ever meet zero operands.
+    // Returns the number of loads.
     auto issue_loads = [&](int it) -> int {
         const int tb = item_chunk(it) * CL + 16 * p;
-        if (tb >= T) return 0;
         const bool full = item_full(it);
         const uint32_t rk = lds0 + BwdLds::kRawRK + (it & 1) * 2 * kTileBytes + 16 * p * kTileRow;
         const uint32_t ww = lds0 + BwdLds::kRawW + (it % 3) * kTileBytes + 16 * p * kTileRow;
@@ -421,7 +461,6 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     for (int s = 0; s < 8; ++s) choff[s] = (uint32_t)((((ch >> 3) ^ s) << 4) + ((ch & 7) << 1)) + (uint32_t)(16 * p * kTileRow);
     auto prepare = [&](int it) {
         const int tb = item_chunk(it) * CL + 16 * p;
-        if (tb >= T) return;
         const bool full = item_full(it);
         const unsigned char *rawrk = smem + BwdLds::kRawRK + (it & 1) * 2 * kTileBytes;
         const unsigned char *raww = smem + BwdLds::kRawW + (it % 3) * kTileBytes;
@@ -474,20 +513,27 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     // item `it` is loaded during iteration it-2 (or the prologue) and prepared during iteration it-1
     GvState gvst;
     if (kAlsoGv) gvst.init();
+    WKV6_STAMP_DECL;
     issue_loads(0);
     wait_younger(nitem > 1 ? issue_loads(1) : 0);
     prepare(0);
     for (int it = 0; it < nitem; ++it) {
+        WKV6_STAMP();
         __syncthreads();
+        WKV6_STAMP();
         // free again: the raw r, k block of item `it` (read by this wave's prepare before the barrier)
         // and the raw w, v, gy blocks of item it-1 (read by the other roles before the barrier)
         const int younger = it + 2 < nitem ? issue_loads(it + 2) : 0;
         if (it + 1 < nitem) {
+            WKV6_STAMP();
             wait_younger(younger);
+            WKV6_STAMP();
             prepare(it + 1);
+            WKV6_STAMP();
         }
         // the gv role, on the waves the operand preparation leaves partly idle
         if (kAlsoGv && item_full(it)) bwd_gv_chunk<kRagged>(gvst, a, smem, a.gv + base, rowbytes, item_chunk(it), it, p, lane);
+        WKV6_STAMP();
     }
     wait_loads<0>();
     __threadfence_block();
@@ -511,6 +557,9 @@ __global__ __launch_bounds__(BwdLayout<kLayout>::kWaves * 64) void chunk_bwd_ker
     static_assert(sizeof(ScanBwdALds) <= BwdLds::kBytes && sizeof(ScanBwdBLds) <= BwdLds::kBytes,
                   "the exact second pass reuses the LDS block");
     if (threadIdx.x == 0) s_wild = 0;
+#ifdef WKV6_TIMING
+    if (threadIdx.x == 0) a.dbg[16 * 256 + 2 * blockIdx.x] = __builtin_readcyclecounter();
+#endif
     __syncthreads();
 
     constexpr int NG = BwdLayout<kLayout>::kGroups;
@@ -532,6 +581,9 @@ __global__ __launch_bounds__(BwdLayout<kLayout>::kWaves * 64) void chunk_bwd_ker
         else if (role == 1) bwd_gv<kSweepStates, kRagged>(a, smem, b, h, q, lane);
         else bwd_consumer<kSweepStates, kRagged, NG, 0>(a, smem, &s_wild, b, h, q, lane);
     }
+#ifdef WKV6_TIMING
+    if (threadIdx.x == 0) a.dbg[16 * 256 + 2 * blockIdx.x + 1] = __builtin_readcyclecounter();
+#endif
     // exact second pass for this (b, h) if any of its tiles left the representable range; the
     // workgroup's own slice of the state workspace (nchunk x 64 x 64 floats = T' x 64) holds P
     if (s_wild) {
@@ -554,7 +606,6 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
                           const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
                           void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, bool states_ready)
 {
-    constexpr int kLayout = 1;
     const size_t lds = BwdLds::kBytes;
     BwdArgs a;
     a.T = (int)T; a.H = (int)H;
@@ -562,15 +613,27 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
     a.u = (const bf16_t *)u; a.gy = (const bf16_t *)gy;
     a.gr = (bf16_t *)gr; a.gk = (bf16_t *)gk; a.gv = (bf16_t *)gv; a.gw = (bf16_t *)gw; a.gu = (bf16_t *)gu;
     a.ckpt = (float *)workspace;
-    auto launch = [&](auto kern) -> hipError_t {
+    a.dbg = reinterpret_cast<long long *>((float *)workspace + (size_t)(B * H) * ((T + CL - 1) / CL) * kN * kN);
+    auto launch = [&](auto kern, int waves) -> hipError_t {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(BwdLayout<kLayout>::kWaves * 64), lds, st, a);
+        hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(waves * 64), lds, st, a);
         return hipGetLastError();
     };
-    const bool ragged = (T % 16) != 0;
-    if (states_ready) return ragged ? launch(chunk_bwd_kernel<false, true, kLayout>) : launch(chunk_bwd_kernel<false, false, kLayout>);
-    return ragged ? launch(chunk_bwd_kernel<true, true, kLayout>) : launch(chunk_bwd_kernel<true, false, kLayout>);
+    const bool ragged = (T % CL) != 0;   // the last chunk has tokens past the end
+    auto run = [&](auto layout_tag) -> hipError_t {
+        constexpr int kLayout = decltype(layout_tag)::value;
+        constexpr int nw = BwdLayout<kLayout>::kWaves;
+        if (states_ready) return ragged ? launch(chunk_bwd_kernel<false, true, kLayout>, nw) : launch(chunk_bwd_kernel<false, false, kLayout>, nw);
+        return ragged ? launch(chunk_bwd_kernel<true, true, kLayout>, nw) : launch(chunk_bwd_kernel<true, false, kLayout>, nw);
+    };
+#ifdef WKV6_DEV_LAYOUTS
+    const char *env = getenv("WKV6_BWD_LAYOUT");
+    const int layout = env ? atoi(env) : 1;
+    if (layout == 0) return run(std::integral_constant<int, 0>());
+    if (layout == 2) return run(std::integral_constant<int, 2>());
+#endif
+    return run(std::integral_constant<int, 1>());
 }
 
 }  // namespace wkv6

@@ -44,7 +44,7 @@ struct FwdLds {
     static constexpr int kBytes = kOp + 2 * kOpBytes;
 };
 
-// kSave: also write the state at every chunk start to `ckpt` (fp32, [b][h][chunk][j][i]) for the
+// kSave: also write the state at every chunk start to `ckpt` (bf16, [b][h][chunk][j][i]) for the
 // backward pass, which then skips its own forward sweep.
 template <typename Ts, bool kSave, bool kRagged>
 __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
@@ -83,11 +83,12 @@ __global__ __launch_bounds__(512) void chunk_fwd_kernel(int T, int H,
         bf16_t *y_h = y + base;
         for (int c = 0; c < nchunk; ++c) {
             if (kSave) {
-                float *dst = ckpt + ((int64_t)blockIdx.x * nchunk + c) * (kN * kN) + 16 * q + l16;
+                // bf16 [chunk][j][i], in the first half of this workgroup's slice of the workspace
+                bf16_t *dst = reinterpret_cast<bf16_t *>(ckpt + (int64_t)blockIdx.x * nchunk * (kN * kN)) + (int64_t)c * (kN * kN) + 16 * q + l16;
 #pragma unroll
                 for (int m = 0; m < 4; ++m)
 #pragma unroll
-                    for (int rr = 0; rr < 4; ++rr) dst[(16 * m + 4 * g + rr) * kN] = S[m][rr];
+                    for (int rr = 0; rr < 4; ++rr) store1(dst + (16 * m + 4 * g + rr) * kN, S[m][rr]);
             }
             __syncthreads();
             const unsigned char *op = smem + FwdLds::kOp + (c & 1) * FwdLds::kOpBytes;

@@ -187,10 +187,19 @@ __device__ __forceinline__ uint32_t tile_off(int t, int ch) {
 // row t0.  Completion is counted by vmcnt; the compiler does not know about these loads, so the
 // caller waits with wait_loads<N>() (N = number of younger loads allowed to stay in flight).
 __device__ __forceinline__ void load_rows8_to_lds(const void *gbase, uint32_t voff, uint32_t lds_addr) {
+    // (the uniform operands are pinned to scalar registers explicitly: an "s" constraint alone does
+    // not move a value the compiler happened to keep in vector registers)
+    const uint64_t gb = reinterpret_cast<uint64_t>(gbase);
+    const uint32_t ub_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)gb);          // (the builtin returns a
+    const uint32_t ub_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(gb >> 32));   //  signed int: no widening casts)
+    const uint64_t ub = ((uint64_t)ub_hi << 32) | (uint64_t)ub_lo;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(gbase) : "memory", "m0");
+                 :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(voff), "s"(ub) : "memory", "m0");
 }
 template <int N> __device__ __forceinline__ void wait_loads() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
+
+// a wave-uniform value the compiler has to treat as newly defined (it stays in a scalar register)
+__device__ __forceinline__ int fresh_s(int x) { asm volatile("" : "+s"(x)); return x; }
 
 __device__ __forceinline__ uint32_t lds_address(const void *p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const unsigned char *)p;
