@@ -40,6 +40,7 @@ namespace wkv6 {
 
 constexpr int CL = 64;   // tokens per chunk
 
+
 // LDS map of the backward kernel (byte offsets into the dynamic block); "item" = one chunk visit
 struct BwdLds {
     static constexpr int kRawRK = 0;                                   // [item & 1][r, k] raw tiles
@@ -199,11 +200,15 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
             const s16x4 rtq = tile_frag_tok(rt, 16 * q, 16 * p, l16, g);
             if (!mine(p)) {
                 // the other group does this tile; only carry the reverse state across it
+                f32x4 Upd[4];   // R~^T gY, off the chain through G
 #pragma unroll
-                for (int m = 0; m < 4; ++m) { Gj[m][0] *= gq; Gj[m][1] *= gq; Gj[m][2] *= gq; Gj[m][3] *= gq; }
+                for (int m = 0; m < 4; ++m) Upd[m] = mfma16(tile_frag_tok(gyt, 16 * m, 16 * p, l16, g), rtq, (f32x4){0.f, 0.f, 0.f, 0.f});
+                settle(Upd[0], Upd[1], Upd[2], Upd[3]);
 #pragma unroll
-                for (int m = 0; m < 4; ++m) Gj[m] = mfma16(tile_frag_tok(gyt, 16 * m, 16 * p, l16, g), rtq, Gj[m]);
-                settle(Gj[0], Gj[1], Gj[2], Gj[3]);
+                for (int m = 0; m < 4; ++m) {
+                    Gj[m][0] = fmaf(Gj[m][0], gq, Upd[m][0]); Gj[m][1] = fmaf(Gj[m][1], gq, Upd[m][1]);
+                    Gj[m][2] = fmaf(Gj[m][2], gq, Upd[m][2]); Gj[m][3] = fmaf(Gj[m][3], gq, Upd[m][3]);
+                }
                 WKV6_STAMP();
                 __builtin_amdgcn_sched_barrier(0);
                 continue;
