@@ -45,7 +45,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c5"])
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c4", "c5"])
     ap.add_argument("--algo", default="auto", choices=["auto", "scan", "chunk"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--plain-pair", action="store_true", help="time forward()+backward() without saved states")
@@ -136,6 +136,38 @@ def bench_stateful(a):
         "dtype": "bf16", "data": "synthetic"}))
 
 
+def bench_model_step(a):
+    """Config 4: one full RWKV-6 training step (24 layers, d_model 2048, 32 heads of 64, FFN 7168,
+    vocab 65536, random init, bf16 autocast, 8 x 1024 uniform random token ids, next-token cross
+    entropy, forward + backward + AdamW) through the torch binding of the operator.  Prints its own
+    JSON line: whole-step tokens/s and the share of the step spent inside the operator."""
+    import torch
+    import rwkv6_harness as hz
+    from rwkv_kernel import RWKVKernelOperator
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(a.seed)
+    B, T = 8, 1024
+    model = hz.RWKV6(RWKVKernelOperator(64, T), **hz.CONFIG4).to(dev)
+    opt = torch.optim.AdamW(model.parameters(), lr=1e-4, fused=True)
+    ids = torch.randint(0, hz.CONFIG4["vocabulary_size"], (B, T + 1), device=dev)
+    steps, warm = min(a.steps, 10), min(a.warmup, 3)
+    losses = [float(hz.train_step(model, opt, ids, torch.bfloat16)) for _ in range(warm)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss = hz.train_step(model, opt, ids, torch.bfloat16)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    losses.append(float(loss))
+    print(json.dumps({
+        "metric": "RWKV-6 1.6B-shaped training step through the torch binding, tokens/s", "n_gpus": 1,
+        "value": B * T / (ms * 1e-3), "unit": "tokens/s", "ms_per_step": ms, "steps": steps, "warmup": warm,
+        "config": {"workload": "c4: 24 layers d=2048 H=32 N=64 FFN=7168 vocab=65536, B=8 T=1024, bf16 autocast, AdamW"},
+        "parameters": sum(p.numel() for p in model.parameters()),
+        "loss_first_last": [losses[0], losses[-1]], "dtype": "bf16", "data": "synthetic"}))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -150,6 +182,9 @@ def main():
     if a.workload == "c5":
         torch.cuda.set_device(0)
         return bench_stateful(a)
+    if a.workload == "c4":
+        torch.cuda.set_device(0)
+        return bench_model_step(a)
     lib = _native.load()
     B, T, H, dt_name = WORKLOADS[a.workload]
     N = 64
