@@ -86,7 +86,7 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
     const int nchunk = (T + CL - 1) / CL;
     // chunk states: bf16 [chunk][j][i] in the first half of this workgroup's workspace slice
-    bf16_t *ck = reinterpret_cast<bf16_t *>(a.ckpt + (int64_t)blockIdx.x * nchunk * (kN * kN));
+    bf16_t *ck = reinterpret_cast<bf16_t *>(a.ckpt + (int64_t)(b * H + h) * nchunk * (kN * kN));
     auto mine = [](int p) { return NG == 1 || (p & 1) == (GRP ^ 1); };   // group 0: tiles 3, 1; group 1: tiles 2, 0
     int item = 0;
     WKV6_STAMP_DECL;
@@ -298,19 +298,27 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
             }
             // exclusive prefix of D over the 16 tokens: 4 in this lane, the rest in the lane groups below
             float pre = E + prefix_rows(D[0] + D[1] + D[2] + D[3], g);
+            float gwo[4];
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                // exp(w) <= kWildLimit here (anything larger sends this (b, h) to the exact second pass)
+                const float ew = fast_exp(w_[rr]);
+                gwo[rr] = -ew * (pre - P[rr]);
+                pre += D[rr];
+            }
+            // the gradient of the first and the last decay is zero by definition (the flow balance
+            // leaves rounding residue there); only the two tiles holding them pay for the test
+            if ((c == 0 && p == 0) || (c == nchunk - 1 && p == (((T - 1) >> 4) & 3))) {
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr)
+                    if (t0 + tk + rr == 0 || t0 + tk + rr == T - 1) gwo[rr] = 0.f;
+            }
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) {
                 const int t = t0 + tk + rr;
-                // exp(w) <= kWildLimit here (anything larger sends this (b, h) to the exact second pass)
-                const float ew = fast_exp(w_[rr]);
-                float gwv = -ew * (pre - P[rr]);
-                pre += D[rr];
-                // the gradient of the first and the last decay is zero by definition (the flow
-                // balance leaves rounding residue there)
-                if (t == 0 || t == T - 1) gwv = 0.f;
                 if (!kRagged || t < T) {
                     const uint32_t o = (uint32_t)t * rowbytes + 2u * (uint32_t)col;
-                    st16(gr_h, o, gro[rr]); st16(gk_h, o, gko[rr]); st16(gw_h, o, gwv);
+                    st16(gr_h, o, gro[rr]); st16(gk_h, o, gko[rr]); st16(gw_h, o, gwo[rr]);
                 }
             }
             WKV6_STAMP();
@@ -593,7 +601,7 @@ __global__ __launch_bounds__(BwdLayout<kLayout>::kWaves * 64) void chunk_bwd_ker
     // workgroup's own slice of the state workspace (nchunk x 64 x 64 floats = T' x 64) holds P
     if (s_wild) {
         const int nchunk = (a.T + CL - 1) / CL;
-        float *ck = a.ckpt + (int64_t)blockIdx.x * nchunk * (kN * kN);
+        float *ck = a.ckpt + (int64_t)(b * a.H + h) * nchunk * (kN * kN);
         __syncthreads();
         scan_bwd_a_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdALds *>(smem), b, h, a.T, a.H, a.r, a.k, a.v, a.w, a.u, a.gy, a.gr, a.gu, ck, kN);
         __threadfence_block();

@@ -107,7 +107,7 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
         WKV6_FSTAMP();
         if (kSave && GRP == 0) {
             // bf16 [chunk][j][i], in the first half of this workgroup's slice of the workspace
-            bf16_t *dst = reinterpret_cast<bf16_t *>(a.ckpt + (int64_t)blockIdx.x * nchunk * (kN * kN)) + (int64_t)c * (kN * kN) + 16 * q + l16;
+            bf16_t *dst = reinterpret_cast<bf16_t *>(a.ckpt + (int64_t)(b * H + h) * nchunk * (kN * kN)) + (int64_t)c * (kN * kN) + 16 * q + l16;
 #pragma unroll
             for (int m = 0; m < 4; ++m)
 #pragma unroll
