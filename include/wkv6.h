@@ -110,7 +110,7 @@ int wkv6_backward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, in
 size_t wkv6_backward_workspace_bytes_ex(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H);
 
 /* Training pair: a forward that also saves what the backward can reuse (with the chunked kernels:
- * the fp32 state at every 64-token chunk start), and the backward that consumes it and therefore
+ * the state at every 64-token chunk start, as bf16), and the backward that consumes it and therefore
  * skips its own forward state sweep.  `saved` is caller-owned device memory of wkv6_saved_bytes()
  * bytes (0 = this path saves nothing; pass NULL), must be left untouched between the two calls,
  * and serves the backward as its workspace too.  No counterpart in the reference, whose backward
