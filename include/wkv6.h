@@ -125,6 +125,18 @@ int wkv6_backward_saved(void *stream, int dtype, int algo, int64_t B, int64_t T,
                         void *gr, void *gk, void *gv, void *gw, void *gu,
                         void *saved, size_t saved_bytes);
 
+/* wkv6_backward_saved with the batch sum of gu fused in: gu (B,C) still receives the per-batch
+ * partials, gu_sum (C elements, output type) their sum over the batch, added up in fp32 from the
+ * stored partials -- the value `gu = torch.sum(gu, 0)` gives the caller in
+ * rwkv_kernel/torch_rwkv_kernel.py:73 (rwkv_kernel/jax_rwkv_kernel.py:166), without the extra
+ * kernel.  `saved` must come from wkv6_forward_save of the same shape (it carries per-head arrival
+ * counters, which the call leaves ready for another backward on the same buffer). */
+int wkv6_backward_saved_sum(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                            const void *r, const void *k, const void *v, const void *w, const void *u,
+                            const void *gy,
+                            void *gr, void *gk, void *gv, void *gw, void *gu, void *gu_sum,
+                            void *saved, size_t saved_bytes);
+
 /* ---- XLA custom-call surface (replaces the pybind module `gpu_ops`,
  * rwkv_kernel/jax_kernel/gpu_ops.cpp:20-43) ---------------------------------------------- */
 

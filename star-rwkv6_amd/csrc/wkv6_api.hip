@@ -94,7 +94,9 @@ size_t wkv6_saved_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, in
     const bool chunk = (algo == WKV6_ALGO_CHUNK && chunk_possible(dtype, T, C)) ||
                        (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
     // sized so that the guarded per-timestep pass of the backward can use the same buffer
-    return chunk ? wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H) : 0;
+    if (!chunk) return 0;
+    const size_t ws = wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H), sv = wkv6::chunk_saved_bytes(B, T, H);
+    return ws > sv ? ws : sv;
 }
 
 int wkv6_forward_save(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
@@ -146,7 +148,7 @@ size_t wkv6_backward_workspace_bytes(int dtype, int64_t B, int64_t T, int64_t C,
 static int backward_impl(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, size_t workspace_bytes,
-                         bool states_ready) {
+                         bool states_ready, void *gu_sum = nullptr) {
     int rc = check_shape(dtype, B, T, C, H);
     if (rc != WKV6_OK) return rc;
     if (!r || !k || !v || !w || !u || !gy || !gr || !gk || !gv || !gw || !gu) return WKV6_ERR_ARG;
@@ -159,9 +161,13 @@ static int backward_impl(void *stream, int dtype, int algo, int64_t B, int64_t T
     if (algo == WKV6_ALGO_CHUNK && !chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;
     const bool chunk = algo == WKV6_ALGO_CHUNK ||
                        (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
-    if (!chunk)
-        return finish(wkv6::scan_backward(st, dtype, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace));
-    return finish(wkv6::chunk_backward(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace, states_ready));
+    if (!chunk) {
+        rc = finish(wkv6::scan_backward(st, dtype, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace));
+        if (rc == WKV6_OK && gu_sum) rc = finish(wkv6::sum_over_batch(st, out_type(dtype), B, C, gu, gu_sum));
+        return rc;
+    }
+    return finish(wkv6::chunk_backward(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace, states_ready,
+                                       states_ready ? gu_sum : nullptr));
 }
 
 int wkv6_backward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
@@ -178,6 +184,17 @@ int wkv6_backward_saved(void *stream, int dtype, int algo, int64_t B, int64_t T,
     // results (and with them the saved states) are discarded anyway
     return backward_impl(stream, dtype, algo, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, saved, saved_bytes,
                          wkv6_saved_bytes(dtype, algo, B, T, C, H) > 0);
+}
+
+int wkv6_backward_saved_sum(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                            const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                            void *gr, void *gk, void *gv, void *gw, void *gu, void *gu_sum,
+                            void *saved, size_t saved_bytes) {
+    if (!gu_sum) return WKV6_ERR_ARG;
+    const size_t need = wkv6_saved_bytes(dtype, algo, B, T, C, H);
+    if (need > 0 && saved_bytes < need) return WKV6_ERR_WORKSPACE;
+    return backward_impl(stream, dtype, algo, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, saved, saved_bytes,
+                         need > 0, gu_sum);
 }
 
 int wkv6_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,

@@ -70,6 +70,9 @@ struct BwdArgs {
     int T, H;
     const bf16_t *r, *k, *v, *w, *u, *gy;
     bf16_t *gr, *gk, *gv, *gw, *gu;
+    bf16_t *gu_sum;   // null, or C elements: receives the sum of gu over the batch
+    int *arrivals;    // per head: workgroups that have delivered their gu partial (zero on entry)
+    int B;
     float *ckpt;
 };
 
@@ -608,16 +611,64 @@ __global__ __launch_bounds__(BwdLayout<kLayout>::kWaves * 64) void chunk_bwd_ker
         __syncthreads();
         scan_bwd_b_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdBLds *>(smem), b, h, a.T, a.H, a.r, a.k, a.v, a.w, a.u, a.gy, ck, kN, a.gk, a.gv, a.gw);
     }
+    // Fused batch sum of gu (what the caller otherwise does with one more kernel): the workgroup that
+    // is the last of its head to deliver adds up the B partials.  The partials travel as written-
+    // through (agent scope) stores into the unused second half of each workgroup's workspace slice,
+    // completed before the arrival counter is bumped; no fence, which would write back the whole L2.
+    if (a.gu_sum != nullptr) {
+        __shared__ int s_last;
+        const int nchunk = (a.T + CL - 1) / CL;
+        const int64_t slice = (int64_t)nchunk * (kN * kN), C = (int64_t)a.H * kN;
+        __threadfence_block();   // this workgroup's partial (consumer group 0 or the second pass) is written
+        __syncthreads();
+        const int tid = threadIdx.x;
+        if (tid < kN) {          // wave 0
+            const float part = load1(a.gu + (int64_t)b * C + h * kN + tid);
+            __hip_atomic_store(a.ckpt + (int64_t)(b * a.H + h) * slice + slice / 2 + tid, part, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            if (tid == 0)
+                s_last = __hip_atomic_fetch_add(a.arrivals + h, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.B - 1;
+        }
+        __syncthreads();
+        if (s_last && tid < kN) {
+            float acc = 0.f;
+            for (int bb = 0; bb < a.B; ++bb)
+                acc += __hip_atomic_load(a.ckpt + (int64_t)(bb * a.H + h) * slice + slice / 2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            store1(a.gu_sum + h * kN + tid, acc);
+            if (tid == 0) __hip_atomic_store(a.arrivals + h, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // armed again
+        }
+    }
 }
 
 size_t chunk_backward_workspace_bytes(int64_t B, int64_t T, int64_t H) {
     const int64_t nchunk = (T + CL - 1) / CL;
     return (size_t)(B * H * nchunk) * kN * kN * sizeof(float);
 }
+size_t chunk_saved_bytes(int64_t B, int64_t T, int64_t H) {
+    return chunk_backward_workspace_bytes(B, T, H) + (((size_t)H * sizeof(int) + 255) & ~(size_t)255);
+}
+
+template <typename T>
+__global__ void sum_over_batch_kernel(int B, int C, const T *__restrict__ p, T *__restrict__ out) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    float acc = 0.f;
+    for (int b = 0; b < B; ++b) acc += load1(p + (int64_t)b * C + c);
+    store1(out + c, acc);
+}
+hipError_t sum_over_batch(hipStream_t st, int out_dtype, int64_t B, int64_t C, const void *partials, void *sum) {
+    const dim3 grid((unsigned)((C + 255) / 256)), block(256);
+    if (out_dtype == kBF16)
+        hipLaunchKernelGGL(sum_over_batch_kernel<bf16_t>, grid, block, 0, st, (int)B, (int)C, (const bf16_t *)partials, (bf16_t *)sum);
+    else
+        hipLaunchKernelGGL(sum_over_batch_kernel<float>, grid, block, 0, st, (int)B, (int)C, (const float *)partials, (float *)sum);
+    return hipGetLastError();
+}
 
 hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
                           const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
-                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, bool states_ready)
+                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, bool states_ready,
+                          void *gu_sum)
 {
     const size_t lds = BwdLds::kBytes;
     BwdArgs a;
@@ -626,6 +677,9 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
     a.u = (const bf16_t *)u; a.gy = (const bf16_t *)gy;
     a.gr = (bf16_t *)gr; a.gk = (bf16_t *)gk; a.gv = (bf16_t *)gv; a.gw = (bf16_t *)gw; a.gu = (bf16_t *)gu;
     a.ckpt = (float *)workspace;
+    a.B = (int)B;
+    a.gu_sum = states_ready ? (bf16_t *)gu_sum : nullptr;
+    a.arrivals = reinterpret_cast<int *>(reinterpret_cast<char *>(workspace) + chunk_backward_workspace_bytes(B, T, H));
     a.dbg = reinterpret_cast<long long *>((float *)workspace + (size_t)(B * H) * ((T + CL - 1) / CL) * kN * kN);
     auto launch = [&](auto kern, int waves) -> hipError_t {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

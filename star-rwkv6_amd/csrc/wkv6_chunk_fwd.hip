@@ -74,6 +74,7 @@ struct FwdArgs {
     bf16_t *y;
     void *sT;
     float *ckpt;
+    int *arrivals;   // with ckpt: per-head counters the backward's fused gu sum starts from zero
 };
 
 // ------------------------------------------------------------------------------------------
@@ -343,6 +344,7 @@ __global__ __launch_bounds__(kFwdThreads) void chunk_fwd_kernel(FwdArgs a)
     // exact second pass for this (b, h) if any of its tiles left the representable range
     __threadfence_block();   // workgroup scope is enough (and a device-scope fence would write back the L2)
     __syncthreads();
+    if (kSave && b == 0 && threadIdx.x == 0) a.arrivals[h] = 0;
     if (s_wild)
         scan_fwd_body<bf16_t, bf16_t, Ts>(*reinterpret_cast<ScanFwdLds *>(smem), b, h, a.T, a.H, a.r, a.k, a.v, a.w, a.u,
                                           reinterpret_cast<const Ts *>(a.s0), a.map, a.y, reinterpret_cast<Ts *>(a.sT));
@@ -357,6 +359,7 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
     a.T = (int)T; a.H = (int)H;
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
     a.s0 = s0; a.map = map; a.y = (bf16_t *)y; a.sT = sT; a.ckpt = (float *)saved_states;
+    a.arrivals = saved_states ? reinterpret_cast<int *>(reinterpret_cast<char *>(saved_states) + chunk_backward_workspace_bytes(B, T, H)) : nullptr;
     a.dbg = saved_states ? reinterpret_cast<long long *>((float *)saved_states + (size_t)(B * H) * ((T + CL - 1) / CL) * kN * kN) : nullptr;
     auto launch = [&](auto kern, auto *) -> hipError_t {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);

@@ -23,9 +23,17 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
                          const void *s0, const int64_t *map, void *y, void *sT, void *saved_states);
 
 size_t chunk_backward_workspace_bytes(int64_t B, int64_t T, int64_t H);
-// states_ready: the workspace already holds the chunk-start states (written by a forward pass)
+// bytes of a forward -> backward hand-over buffer: the workspace plus one arrival counter per head
+// (zeroed by the saving forward, used by the backward's fused batch sum of gu)
+size_t chunk_saved_bytes(int64_t B, int64_t T, int64_t H);
+// states_ready: the workspace already holds the chunk-start states (written by a forward pass).
+// gu_sum (may be null; needs states_ready and a buffer of chunk_saved_bytes): also write sum_b gu[b].
 hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
                           const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
-                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, bool states_ready);
+                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, bool states_ready,
+                          void *gu_sum);
+
+// sum over the batch of (B, C) partials -> (C), both in the output type (for the paths without a fused sum)
+hipError_t sum_over_batch(hipStream_t st, int out_dtype, int64_t B, int64_t C, const void *partials, void *sum);
 
 }  // namespace wkv6

@@ -31,6 +31,7 @@ SIGNATURES = {
     "wkv6_saved_bytes": (_sz, [_int, _int] + [_i64] * 4),
     "wkv6_forward_save": (_int, [_p, _int, _int] + [_i64] * 4 + [_p] * 6 + [_p, _sz]),
     "wkv6_backward_saved": (_int, [_p, _int, _int] + [_i64] * 4 + [_p] * 11 + [_p, _sz]),
+    "wkv6_backward_saved_sum": (_int, [_p, _int, _int] + [_i64] * 4 + [_p] * 12 + [_p, _sz]),
     "wkv6_create_descriptor": (_sz, [_int] * 7 + [_p]),
     "wkv_forward": (None, [_p, ctypes.POINTER(_p), ctypes.c_char_p, _sz]),
     "wkv_backward": (None, [_p, ctypes.POINTER(_p), ctypes.c_char_p, _sz]),

@@ -82,9 +82,12 @@ class _WKV6(torch.autograd.Function):
             with torch.cuda.device(gy.device):
                 saved = ctx.saved_states
                 if saved is not None:
+                    # the batch sum of gu (rwkv_kernel/torch_rwkv_kernel.py:73) comes out of the same launch
                     ctx.saved_states = None
-                    _native.check(lib.wkv6_backward_saved(_stream(), code, ctx.algo, B, T, C, H, *args,
-                                                          _ptr(saved), saved.numel()))
+                    gu_sum = torch.empty(C, device=gy.device, dtype=odt)
+                    _native.check(lib.wkv6_backward_saved_sum(_stream(), code, ctx.algo, B, T, C, H, *args, _ptr(gu_sum),
+                                                              _ptr(saved), saved.numel()))
+                    return (None, None, None, None, gr, gk, gv, gw, gu_sum.reshape(u.shape), None)
                 else:
                     ws_bytes = lib.wkv6_backward_workspace_bytes_ex(code, ctx.algo, B, T, C, H)
                     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=gy.device) if ws_bytes else None

@@ -308,7 +308,7 @@ def test_plain_backward_equals_saved_backward(op, oracle):
         y = torch.empty_like(r)
         outs = [torch.empty_like(r) for _ in range(4)] + [torch.empty(B, C, dtype=r.dtype, device="cuda")]
         n = lib.wkv6_saved_bytes(_native.BF16, CHUNK, B, T, C, H)
-        assert n == lib.wkv6_backward_workspace_bytes_ex(_native.BF16, CHUNK, B, T, C, H) > 0
+        assert n >= lib.wkv6_backward_workspace_bytes_ex(_native.BF16, CHUNK, B, T, C, H) > 0   # + arrival counters
         buf = torch.empty(n, dtype=torch.uint8, device="cuda")
         if mode == "plain":
             _native.check(lib.wkv6_forward_ex(st, _native.BF16, CHUNK, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(y), None, 0))
@@ -330,3 +330,42 @@ def test_plain_backward_equals_saved_backward(op, oracle):
     for a, b in zip(res[0][1:5], res[1][1:5]):
         assert (a.float() - b.float()).abs().max() <= 5e-3 * b.float().abs().max()
     assert lib.wkv6_saved_bytes(_native.F32, SCAN, B, T, C, H) == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,T,H,dt", [(8, 256, 8, "bf16"), (5, 100, 3, "bf16"), (1, 64, 2, "bf16"), (3, 40, 2, "f32")])
+def test_fused_gu_batch_sum(op, oracle, B, T, H, dt):
+    """wkv6_backward_saved_sum: gu_sum is the sum over the batch of the partials it also returns
+    (summed in fp32, rounded once: what torch.sum does for the caller, rwkv_kernel/torch_rwkv_kernel.py:73),
+    on two consecutive backward calls over the same hand-over buffer, and for head counts that do
+    and do not divide over the XCDs evenly."""
+    from rwkv_kernel import _native
+    lib = _native.load()
+    N, C = 64, H * 64
+    dtype = {"bf16": torch.bfloat16, "f32": torch.float32}[dt]
+    code = {"bf16": _native.BF16, "f32": _native.F32}[dt]
+    r, k, v, w, u, gy = (x.to(dtype).cuda().contiguous() for x in oracle.make_inputs(B, T, H, N, 11))
+    y = torch.empty_like(r)
+    gr, gk, gv, gw = (torch.empty_like(r) for _ in range(4))
+    # (for the per-timestep path nothing is saved and the same buffer is just the backward's workspace)
+    n = max(lib.wkv6_saved_bytes(code, _native.ALGO_AUTO, B, T, C, H),
+            lib.wkv6_backward_workspace_bytes_ex(code, _native.ALGO_AUTO, B, T, C, H), 16)
+    saved = torch.empty(n, dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    P = lambda t: t.data_ptr()
+    _native.check(lib.wkv6_forward_save(st, code, _native.ALGO_AUTO, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(y), P(saved), n))
+    for _ in range(2):
+        gu = torch.full((B, C), float("nan"), dtype=dtype, device="cuda")
+        gs = torch.full((C,), float("nan"), dtype=dtype, device="cuda")
+        _native.check(lib.wkv6_backward_saved_sum(st, code, _native.ALGO_AUTO, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy),
+                                                  P(gr), P(gk), P(gv), P(gw), P(gu), P(gs), P(saved), n))
+        torch.cuda.synchronize()
+        want = torch.sum(gu.float(), 0).to(dtype)
+        assert torch.isfinite(gs).all()
+        assert torch.equal(gs, want) or float((gs.float() - want.float()).abs().max()) <= 2 ** -7 * float(want.float().abs().max())
+    # and the partials are the ones the plain call gives
+    gu2 = torch.empty_like(gu)
+    _native.check(lib.wkv6_backward_saved(st, code, _native.ALGO_AUTO, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy),
+                                          P(gr), P(gk), P(gv), P(gw), P(gu2), P(saved), n))
+    torch.cuda.synchronize()
+    assert torch.equal(gu, gu2)
