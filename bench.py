@@ -284,7 +284,7 @@ def main():
         "dtype": dt_name, "data": "synthetic",
         "config": {"workload": "%s: WKV6 fwd+bwd B=%d T=%d C=%d H=%d N=%d %s I/O fp32 state" % (
             a.workload, B, T, C, H, N, dt_name), "algo": algo_used, "tokens_per_step": tokens,
-            "calls": "forward+backward" if (a.plain_pair or not nsave) else "forward_save+backward_saved"},
+            "calls": "forward+backward" if (a.plain_pair or not nsave) else "forward_save+backward_saved_sum"},
         "roofline": {
             "bound": "hbm", "kernel": "wkv6_%s (%s)" % ("backward" if dom == "bwd" else "forward", algo_used),
             "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
