@@ -369,3 +369,49 @@ def test_fused_gu_batch_sum(op, oracle, B, T, H, dt):
                                           P(gr), P(gk), P(gv), P(gw), P(gu2), P(saved), n))
     torch.cuda.synchronize()
     assert torch.equal(gu, gu2)
+
+
+@pytest.mark.gpu
+def test_training_pair_replays_in_a_hip_graph(op, oracle):
+    """forward_save + backward_saved_sum captured once into a graph (the library allocates nothing
+    and only enqueues on the given stream), replayed several times with eager work and
+    synchronisations in between; every replay must reproduce the eager results bit for bit."""
+    from rwkv_kernel import _native
+    lib = _native.load()
+    B, T, H, N = 2, 256, 4, 64
+    C = H * N
+    r, k, v, w, u, gy = (x.to(torch.bfloat16).cuda().contiguous() for x in oracle.make_inputs(B, T, H, N, 21))
+    n = lib.wkv6_saved_bytes(_native.BF16, _native.ALGO_AUTO, B, T, C, H)
+    saved = torch.empty(n, dtype=torch.uint8, device="cuda")
+    outs = {name: torch.empty_like(r) for name in ("y", "gr", "gk", "gv", "gw")}
+    outs["gu"] = torch.empty(B, C, dtype=r.dtype, device="cuda")
+    outs["gs"] = torch.empty(C, dtype=r.dtype, device="cuda")
+    P = lambda t: t.data_ptr()
+
+    def step():
+        st = torch.cuda.current_stream().cuda_stream
+        _native.check(lib.wkv6_forward_save(st, _native.BF16, _native.ALGO_AUTO, B, T, C, H,
+                                            P(r), P(k), P(v), P(w), P(u), P(outs["y"]), P(saved), n))
+        _native.check(lib.wkv6_backward_saved_sum(st, _native.BF16, _native.ALGO_AUTO, B, T, C, H,
+                                                  P(r), P(k), P(v), P(w), P(u), P(gy), P(outs["gr"]), P(outs["gk"]),
+                                                  P(outs["gv"]), P(outs["gw"]), P(outs["gu"]), P(outs["gs"]), P(saved), n))
+
+    step()
+    torch.cuda.synchronize()
+    eager = {name: t.clone() for name, t in outs.items()}
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                      # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(3):
+        for t in outs.values():
+            t.fill_(float("nan"))   # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, t in outs.items():
+            assert torch.equal(t, eager[name]), (rep, name)
