@@ -93,6 +93,12 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     auto mine = [](int p) { return NG == 1 || (p & 1) == (GRP ^ 1); };   // group 0: tiles 3, 1; group 1: tiles 2, 0
     int item = 0;
     WKV6_STAMP_DECL;
+#ifdef WKV6_PRIO_A
+    if (GRP == 0) __builtin_amdgcn_s_setprio(WKV6_PRIO_A);
+#endif
+#ifdef WKV6_PRIO_B
+    if (GRP == 1) __builtin_amdgcn_s_setprio(WKV6_PRIO_B);
+#endif
     if (kSweepStates) {
         // phase 1: S^T (rows i, column j = col), checkpoint at every chunk start; group 0 only
         f32x4 S[4];
@@ -317,11 +323,16 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
                     if (t0 + tk + rr == 0 || t0 + tk + rr == T - 1) gwo[rr] = 0.f;
             }
 #pragma unroll
-            for (int rr = 0; rr < 4; ++rr) {
+            for (int rr = 0; rr < 4; rr += 2) {   // two tokens share one conversion per tensor
+                const uint32_t pr2 = pack_bf16x2(gro[rr], gro[rr + 1]), pk2 = pack_bf16x2(gko[rr], gko[rr + 1]);
+                const uint32_t pw2 = pack_bf16x2(gwo[rr], gwo[rr + 1]);
                 const int t = t0 + tk + rr;
+                const uint32_t o = (uint32_t)t * rowbytes + 2u * (uint32_t)col;
                 if (!kRagged || t < T) {
-                    const uint32_t o = (uint32_t)t * rowbytes + 2u * (uint32_t)col;
-                    st16(gr_h, o, gro[rr]); st16(gk_h, o, gko[rr]); st16(gw_h, o, gwo[rr]);
+                    st16_lo(gr_h, o, pr2); st16_lo(gk_h, o, pk2); st16_lo(gw_h, o, pw2);
+                }
+                if (!kRagged || t + 1 < T) {
+                    st16_hi(gr_h, o + rowbytes, pr2); st16_hi(gk_h, o + rowbytes, pk2); st16_hi(gw_h, o + rowbytes, pw2);
                 }
             }
             WKV6_STAMP();
@@ -475,19 +486,26 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     uint32_t choff[8];
 #pragma unroll
     for (int s = 0; s < 8; ++s) choff[s] = (uint32_t)((((ch >> 3) ^ s) << 4) + ((ch & 7) << 1)) + (uint32_t)(16 * p * kTileRow);
+    const float kLog2Log2e = 0.5287663729448977f;   // log2(log2(e)): exp(w) log2(e) = 2^(w log2(e) + this)
     auto prepare = [&](int it) {
         const int tb = item_chunk(it) * CL + 16 * p;
         const bool full = item_full(it);
-        const unsigned char *rawrk = smem + BwdLds::kRawRK + (it & 1) * 2 * kTileBytes;
-        const unsigned char *raww = smem + BwdLds::kRawW + (it % 3) * kTileBytes;
-        unsigned char *op = smem + BwdLds::kOp + (it & 1) * BwdLds::kOpBytes;
+        // lane addresses of the 8 swizzle phases in the three blocks this item uses (the row and tensor
+        // offsets on top of them are instruction immediates)
+        const unsigned char *a_rk[8], *a_w[8];
+        unsigned char *a_op[8];
+#pragma unroll
+        for (int sw = 0; sw < 8; ++sw) {
+            a_rk[sw] = smem + (BwdLds::kRawRK + (it & 1) * 2 * kTileBytes + choff[sw]);
+            a_w[sw] = smem + (BwdLds::kRawW + (it % 3) * kTileBytes + choff[sw]);
+            a_op[sw] = smem + (BwdLds::kOp + (it & 1) * BwdLds::kOpBytes + choff[sw]);
+        }
         float fr[16], fk[16], fw[16];
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            const uint32_t o = choff[e & 7] + e * kTileRow;
-            uint32_t ra = *reinterpret_cast<const uint16_t *>(rawrk + o);
-            uint32_t rk = *reinterpret_cast<const uint16_t *>(rawrk + kTileBytes + o);
-            uint32_t rw = *reinterpret_cast<const uint16_t *>(raww + o);
+            uint32_t ra = *reinterpret_cast<const uint16_t *>(a_rk[e & 7] + e * kTileRow);
+            uint32_t rk = *reinterpret_cast<const uint16_t *>(a_rk[e & 7] + kTileBytes + e * kTileRow);
+            uint32_t rw = *reinterpret_cast<const uint16_t *>(a_w[e & 7] + e * kTileRow);
             if (!full) ra = 0u;   // r is not loaded for the phase 1 items
             if (kRagged && tb + e >= T) { ra = 0u; rk = 0u; rw = 0xff80u; }
             fr[e] = bf16_bits_to_float(ra); fk[e] = bf16_bits_to_float(rk); fw[e] = bf16_bits_to_float(rw);
@@ -497,7 +515,7 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
         float cs2 = 0.f, pa = 1.f;
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-            const float ew2 = exp2_fast(fw[e] * kLog2e) * kLog2e;   // exp(w) * log2(e)
+            const float ew2 = exp2_fast(fmaf(fw[e], kLog2e, kLog2Log2e));   // exp(w) * log2(e)
             fa[e] = pa;
             xr[e] = fr[e] * pa;
             cs2 += ew2;
@@ -512,14 +530,15 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
         for (int e = 0; e < 16; e += 2) {
             const uint32_t pr2 = pack_bf16x2(xr[e], xr[e + 1]), pk2 = pack_bf16x2(xk[e], xk[e + 1]);
             const uint32_t pf2 = pack_bf16x2(fa[e], fa[e + 1]);
-            const uint32_t o0 = choff[e & 7] + e * kTileRow, o1 = choff[(e + 1) & 7] + (e + 1) * kTileRow;
-            *reinterpret_cast<uint16_t *>(op + BwdLds::kOpRt + o0) = (uint16_t)pr2;
-            *reinterpret_cast<uint16_t *>(op + BwdLds::kOpRt + o1) = (uint16_t)(pr2 >> 16);
-            *reinterpret_cast<uint16_t *>(op + BwdLds::kOpKt + o0) = (uint16_t)pk2;
-            *reinterpret_cast<uint16_t *>(op + BwdLds::kOpKt + o1) = (uint16_t)(pk2 >> 16);
-            *reinterpret_cast<uint16_t *>(op + BwdLds::kOpFr + o0) = (uint16_t)pf2;
-            *reinterpret_cast<uint16_t *>(op + BwdLds::kOpFr + o1) = (uint16_t)(pf2 >> 16);
+            unsigned char *o0 = a_op[e & 7] + e * kTileRow, *o1 = a_op[(e + 1) & 7] + (e + 1) * kTileRow;
+            *reinterpret_cast<uint16_t *>(o0 + BwdLds::kOpRt) = (uint16_t)pr2;
+            *reinterpret_cast<uint16_t *>(o1 + BwdLds::kOpRt) = (uint16_t)(pr2 >> 16);
+            *reinterpret_cast<uint16_t *>(o0 + BwdLds::kOpKt) = (uint16_t)pk2;
+            *reinterpret_cast<uint16_t *>(o1 + BwdLds::kOpKt) = (uint16_t)(pk2 >> 16);
+            *reinterpret_cast<uint16_t *>(o0 + BwdLds::kOpFr) = (uint16_t)pf2;
+            *reinterpret_cast<uint16_t *>(o1 + BwdLds::kOpFr) = (uint16_t)(pf2 >> 16);
         }
+        unsigned char *op = smem + BwdLds::kOp + (it & 1) * BwdLds::kOpBytes;
         reinterpret_cast<float *>(op + BwdLds::kOpG)[p * kN + ch] = pa;
         if (full) {
             const float tr = transpose_reduce16(pr, lane);
@@ -530,6 +549,9 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     GvState gvst;
     if (kAlsoGv) gvst.init();
     WKV6_STAMP_DECL;
+#ifdef WKV6_PRIO_P
+    __builtin_amdgcn_s_setprio(WKV6_PRIO_P);
+#endif
     issue_loads(0);
     wait_younger(nitem > 1 ? issue_loads(1) : 0);
     prepare(0);

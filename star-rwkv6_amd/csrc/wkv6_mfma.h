@@ -92,6 +92,13 @@ __device__ __forceinline__ uint32_t ld16(const void *base, uint32_t byteoff) {
     return *reinterpret_cast<const uint16_t *>(reinterpret_cast<const char *>(base) + byteoff);
 }
 
+// the low / the high bf16 of a packed pair
+__device__ __forceinline__ void st16_lo(void *base, uint32_t byteoff, uint32_t pair) {
+    *reinterpret_cast<uint16_t *>(reinterpret_cast<char *>(base) + byteoff) = (uint16_t)pair;
+}
+__device__ __forceinline__ void st16_hi(void *base, uint32_t byteoff, uint32_t pair) {
+    *reinterpret_cast<uint16_t *>(reinterpret_cast<char *>(base) + byteoff) = (uint16_t)(pair >> 16);
+}
 __device__ __forceinline__ void st16(void *base, uint32_t byteoff, float x) {
     *reinterpret_cast<uint16_t *>(reinterpret_cast<char *>(base) + byteoff) = (uint16_t)pack_bf16x2(x, 0.f);
 }
@@ -115,19 +122,33 @@ __device__ __forceinline__ bf16x8 acc_as_operand(const f32x4 &a, const f32x4 &b)
     return make_bf16x8(pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]), pack_bf16x2(b[0], b[1]), pack_bf16x2(b[2], b[3]));
 }
 
-// sum over the 64 lanes of 16 per-lane values; lane l receives the total of value (l>>2)&15
+// sum over the 64 lanes of 16 per-lane values; lane l receives the total of value (l>>2)&15.
+// The two folds across the 16-lane rows use the row-swap instructions (one swap hands both
+// partners what they need), the folds inside a row DPP / the swizzle crossbar.
+__device__ __forceinline__ float add_swapped32(float a, float b) {   // rows 0,1: a folded over lane^32; rows 2,3: b
+    const u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float add_swapped16(float a, float b) {   // rows 0,2: a folded over lane^16; rows 1,3: b
+    const u32x2 r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 __device__ __forceinline__ float transpose_reduce16(const float (&p)[16], int lane) {
     float x8[8], x4[4], x2[2];
-    const bool b5 = lane & 32, b4 = lane & 16, b3 = lane & 8, b2 = lane & 4;
 #pragma unroll
-    for (int a = 0; a < 8; ++a) x8[a] = (b5 ? p[a + 8] : p[a]) + __shfl_xor(b5 ? p[a] : p[a + 8], 32);
+    for (int a = 0; a < 8; ++a) x8[a] = add_swapped32(p[a], p[a + 8]);      // value a | a+8 by wave half
 #pragma unroll
-    for (int a = 0; a < 4; ++a) x4[a] = (b4 ? x8[a + 4] : x8[a]) + __shfl_xor(b4 ? x8[a] : x8[a + 4], 16);
+    for (int a = 0; a < 4; ++a) x4[a] = add_swapped16(x8[a], x8[a + 4]);    // row rho holds value a + 4 rho
+    const bool b3 = lane & 8, b2 = lane & 4;
 #pragma unroll
-    for (int a = 0; a < 2; ++a) x2[a] = (b3 ? x4[a + 2] : x4[a]) + __shfl_xor(b3 ? x4[a] : x4[a + 2], 8);
-    float x = (b2 ? x2[1] : x2[0]) + __shfl_xor(b2 ? x2[0] : x2[1], 4);
-    x += __shfl_xor(x, 2);
-    x += __shfl_xor(x, 1);
+    for (int a = 0; a < 2; ++a) {
+        const float keep = b3 ? x4[a + 2] : x4[a], give = b3 ? x4[a] : x4[a + 2];
+        x2[a] = keep + __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(give), 0x128, 0xF, 0xF, true));   // row_ror:8 = lane^8
+    }
+    const float keep = b2 ? x2[1] : x2[0], give = b2 ? x2[0] : x2[1];
+    float x = keep + __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(give), 0x101F));   // lane^4
+    x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0x4E, 0xF, 0xF, true));       // lane^2
+    x += xor1(x);
     return x;
 }
 
