@@ -65,6 +65,10 @@ static_assert(BwdLds::kBytes <= 160 * 1024, "LDS block of the backward kernel");
 #define WKV6_STAMP_DECL do { } while (0)
 #endif
 
+#ifndef WKV6_ABLATE
+#define WKV6_ABLATE 0   // timing experiments only: 1 no tile loads, 2 no state loads, 4 no gr/gk/gw stores, 8 no gv stores
+#endif
+
 struct BwdArgs {
     long long *dbg;
     int T, H;
@@ -93,12 +97,6 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     auto mine = [](int p) { return NG == 1 || (p & 1) == (GRP ^ 1); };   // group 0: tiles 3, 1; group 1: tiles 2, 0
     int item = 0;
     WKV6_STAMP_DECL;
-#ifdef WKV6_PRIO_A
-    if (GRP == 0) __builtin_amdgcn_s_setprio(WKV6_PRIO_A);
-#endif
-#ifdef WKV6_PRIO_B
-    if (GRP == 1) __builtin_amdgcn_s_setprio(WKV6_PRIO_B);
-#endif
     if (kSweepStates) {
         // phase 1: S^T (rows i, column j = col), checkpoint at every chunk start; group 0 only
         f32x4 S[4];
@@ -139,26 +137,44 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     float gu_acc = 0.f;
     bf16_t *gr_h = a.gr + base, *gk_h = a.gk + base, *gw_h = a.gw + base;
     const uint32_t rowbytes = (uint32_t)C * 2u;
-    // checkpointed forward state of a chunk, as loaded (packed bf16)
+    // Checkpointed forward state as loaded (packed bf16), requested one visit ahead.  A wave's loads
+    // and stores complete in program order, so this load is not reported complete before the
+    // gradient stores issued ahead of it have reached the L2; the request therefore goes out as early
+    // in the visit as the registers allow, and the wait for it comes at the very end.
     uint2 Sraw[4];
-    auto load_state = [&](int c) {
+    auto load_state = [&](int c, uint2 (&dst)[4]) {
+        if ((WKV6_ABLATE & 2) && T > 0) { dst[0] = dst[1] = dst[2] = dst[3] = make_uint2(0u, 0u); return; }
         const bf16_t *src = ck + (int64_t)c * (kN * kN) + col * kN;
 #pragma unroll
-        for (int m = 0; m < 4; ++m) Sraw[m] = *reinterpret_cast<const uint2 *>(src + 16 * m + 4 * g);
+        for (int m = 0; m < 4; ++m) dst[m] = *reinterpret_cast<const uint2 *>(src + 16 * m + 4 * g);
     };
     // One chunk visit.  All four tiles are always processed (tokens past the end were prepared as
     // r = k = 0, decay 1, so they leave both states alone and contribute nothing), which keeps the
     // body free of branches that change the number of memory operations: the wait for the
-    // prefetched next state (the fake use at the end) is then counted exactly instead of draining
-    // this wave's stores every chunk.
-    if (!kSweepStates && nchunk > 0) load_state(nchunk - 1);
-    for (int c = nchunk - 1; c >= 0; --c, ++item) {
+    // prefetched state of the next visit (the fake use at the end) is then counted exactly instead
+    // of draining this wave's stores every chunk.
+    // gr, gk, gw of the 4 tokens from `tfirst` on, channel col, as packed pairs {gr01, gk01, gw01, gr23, gk23, gw23}
+    auto store_tile = [&](int tfirst, const uint32_t (&pk)[6]) {
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+            const int t = tfirst + 2 * hh;
+            const uint32_t o = (uint32_t)t * rowbytes + 2u * (uint32_t)col;
+            if ((WKV6_ABLATE & 4) && T > 0) continue;
+            if (!kRagged || t < T) {
+                st16_lo(gr_h, o, pk[3 * hh]); st16_lo(gk_h, o, pk[3 * hh + 1]); st16_lo(gw_h, o, pk[3 * hh + 2]);
+            }
+            if (!kRagged || t + 1 < T) {
+                st16_hi(gr_h, o + rowbytes, pk[3 * hh]); st16_hi(gk_h, o + rowbytes, pk[3 * hh + 1]); st16_hi(gw_h, o + rowbytes, pk[3 * hh + 2]);
+            }
+        }
+    };
+    auto visit = [&](int c, uint2 (&Sraw)[4]) {
         WKV6_STAMP();
         __syncthreads();
         WKV6_STAMP();
         // with kSweepStates the checkpoints were written by this kernel a moment ago: read them
-        // here; otherwise the load was issued during the previous chunk
-        if (kSweepStates) load_state(c);
+        // here; otherwise the load was issued two visits ago
+        if (kSweepStates) load_state(c, Sraw);
         // Uniform block offsets of this item.  They pass through fresh_s() before every tile, which
         // keeps the compiler from forming (block + lane offset) for all tiles at once and holding
         // two dozen address registers across the chunk.
@@ -186,6 +202,9 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
             SopL[0] = make_bf16x8(Sraw[0].x, Sraw[0].y, Sraw[1].x, Sraw[1].y);
             SopH[0] = make_bf16x8(Sraw[2].x, Sraw[2].y, Sraw[3].x, Sraw[3].y);
         }
+        // the registers of the packed state are free again: request the next visit's (chunk 0
+        // fetches itself once more, unused)
+        if (!kSweepStates) load_state(c > 0 ? c - 1 : 0, Sraw);
 #pragma unroll
         for (int p = 0; p < 3; ++p) {
             if (NG == 2 && GRP == 1 && p == 2) continue;   // group 1 needs the states of tiles 0 and 2 only
@@ -198,8 +217,6 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
             for (int m = 0; m < 4; ++m) { S[m][0] *= gq; S[m][1] *= gq; S[m][2] *= gq; S[m][3] *= gq; }
             if (mine(p + 1)) { SopL[p + 1] = acc_as_operand(S[0], S[1]); SopH[p + 1] = acc_as_operand(S[2], S[3]); }
         }
-        // S is free again: fetch the next chunk's state under this chunk's work (chunk 0 fetches itself again, unused)
-        if (!kSweepStates) load_state(c > 0 ? c - 1 : 0);
         WKV6_STAMP();
         __builtin_amdgcn_sched_barrier(0);   // keep the scheduler from interleaving the tiles (register pressure)
 #pragma unroll
@@ -322,26 +339,25 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
                 for (int rr = 0; rr < 4; ++rr)
                     if (t0 + tk + rr == 0 || t0 + tk + rr == T - 1) gwo[rr] = 0.f;
             }
-#pragma unroll
-            for (int rr = 0; rr < 4; rr += 2) {   // two tokens share one conversion per tensor
-                const uint32_t pr2 = pack_bf16x2(gro[rr], gro[rr + 1]), pk2 = pack_bf16x2(gko[rr], gko[rr + 1]);
-                const uint32_t pw2 = pack_bf16x2(gwo[rr], gwo[rr + 1]);
-                const int t = t0 + tk + rr;
-                const uint32_t o = (uint32_t)t * rowbytes + 2u * (uint32_t)col;
-                if (!kRagged || t < T) {
-                    st16_lo(gr_h, o, pr2); st16_lo(gk_h, o, pk2); st16_lo(gw_h, o, pw2);
-                }
-                if (!kRagged || t + 1 < T) {
-                    st16_hi(gr_h, o + rowbytes, pr2); st16_hi(gk_h, o + rowbytes, pk2); st16_hi(gw_h, o + rowbytes, pw2);
-                }
-            }
+            // two tokens share one conversion per tensor
+            const uint32_t packed[6] = {pack_bf16x2(gro[0], gro[1]), pack_bf16x2(gko[0], gko[1]), pack_bf16x2(gwo[0], gwo[1]),
+                                        pack_bf16x2(gro[2], gro[3]), pack_bf16x2(gko[2], gko[3]), pack_bf16x2(gwo[2], gwo[3])};
+            store_tile(t0 + tk, packed);
             WKV6_STAMP();
             __builtin_amdgcn_sched_barrier(0);
         }
-        // fake use of the prefetched state: the wait for its loads lands here, after this chunk's
+        // fake use of the next visit's state: the wait for its loads lands here, after this visit's
         // stores in program order and with their number known
         if (!kSweepStates) asm volatile("" : "+v"(Sraw[0]), "+v"(Sraw[1]), "+v"(Sraw[2]), "+v"(Sraw[3]));
+        ++item;
+    };
+    if (!kSweepStates && nchunk > 0) {
+        load_state(nchunk - 1, Sraw);
+        // have the first state arrive here: a wait for it inside the loop would be sized for this
+        // path (nothing younger in flight) and drain the stores on every visit
+        asm volatile("" : "+v"(Sraw[0]), "+v"(Sraw[1]), "+v"(Sraw[2]), "+v"(Sraw[3]));
     }
+    for (int c = nchunk - 1; c >= 0; --c) visit(c, Sraw);
     // gu: fold the four lane groups (different tokens, same channel), then the consumer groups
     gu_acc = sum_rows(gu_acc);
     if (NG == 2 && GRP == 1 && g == 0) reinterpret_cast<float *>(smem + BwdLds::kGu)[col] = gu_acc;
@@ -409,6 +425,7 @@ __device__ __forceinline__ void bwd_gv_chunk(GvState &st, const BwdArgs &a, cons
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
             const int t = t0 + tk + rr;
+            if ((WKV6_ABLATE & 8) && T > 0) continue;
             if (!kRagged || t < T) st16(gv_h, (uint32_t)t * rowbytes + 2u * (uint32_t)col, GV[rr]);
         }
     }
@@ -460,6 +477,7 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     // turns them into r = k = 0, w = -inf (decay 1), and the v, gy rows only ever meet zero operands.
     // Returns the number of loads.
     auto issue_loads = [&](int it) -> int {
+        if ((WKV6_ABLATE & 1) && T > 0) return 0;
         const int tb = item_chunk(it) * CL + 16 * p;
         const bool full = item_full(it);
         const uint32_t rk = lds0 + BwdLds::kRawRK + (it & 1) * 2 * kTileBytes + 16 * p * kTileRow;
@@ -479,8 +497,20 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
         }
         return full ? 10 : 6;
     };
-    auto wait_younger = [&](int n) {   // n = loads issued after the ones being waited for
-        if (n == 10) wait_loads<10>(); else if (n == 6) wait_loads<6>(); else wait_loads<0>();
+    // Waits for this wave's tile loads of one item.  `n` = operations issued after them: the loads
+    // of the following item and, with the gv role on this wave, the 16 gv stores of the chunk
+    // visit in between (memory operations of a wave complete in program order; the stores are left
+    // in flight -- waiting for them costs more than a microsecond per chunk under load).
+    auto wait_younger = [&](int n) {
+        if ((WKV6_ABLATE & 1) && T > 0) return;
+        switch (n) {
+        case 26: wait_loads<26>(); break;
+        case 22: wait_loads<22>(); break;
+        case 16: wait_loads<16>(); break;
+        case 10: wait_loads<10>(); break;
+        case 6: wait_loads<6>(); break;
+        default: wait_loads<0>(); break;
+        }
     };
     // per-lane byte offsets of channel `ch` inside a tile row, for the 8 swizzle phases
     uint32_t choff[8];
@@ -549,9 +579,6 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     GvState gvst;
     if (kAlsoGv) gvst.init();
     WKV6_STAMP_DECL;
-#ifdef WKV6_PRIO_P
-    __builtin_amdgcn_s_setprio(WKV6_PRIO_P);
-#endif
     issue_loads(0);
     wait_younger(nitem > 1 ? issue_loads(1) : 0);
     prepare(0);
@@ -564,7 +591,9 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
         const int younger = it + 2 < nitem ? issue_loads(it + 2) : 0;
         if (it + 1 < nitem) {
             WKV6_STAMP();
-            wait_younger(younger);
+            // (with a ragged tail the number of gv stores issued is not fixed: wait for everything older)
+            const int gv_stores = (kAlsoGv && !kRagged && it >= 1 && item_full(it - 1)) ? 16 : 0;
+            wait_younger(younger + gv_stores);
             WKV6_STAMP();
             prepare(it + 1);
             WKV6_STAMP();
@@ -595,6 +624,7 @@ __global__ __launch_bounds__(BwdLayout<kLayout>::kWaves * 64) void chunk_bwd_ker
     static_assert(sizeof(ScanBwdALds) <= BwdLds::kBytes && sizeof(ScanBwdBLds) <= BwdLds::kBytes,
                   "the exact second pass reuses the LDS block");
     if (threadIdx.x == 0) s_wild = 0;
+    if (WKV6_ABLATE & 1) for (int i = threadIdx.x; i < BwdLds::kBytes / 4; i += blockDim.x) reinterpret_cast<uint32_t *>(smem)[i] = 0u;
 #ifdef WKV6_TIMING
     if (threadIdx.x == 0) a.dbg[16 * 256 + 2 * blockIdx.x] = __builtin_readcyclecounter();
 #endif
