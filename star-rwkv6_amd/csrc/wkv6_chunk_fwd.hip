@@ -1,7 +1,8 @@
 // WKV6 in chunk-parallel form for gfx950: bf16 MFMA for the dense products, fp32 state.
 //
-// One workgroup (16 waves) per (batch, head).  Time is cut into chunks of 64 tokens, each chunk
-// into 4 tiles of 16 tokens.  The fp32 state S[j][i] lives in the MFMA accumulators of the
+// One workgroup (12 waves) per (batch, head) pair, or -- with more pairs than compute units -- one
+// workgroup per compute unit that runs its pairs back to back through the same pipeline.  Time is
+// cut into chunks of 64 tokens, each chunk into 4 tiles of 16 tokens.  The fp32 state S[j][i] lives in the MFMA accumulators of the
 // "consumer" waves (wave q of a group owns value columns 16q..16q+15) and is advanced one tile at a time:
 //
 //   c_t = sum_{s<t} exp(w_s) inside the tile (so exp(-c_t) is the decay from the tile start to t)
@@ -12,8 +13,8 @@
 //   S       <- diag(g) (S + K~^T V)   (64x16x16 MFMA, K index s)
 //
 // Data path.  The raw r, k, w, v rows of a chunk go from global memory straight into LDS tiles
-// (16-byte pieces, no registers), two chunks ahead of their use.  The eight "producer" waves (two per
-// tile, eight tokens each, lane = channel) read r, k, w from there, compute R~, K~, g and the diagonal
+// (16-byte pieces, no registers), two chunks ahead of their use.  The four "producer" waves (one per
+// tile, lane = channel) read r, k, w from there, compute R~, K~, g and the diagonal
 // in fp32 for the NEXT chunk and write them back as bf16 tiles while the consumers run the MFMAs of
 // the current one; the consumers (two groups of four waves that both carry the state but share out
 // the per-tile output work) take V directly from its raw tile.  Every tile is stored once,
@@ -68,6 +69,7 @@ constexpr int kFwdThreads = 4 * (kFwdHalves + kFwdGroups) * 64;
 struct FwdArgs {
     long long *dbg;
     int T, H;
+    int nitems;      // B * H (batch, head) pairs; with kMulti a workgroup takes every gridDim.x-th of them
     const bf16_t *r, *k, *v, *w, *u;
     const void *s0;
     const int64_t *map;
@@ -81,107 +83,126 @@ struct FwdArgs {
 // Consumer group GRP of two: both groups carry the state through every tile (4 MFMAs and a
 // scaling), group 0 produces y for tiles 0 and 2, group 1 for tiles 1 and 3.
 // ------------------------------------------------------------------------------------------
-template <typename Ts, bool kSave, bool kRagged, int NG, int GRP>
-__device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned char *smem, int b, int h, int q, int lane)
+template <typename Ts, bool kSave, bool kRagged, bool kMulti, int NG, int GRP>
+__device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned char *smem, int q, int lane)
 {
     const int T = a.T, H = a.H;
     const int g = lane >> 4, l16 = lane & 15;
     const int64_t C = (int64_t)H * kN;
-    const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
     const int nchunk = (T + CL - 1) / CL;
+    const int stride = (int)gridDim.x;
+    const int n_my = kMulti ? (a.nitems - (int)blockIdx.x + stride - 1) / stride : 1;
     const Ts *s0 = reinterpret_cast<const Ts *>(a.s0);
-    f32x4 S[4];
-    if (s0 != nullptr) {
+    // initial state of a (batch, head) pair as stored (converted when the pair starts)
+    Ts Sraw[16];
+    auto request_state = [&](int bh) {
+        const int b = bh / H, h = bh - b * H;
         const int64_t row = a.map ? a.map[b] : (int64_t)b;
         const Ts *p = s0 + (row * H + h) * kN * kN + 16 * q + l16;
 #pragma unroll
         for (int m = 0; m < 4; ++m)
 #pragma unroll
-            for (int rr = 0; rr < 4; ++rr) S[m][rr] = load1(p + (16 * m + 4 * g + rr) * kN);
-    } else {
-#pragma unroll
-        for (int m = 0; m < 4; ++m) S[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    }
-    bf16_t *y_h = a.y + base;
+            for (int rr = 0; rr < 4; ++rr) Sraw[4 * m + rr] = p[(16 * m + 4 * g + rr) * kN];
+    };
+    if (s0 != nullptr) request_state((int)blockIdx.x);
     WKV6_FSTAMP_DECL;
-    for (int c = 0; c < nchunk; ++c) {
-        WKV6_FSTAMP();
-        if (kSave && GRP == 0) {
-            // bf16 [chunk][j][i], in the first half of this workgroup's slice of the workspace
-            bf16_t *dst = reinterpret_cast<bf16_t *>(a.ckpt + (int64_t)(b * H + h) * nchunk * (kN * kN)) + (int64_t)c * (kN * kN) + 16 * q + l16;
+    int it = 0;   // chunk visits of this workgroup so far: picks the LDS buffers
+    for (int n = 0, bh = (int)blockIdx.x; n < n_my; ++n, bh += stride) {
+        const int b = bh / H, h = bh - b * H;
+        const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
+        f32x4 S[4];
+        if (s0 != nullptr) {
 #pragma unroll
             for (int m = 0; m < 4; ++m)
 #pragma unroll
-                for (int rr = 0; rr < 4; ++rr) store1(dst + (16 * m + 4 * g + rr) * kN, S[m][rr]);
+                for (int rr = 0; rr < 4; ++rr) S[m][rr] = (float)Sraw[4 * m + rr];
+        } else {
+#pragma unroll
+            for (int m = 0; m < 4; ++m) S[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
         }
-        WKV6_FSTAMP();
-        __syncthreads();
-        WKV6_FSTAMP();
-        // Tokens past the end were prepared as r = k = 0, decay 1: their tiles leave the state alone,
-        // and their y rows are not stored.
-        int op_off = FwdLds::kOp + (c & 1) * FwdLds::kOpBytes, v_off = FwdLds::kRawV + (c % 3) * kTileBytes;
-        const int t0 = c * CL;
+        bf16_t *y_h = a.y + base;
+        if (kSave && GRP == 0 && b == 0 && q == 0 && lane == 0) a.arrivals[h] = 0;
+        for (int c = 0; c < nchunk; ++c, ++it) {
+            WKV6_FSTAMP();
+            if (kSave && GRP == 0) {
+                // bf16 [chunk][j][i], in the first half of this pair's slice of the workspace
+                bf16_t *dst = reinterpret_cast<bf16_t *>(a.ckpt + (int64_t)bh * nchunk * (kN * kN)) + (int64_t)c * (kN * kN) + 16 * q + l16;
 #pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            // (fresh_s: form the tile addresses per tile instead of holding them all across the chunk)
-            op_off = fresh_s(op_off); v_off = fresh_s(v_off);
-            const unsigned char *rt = smem + op_off + FwdLds::kOpRt, *kt = smem + op_off + FwdLds::kOpKt;
-            const float *gv_ = reinterpret_cast<const float *>(smem + op_off + FwdLds::kOpG);
-            const float *ruk = reinterpret_cast<const float *>(smem + op_off + FwdLds::kOpRuk);
-            const unsigned char *vt = smem + v_off;
-            const s16x4 vf = tile_frag_tok(vt, 16 * q, 16 * p, l16, g);
-            // U = K~^T V in accumulators of its own: these MFMAs do not wait for the state, which keeps
-            // the chain from one tile's state to the next down to the VALU update at the end
-            f32x4 U[4];
+                for (int m = 0; m < 4; ++m)
 #pragma unroll
-            for (int m = 0; m < 4; ++m) U[m] = mfma16(tile_frag_tok(kt, 16 * m, 16 * p, l16, g), vf, (f32x4){0.f, 0.f, 0.f, 0.f});
-            if (NG == 1 || (p & 1) == GRP) {
-                const int row = 16 * p + l16;
-                const bf16x8 rf0 = tile_frag_ch(rt, row, 0, g), rf1 = tile_frag_ch(rt, row, 1, g);
-                const bf16x8 kf0 = tile_frag_ch(kt, row, 0, g), kf1 = tile_frag_ch(kt, row, 1, g);
-                const float rukv = ruk[row];
-                // A^T[s][t] = K~_s . R~_t  (accumulator rows s = 4g+r, column t = l16)
-                f32x4 AT = {0.f, 0.f, 0.f, 0.f};
-                AT = mfma32(kf0, rf0, AT);
-                AT = mfma32(kf1, rf1, AT);
-                // Y = R~ S
-                f32x4 Y = {0.f, 0.f, 0.f, 0.f};
-                Y = mfma32(rf0, acc_as_operand(S[0], S[1]), Y);
-                Y = mfma32(rf1, acc_as_operand(S[2], S[3]), Y);
-                settle(AT);
-#pragma unroll
-                for (int rr = 0; rr < 4; ++rr) {
-                    const int s = 4 * g + rr;
-                    AT[rr] = (l16 > s) ? AT[rr] : ((l16 == s) ? rukv : 0.f);
-                }
-                // Y += A V : the masked A^T accumulator IS the A operand (row t = l16, k-slots s = 4g+r)
-                chain_gap(Y);
-                Y = mfma16(make_s16x4(pack_bf16x2(AT[0], AT[1]), pack_bf16x2(AT[2], AT[3])), vf, Y);
-                settle(Y);
-#pragma unroll
-                for (int rr = 0; rr < 4; ++rr) {
-                    const int t = t0 + 16 * p + 4 * g + rr;
-                    if (!kRagged || t < T) st16(y_h, (uint32_t)t * (uint32_t)C * 2u + 2u * (uint32_t)(16 * q + l16), Y[rr]);
-                }
-            }
-            // S <- diag(g) (S + U)
-            settle(U[0], U[1], U[2], U[3]);
-#pragma unroll
-            for (int m = 0; m < 4; ++m) {
-                const float4 gg = *reinterpret_cast<const float4 *>(&gv_[p * kN + 16 * m + 4 * g]);
-                S[m][0] = (S[m][0] + U[m][0]) * gg.x; S[m][1] = (S[m][1] + U[m][1]) * gg.y;
-                S[m][2] = (S[m][2] + U[m][2]) * gg.z; S[m][3] = (S[m][3] + U[m][3]) * gg.w;
+                    for (int rr = 0; rr < 4; ++rr) store1(dst + (16 * m + 4 * g + rr) * kN, S[m][rr]);
             }
             WKV6_FSTAMP();
-            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
+            WKV6_FSTAMP();
+            // the next pair's initial state is requested one chunk visit ahead of its use
+            if (kMulti && s0 != nullptr && c == nchunk - 1 && n + 1 < n_my) request_state(bh + stride);
+            // Tokens past the end were prepared as r = k = 0, decay 1: their tiles leave the state alone,
+            // and their y rows are not stored.
+            int op_off = FwdLds::kOp + (it & 1) * FwdLds::kOpBytes, v_off = FwdLds::kRawV + (it % 3) * kTileBytes;
+            const int t0 = c * CL;
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                // (fresh_s: form the tile addresses per tile instead of holding them all across the chunk)
+                op_off = fresh_s(op_off); v_off = fresh_s(v_off);
+                const unsigned char *rt = smem + op_off + FwdLds::kOpRt, *kt = smem + op_off + FwdLds::kOpKt;
+                const float *gv_ = reinterpret_cast<const float *>(smem + op_off + FwdLds::kOpG);
+                const float *ruk = reinterpret_cast<const float *>(smem + op_off + FwdLds::kOpRuk);
+                const unsigned char *vt = smem + v_off;
+                const s16x4 vf = tile_frag_tok(vt, 16 * q, 16 * p, l16, g);
+                // U = K~^T V in accumulators of its own: these MFMAs do not wait for the state, which keeps
+                // the chain from one tile's state to the next down to the VALU update at the end
+                f32x4 U[4];
+#pragma unroll
+                for (int m = 0; m < 4; ++m) U[m] = mfma16(tile_frag_tok(kt, 16 * m, 16 * p, l16, g), vf, (f32x4){0.f, 0.f, 0.f, 0.f});
+                if (NG == 1 || (p & 1) == GRP) {
+                    const int row = 16 * p + l16;
+                    const bf16x8 rf0 = tile_frag_ch(rt, row, 0, g), rf1 = tile_frag_ch(rt, row, 1, g);
+                    const bf16x8 kf0 = tile_frag_ch(kt, row, 0, g), kf1 = tile_frag_ch(kt, row, 1, g);
+                    const float rukv = ruk[row];
+                    // A^T[s][t] = K~_s . R~_t  (accumulator rows s = 4g+r, column t = l16)
+                    f32x4 AT = {0.f, 0.f, 0.f, 0.f};
+                    AT = mfma32(kf0, rf0, AT);
+                    AT = mfma32(kf1, rf1, AT);
+                    // Y = R~ S
+                    f32x4 Y = {0.f, 0.f, 0.f, 0.f};
+                    Y = mfma32(rf0, acc_as_operand(S[0], S[1]), Y);
+                    Y = mfma32(rf1, acc_as_operand(S[2], S[3]), Y);
+                    settle(AT);
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) {
+                        const int s = 4 * g + rr;
+                        AT[rr] = (l16 > s) ? AT[rr] : ((l16 == s) ? rukv : 0.f);
+                    }
+                    // Y += A V : the masked A^T accumulator IS the A operand (row t = l16, k-slots s = 4g+r)
+                    chain_gap(Y);
+                    Y = mfma16(make_s16x4(pack_bf16x2(AT[0], AT[1]), pack_bf16x2(AT[2], AT[3])), vf, Y);
+                    settle(Y);
+#pragma unroll
+                    for (int rr = 0; rr < 4; ++rr) {
+                        const int t = t0 + 16 * p + 4 * g + rr;
+                        if (!kRagged || t < T) st16(y_h, (uint32_t)t * (uint32_t)C * 2u + 2u * (uint32_t)(16 * q + l16), Y[rr]);
+                    }
+                }
+                // S <- diag(g) (S + U)
+                settle(U[0], U[1], U[2], U[3]);
+#pragma unroll
+                for (int m = 0; m < 4; ++m) {
+                    const float4 gg = *reinterpret_cast<const float4 *>(&gv_[p * kN + 16 * m + 4 * g]);
+                    S[m][0] = (S[m][0] + U[m][0]) * gg.x; S[m][1] = (S[m][1] + U[m][1]) * gg.y;
+                    S[m][2] = (S[m][2] + U[m][2]) * gg.z; S[m][3] = (S[m][3] + U[m][3]) * gg.w;
+                }
+                WKV6_FSTAMP();
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-    }
-    if (a.sT != nullptr && GRP == 0) {
-        Ts *p = reinterpret_cast<Ts *>(a.sT) + ((int64_t)b * H + h) * kN * kN + 16 * q + l16;
+        if (a.sT != nullptr && GRP == 0) {
+            Ts *p = reinterpret_cast<Ts *>(a.sT) + (int64_t)bh * kN * kN + 16 * q + l16;
 #pragma unroll
-        for (int m = 0; m < 4; ++m)
+            for (int m = 0; m < 4; ++m)
 #pragma unroll
-            for (int rr = 0; rr < 4; ++rr) store1(p + (16 * m + 4 * g + rr) * kN, S[m][rr]);
+                for (int rr = 0; rr < 4; ++rr) store1(p + (16 * m + 4 * g + rr) * kN, S[m][rr]);
+        }
     }
 }
 
@@ -190,33 +211,43 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
 // wave 2p+hf <-> tokens 8hf..8hf+7 of tile p; the second-half wave redoes the first half's exp(w)
 // to get its starting decay.
 // ------------------------------------------------------------------------------------------
-template <bool kRagged, int kHalves>
-__device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *smem, int *s_wild, int b, int h, int pw, int lane)
+template <bool kRagged, bool kMulti, int kHalves>
+__device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *smem, int *s_wild, int pw, int lane)
 {
     constexpr int NT = 16 / kHalves;   // tokens per wave and chunk
     const int T = a.T, H = a.H;
     const int p = kHalves == 2 ? pw >> 1 : pw, hf = kHalves == 2 ? pw & 1 : 0;
     const int ch = lane;
     const int64_t C = (int64_t)H * kN;
-    const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
     const int nchunk = (T + CL - 1) / CL;
-    const float uc = load1(a.u + h * kN + ch);
-    const bf16_t *rb = a.r + base, *kb_ = a.k + base, *vb = a.v + base, *wb = a.w + base;   // uniform
+    const int stride = (int)gridDim.x;
+    const int n_my = kMulti ? (a.nitems - (int)blockIdx.x + stride - 1) / stride : 1;
+    const int nvisit = n_my * nchunk;   // chunk visits of this workgroup, pair after pair
     const uint32_t rowbytes = (uint32_t)C * 2u;
     const uint32_t lds0 = lds_address(smem);
     // this lane's part of an 8-row block load: row (lane >> 3), 16-byte piece swizzled with the row
     const int lrow = lane >> 3;
     const uint32_t lpiece = (uint32_t)(((lane & 7) ^ lrow) << 4);
+    // The load stream and the preparation stream each walk the visits in order; `ld_*` / `pp_*` are
+    // the (pair, chunk) the next load / preparation belongs to.
+    int ld_c = 0, ld_bh = (int)blockIdx.x;
+    const bf16_t *rb, *kb_, *vb, *wb;   // uniform: this pair's first row
+    auto point_loads = [&]() {
+        const int b = ld_bh / H, h = ld_bh - b * H;
+        const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
+        rb = a.r + base; kb_ = a.k + base; vb = a.v + base; wb = a.w + base;
+    };
+    point_loads();
     // Rows past the end of the sequence are fetched from row T-1 (valid memory); the operand
     // preparation turns them into r = k = 0, w = -inf (decay 1), and the v rows only ever meet zero
     // operands.  Each wave loads what it reads itself (with kHalves = 2 the second-half wave also
     // the first half's w rows), so its own vmcnt covers its inputs; v is picked up by the consumers
     // a barrier later.
     constexpr int kLoads = kHalves == 2 ? 5 : 8;   // per chunk and wave
-    auto issue_loads = [&](int c) {
-        const int tb = c * CL + 16 * p;
-        const uint32_t rkw = lds0 + FwdLds::kRawRKW + (c & 1) * 3 * kTileBytes + 16 * p * kTileRow;
-        const uint32_t vv = lds0 + FwdLds::kRawV + (c % 3) * kTileBytes + 16 * p * kTileRow;
+    auto issue_loads = [&](int it) {   // visit `it` = the load stream's current (pair, chunk)
+        const int tb = ld_c * CL + 16 * p;
+        const uint32_t rkw = lds0 + FwdLds::kRawRKW + (it & 1) * 3 * kTileBytes + 16 * p * kTileRow;
+        const uint32_t vv = lds0 + FwdLds::kRawV + (it % 3) * kTileBytes + 16 * p * kTileRow;
         if (kHalves == 2) {
             // (the first-half wave loads its w block twice, which keeps the count uniform)
             const int t_first = tb + lrow;
@@ -232,16 +263,19 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
             load_rows8_to_lds(kb_, o, rkw + kTileBytes + 8 * blk * kTileRow);
             load_rows8_to_lds(vb, o, vv + 8 * blk * kTileRow);
         }
+        if (++ld_c == nchunk && kMulti) { ld_c = 0; ld_bh += stride; if (ld_bh < a.nitems) point_loads(); }
     };
+    int pp_c = 0, pp_n = 0, pp_h = (int)blockIdx.x % H;
+    float uc = load1(a.u + pp_h * kN + ch);
     // per-lane byte offsets of channel `ch` inside a tile row, for the 8 swizzle phases
     uint32_t choff[8];
 #pragma unroll
     for (int s = 0; s < 8; ++s) choff[s] = (uint32_t)((((ch >> 3) ^ s) << 4) + ((ch & 7) << 1)) + (uint32_t)(16 * p * kTileRow);
     const float kLog2Log2e = 0.5287663729448977f;   // log2(log2(e)): exp(w) log2(e) = 2^(w log2(e) + this)
-    auto prepare = [&](int c) {
-        const unsigned char *raw = smem + FwdLds::kRawRKW + (c & 1) * 3 * kTileBytes;
-        unsigned char *op = smem + FwdLds::kOp + (c & 1) * FwdLds::kOpBytes;
-        const int tb = c * CL + 16 * p;
+    auto prepare = [&](int it) {   // visit `it` = the preparation stream's current (pair, chunk)
+        const unsigned char *raw = smem + FwdLds::kRawRKW + (it & 1) * 3 * kTileBytes;
+        unsigned char *op = smem + FwdLds::kOp + (it & 1) * FwdLds::kOpBytes;
+        const int tb = pp_c * CL + 16 * p;
         const int e0 = 8 * hf;   // first token of this wave inside the tile
         // exponents are kept in base 2 (one v_exp_f32 each, no extra scaling multiply)
         float cs2 = 0.f, pa = 1.f;
@@ -287,7 +321,7 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
         if (kHalves == 1 || hf) {
             // the whole tile's decay: g, and the range check of exp(+c)
             if (__builtin_amdgcn_ballot_w64(!(cs2 <= kWildLimit * kLog2e)) != 0ull) {
-                if (lane == 0) *s_wild = 1;
+                if (lane == 0) s_wild[pp_n] = 1;
             }
             reinterpret_cast<float *>(op + FwdLds::kOpG)[p * kN + ch] = pa;
         }
@@ -299,24 +333,31 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
             const float tot = transpose_reduce16(pr, lane);
             if ((lane & 3) == 0) ruk[(lane >> 2) & 15] = tot;
         }
+        if (++pp_c == nchunk && kMulti) {   // the next preparation opens the next pair: its head's u
+            pp_c = 0; ++pp_n;
+            if (pp_n < n_my) {
+                pp_h = ((int)blockIdx.x + pp_n * stride) % H;
+                uc = load1(a.u + pp_h * kN + ch);
+            }
+        }
     };
     WKV6_FSTAMP_DECL;
-    // chunk c is loaded during iteration c-2 (or the prologue), prepared during iteration c-1
+    // visit `it` is loaded during visit it-2 (or the prologue), prepared during visit it-1
     issue_loads(0);
-    if (nchunk > 1) { issue_loads(1); wait_loads<kLoads>(); } else wait_loads<0>();
+    if (nvisit > 1) { issue_loads(1); wait_loads<kLoads>(); } else wait_loads<0>();
     prepare(0);
-    for (int c = 0; c < nchunk; ++c) {
+    for (int it = 0; it < nvisit; ++it) {
         WKV6_FSTAMP();
         __syncthreads();
         WKV6_FSTAMP();
-        // the raw r, k, w block of chunk c (read by this wave's prepare(c) before the barrier) and the
-        // raw v block of chunk c-1 (read by the consumers before the barrier) are free again
-        if (c + 2 < nchunk) issue_loads(c + 2);
+        // the raw r, k, w block of visit `it` (read by this wave's prepare(it) before the barrier) and the
+        // raw v block of visit it-1 (read by the consumers before the barrier) are free again
+        if (it + 2 < nvisit) issue_loads(it + 2);
         WKV6_FSTAMP();
-        if (c + 1 < nchunk) {
-            if (c + 2 < nchunk) wait_loads<kLoads>(); else wait_loads<0>();
+        if (it + 1 < nvisit) {
+            if (it + 2 < nvisit) wait_loads<kLoads>(); else wait_loads<0>();
             WKV6_FSTAMP();
-            prepare(c + 1);
+            prepare(it + 1);
             WKV6_FSTAMP();
         }
     }
@@ -325,57 +366,89 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
 
 // kSave: also write the state at every chunk start to `ckpt` (bf16, [b][h][chunk][j][i]) for the
 // backward pass, which then skips its own forward sweep.  kRagged: T is not a multiple of 64.
-template <typename Ts, bool kSave, bool kRagged>
+// kMulti: more (batch, head) pairs than workgroups -- each workgroup takes every gridDim.x-th pair and
+// runs them back to back through one pipeline, so the loads of a pair's first chunks overlap the
+// previous pair's last ones (a workgroup fills the CU's LDS, so nothing else would hide them).
+constexpr int kMaxPairsPerWorkgroup = 32;
+template <typename Ts, bool kSave, bool kRagged, bool kMulti>
 __global__ __launch_bounds__(kFwdThreads) void chunk_fwd_kernel(FwdArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ int s_wild;
+    __shared__ int s_wild[kMaxPairsPerWorkgroup];
     static_assert(sizeof(ScanFwdLds) <= FwdLds::kBytes, "the exact second pass reuses the LDS block");
-    if (threadIdx.x == 0) s_wild = 0;
+    if (threadIdx.x < kMaxPairsPerWorkgroup) s_wild[threadIdx.x] = 0;
     __syncthreads();
 
-    const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int role = wave >> 2, q = wave & 3;
-    if (role < kFwdHalves) fwd_producer<kRagged, kFwdHalves>(a, smem, &s_wild, b, h, wave, lane);
-    else if (kFwdGroups == 1 || role == kFwdHalves) fwd_consumer<Ts, kSave, kRagged, kFwdGroups, 0>(a, smem, b, h, q, lane);
-    else fwd_consumer<Ts, kSave, kRagged, kFwdGroups, 1>(a, smem, b, h, q, lane);
-    // exact second pass for this (b, h) if any of its tiles left the representable range
+    if (role < kFwdHalves) fwd_producer<kRagged, kMulti, kFwdHalves>(a, smem, s_wild, wave, lane);
+    else if (kFwdGroups == 1 || role == kFwdHalves) fwd_consumer<Ts, kSave, kRagged, kMulti, kFwdGroups, 0>(a, smem, q, lane);
+    else fwd_consumer<Ts, kSave, kRagged, kMulti, kFwdGroups, 1>(a, smem, q, lane);
+    // exact second pass for every pair of this workgroup that had a tile leave the representable range
     __threadfence_block();   // workgroup scope is enough (and a device-scope fence would write back the L2)
     __syncthreads();
-    if (kSave && b == 0 && threadIdx.x == 0) a.arrivals[h] = 0;
-    if (s_wild)
-        scan_fwd_body<bf16_t, bf16_t, Ts>(*reinterpret_cast<ScanFwdLds *>(smem), b, h, a.T, a.H, a.r, a.k, a.v, a.w, a.u,
+    const int stride = (int)gridDim.x;
+    const int n_my = kMulti ? (a.nitems - (int)blockIdx.x + stride - 1) / stride : 1;
+    for (int n = 0; n < n_my; ++n) {
+        if (!s_wild[n]) continue;   // uniform over the workgroup
+        const int bh = (int)blockIdx.x + n * stride;
+        __syncthreads();
+        scan_fwd_body<bf16_t, bf16_t, Ts>(*reinterpret_cast<ScanFwdLds *>(smem), bh / a.H, bh % a.H, a.T, a.H, a.r, a.k, a.v, a.w, a.u,
                                           reinterpret_cast<const Ts *>(a.s0), a.map, a.y, reinterpret_cast<Ts *>(a.sT));
+    }
+}
+
+// compute units of the current device (an immutable device property, looked up once per device)
+static int compute_units() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+template <typename Ts, bool kSave, bool kRagged, bool kMulti>
+static hipError_t launch_fwd(hipStream_t st, const FwdArgs &a, unsigned grid) {
+    auto kern = chunk_fwd_kernel<Ts, kSave, kRagged, kMulti>;
+    const size_t lds = FwdLds::kBytes;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kFwdThreads), lds, st, a);
+    return hipGetLastError();
+}
+template <typename Ts, bool kSave, bool kRagged>
+static hipError_t launch_fwd(hipStream_t st, const FwdArgs &a, bool multi, unsigned grid) {
+    return multi ? launch_fwd<Ts, kSave, kRagged, true>(st, a, grid) : launch_fwd<Ts, kSave, kRagged, false>(st, a, grid);
+}
+template <typename Ts>
+static hipError_t launch_fwd(hipStream_t st, const FwdArgs &a, bool save, bool ragged, bool multi, unsigned grid) {
+    if (save) return ragged ? launch_fwd<Ts, true, true>(st, a, multi, grid) : launch_fwd<Ts, true, false>(st, a, multi, grid);
+    return ragged ? launch_fwd<Ts, false, true>(st, a, multi, grid) : launch_fwd<Ts, false, false>(st, a, multi, grid);
 }
 
 hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u,
                          const void *s0, const int64_t *map, void *y, void *sT, void *saved_states)
 {
-    const size_t lds = FwdLds::kBytes;
     FwdArgs a;
-    a.T = (int)T; a.H = (int)H;
+    a.T = (int)T; a.H = (int)H; a.nitems = (int)(B * H);
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
     a.s0 = s0; a.map = map; a.y = (bf16_t *)y; a.sT = sT; a.ckpt = (float *)saved_states;
     a.arrivals = saved_states ? reinterpret_cast<int *>(reinterpret_cast<char *>(saved_states) + chunk_backward_workspace_bytes(B, T, H)) : nullptr;
     a.dbg = saved_states ? reinterpret_cast<long long *>((float *)saved_states + (size_t)(B * H) * ((T + CL - 1) / CL) * kN * kN + 1024) : nullptr;
-    auto launch = [&](auto kern, auto *) -> hipError_t {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(kFwdThreads), lds, st, a);
-        return hipGetLastError();
-    };
+    // One workgroup per pair while they all fit on the chip at once; beyond that one workgroup per
+    // compute unit (more only if a workgroup would otherwise get more pairs than it keeps flags for).
+    const int64_t pairs = B * H, cus = compute_units();
+    const bool multi = pairs > cus;
+    const int64_t grid = !multi ? pairs : (pairs + cus * kMaxPairsPerWorkgroup - 1) / (cus * kMaxPairsPerWorkgroup) * cus;
     const bool save = saved_states != nullptr, ragged = (T % CL) != 0;
-    float *f32tag = nullptr;
-    bf16_t *bf16tag = nullptr;
-    if (state_dtype == kF32) {
-        if (ragged) return save ? launch(chunk_fwd_kernel<float, true, true>, f32tag) : launch(chunk_fwd_kernel<float, false, true>, f32tag);
-        return save ? launch(chunk_fwd_kernel<float, true, false>, f32tag) : launch(chunk_fwd_kernel<float, false, false>, f32tag);
-    }
-    if (ragged) return save ? launch(chunk_fwd_kernel<bf16_t, true, true>, bf16tag) : launch(chunk_fwd_kernel<bf16_t, false, true>, bf16tag);
-    return save ? launch(chunk_fwd_kernel<bf16_t, true, false>, bf16tag) : launch(chunk_fwd_kernel<bf16_t, false, false>, bf16tag);
+    return state_dtype == kF32 ? launch_fwd<float>(st, a, save, ragged, multi, (unsigned)grid)
+                               : launch_fwd<bf16_t>(st, a, save, ragged, multi, (unsigned)grid);
 }
 
 }  // namespace wkv6

@@ -278,6 +278,44 @@ def test_chunk_falls_back_on_extreme_decay(op, oracle):
         check_close(name, to_np(g).reshape(gr.shape), gr, torch.bfloat16, is_grad=True)
 
 
+# More (batch, head) pairs than the chip has compute units: a forward workgroup then runs several
+# pairs back to back through one pipeline (the state, the head's u, the saved states and the
+# fallback flag all switch at the pair boundaries).
+@pytest.mark.parametrize("B,T,H", [(75, 64, 4), (43, 150, 7), (300, 32, 1)])
+def test_chunk_many_pairs_fwd_bwd_bf16(op, oracle, B, T, H):
+    _case(op, oracle, B, T, H, 90 + T, torch.bfloat16, CHUNK)
+
+
+def test_chunk_many_pairs_state_in_out(op, oracle):
+    B, T, H, N = 90, 130, 4, 64
+    ins = oracle.make_inputs(B, T, H, N, 55, with_state=True)
+    dev, ref = cast_inputs(ins[:5], torch.bfloat16)
+    op.algo = CHUNK
+    for sdt in (torch.bfloat16, torch.float32):
+        s_dev, s_ref = cast_inputs([ins[6][:7]], sdt)
+        smap = [(3 * i) % 7 for i in range(B)]
+        y, sT = op(*dev, return_state=True, init_state=s_dev[0], state_map=smap)
+        torch.cuda.synchronize()
+        y_ref, sT_ref = oracle.forward_c(*ref, N, s_ref[0], smap)
+        check_close("y", y, y_ref, torch.bfloat16)
+        check_close("sT", sT, sT_ref, torch.bfloat16)
+
+
+def test_chunk_many_pairs_fall_back_pair_by_pair(op, oracle):
+    # pairs 1 and 300 of 320 leave the representable range: each is redone exactly, whichever
+    # position it has in its workgroup's list, and the others keep their MFMA results
+    B, T, H, N = 80, 128, 4, 64
+    ins = oracle.make_inputs(B, T, H, N, 56)
+    ins[3][0, 40:60, 70:90] = 6.0        # pair (0, 1)
+    ins[3][75, 100:120, 10:20] = 6.0     # pair (75, 0) = 300
+    dev, ref = cast_inputs(ins[:5], torch.bfloat16)
+    gy_dev, gy_ref = cast_inputs(ins[5:6], torch.bfloat16)
+    y, grads = _run_fwd_bwd(op, dev + gy_dev, CHUNK)
+    check_close("y", y, oracle.forward_c(*ref, N)[0], torch.bfloat16)
+    for name, g, gr in zip("gr gk gv gw gu".split(), grads, oracle.backward_c(*ref, gy_ref[0], N)):
+        check_close(name, to_np(g).reshape(gr.shape), gr, torch.bfloat16, is_grad=True)
+
+
 def test_chunk_matches_scan_on_padding_mask(op, oracle):
     B, T, H, N = 1, 96, 1, 64
     ins = oracle.make_inputs(B, T, H, N, 54)
