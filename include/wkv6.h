@@ -85,6 +85,22 @@ int wkv6_forward_with_state_ex(void *stream, int dtype, int state_dtype, int alg
                                void *workspace, size_t workspace_bytes);
 size_t wkv6_forward_workspace_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H);
 
+/* Forward (inference) with the layer's output stage fused in; y itself is not written:
+ *     out[b,t,h,:] = (layer_norm(y[b,t,h,:], gn_eps) * gn_scale[h,:] + gn_offset[h,:]) * gate[b,t,h,:]
+ * i.e. what the caller of the operator does next in the reference model: the per-head group
+ * normalisation with learned scale and offset and the gate, rwkv6_model.py:94-99 (GroupNorm.call,
+ * mean and variance over one head's channels) and :158-160 (TimeMix.call: x = group_norm(x) * g).
+ * No counterpart in the reference's native code, which leaves these to framework kernels (one more
+ * write and two more reads of a (B,T,C) tensor per layer).  bf16 tensors only (WKV6_ERR_UNSUPPORTED
+ * otherwise); gn_scale, gn_offset: (H, 64) fp32 in device memory; gate, out: (B,T,C) in `dtype`;
+ * state arguments as in wkv6_forward_with_state_ex (ys may be NULL).  No gradient. */
+int wkv6_forward_gn_gate(void *stream, int dtype, int state_dtype,
+                         int64_t B, int64_t T, int64_t C, int64_t H,
+                         int has_init_state, const int64_t *state_map,
+                         const void *r, const void *k, const void *v, const void *w, const void *u,
+                         const void *s, const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
+                         void *out, void *ys);
+
 /* Backward of the stateless forward: gr,gk,gv,gw (B,T,C) and gu (B,C), all in the output type.
  * Replaces backward_{bf16,fp16,fp32}(B,T,C,H,r,k,v,w,u,gy,gr,gk,gv,gw,gu),
  * rwkv_kernel/torch_kernel/wkv6_op.cpp:33-41 (kernel_backward_101/102/103/201,

@@ -186,6 +186,22 @@ def closed_form_np(r, k, v, w, u, head_size, init_state=None):
     return y
 
 
+def group_norm_gate_np(y, gate, scale, offset, head_size, epsilon=64e-5):
+    """What the caller does with the operator's output in the reference model, in float64:
+    per-head layer norm of y with scale and offset (rwkv6_model.py:94-99: mean and variance over
+    one head's channels, 1/sqrt(var + epsilon)), then the gate (rwkv6_model.py:158-160)."""
+    y = np.asarray(y, dtype=np.float64)
+    B, T, C = y.shape
+    N = head_size
+    H = C // N
+    x = y.reshape(B, T, H, N)
+    mu = x.mean(-1, keepdims=True)
+    var = ((x - mu) ** 2).mean(-1, keepdims=True)
+    x = (x - mu) / np.sqrt(var + epsilon)
+    x = x * np.asarray(scale, dtype=np.float64).reshape(1, 1, H, N) + np.asarray(offset, dtype=np.float64).reshape(1, 1, H, N)
+    return x.reshape(B, T, C) * np.asarray(gate, dtype=np.float64)
+
+
 def make_inputs(B, T, H, N, seed, with_gy=True, with_state=False):
     """The benchmark's seeded distributions, drawn on the CPU in float32:
     r,k,v ~ N(0,1); w = x ~ U(-6,1) passed raw; u ~ N(0,0.5^2) (H,N); gy ~ N(0,1);

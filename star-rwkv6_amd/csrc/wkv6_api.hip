@@ -89,6 +89,25 @@ int wkv6_forward_with_state_ex(void *stream, int dtype, int state_dtype, int alg
                         nullptr);
 }
 
+int wkv6_forward_gn_gate(void *stream, int dtype, int state_dtype,
+                         int64_t B, int64_t T, int64_t C, int64_t H,
+                         int has_init_state, const int64_t *state_map,
+                         const void *r, const void *k, const void *v, const void *w, const void *u,
+                         const void *s, const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
+                         void *out, void *ys) {
+    int rc = check_shape(dtype, B, T, C, H);
+    if (rc != WKV6_OK) return rc;
+    if (!r || !k || !v || !w || !u || !gate || !gn_scale || !gn_offset || !out) return WKV6_ERR_ARG;
+    if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(gate) || !aligned16(out)) return WKV6_ERR_ARG;
+    if (has_init_state && !s) return WKV6_ERR_ARG;
+    if (!(gn_eps >= 0.f)) return WKV6_ERR_ARG;
+    if (state_dtype != out_type(dtype) && state_dtype != WKV6_F32) return WKV6_ERR_ARG;
+    if (!chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;   // bf16 tensors only
+    return finish(wkv6::chunk_forward_fused((hipStream_t)stream, state_dtype, B, T, H, r, k, v, w, u,
+                                            has_init_state ? s : nullptr, has_init_state ? state_map : nullptr,
+                                            gate, gn_scale, gn_offset, gn_eps, out, ys));
+}
+
 size_t wkv6_saved_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
     if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
     const bool chunk = (algo == WKV6_ALGO_CHUNK && chunk_possible(dtype, T, C)) ||

@@ -44,7 +44,19 @@ struct FwdLds {
     static constexpr int kOpRt = 0, kOpKt = kTileBytes, kOpG = 2 * kTileBytes, kOpRuk = kOpG + 4 * kN * 4;
     static constexpr int kOpBytes = kOpRuk + CL * 4;
     static constexpr int kBytes = kOp + 2 * kOpBytes;
+    // only with the fused output stage (group norm and gate):
+    static constexpr int kYStage = kBytes;                              // [2 visit parities] y of one chunk, bf16
+    static constexpr int kRawG = kYStage + 2 * kTileBytes;              // [4] raw gate tiles (visit & 3)
+    static constexpr int kBytesFused = kRawG + 4 * kTileBytes;
 };
+
+// With the fused output stage y does not go to global memory: the consumers leave each chunk in LDS
+// as [token][64 channels] rows of 128 bytes, and a producer wave reads whole rows (lane = channel)
+// one visit later.  The 32-byte slot of a consumer wave's 16 channels is XORed with bits 2..3 of the
+// token, so that the four token rows one accumulator store touches fall into different banks.
+__device__ __forceinline__ uint32_t ystage_off(int t, int ch) {
+    return ((uint32_t)t << 7) + (((((uint32_t)ch >> 4) ^ ((uint32_t)t >> 2)) & 3u) << 5) + (((uint32_t)ch & 15u) << 1);
+}
 
 // development aid (-DWKV6_TIMING): cycle stamps of workgroup 0, 256 slots per wave, behind the workspace
 #ifdef WKV6_TIMING
@@ -77,13 +89,18 @@ struct FwdArgs {
     void *sT;
     float *ckpt;
     int *arrivals;   // with ckpt: per-head counters the backward's fused gu sum starts from zero
+    // fused output stage: out = (group_norm_head(y) * gn_scale + gn_offset) * gate, y itself is not written
+    const bf16_t *gate;
+    const float *gn_scale, *gn_offset;   // (H, 64)
+    float gn_eps;
+    bf16_t *out;
 };
 
 // ------------------------------------------------------------------------------------------
 // Consumer group GRP of two: both groups carry the state through every tile (4 MFMAs and a
 // scaling), group 0 produces y for tiles 0 and 2, group 1 for tiles 1 and 3.
 // ------------------------------------------------------------------------------------------
-template <typename Ts, bool kSave, bool kRagged, bool kMulti, int NG, int GRP>
+template <typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse, int NG, int GRP>
 __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned char *smem, int q, int lane)
 {
     const int T = a.T, H = a.H;
@@ -178,10 +195,20 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
                     chain_gap(Y);
                     Y = mfma16(make_s16x4(pack_bf16x2(AT[0], AT[1]), pack_bf16x2(AT[2], AT[3])), vf, Y);
                     settle(Y);
+                    if (kFuse) {
+                        unsigned char *ys = const_cast<unsigned char *>(smem) + FwdLds::kYStage + (it & 1) * kTileBytes;
+                        const uint32_t y01 = pack_bf16x2(Y[0], Y[1]), y23 = pack_bf16x2(Y[2], Y[3]);
+                        const int tk = 16 * p + 4 * g, chn = 16 * q + l16;
+                        *reinterpret_cast<uint16_t *>(ys + ystage_off(tk, chn)) = (uint16_t)y01;
+                        *reinterpret_cast<uint16_t *>(ys + ystage_off(tk + 1, chn)) = (uint16_t)(y01 >> 16);
+                        *reinterpret_cast<uint16_t *>(ys + ystage_off(tk + 2, chn)) = (uint16_t)y23;
+                        *reinterpret_cast<uint16_t *>(ys + ystage_off(tk + 3, chn)) = (uint16_t)(y23 >> 16);
+                    } else {
 #pragma unroll
-                    for (int rr = 0; rr < 4; ++rr) {
-                        const int t = t0 + 16 * p + 4 * g + rr;
-                        if (!kRagged || t < T) st16(y_h, (uint32_t)t * (uint32_t)C * 2u + 2u * (uint32_t)(16 * q + l16), Y[rr]);
+                        for (int rr = 0; rr < 4; ++rr) {
+                            const int t = t0 + 16 * p + 4 * g + rr;
+                            if (!kRagged || t < T) st16(y_h, (uint32_t)t * (uint32_t)C * 2u + 2u * (uint32_t)(16 * q + l16), Y[rr]);
+                        }
                     }
                 }
                 // S <- diag(g) (S + U)
@@ -204,6 +231,7 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
                 for (int rr = 0; rr < 4; ++rr) store1(p + (16 * m + 4 * g + rr) * kN, S[m][rr]);
         }
     }
+    if (kFuse) __syncthreads();   // the producers finish the last visit's output behind this one
 }
 
 // ------------------------------------------------------------------------------------------
@@ -211,7 +239,7 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
 // wave 2p+hf <-> tokens 8hf..8hf+7 of tile p; the second-half wave redoes the first half's exp(w)
 // to get its starting decay.
 // ------------------------------------------------------------------------------------------
-template <bool kRagged, bool kMulti, int kHalves>
+template <bool kRagged, bool kMulti, bool kFuse, int kHalves>
 __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *smem, int *s_wild, int pw, int lane)
 {
     constexpr int NT = 16 / kHalves;   // tokens per wave and chunk
@@ -231,11 +259,12 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
     // The load stream and the preparation stream each walk the visits in order; `ld_*` / `pp_*` are
     // the (pair, chunk) the next load / preparation belongs to.
     int ld_c = 0, ld_bh = (int)blockIdx.x;
-    const bf16_t *rb, *kb_, *vb, *wb;   // uniform: this pair's first row
+    const bf16_t *rb, *kb_, *vb, *wb, *gb = nullptr;   // uniform: this pair's first row (gb: gate, fused output stage)
     auto point_loads = [&]() {
         const int b = ld_bh / H, h = ld_bh - b * H;
         const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
         rb = a.r + base; kb_ = a.k + base; vb = a.v + base; wb = a.w + base;
+        if (kFuse) gb = a.gate + base;
     };
     point_loads();
     // Rows past the end of the sequence are fetched from row T-1 (valid memory); the operand
@@ -243,7 +272,8 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
     // operands.  Each wave loads what it reads itself (with kHalves = 2 the second-half wave also
     // the first half's w rows), so its own vmcnt covers its inputs; v is picked up by the consumers
     // a barrier later.
-    constexpr int kLoads = kHalves == 2 ? 5 : 8;   // per chunk and wave
+    static_assert(!kFuse || kHalves == 1, "the fused output stage is written for one producer wave per tile");
+    constexpr int kLoads = (kHalves == 2 ? 5 : 8) + (kFuse ? 2 : 0);   // per chunk and wave
     auto issue_loads = [&](int it) {   // visit `it` = the load stream's current (pair, chunk)
         const int tb = ld_c * CL + 16 * p;
         const uint32_t rkw = lds0 + FwdLds::kRawRKW + (it & 1) * 3 * kTileBytes + 16 * p * kTileRow;
@@ -262,15 +292,55 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
             load_rows8_to_lds(rb, o, rkw + 8 * blk * kTileRow);
             load_rows8_to_lds(kb_, o, rkw + kTileBytes + 8 * blk * kTileRow);
             load_rows8_to_lds(vb, o, vv + 8 * blk * kTileRow);
+            if (kFuse) load_rows8_to_lds(gb, o, lds0 + FwdLds::kRawG + (it & 3) * kTileBytes + (16 * p + 8 * blk) * kTileRow);
         }
         if (++ld_c == nchunk && kMulti) { ld_c = 0; ld_bh += stride; if (ld_bh < a.nitems) point_loads(); }
     };
-    int pp_c = 0, pp_n = 0, pp_h = (int)blockIdx.x % H;
-    float uc = load1(a.u + pp_h * kN + ch);
     // per-lane byte offsets of channel `ch` inside a tile row, for the 8 swizzle phases
     uint32_t choff[8];
 #pragma unroll
     for (int s = 0; s < 8; ++s) choff[s] = (uint32_t)((((ch >> 3) ^ s) << 4) + ((ch & 7) << 1)) + (uint32_t)(16 * p * kTileRow);
+    // Fused output stage for the chunk the consumers staged during the previous visit; wave p takes
+    // tile p, lane = channel:  out = ((y - mean) * rstd * gn_scale + gn_offset) * gate, mean and
+    // variance over the head's 64 channels of a token (two passes, like a layer norm).
+    int fl_c = 0, fl_bh = (int)blockIdx.x;
+    bf16_t *ob = nullptr;
+    float gsc = 0.f, gof = 0.f;
+    auto point_output = [&]() {
+        const int b = fl_bh / H, h = fl_bh - b * H;
+        ob = a.out + (int64_t)b * T * C + (int64_t)h * kN;
+        gsc = a.gn_scale[h * kN + ch];
+        gof = a.gn_offset[h * kN + ch];
+    };
+    if (kFuse) point_output();
+    auto output_stage = [&](int it) {   // visit `it` = the output stream's current (pair, chunk)
+        const unsigned char *ys = smem + FwdLds::kYStage + (it & 1) * kTileBytes;
+        const unsigned char *gt = smem + FwdLds::kRawG + (it & 3) * kTileBytes;
+        float yv[16], dv[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            yv[e] = bf16_bits_to_float(*reinterpret_cast<const uint16_t *>(ys + ystage_off(16 * p + e, ch)));
+        // lane l of the reduction holds the total of token (l >> 2) & 15
+        const float mu_own = transpose_reduce16(yv, lane) * (1.f / kN);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const float mu = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(mu_own), 4 * e));
+            yv[e] -= mu;
+            dv[e] = yv[e] * yv[e];
+        }
+        const float rstd_own = __builtin_amdgcn_rsqf(transpose_reduce16(dv, lane) * (1.f / kN) + a.gn_eps);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+            const float rstd = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(rstd_own), 4 * e));
+            const float gate = bf16_bits_to_float(*reinterpret_cast<const uint16_t *>(gt + choff[e & 7] + e * kTileRow));
+            const int t = fl_c * CL + 16 * p + e;
+            const float o = fmaf(yv[e] * rstd, gsc, gof) * gate;
+            if (!kRagged || t < T) st16(ob, (uint32_t)t * rowbytes + 2u * (uint32_t)ch, o);
+        }
+        if (++fl_c == nchunk && kMulti) { fl_c = 0; fl_bh += stride; if (fl_bh < a.nitems) point_output(); }
+    };
+    int pp_c = 0, pp_n = 0, pp_h = (int)blockIdx.x % H;
+    float uc = load1(a.u + pp_h * kN + ch);
     const float kLog2Log2e = 0.5287663729448977f;   // log2(log2(e)): exp(w) log2(e) = 2^(w log2(e) + this)
     auto prepare = [&](int it) {   // visit `it` = the preparation stream's current (pair, chunk)
         const unsigned char *raw = smem + FwdLds::kRawRKW + (it & 1) * 3 * kTileBytes;
@@ -351,26 +421,60 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
         __syncthreads();
         WKV6_FSTAMP();
         // the raw r, k, w block of visit `it` (read by this wave's prepare(it) before the barrier) and the
-        // raw v block of visit it-1 (read by the consumers before the barrier) are free again
+        // raw v block of visit it-1 (read by the consumers before the barrier) are free again.
+        // The output stage's 16 stores go out behind the loads and are not waited for: a wave's
+        // memory operations complete in program order, and the loads waited for below are older
+        // than both.  (With a ragged end the number of store instructions issued is not fixed;
+        // they go first then and are waited for with the loads.)
+        const bool outputs = kFuse && it > 0;
+        if (outputs && kRagged) output_stage(it - 1);
         if (it + 2 < nvisit) issue_loads(it + 2);
+        if (outputs && !kRagged) output_stage(it - 1);
         WKV6_FSTAMP();
         if (it + 1 < nvisit) {
-            if (it + 2 < nvisit) wait_loads<kLoads>(); else wait_loads<0>();
+            const bool stores_behind = outputs && !kRagged;
+            if (it + 2 < nvisit) { if (stores_behind) wait_loads<kLoads + 16>(); else wait_loads<kLoads>(); }
+            else { if (stores_behind) wait_loads<16>(); else wait_loads<0>(); }
             WKV6_FSTAMP();
             prepare(it + 1);
             WKV6_FSTAMP();
         }
     }
+    if (kFuse) {
+        __syncthreads();
+        output_stage(nvisit - 1);
+    }
     wait_loads<0>();
 }
 
-// kSave: also write the state at every chunk start to `ckpt` (bf16, [b][h][chunk][j][i]) for the
-// backward pass, which then skips its own forward sweep.  kRagged: T is not a multiple of 64.
 // kMulti: more (batch, head) pairs than workgroups -- each workgroup takes every gridDim.x-th pair and
 // runs them back to back through one pipeline, so the loads of a pair's first chunks overlap the
 // previous pair's last ones (a workgroup fills the CU's LDS, so nothing else would hide them).
 constexpr int kMaxPairsPerWorkgroup = 32;
-template <typename Ts, bool kSave, bool kRagged, bool kMulti>
+// The exact second pass leaves y in `out`; this turns one pair's rows into the fused output in place
+// (a wave per token, lane = channel).
+__device__ __forceinline__ void output_stage_in_place(const FwdArgs &a, int bh) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwave = blockDim.x >> 6;
+    const int b = bh / a.H, h = bh - b * a.H;
+    const int64_t C = (int64_t)a.H * kN;
+    bf16_t *rowp = a.out + (int64_t)b * a.T * C + (int64_t)h * kN + lane;
+    const bf16_t *gp = a.gate + (int64_t)b * a.T * C + (int64_t)h * kN + lane;
+    const float gsc = a.gn_scale[h * kN + lane], gof = a.gn_offset[h * kN + lane];
+    for (int t = wave; t < a.T; t += nwave) {
+        const float y = load1(rowp + (int64_t)t * C);
+        float sum = y;
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) sum += __shfl_xor(sum, m);
+        const float d = y - sum * (1.f / kN);
+        float sq = d * d;
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) sq += __shfl_xor(sq, m);
+        const float rstd = __builtin_amdgcn_rsqf(sq * (1.f / kN) + a.gn_eps);
+        store1(rowp + (int64_t)t * C, fmaf(d * rstd, gsc, gof) * load1(gp + (int64_t)t * C));
+    }
+}
+
+template <typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse>
 __global__ __launch_bounds__(kFwdThreads) void chunk_fwd_kernel(FwdArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -382,9 +486,9 @@ __global__ __launch_bounds__(kFwdThreads) void chunk_fwd_kernel(FwdArgs a)
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int role = wave >> 2, q = wave & 3;
-    if (role < kFwdHalves) fwd_producer<kRagged, kMulti, kFwdHalves>(a, smem, s_wild, wave, lane);
-    else if (kFwdGroups == 1 || role == kFwdHalves) fwd_consumer<Ts, kSave, kRagged, kMulti, kFwdGroups, 0>(a, smem, q, lane);
-    else fwd_consumer<Ts, kSave, kRagged, kMulti, kFwdGroups, 1>(a, smem, q, lane);
+    if (role < kFwdHalves) fwd_producer<kRagged, kMulti, kFuse, kFwdHalves>(a, smem, s_wild, wave, lane);
+    else if (kFwdGroups == 1 || role == kFwdHalves) fwd_consumer<Ts, kSave, kRagged, kMulti, kFuse, kFwdGroups, 0>(a, smem, q, lane);
+    else fwd_consumer<Ts, kSave, kRagged, kMulti, kFuse, kFwdGroups, 1>(a, smem, q, lane);
     // exact second pass for every pair of this workgroup that had a tile leave the representable range
     __threadfence_block();   // workgroup scope is enough (and a device-scope fence would write back the L2)
     __syncthreads();
@@ -395,7 +499,12 @@ __global__ __launch_bounds__(kFwdThreads) void chunk_fwd_kernel(FwdArgs a)
         const int bh = (int)blockIdx.x + n * stride;
         __syncthreads();
         scan_fwd_body<bf16_t, bf16_t, Ts>(*reinterpret_cast<ScanFwdLds *>(smem), bh / a.H, bh % a.H, a.T, a.H, a.r, a.k, a.v, a.w, a.u,
-                                          reinterpret_cast<const Ts *>(a.s0), a.map, a.y, reinterpret_cast<Ts *>(a.sT));
+                                          reinterpret_cast<const Ts *>(a.s0), a.map, kFuse ? a.out : a.y, reinterpret_cast<Ts *>(a.sT));
+        if (kFuse) {
+            __threadfence_block();
+            __syncthreads();
+            output_stage_in_place(a, bh);
+        }
     }
 }
 
@@ -412,43 +521,69 @@ static int compute_units() {
     return cached[dev];
 }
 
-template <typename Ts, bool kSave, bool kRagged, bool kMulti>
+template <typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse>
 static hipError_t launch_fwd(hipStream_t st, const FwdArgs &a, unsigned grid) {
-    auto kern = chunk_fwd_kernel<Ts, kSave, kRagged, kMulti>;
-    const size_t lds = FwdLds::kBytes;
+    auto kern = chunk_fwd_kernel<Ts, kSave, kRagged, kMulti, kFuse>;
+    const size_t lds = kFuse ? FwdLds::kBytesFused : FwdLds::kBytes;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kFwdThreads), lds, st, a);
     return hipGetLastError();
 }
-template <typename Ts, bool kSave, bool kRagged>
+template <typename Ts, bool kSave, bool kRagged, bool kFuse>
 static hipError_t launch_fwd(hipStream_t st, const FwdArgs &a, bool multi, unsigned grid) {
-    return multi ? launch_fwd<Ts, kSave, kRagged, true>(st, a, grid) : launch_fwd<Ts, kSave, kRagged, false>(st, a, grid);
+    return multi ? launch_fwd<Ts, kSave, kRagged, true, kFuse>(st, a, grid) : launch_fwd<Ts, kSave, kRagged, false, kFuse>(st, a, grid);
 }
 template <typename Ts>
 static hipError_t launch_fwd(hipStream_t st, const FwdArgs &a, bool save, bool ragged, bool multi, unsigned grid) {
-    if (save) return ragged ? launch_fwd<Ts, true, true>(st, a, multi, grid) : launch_fwd<Ts, true, false>(st, a, multi, grid);
-    return ragged ? launch_fwd<Ts, false, true>(st, a, multi, grid) : launch_fwd<Ts, false, false>(st, a, multi, grid);
+    if (save) return ragged ? launch_fwd<Ts, true, true, false>(st, a, multi, grid) : launch_fwd<Ts, true, false, false>(st, a, multi, grid);
+    return ragged ? launch_fwd<Ts, false, true, false>(st, a, multi, grid) : launch_fwd<Ts, false, false, false>(st, a, multi, grid);
+}
+template <typename Ts>
+static hipError_t launch_fwd_fused(hipStream_t st, const FwdArgs &a, bool ragged, bool multi, unsigned grid) {
+    return ragged ? launch_fwd<Ts, false, true, true>(st, a, multi, grid) : launch_fwd<Ts, false, false, true>(st, a, multi, grid);
+}
+
+// One workgroup per pair while they all fit on the chip at once; beyond that one workgroup per
+// compute unit (more only if a workgroup would otherwise get more pairs than it keeps flags for).
+static unsigned forward_grid(int64_t pairs, bool *multi) {
+    const int64_t cus = compute_units();
+    *multi = pairs > cus;
+    return (unsigned)(!*multi ? pairs : (pairs + cus * kMaxPairsPerWorkgroup - 1) / (cus * kMaxPairsPerWorkgroup) * cus);
 }
 
 hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u,
                          const void *s0, const int64_t *map, void *y, void *sT, void *saved_states)
 {
-    FwdArgs a;
+    FwdArgs a = {};
     a.T = (int)T; a.H = (int)H; a.nitems = (int)(B * H);
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
     a.s0 = s0; a.map = map; a.y = (bf16_t *)y; a.sT = sT; a.ckpt = (float *)saved_states;
     a.arrivals = saved_states ? reinterpret_cast<int *>(reinterpret_cast<char *>(saved_states) + chunk_backward_workspace_bytes(B, T, H)) : nullptr;
     a.dbg = saved_states ? reinterpret_cast<long long *>((float *)saved_states + (size_t)(B * H) * ((T + CL - 1) / CL) * kN * kN + 1024) : nullptr;
-    // One workgroup per pair while they all fit on the chip at once; beyond that one workgroup per
-    // compute unit (more only if a workgroup would otherwise get more pairs than it keeps flags for).
-    const int64_t pairs = B * H, cus = compute_units();
-    const bool multi = pairs > cus;
-    const int64_t grid = !multi ? pairs : (pairs + cus * kMaxPairsPerWorkgroup - 1) / (cus * kMaxPairsPerWorkgroup) * cus;
+    bool multi;
+    const unsigned grid = forward_grid(B * H, &multi);
     const bool save = saved_states != nullptr, ragged = (T % CL) != 0;
-    return state_dtype == kF32 ? launch_fwd<float>(st, a, save, ragged, multi, (unsigned)grid)
-                               : launch_fwd<bf16_t>(st, a, save, ragged, multi, (unsigned)grid);
+    return state_dtype == kF32 ? launch_fwd<float>(st, a, save, ragged, multi, grid)
+                               : launch_fwd<bf16_t>(st, a, save, ragged, multi, grid);
+}
+
+hipError_t chunk_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
+                               const void *r, const void *k, const void *v, const void *w, const void *u,
+                               const void *s0, const int64_t *map, const void *gate, const float *gn_scale,
+                               const float *gn_offset, float gn_eps, void *out, void *sT)
+{
+    FwdArgs a = {};
+    a.T = (int)T; a.H = (int)H; a.nitems = (int)(B * H);
+    a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
+    a.s0 = s0; a.map = map; a.sT = sT;
+    a.gate = (const bf16_t *)gate; a.gn_scale = gn_scale; a.gn_offset = gn_offset; a.gn_eps = gn_eps; a.out = (bf16_t *)out;
+    bool multi;
+    const unsigned grid = forward_grid(B * H, &multi);
+    const bool ragged = (T % CL) != 0;
+    return state_dtype == kF32 ? launch_fwd_fused<float>(st, a, ragged, multi, grid)
+                               : launch_fwd_fused<bf16_t>(st, a, ragged, multi, grid);
 }
 
 }  // namespace wkv6

@@ -22,6 +22,12 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
                          const void *r, const void *k, const void *v, const void *w, const void *u,
                          const void *s0, const int64_t *map, void *y, void *sT, void *saved_states);
 
+// forward with the layer's output stage fused in: out = (group_norm_head(y) * gn_scale + gn_offset) * gate
+hipError_t chunk_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
+                               const void *r, const void *k, const void *v, const void *w, const void *u,
+                               const void *s0, const int64_t *map, const void *gate, const float *gn_scale,
+                               const float *gn_offset, float gn_eps, void *out, void *sT);
+
 size_t chunk_backward_workspace_bytes(int64_t B, int64_t T, int64_t H);
 // bytes of a forward -> backward hand-over buffer: the workspace plus one arrival counter per head
 // (zeroed by the saving forward, used by the backward's fused batch sum of gu)

@@ -134,7 +134,8 @@ class RWKVKernelOperator:
         self.normal_kernenl = _WKV6
         self.kernel_with_state = _forward_with_state
 
-    def __call__(self, r, k, v, w, u, return_state=False, init_state=None, state_map=None):
+    def _check(self, r, k, v, w, u, init_state, state_map):
+        """Argument checks shared by every entry; returns (B, T, C, H, N, u, init_state, state_map)."""
         B, T, C = r.shape
         N = self.head_size
         assert C % N == 0
@@ -167,28 +168,64 @@ class RWKVKernelOperator:
                 assert state_map.dtype in (torch.int32, torch.int64), "state_map must be int32/int64 of shape (batch,)"
                 state_map = state_map.to(torch.int64)
             assert tuple(state_map.shape) == (B,), "state_map must have shape (batch,)"
+        return B, T, C, H, N, u, init_state, state_map
 
+    def _resolve_state(self, B, r, init_state, state_map):
+        """Default / validated state_map on the device (None = identity), contiguous init_state."""
+        if init_state is None:
+            assert state_map is None, "state_map needs init_state"
+            return None, None
+        n_state = init_state.shape[0]
+        if state_map is None:
+            assert n_state == 1 or n_state == B, "cannot infer state_map; pass it explicitly"
+            if n_state == 1 and B > 1:
+                key = (B, r.device)
+                if key not in self._zero_maps:
+                    self._zero_maps[key] = torch.zeros(B, dtype=torch.int64, device=r.device)
+                state_map = self._zero_maps[key]
+            # n_state == B: identity, expressed as "no map" so that a decode loop pays
+            # neither a host-to-device copy nor a range check per step
+        else:
+            assert bool((state_map >= 0).all()) and bool((state_map < n_state).all()), \
+                "state_map values must lie in [0, %d)" % n_state
+            state_map = state_map.to(r.device).contiguous()
+        return init_state.contiguous(), state_map
+
+    def __call__(self, r, k, v, w, u, return_state=False, init_state=None, state_map=None):
+        B, T, C, H, N, u, init_state, state_map = self._check(r, k, v, w, u, init_state, state_map)
         if return_state:
-            if init_state is None:
-                assert state_map is None, "state_map needs init_state"
-            else:
-                n_state = init_state.shape[0]
-                if state_map is None:
-                    assert n_state == 1 or n_state == B, "cannot infer state_map; pass it explicitly"
-                    if n_state == 1 and B > 1:
-                        key = (B, r.device)
-                        if key not in self._zero_maps:
-                            self._zero_maps[key] = torch.zeros(B, dtype=torch.int64, device=r.device)
-                        state_map = self._zero_maps[key]
-                    # n_state == B: identity, expressed as "no map" so that a decode loop pays
-                    # neither a host-to-device copy nor a range check per step
-                else:
-                    assert bool((state_map >= 0).all()) and bool((state_map < n_state).all()), \
-                        "state_map values must lie in [0, %d)" % n_state
-                    state_map = state_map.to(r.device).contiguous()
-                init_state = init_state.contiguous()
+            init_state, state_map = self._resolve_state(B, r, init_state, state_map)
             for x in (r, k, v, w, u):
                 assert x.is_contiguous()
             return _forward_with_state(B, T, C, H, state_map, r, k, v, w, u, init_state, self.algo)
         o = _WKV6.apply(B, T, C, H, r, k, v, w, u, self.algo)
         return o, None
+
+    def forward_gn_gate(self, r, k, v, w, u, gate, gn_scale, gn_offset, epsilon=64e-5,
+                        return_state=False, init_state=None, state_map=None):
+        """Inference forward with the layer's next two steps fused into the kernel's output stage:
+        returns ``(group_norm(y) * gate, state)`` where group_norm is the per-head layer norm with
+        scale and offset of rwkv6_model.py:94-99 and ``* gate`` is rwkv6_model.py:158-160; y itself is
+        never written.  bf16 tensors; gn_scale / gn_offset hold one value per channel.  No gradient.
+        Not part of the reference's operator."""
+        B, T, C, H, N, u, init_state, state_map = self._check(r, k, v, w, u, init_state, state_map)
+        assert r.dtype == torch.bfloat16, "the fused output stage takes bf16 tensors"
+        assert gate.shape == r.shape and gate.dtype == r.dtype and gate.device == r.device
+        assert gn_scale.numel() == C and gn_offset.numel() == C
+        init_state, state_map = self._resolve_state(B, r, init_state, state_map)
+        for x in (r, k, v, w, u, gate):
+            assert x.is_contiguous()
+        lib = _native.load()
+        with torch.no_grad():
+            sc = gn_scale.detach().to(device=r.device, dtype=torch.float32).contiguous()
+            of = gn_offset.detach().to(device=r.device, dtype=torch.float32).contiguous()
+            sdt = init_state.dtype if init_state is not None else torch.float32
+            out = torch.empty_like(r)
+            ys = torch.empty((B, H, N, N), device=r.device, dtype=sdt) if return_state else None
+            with torch.cuda.device(r.device):
+                _native.check(lib.wkv6_forward_gn_gate(
+                    _stream(), _DTYPE_CODE[r.dtype], _DTYPE_CODE[sdt], B, T, C, H,
+                    int(init_state is not None), _ptr(state_map),
+                    _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(init_state), _ptr(gate), _ptr(sc), _ptr(of),
+                    float(epsilon), _ptr(out), _ptr(ys)))
+        return out, ys

@@ -316,6 +316,47 @@ def test_chunk_many_pairs_fall_back_pair_by_pair(op, oracle):
         check_close(name, to_np(g).reshape(gr.shape), gr, torch.bfloat16, is_grad=True)
 
 
+# Fused output stage (inference): out = group_norm(y) * gate straight from the kernel, y never stored.
+# Checked against the oracle's y (float64, fed the bf16-rounded inputs) pushed through the float64
+# restatement of the model's group norm and gate.  Tolerance: the bf16 one of the operator,
+# relative to the largest reference value (the kernel normalises the bf16-rounded y, as a caller
+# would).
+@pytest.mark.parametrize("B,T,H,with_state", [(2, 64, 2, False), (3, 150, 2, True), (1, 1000, 3, False),
+                                              (70, 96, 4, True), (1, 16, 1, False)])
+def test_fused_group_norm_gate(op, oracle, B, T, H, with_state):
+    N = 64
+    ins = oracle.make_inputs(B, T, H, N, 70 + T, with_state=True)
+    dev, ref = cast_inputs(ins[:5], torch.bfloat16)
+    g = torch.Generator().manual_seed(T)
+    gate = torch.randn(B, T, H * N, generator=g)
+    gate_dev, gate_ref = cast_inputs([gate], torch.bfloat16)
+    scale = torch.rand(H, N, generator=g) + 0.5
+    offset = torch.randn(H, N, generator=g) * 0.3
+    s0 = ins[6].float() if with_state else None
+    out, sT = op.forward_gn_gate(*dev, gate_dev[0], scale.cuda(), offset.cuda(), 64e-5, return_state=True,
+                                 init_state=s0.cuda() if with_state else None)
+    torch.cuda.synchronize()
+    y_ref, sT_ref = oracle.forward_c(*ref, N, to_np(s0) if with_state else None)
+    want = oracle.group_norm_gate_np(y_ref, gate_ref[0], scale.numpy(), offset.numpy(), N, 64e-5)
+    check_close("out", out, want, torch.bfloat16)
+    check_close("sT", sT, sT_ref, torch.bfloat16)
+
+
+def test_fused_group_norm_gate_on_a_fallback_pair(op, oracle):
+    # a pair that leaves the chunked form's range is redone exactly and then normalised in place
+    B, T, H, N = 2, 128, 2, 64
+    ins = oracle.make_inputs(B, T, H, N, 77)
+    ins[3][1, 40:60, 70:90] = 6.0
+    dev, ref = cast_inputs(ins[:5], torch.bfloat16)
+    g = torch.Generator().manual_seed(5)
+    gate_dev, gate_ref = cast_inputs([torch.randn(B, T, H * N, generator=g)], torch.bfloat16)
+    scale, offset = torch.rand(H, N, generator=g) + 0.5, torch.randn(H, N, generator=g) * 0.3
+    out, _ = op.forward_gn_gate(*dev, gate_dev[0], scale.cuda(), offset.cuda())
+    torch.cuda.synchronize()
+    want = oracle.group_norm_gate_np(oracle.forward_c(*ref, N)[0], gate_ref[0], scale.numpy(), offset.numpy(), N)
+    check_close("out", out, want, torch.bfloat16)
+
+
 def test_chunk_matches_scan_on_padding_mask(op, oracle):
     B, T, H, N = 1, 96, 1, 64
     ins = oracle.make_inputs(B, T, H, N, 54)

@@ -190,3 +190,27 @@ def test_golden_fixture_matches_oracle(oracle):
     np.testing.assert_allclose(y0, z["y"], rtol=1e-12, atol=1e-12)
     for name, a in zip("gr gk gv gw gu".split(), oracle.backward_c(z["r"], z["k"], z["v"], z["w"], z["u"], z["gy"], N)):
         np.testing.assert_allclose(a, z[name], rtol=1e-11, atol=1e-12, err_msg=name)
+
+
+def test_group_norm_gate_is_a_per_head_layer_norm(oracle):
+    # the restated output stage against the library routine it reduces to, and against the gate
+    # being a plain elementwise factor; a wrong axis, a missing epsilon or population/sample
+    # variance mix-up all fail here
+    import torch
+    import torch.nn.functional as F
+
+    g = torch.Generator().manual_seed(7)
+    B, T, H, N = 2, 5, 3, 64
+    y = torch.randn(B, T, H * N, generator=g, dtype=torch.float64) * 3 + 0.7
+    gate = torch.randn(B, T, H * N, generator=g, dtype=torch.float64)
+    scale = torch.randn(H, N, generator=g, dtype=torch.float64)
+    offset = torch.randn(H, N, generator=g, dtype=torch.float64)
+    for eps in (64e-5, 1e-2):
+        ln = F.layer_norm(y.reshape(B, T, H, N), (N,), None, None, eps)
+        want = ((ln * scale + offset).reshape(B, T, H * N) * gate).numpy()
+        got = oracle.group_norm_gate_np(y.numpy(), gate.numpy(), scale.numpy(), offset.numpy(), N, eps)
+        assert np.abs(got - want).max() < 1e-12
+    # tiny variance: epsilon decides the scale (a row of equal values maps to the offset)
+    flat = np.full((1, 1, N), 2.5)
+    out = oracle.group_norm_gate_np(flat, np.ones_like(flat), np.ones((1, N)), np.full((1, N), 0.25), N)
+    assert np.abs(out - 0.25).max() < 1e-12
