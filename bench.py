@@ -122,6 +122,12 @@ def bench_stateful(a):
         return e0.elapsed_time(e1) / reps
 
     pre_ms = timed(lambda: call(pre, Tp, yp, h0, sa), 20)
+    # the same prefill with the layer's group norm and gate fused into the kernel's output stage
+    gate = torch.randn(B, Tp, C, device=dev).to(torch.bfloat16)
+    gn_scale, gn_offset = torch.ones(H, N, device=dev), torch.zeros(H, N, device=dev)
+    fused_ms = timed(lambda: _native.check(lib.wkv6_forward_gn_gate(
+        st, _native.BF16, _native.F32, B, Tp, C, H, 1, None, P(pre[0]), P(pre[1]), P(pre[2]), P(pre[3]), P(u), P(h0),
+        P(gate), P(gn_scale), P(gn_offset), 64e-5, P(yp), P(sa))), 20)
 
     def two_steps():
         call(one, 1, y1, sa, sb); call(one, 1, y1, sb, sa)
@@ -132,6 +138,7 @@ def bench_stateful(a):
         "metric": "WKV6 stateful forward, B64 C2048 H32 bf16 activations, fp32 state", "n_gpus": 1,
         "config": {"workload": "c5: prefill T=512 then T=1 decode steps with carried state"},
         "prefill_Mtokens_per_s": B * Tp / (pre_ms * 1e-3) / 1e6, "prefill_ms": pre_ms,
+        "prefill_with_group_norm_and_gate_ms": fused_ms,
         "decode_steps_per_s": 1.0 / (dec_ms * 1e-3), "decode_us_per_step": dec_ms * 1e3,
         "decode_state_GBps": state_bytes / (dec_ms * 1e-3) / 1e9,
         "decode_frac_of_hbm_peak": state_bytes / (dec_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,

@@ -47,7 +47,8 @@ struct FwdLds {
     // only with the fused output stage (group norm and gate):
     static constexpr int kYStage = kBytes;                              // [2 visit parities] y of one chunk, bf16
     static constexpr int kRawG = kYStage + 2 * kTileBytes;              // [4] raw gate tiles (visit & 3)
-    static constexpr int kBytesFused = kRawG + 4 * kTileBytes;
+    static constexpr int kGnTab = kRawG + 4 * kTileBytes;               // [4][scale, offset][64] floats of the visit's head
+    static constexpr int kBytesFused = kGnTab + 4 * 2 * kN * 4;
 };
 
 // With the fused output stage y does not go to global memory: the consumers leave each chunk in LDS
@@ -258,10 +259,11 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
     const uint32_t lpiece = (uint32_t)(((lane & 7) ^ lrow) << 4);
     // The load stream and the preparation stream each walk the visits in order; `ld_*` / `pp_*` are
     // the (pair, chunk) the next load / preparation belongs to.
-    int ld_c = 0, ld_bh = (int)blockIdx.x;
+    int ld_c = 0, ld_bh = (int)blockIdx.x, ld_h = 0;
     const bf16_t *rb, *kb_, *vb, *wb, *gb = nullptr;   // uniform: this pair's first row (gb: gate, fused output stage)
     auto point_loads = [&]() {
         const int b = ld_bh / H, h = ld_bh - b * H;
+        ld_h = h;
         const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
         rb = a.r + base; kb_ = a.k + base; vb = a.v + base; wb = a.w + base;
         if (kFuse) gb = a.gate + base;
@@ -274,6 +276,7 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
     // a barrier later.
     static_assert(!kFuse || kHalves == 1, "the fused output stage is written for one producer wave per tile");
     constexpr int kLoads = (kHalves == 2 ? 5 : 8) + (kFuse ? 2 : 0);   // per chunk and wave
+    constexpr int kLoads0 = kLoads + (kFuse ? 2 : 0);                  // wave 0 also brings the norm's scale and offset
     auto issue_loads = [&](int it) {   // visit `it` = the load stream's current (pair, chunk)
         const int tb = ld_c * CL + 16 * p;
         const uint32_t rkw = lds0 + FwdLds::kRawRKW + (it & 1) * 3 * kTileBytes + 16 * p * kTileRow;
@@ -294,7 +297,22 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
             load_rows8_to_lds(vb, o, vv + 8 * blk * kTileRow);
             if (kFuse) load_rows8_to_lds(gb, o, lds0 + FwdLds::kRawG + (it & 3) * kTileBytes + (16 * p + 8 * blk) * kTileRow);
         }
+        if (kFuse && pw == 0 && lane < 16) {
+            // scale and offset of this visit's head (64 floats each), read by all four waves' output stage
+            const uint32_t tab = lds0 + FwdLds::kGnTab + (it & 3) * (2 * kN * 4);
+            load_rows8_to_lds(a.gn_scale + ld_h * kN, (uint32_t)lane * 16u, tab);
+            load_rows8_to_lds(a.gn_offset + ld_h * kN, (uint32_t)lane * 16u, tab + kN * 4);
+        }
         if (++ld_c == nchunk && kMulti) { ld_c = 0; ld_bh += stride; if (ld_bh < a.nitems) point_loads(); }
+    };
+    // waits until at most `stores` + this wave's loads of one visit are in flight
+    auto wait_visit_loads = [&](bool next_in_flight, bool stores_behind) {
+        if (next_in_flight) {
+            if (stores_behind) { if (pw == 0) wait_loads<kLoads0 + 16>(); else wait_loads<kLoads + 16>(); }
+            else { if (pw == 0) wait_loads<kLoads0>(); else wait_loads<kLoads>(); }
+        } else {
+            if (stores_behind) wait_loads<16>(); else wait_loads<0>();
+        }
     };
     // per-lane byte offsets of channel `ch` inside a tile row, for the 8 swizzle phases
     uint32_t choff[8];
@@ -305,17 +323,16 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
     // variance over the head's 64 channels of a token (two passes, like a layer norm).
     int fl_c = 0, fl_bh = (int)blockIdx.x;
     bf16_t *ob = nullptr;
-    float gsc = 0.f, gof = 0.f;
     auto point_output = [&]() {
         const int b = fl_bh / H, h = fl_bh - b * H;
         ob = a.out + (int64_t)b * T * C + (int64_t)h * kN;
-        gsc = a.gn_scale[h * kN + ch];
-        gof = a.gn_offset[h * kN + ch];
     };
     if (kFuse) point_output();
     auto output_stage = [&](int it) {   // visit `it` = the output stream's current (pair, chunk)
         const unsigned char *ys = smem + FwdLds::kYStage + (it & 1) * kTileBytes;
         const unsigned char *gt = smem + FwdLds::kRawG + (it & 3) * kTileBytes;
+        const float *tab = reinterpret_cast<const float *>(smem + FwdLds::kGnTab + (it & 3) * (2 * kN * 4));
+        const float gsc = tab[ch], gof = tab[kN + ch];
         float yv[16], dv[16];
 #pragma unroll
         for (int e = 0; e < 16; ++e)
@@ -414,7 +431,8 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
     WKV6_FSTAMP_DECL;
     // visit `it` is loaded during visit it-2 (or the prologue), prepared during visit it-1
     issue_loads(0);
-    if (nvisit > 1) { issue_loads(1); wait_loads<kLoads>(); } else wait_loads<0>();
+    if (nvisit > 1) issue_loads(1);
+    wait_visit_loads(nvisit > 1, false);
     prepare(0);
     for (int it = 0; it < nvisit; ++it) {
         WKV6_FSTAMP();
@@ -432,9 +450,7 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
         if (outputs && !kRagged) output_stage(it - 1);
         WKV6_FSTAMP();
         if (it + 1 < nvisit) {
-            const bool stores_behind = outputs && !kRagged;
-            if (it + 2 < nvisit) { if (stores_behind) wait_loads<kLoads + 16>(); else wait_loads<kLoads>(); }
-            else { if (stores_behind) wait_loads<16>(); else wait_loads<0>(); }
+            wait_visit_loads(it + 2 < nvisit, outputs && !kRagged);
             WKV6_FSTAMP();
             prepare(it + 1);
             WKV6_FSTAMP();

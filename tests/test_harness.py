@@ -108,3 +108,33 @@ def test_model_step_hip_operator_matches_python_loop(dtype):
         denom = float(g_ref[n].abs().max()) + 1e-12
         worst = max(worst, float((g_gpu[n] - g_ref[n]).abs().max()) / denom)
     assert worst <= (2e-3 if dtype is None else 8e-2), worst
+
+
+@pytest.mark.gpu
+def test_inference_forward_uses_the_fused_output_stage():
+    """Without gradients and in bf16 the time-mix layer takes group norm and gate from the
+    operator's own output stage; the logits agree with the unfused bf16 path and with the fp32
+    python-loop model on the CPU."""
+    from rwkv_kernel import RWKVKernelOperator
+    T = 96
+    ref = _toy(OPSKernelOperator(64, T), seed=6)
+    dev = torch.device("cuda:0")
+    gpu = _toy(RWKVKernelOperator(64, T), seed=6).to(dev)
+    gpu.load_state_dict(ref.state_dict())
+    torch.manual_seed(7)
+    ids = torch.randint(0, TOY["vocabulary_size"], (3, T))
+    calls = []
+    op = gpu.blocks[0].time_mix.rwkv_kernel
+    inner = op.forward_gn_gate
+    op.forward_gn_gate = lambda *a, **kw: (calls.append(1), inner(*a, **kw))[1]
+    with torch.no_grad():
+        want = ref(ids).float()
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            fused = gpu(ids.to(dev)).float().cpu()
+    assert len(calls) == TOY["num_layers"]
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        unfused = gpu(ids.to(dev)).float().cpu()   # gradients enabled: the unfused path
+    assert len(calls) == TOY["num_layers"]
+    scale = float(want.abs().max())
+    assert float((fused - want).abs().max()) <= 5e-2 * scale
+    assert float((fused - unfused.detach()).abs().max()) <= 3e-2 * scale
