@@ -153,6 +153,21 @@ int wkv6_backward_saved_sum(void *stream, int dtype, int algo, int64_t B, int64_
                             void *gr, void *gk, void *gv, void *gw, void *gu, void *gu_sum,
                             void *saved, size_t saved_bytes);
 
+/* Backward with gradients through the state (no counterpart in the reference, whose backward is
+ * defined for the stateless call only, rwkv_kernel/torch_rwkv_kernel.py:100-168; it is what carrying
+ * the state across calls, rwkv_kernel/__init__.py:14-38, needs for truncated back-propagation over
+ * pieces of a longer sequence).  Gradient of  sum(y*gy) + sum(S_T*gsT)  for the forward started from
+ * S_0 = s0:  s0, gsT, gs0 are fp32 (B,H,64,64) in [key][value] order; s0 NULL = zero initial state,
+ * gsT NULL = no gradient arrives at the final state, gs0 NULL = dL/dS_0 not wanted.  With a state
+ * the first / last decay do receive a gradient (gw[:,0], gw[:,T-1] are not forced to zero).  All
+ * three NULL gives wkv6_backward_ex.  gu is (B,C) per-batch partials as in wkv6_backward. */
+size_t wkv6_backward_with_state_workspace_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H);
+int wkv6_backward_with_state(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                             const void *r, const void *k, const void *v, const void *w, const void *u,
+                             const float *s0, const void *gy, const float *gsT,
+                             void *gr, void *gk, void *gv, void *gw, void *gu, float *gs0,
+                             void *workspace, size_t workspace_bytes);
+
 /* ---- XLA custom-call surface (replaces the pybind module `gpu_ops`,
  * rwkv_kernel/jax_kernel/gpu_ops.cpp:20-43) ---------------------------------------------- */
 

@@ -72,13 +72,16 @@ int FN(wkv6_oracle_forward)(int64_t B, int64_t T, int64_t H, int64_t N,
     return bad ? -1 : 0;
 }
 
-/* Backward of the stateless forward (S_0 = 0, no gradient into or out of the state).
+/* Backward.  S_0 = s0[b] (or 0 when s0 is NULL), G_T = gsT[b] (or 0): with both NULL this is the
+ * backward of the stateless forward the reference defines (no gradient into or out of the state);
+ * with states it is the gradient of  sum(y*gy) + sum(S_T*gsT)  and gs0 (if not NULL) receives
+ * dL/dS_0 = G_0.  States are (B,H,N,N) in [key][value] order.
  * gu is written as per-batch partials (B,C), as the reference kernels do
  * (rwkv_kernels.cu:249); the batch sum is the caller's. */
-int FN(wkv6_oracle_backward)(int64_t B, int64_t T, int64_t H, int64_t N,
-                             const REAL *r, const REAL *k, const REAL *v, const REAL *w, const REAL *u,
-                             const REAL *gy,
-                             REAL *gr, REAL *gk, REAL *gv, REAL *gw, REAL *gu)
+static int backward_impl(int64_t B, int64_t T, int64_t H, int64_t N,
+                         const REAL *r, const REAL *k, const REAL *v, const REAL *w, const REAL *u,
+                         const REAL *s0, const REAL *gy, const REAL *gsT,
+                         REAL *gr, REAL *gk, REAL *gv, REAL *gw, REAL *gu, REAL *gs0)
 {
     const int64_t C = H * N, NN = N * N;
     int bad = 0;
@@ -90,7 +93,9 @@ int FN(wkv6_oracle_backward)(int64_t B, int64_t T, int64_t H, int64_t N,
         if (!Sall || !G) { bad |= 1; free(Sall); free(G); continue; }
         const REAL *uh = u + h * N;
         /* forward sweep, keeping every state */
-        memset(Sall, 0, (size_t)NN * sizeof(REAL));
+        if (s0) memcpy(Sall, s0 + bh * NN, (size_t)NN * sizeof(REAL));
+        else memset(Sall, 0, (size_t)NN * sizeof(REAL));
+        if (gsT) memcpy(G, gsT + bh * NN, (size_t)NN * sizeof(REAL));
         for (int64_t t = 0; t + 1 < T; ++t) {
             const int64_t o = (b * T + t) * C + h * N;
             const REAL *S = Sall + t * NN;
@@ -126,8 +131,25 @@ int FN(wkv6_oracle_backward)(int64_t B, int64_t T, int64_t H, int64_t N,
                 gu[b * C + h * N + j] += rj * kj * vgy;
             }
         }
+        if (gs0) memcpy(gs0 + bh * NN, G, (size_t)NN * sizeof(REAL));
         free(Sall);
         free(G);
     }
     return bad ? -1 : 0;
+}
+
+int FN(wkv6_oracle_backward)(int64_t B, int64_t T, int64_t H, int64_t N,
+                             const REAL *r, const REAL *k, const REAL *v, const REAL *w, const REAL *u,
+                             const REAL *gy,
+                             REAL *gr, REAL *gk, REAL *gv, REAL *gw, REAL *gu)
+{
+    return backward_impl(B, T, H, N, r, k, v, w, u, NULL, gy, NULL, gr, gk, gv, gw, gu, NULL);
+}
+
+int FN(wkv6_oracle_backward_state)(int64_t B, int64_t T, int64_t H, int64_t N,
+                                   const REAL *r, const REAL *k, const REAL *v, const REAL *w, const REAL *u,
+                                   const REAL *s0, const REAL *gy, const REAL *gsT,
+                                   REAL *gr, REAL *gk, REAL *gv, REAL *gw, REAL *gu, REAL *gs0)
+{
+    return backward_impl(B, T, H, N, r, k, v, w, u, s0, gy, gsT, gr, gk, gv, gw, gu, gs0);
 }

@@ -50,6 +50,9 @@ def _load():
             g = getattr(_lib, "wkv6_oracle_backward" + sfx)
             g.restype = ctypes.c_int
             g.argtypes = [i64] * 4 + [p] * 11
+            gs = getattr(_lib, "wkv6_oracle_backward_state" + sfx)
+            gs.restype = ctypes.c_int
+            gs.argtypes = [i64] * 4 + [p] * 14
     return _lib
 
 
@@ -106,6 +109,31 @@ def backward_c(r, k, v, w, u, gy, head_size, dtype=np.float64):
     if rc != 0:
         raise MemoryError("oracle backward failed")
     return gr, gk, gv, gw, gu.sum(0).reshape(H, N)
+
+
+def backward_state_c(r, k, v, w, u, gy, head_size, init_state=None, g_state=None, dtype=np.float64):
+    """Gradients of  sum(y*gy) + sum(S_T*g_state)  with S_0 = init_state (B,H,N,N; None = 0):
+    gr, gk, gv, gw, gu(H,N), gs0 (B,H,N,N) from the C oracle (adjoint form).  The operator the
+    reference defines has no gradient through the state; this is the extension the carried-state
+    API suggests (dL/dS_0 = G_0, G_T = g_state)."""
+    lib = _load()
+    r, k, v, w, gy = (_as(x, dtype) for x in (r, k, v, w, gy))
+    B, T, C = r.shape
+    N = head_size
+    H = C // N
+    u = _as(u, dtype).reshape(H, N)
+    s0 = None if init_state is None else _as(init_state, dtype).reshape(B, H, N, N)
+    gsT = None if g_state is None else _as(g_state, dtype).reshape(B, H, N, N)
+    gr, gk, gv, gw = (np.empty((B, T, C), dtype) for _ in range(4))
+    gu = np.empty((B, C), dtype)
+    gs0 = np.empty((B, H, N, N), dtype)
+    sfx = "_f64" if dtype == np.float64 else "_f32"
+    rc = getattr(lib, "wkv6_oracle_backward_state" + sfx)(
+        B, T, H, N, _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(s0), _ptr(gy), _ptr(gsT),
+        _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu), _ptr(gs0))
+    if rc != 0:
+        raise MemoryError("oracle backward failed")
+    return gr, gk, gv, gw, gu.sum(0).reshape(H, N), gs0
 
 
 def loop_torch(r, k, v, w, u, head_size, init_state=None, state_map=None):

@@ -216,6 +216,36 @@ int wkv6_backward_saved_sum(void *stream, int dtype, int algo, int64_t B, int64_
                          need > 0, gu_sum);
 }
 
+size_t wkv6_backward_with_state_workspace_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
+    if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
+    size_t need = wkv6::scan_backward_state_workspace_bytes(B, T, C);
+    const size_t c = wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H);
+    return c > need ? c : need;
+}
+
+int wkv6_backward_with_state(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                             const void *r, const void *k, const void *v, const void *w, const void *u,
+                             const float *s0, const void *gy, const float *gsT,
+                             void *gr, void *gk, void *gv, void *gw, void *gu, float *gs0,
+                             void *workspace, size_t workspace_bytes) {
+    int rc = check_shape(dtype, B, T, C, H);
+    if (rc != WKV6_OK) return rc;
+    if (!r || !k || !v || !w || !u || !gy || !gr || !gk || !gv || !gw || !gu) return WKV6_ERR_ARG;
+    if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(gy) || !aligned16(gr) ||
+        !aligned16(gk) || !aligned16(gv) || !aligned16(gw)) return WKV6_ERR_ARG;
+    if ((s0 && !aligned16(s0)) || (gsT && !aligned16(gsT)) || (gs0 && !aligned16(gs0))) return WKV6_ERR_ARG;
+    if (algo < WKV6_ALGO_AUTO || algo > WKV6_ALGO_CHUNK) return WKV6_ERR_ARG;
+    const size_t need = wkv6_backward_with_state_workspace_bytes(dtype, algo, B, T, C, H);
+    if (!workspace || workspace_bytes < need || !aligned16(workspace)) return WKV6_ERR_WORKSPACE;
+    if (algo == WKV6_ALGO_CHUNK && !chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t)stream;
+    const bool chunk = algo == WKV6_ALGO_CHUNK || (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
+    if (!chunk)
+        return finish(wkv6::scan_backward_state(st, dtype, B, T, H, r, k, v, w, u, s0, gy, gsT, gr, gk, gv, gw, gu, gs0, workspace));
+    return finish(wkv6::chunk_backward(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace, false, nullptr,
+                                       s0, gsT, gs0));
+}
+
 int wkv6_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
                   const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
                   void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, size_t workspace_bytes) {

@@ -78,6 +78,9 @@ struct BwdArgs {
     int *arrivals;    // per head: workgroups that have delivered their gu partial (zero on entry)
     int B;
     float *ckpt;
+    // gradients through the state (all null for the stateless operator): fp32 (B,H,64,64) [key][value]
+    const float *s0, *gsT;   // initial state; gradient arriving at the final state
+    float *gs0;              // receives dL/dS_0
 };
 
 // ------------------------------------------------------------------------------------------
@@ -101,7 +104,10 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
         // phase 1: S^T (rows i, column j = col), checkpoint at every chunk start; group 0 only
         f32x4 S[4];
 #pragma unroll
-        for (int m = 0; m < 4; ++m) S[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int m = 0; m < 4; ++m) {
+            S[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            if (a.s0) S[m] = *reinterpret_cast<const f32x4 *>(a.s0 + (int64_t)(b * H + h) * (kN * kN) + col * kN + 16 * m + 4 * g);
+        }
         for (int c = 0; c < nchunk; ++c, ++item) {
             __syncthreads();
             if (GRP != 0) continue;
@@ -132,7 +138,10 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     float *vgyw = reinterpret_cast<float *>(smem + BwdLds::kVgy) + (4 * GRP + q) * 16;
     f32x4 Gj[4];   // reverse state, rows i, column j = col (the copy with rows j lives in the gv waves)
 #pragma unroll
-    for (int m = 0; m < 4; ++m) Gj[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int m = 0; m < 4; ++m) {
+        Gj[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        if (a.gsT) Gj[m] = *reinterpret_cast<const f32x4 *>(a.gsT + (int64_t)(b * H + h) * (kN * kN) + col * kN + 16 * m + 4 * g);
+    }
     const float uj = load1(a.u + h * kN + col);
     float gu_acc = 0.f;
     bf16_t *gr_h = a.gr + base, *gk_h = a.gk + base, *gw_h = a.gw + base;
@@ -334,10 +343,11 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
             }
             // the gradient of the first and the last decay is zero by definition (the flow balance
             // leaves rounding residue there); only the two tiles holding them pay for the test
+            // (with a non-zero initial state / a gradient arriving at the final state they are not zero)
             if ((c == 0 && p == 0) || (c == nchunk - 1 && p == (((T - 1) >> 4) & 3))) {
 #pragma unroll
                 for (int rr = 0; rr < 4; ++rr)
-                    if (t0 + tk + rr == 0 || t0 + tk + rr == T - 1) gwo[rr] = 0.f;
+                    if ((t0 + tk + rr == 0 && !a.s0) || (t0 + tk + rr == T - 1 && !a.gsT)) gwo[rr] = 0.f;
             }
             // two tokens share one conversion per tensor
             const uint32_t packed[6] = {pack_bf16x2(gro[0], gro[1]), pack_bf16x2(gko[0], gko[1]), pack_bf16x2(gwo[0], gwo[1]),
@@ -358,6 +368,11 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
         asm volatile("" : "+v"(Sraw[0]), "+v"(Sraw[1]), "+v"(Sraw[2]), "+v"(Sraw[3]));
     }
     for (int c = nchunk - 1; c >= 0; --c) visit(c, Sraw);
+    if (a.gs0 && GRP == 0) {   // the reverse state has arrived at t = 0: dL/dS_0
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+            *reinterpret_cast<f32x4 *>(a.gs0 + (int64_t)(b * H + h) * (kN * kN) + col * kN + 16 * m + 4 * g) = Gj[m];
+    }
     // gu: fold the four lane groups (different tokens, same channel), then the consumer groups
     gu_acc = sum_rows(gu_acc);
     if (NG == 2 && GRP == 1 && g == 0) reinterpret_cast<float *>(smem + BwdLds::kGu)[col] = gu_acc;
@@ -374,9 +389,12 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
 // ------------------------------------------------------------------------------------------
 struct GvState {
     f32x4 Gi[4];
-    __device__ __forceinline__ void init() {
+    // gsT: this pair's [key][value] block or null; the copy here has rows j = 16m + 4g + rr, column i = col
+    __device__ __forceinline__ void init(const float *gsT, int col, int g) {
 #pragma unroll
-        for (int m = 0; m < 4; ++m) Gi[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int m = 0; m < 4; ++m)
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) Gi[m][rr] = gsT ? gsT[(16 * m + 4 * g + rr) * kN + col] : 0.f;
     }
 };
 // the tiles of chunk c (phase 2 item `item`), last to first
@@ -439,7 +457,7 @@ __device__ __forceinline__ void bwd_gv(const BwdArgs &a, unsigned char *smem, in
     const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
     const int nchunk = (T + CL - 1) / CL;
     GvState st;
-    st.init();
+    st.init(a.gsT ? a.gsT + (int64_t)(b * H + h) * (kN * kN) : nullptr, 16 * q + (lane & 15), lane >> 4);
     int item = 0;
     if (kSweepStates)
         for (; item < nchunk; ++item) __syncthreads();
@@ -577,7 +595,7 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     };
     // item `it` is loaded during iteration it-2 (or the prologue) and prepared during iteration it-1
     GvState gvst;
-    if (kAlsoGv) gvst.init();
+    if (kAlsoGv) gvst.init(a.gsT ? a.gsT + (int64_t)(b * H + h) * (kN * kN) : nullptr, 16 * p + (lane & 15), lane >> 4);
     WKV6_STAMP_DECL;
     issue_loads(0);
     wait_younger(nitem > 1 ? issue_loads(1) : 0);
@@ -621,6 +639,7 @@ __global__ __launch_bounds__(BwdLayout<kLayout>::kWaves * 64) void chunk_bwd_ker
 {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_wild;
+    __shared__ float s_ft[kN];   // exact second pass with state gradients: the anchor of the gw sums
     static_assert(sizeof(ScanBwdALds) <= BwdLds::kBytes && sizeof(ScanBwdBLds) <= BwdLds::kBytes,
                   "the exact second pass reuses the LDS block");
     if (threadIdx.x == 0) s_wild = 0;
@@ -657,11 +676,16 @@ __global__ __launch_bounds__(BwdLayout<kLayout>::kWaves * 64) void chunk_bwd_ker
     if (s_wild) {
         const int nchunk = (a.T + CL - 1) / CL;
         float *ck = a.ckpt + (int64_t)(b * a.H + h) * nchunk * (kN * kN);
+        const int64_t so = (int64_t)(b * a.H + h) * (kN * kN);
+        const float *s0p = a.s0 ? a.s0 + so : nullptr, *gsTp = a.gsT ? a.gsT + so : nullptr;
+        const bool states = a.s0 || a.gsT || a.gs0;
         __syncthreads();
-        scan_bwd_a_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdALds *>(smem), b, h, a.T, a.H, a.r, a.k, a.v, a.w, a.u, a.gy, a.gr, a.gu, ck, kN);
+        scan_bwd_a_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdALds *>(smem), b, h, a.T, a.H, a.r, a.k, a.v, a.w, a.u, a.gy, a.gr, a.gu, ck, kN,
+                                        s0p, gsTp, states ? s_ft : nullptr);
         __threadfence_block();
         __syncthreads();
-        scan_bwd_b_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdBLds *>(smem), b, h, a.T, a.H, a.r, a.k, a.v, a.w, a.u, a.gy, ck, kN, a.gk, a.gv, a.gw);
+        scan_bwd_b_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdBLds *>(smem), b, h, a.T, a.H, a.r, a.k, a.v, a.w, a.u, a.gy, ck, kN, a.gk, a.gv, a.gw,
+                                        gsTp, states ? s_ft : nullptr, a.gs0 ? a.gs0 + so : nullptr, a.s0 == nullptr);
     }
     // Fused batch sum of gu (what the caller otherwise does with one more kernel): the workgroup that
     // is the last of its head to deliver adds up the B partials.  The partials travel as written-
@@ -720,10 +744,11 @@ hipError_t sum_over_batch(hipStream_t st, int out_dtype, int64_t B, int64_t C, c
 hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
                           const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
                           void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, bool states_ready,
-                          void *gu_sum)
+                          void *gu_sum, const float *s0, const float *gsT, float *gs0)
 {
     const size_t lds = BwdLds::kBytes;
     BwdArgs a;
+    a.s0 = s0; a.gsT = gsT; a.gs0 = gs0;
     a.T = (int)T; a.H = (int)H;
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w;
     a.u = (const bf16_t *)u; a.gy = (const bf16_t *)gy;

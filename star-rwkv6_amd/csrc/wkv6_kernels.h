@@ -17,6 +17,14 @@ hipError_t scan_backward(hipStream_t st, int dtype, int64_t B, int64_t T, int64_
                          const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace);
 
+// with gradients through the state: S_0 = s0 (null = 0), G_T = gsT (null = 0), gs0 = dL/dS_0 (may be null);
+// states are fp32 (B,H,64,64) [key][value]
+size_t scan_backward_state_workspace_bytes(int64_t B, int64_t T, int64_t C);
+hipError_t scan_backward_state(hipStream_t st, int dtype, int64_t B, int64_t T, int64_t H,
+                               const void *r, const void *k, const void *v, const void *w, const void *u,
+                               const float *s0, const void *gy, const float *gsT,
+                               void *gr, void *gk, void *gv, void *gw, void *gu, float *gs0, void *workspace);
+
 // --- chunk-parallel MFMA form, bf16 tensors only (wkv6_chunk.hip) ---
 hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u,
@@ -37,7 +45,8 @@ size_t chunk_saved_bytes(int64_t B, int64_t T, int64_t H);
 hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
                           const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
                           void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, bool states_ready,
-                          void *gu_sum);
+                          void *gu_sum, const float *s0 = nullptr, const float *gsT = nullptr, float *gs0 = nullptr);
+// s0 / gsT / gs0: gradients through the state, as in scan_backward_state (with states_ready = false)
 
 // sum over the batch of (B, C) partials -> (C), both in the output type (for the paths without a fused sum)
 hipError_t sum_over_batch(hipStream_t st, int out_dtype, int64_t B, int64_t C, const void *partials, void *sum);

@@ -33,12 +33,16 @@ template <typename Tin, typename Tout>
 __global__ __launch_bounds__(256) void scan_bwd_a_kernel(int T, int H,
         const Tin *__restrict__ r, const Tin *__restrict__ k, const Tin *__restrict__ v,
         const Tin *__restrict__ w, const Tin *__restrict__ u, const Tout *__restrict__ gy,
-        Tout *__restrict__ gr, Tout *__restrict__ gu, float *__restrict__ wsP)
+        Tout *__restrict__ gr, Tout *__restrict__ gu, float *__restrict__ wsP,
+        const float *__restrict__ s0, const float *__restrict__ gsT, float *__restrict__ fT)
 {
     __shared__ ScanBwdALds lds;
     const int b = blockIdx.x / H, h = blockIdx.x % H;
     const int64_t C = (int64_t)H * kN;
-    scan_bwd_a_body<Tin, Tout>(lds, b, h, T, H, r, k, v, w, u, gy, gr, gu, wsP + (int64_t)b * T * C + h * kN, C);
+    const int64_t pair = blockIdx.x;
+    scan_bwd_a_body<Tin, Tout>(lds, b, h, T, H, r, k, v, w, u, gy, gr, gu, wsP + (int64_t)b * T * C + h * kN, C,
+                               s0 ? s0 + pair * kN * kN : nullptr, gsT ? gsT + pair * kN * kN : nullptr,
+                               fT ? fT + pair * kN : nullptr);
 }
 
 template <typename Tin, typename Tout>
@@ -46,12 +50,16 @@ __global__ __launch_bounds__(512) void scan_bwd_b_kernel(int T, int H,
         const Tin *__restrict__ r, const Tin *__restrict__ k, const Tin *__restrict__ v,
         const Tin *__restrict__ w, const Tin *__restrict__ u, const Tout *__restrict__ gy,
         const float *__restrict__ wsP,
-        Tout *__restrict__ gk, Tout *__restrict__ gv, Tout *__restrict__ gw)
+        Tout *__restrict__ gk, Tout *__restrict__ gv, Tout *__restrict__ gw,
+        const float *__restrict__ gsT, const float *__restrict__ fT, float *__restrict__ gs0, int first_decay_unused)
 {
     __shared__ ScanBwdBLds lds;
     const int b = blockIdx.x / H, h = blockIdx.x % H;
     const int64_t C = (int64_t)H * kN;
-    scan_bwd_b_body<Tin, Tout>(lds, b, h, T, H, r, k, v, w, u, gy, wsP + (int64_t)b * T * C + h * kN, C, gk, gv, gw);
+    const int64_t pair = blockIdx.x;
+    scan_bwd_b_body<Tin, Tout>(lds, b, h, T, H, r, k, v, w, u, gy, wsP + (int64_t)b * T * C + h * kN, C, gk, gv, gw,
+                               gsT ? gsT + pair * kN * kN : nullptr, fT ? fT + pair * kN : nullptr,
+                               gs0 ? gs0 + pair * kN * kN : nullptr, first_decay_unused != 0);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -85,20 +93,27 @@ hipError_t scan_forward(hipStream_t st, int dtype, int state_dtype, int64_t B, i
 template <typename Tin, typename Tout>
 static hipError_t launch_bwd(hipStream_t st, int64_t B, int64_t T, int64_t H, const void *r, const void *k,
                              const void *v, const void *w, const void *u, const void *gy, void *gr, void *gk,
-                             void *gv, void *gw, void *gu, float *wsP)
+                             void *gv, void *gw, void *gu, float *wsP,
+                             const float *s0 = nullptr, const float *gsT = nullptr, float *gs0 = nullptr)
 {
+    // with state gradients: F_T (one value per channel and batch row) sits behind P in the workspace
+    float *fT = (s0 || gsT || gs0) ? wsP + B * T * H * kN : nullptr;
     hipLaunchKernelGGL((scan_bwd_a_kernel<Tin, Tout>), dim3((unsigned)(B * H)), dim3(256), 0, st, (int)T, (int)H,
                        (const Tin *)r, (const Tin *)k, (const Tin *)v, (const Tin *)w, (const Tin *)u,
-                       (const Tout *)gy, (Tout *)gr, (Tout *)gu, wsP);
+                       (const Tout *)gy, (Tout *)gr, (Tout *)gu, wsP, s0, gsT, fT);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((scan_bwd_b_kernel<Tin, Tout>), dim3((unsigned)(B * H)), dim3(512), 0, st, (int)T, (int)H,
                        (const Tin *)r, (const Tin *)k, (const Tin *)v, (const Tin *)w, (const Tin *)u,
-                       (const Tout *)gy, (const float *)wsP, (Tout *)gk, (Tout *)gv, (Tout *)gw);
+                       (const Tout *)gy, (const float *)wsP, (Tout *)gk, (Tout *)gv, (Tout *)gw,
+                       gsT, (const float *)fT, gs0, s0 ? 0 : 1);
     return hipGetLastError();
 }
 
 size_t scan_backward_workspace_bytes(int64_t B, int64_t T, int64_t C) { return (size_t)(B * T * C) * sizeof(float); }
+size_t scan_backward_state_workspace_bytes(int64_t B, int64_t T, int64_t C) {
+    return (size_t)(B * T * C + B * C) * sizeof(float);
+}
 
 hipError_t scan_backward(hipStream_t st, int dtype, int64_t B, int64_t T, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
@@ -109,6 +124,19 @@ hipError_t scan_backward(hipStream_t st, int dtype, int64_t B, int64_t T, int64_
     case kF32: return launch_bwd<float, float>(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, wsP);
     case kF16: return launch_bwd<f16_t, float>(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, wsP);
     default:   return launch_bwd<bf16_t, bf16_t>(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, wsP);
+    }
+}
+
+hipError_t scan_backward_state(hipStream_t st, int dtype, int64_t B, int64_t T, int64_t H,
+                               const void *r, const void *k, const void *v, const void *w, const void *u,
+                               const float *s0, const void *gy, const float *gsT,
+                               void *gr, void *gk, void *gv, void *gw, void *gu, float *gs0, void *workspace)
+{
+    float *wsP = (float *)workspace;
+    switch (dtype) {
+    case kF32: return launch_bwd<float, float>(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, wsP, s0, gsT, gs0);
+    case kF16: return launch_bwd<f16_t, float>(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, wsP, s0, gsT, gs0);
+    default:   return launch_bwd<bf16_t, bf16_t>(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, wsP, s0, gsT, gs0);
     }
 }
 

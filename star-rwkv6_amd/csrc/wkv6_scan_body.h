@@ -166,8 +166,12 @@ template <typename Tin, typename Tout>
 __device__ __forceinline__ void scan_bwd_a_body(ScanBwdALds &L, int b, int h, int T, int H,
         const Tin *__restrict__ r, const Tin *__restrict__ k, const Tin *__restrict__ v,
         const Tin *__restrict__ w, const Tin *__restrict__ u, const Tout *__restrict__ gy,
-        Tout *__restrict__ gr, Tout *__restrict__ gu, float *__restrict__ wsP, int64_t pstride)
+        Tout *__restrict__ gr, Tout *__restrict__ gu, float *__restrict__ wsP, int64_t pstride,
+        const float *__restrict__ s0 = nullptr, const float *__restrict__ gsT = nullptr, float *fT = nullptr)
 {
+    // State gradients (all three null for the stateless operator): s0 = this pair's initial state
+    // [key][value] fp32; gsT = the gradient arriving at its final state; fT[64] receives
+    // F_T[j] = sum_i S_T[j][i] gsT[j][i], the anchor of the gw suffix sums of sweep B.
     auto &s_r = L.s_r; auto &s_k = L.s_k; auto &s_d = L.s_d; auto &s_v = L.s_v; auto &s_g = L.s_g;
     auto &s_part = L.s_part; auto &s_vgy = L.s_vgy; auto &s_u = L.s_u;
     const int tid = threadIdx.x, lane = tid & 63, q = tid >> 6;
@@ -187,7 +191,7 @@ __device__ __forceinline__ void scan_bwd_a_body(ScanBwdALds &L, int b, int h, in
 
     float s[16];
 #pragma unroll
-    for (int ii = 0; ii < 16; ++ii) s[ii] = 0.f;
+    for (int ii = 0; ii < 16; ++ii) s[ii] = s0 ? s0[lane * kN + 16 * q + ii] : 0.f;
     if (tid < kN) s_u[tid] = load1(u + h * kN + tid);
     float gu_acc[4] = {0.f, 0.f, 0.f, 0.f};
 
@@ -288,10 +292,17 @@ __device__ __forceinline__ void scan_bwd_a_body(ScanBwdALds &L, int b, int h, in
 #pragma unroll
         for (int i = 0; i < 4; ++i) s_part[0][q][lane * 4 + i] = gu_acc[i];
     }
+    if (fT) {   // s now holds S_T
+        float f = 0.f;
+#pragma unroll
+        for (int ii = 0; ii < 16; ++ii) f = fmaf(s[ii], gsT ? gsT[lane * kN + 16 * q + ii] : 0.f, f);
+        s_part[1][q][lane] = f;
+    }
     __syncthreads();
     if (tid < kN) {
         const float g = s_part[0][0][tid] + s_part[0][1][tid] + s_part[0][2][tid] + s_part[0][3][tid];
         store1(gu + (int64_t)b * C + h * kN + tid, g);
+        if (fT) fT[tid] = s_part[1][0][tid] + s_part[1][1][tid] + s_part[1][2][tid] + s_part[1][3][tid];
     }
 }
 
@@ -319,8 +330,13 @@ __device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLds &L, int b, int h, in
         const Tin *__restrict__ r, const Tin *__restrict__ k, const Tin *__restrict__ v,
         const Tin *__restrict__ w, const Tin *__restrict__ u, const Tout *__restrict__ gy,
         const float *__restrict__ wsP, int64_t pstride,
-        Tout *__restrict__ gk, Tout *__restrict__ gv, Tout *__restrict__ gw)
+        Tout *__restrict__ gk, Tout *__restrict__ gv, Tout *__restrict__ gw,
+        const float *__restrict__ gsT = nullptr, const float *fT = nullptr, float *__restrict__ gs0 = nullptr,
+        bool first_decay_unused = true)
 {
+    // State gradients (null / true for the stateless operator): the reverse state starts from gsT
+    // (this pair's [key][value] fp32 block) and ends as gs0 = dL/dS_0; fT[64] anchors the gw suffix
+    // sums (sweep A); first_decay_unused = the initial state is zero, so d_0 reaches no output.
     auto &s_r = L.s_r; auto &s_k = L.s_k; auto &s_d = L.s_d; auto &s_v = L.s_v; auto &s_g = L.s_g;
     auto &s_pk = L.s_pk; auto &s_pv = L.s_pv; auto &s_e = L.s_e;
     auto &s_vgy = L.s_vgy; auto &s_ruk = L.s_ruk; auto &s_u = L.s_u;
@@ -346,9 +362,14 @@ __device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLds &L, int b, int h, in
 
     float g[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) g[i] = 0.f;
+    for (int i = 0; i < 16; ++i)
+        g[i] = !gsT ? 0.f : role_k ? gsT[lane * kN + 16 * q + i] : gsT[(16 * q + i) * kN + lane];
     if (tid < kN) s_u[tid] = load1(u + h * kN + tid);
     float carry[4] = {0.f, 0.f, 0.f, 0.f};  // sum over later tiles of (P - Q), finaliser channels
+    if (fT && tid < 256) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) carry[i] = fT[fc + i];
+    }
 
     auto prefetch = [&](int t0) {
         const int t = t0 + st;
@@ -509,7 +530,8 @@ __device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLds &L, int b, int h, in
                 }
                 // the first and last decay never reach an output: exactly zero, as the reference
                 // kernel writes them (rwkv_kernels.cu:381,406), not the rounding residue of P - Q
-                if (t0 + ft == 0 || t0 + ft == T - 1) { o4[0] = o4[1] = o4[2] = o4[3] = 0.f; }
+                // (with a gradient arriving at the final state / a non-zero initial state they do)
+                if ((t0 + ft == 0 && first_decay_unused) || (t0 + ft == T - 1 && !gsT)) { o4[0] = o4[1] = o4[2] = o4[3] = 0.f; }
                 store4(gw + of, o4[0], o4[1], o4[2], o4[3]);
             }
 #pragma unroll
@@ -517,6 +539,10 @@ __device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLds &L, int b, int h, in
         }
         // s_e is next written two barriers from here; staging overwrites only tiles whose readers
         // are done (finalisers read s_r/s_k/s_g/s_vgy/s_ruk before the barrier above).
+    }
+    if (gs0 && role_k) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) gs0[lane * kN + 16 * q + i] = g[i];
     }
 }
 

@@ -29,6 +29,8 @@ SIGNATURES = {
     "wkv6_forward_ex": (_int, [_p, _int, _int] + [_i64] * 4 + [_p] * 6 + [_p, _sz]),
     "wkv6_backward_ex": (_int, [_p, _int, _int] + [_i64] * 4 + [_p] * 11 + [_p, _sz]),
     "wkv6_backward_workspace_bytes_ex": (_sz, [_int, _int] + [_i64] * 4),
+    "wkv6_backward_with_state_workspace_bytes": (_sz, [_int, _int] + [_i64] * 4),
+    "wkv6_backward_with_state": (_int, [_p, _int, _int] + [_i64] * 4 + [_p] * 14 + [_p, _sz]),
     "wkv6_saved_bytes": (_sz, [_int, _int] + [_i64] * 4),
     "wkv6_forward_save": (_int, [_p, _int, _int] + [_i64] * 4 + [_p] * 6 + [_p, _sz]),
     "wkv6_backward_saved": (_int, [_p, _int, _int] + [_i64] * 4 + [_p] * 11 + [_p, _sz]),

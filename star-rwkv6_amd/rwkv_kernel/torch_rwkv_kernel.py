@@ -97,7 +97,7 @@ class _WKV6(torch.autograd.Function):
             return (None, None, None, None, gr, gk, gv, gw, gu, None)
 
 
-def _forward_with_state(B, T, C, H, state_map, r, k, v, w, u, init_state, algo=_native.ALGO_AUTO):
+def _forward_with_state(B, T, C, H, state_map, r, k, v, w, u, init_state, algo=_native.ALGO_AUTO, state_dtype=None):
     """Stateful forward, no gradient (rwkv_kernel/torch_rwkv_kernel.py:76-95)."""
     lib = _native.load()
     with torch.no_grad():
@@ -105,7 +105,7 @@ def _forward_with_state(B, T, C, H, state_map, r, k, v, w, u, init_state, algo=_
         assert init_state is not None or state_map is None, "state_map needs init_state"
         assert state_map is None or state_map.dtype == torch.int64
         odt = _out_dtype(r.dtype)
-        sdt = init_state.dtype if init_state is not None else odt
+        sdt = init_state.dtype if init_state is not None else (state_dtype or odt)
         N = C // H
         y = torch.empty((B, T, C), device=r.device, dtype=odt)
         ys = torch.empty((B, H, N, N), device=r.device, dtype=sdt)
@@ -115,6 +115,46 @@ def _forward_with_state(B, T, C, H, state_map, r, k, v, w, u, init_state, algo=_
                 int(init_state is not None), _ptr(state_map),
                 _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(init_state), _ptr(y), _ptr(ys), None, 0))
     return y, ys
+
+
+class _WKV6State(torch.autograd.Function):
+    """Stateful operator WITH gradients through the state: y, S_T = f(r, k, v, w, u, S_0), states fp32
+    (B,H,N,N), one per batch row.  Not part of the reference, whose stateful call carries no gradient
+    (rwkv_kernel/torch_rwkv_kernel.py:145-168); it makes back-propagation over a sequence cut into
+    pieces possible (the state's gradient is handed from one piece to the one before)."""
+
+    @staticmethod
+    def forward(ctx, B, T, C, H, r, k, v, w, u, s0, algo):
+        ctx.dims = (B, T, C, H)
+        ctx.algo = algo
+        ctx.has_s0 = s0 is not None
+        ctx.set_materialize_grads(False)   # an unused output arrives as None, not as a tensor of zeros
+        y, sT = _forward_with_state(B, T, C, H, None, r, k, v, w, u, s0, algo, state_dtype=torch.float32)
+        ctx.save_for_backward(r, k, v, w, u, *((s0,) if s0 is not None else ()))
+        return y, sT
+
+    @staticmethod
+    def backward(ctx, gy, gsT):
+        lib = _native.load()
+        B, T, C, H = ctx.dims
+        r, k, v, w, u = ctx.saved_tensors[:5]
+        s0 = ctx.saved_tensors[5] if ctx.has_s0 else None
+        with torch.no_grad():
+            odt = _out_dtype(r.dtype)
+            gy = torch.zeros((B, T, C), device=r.device, dtype=odt) if gy is None else gy.to(odt).contiguous()
+            gsT = None if gsT is None else gsT.float().contiguous()
+            gr, gk, gv, gw = (torch.empty((B, T, C), device=r.device, dtype=odt) for _ in range(4))
+            gu = torch.empty((B, C), device=r.device, dtype=odt)
+            gs0 = torch.empty((B, H, C // H, C // H), device=r.device, dtype=torch.float32) if ctx.has_s0 else None
+            code = _DTYPE_CODE[r.dtype]
+            with torch.cuda.device(r.device):
+                n = lib.wkv6_backward_with_state_workspace_bytes(code, ctx.algo, B, T, C, H)
+                ws = torch.empty(max(int(n), 16), device=r.device, dtype=torch.uint8)
+                _native.check(lib.wkv6_backward_with_state(
+                    _stream(), code, ctx.algo, B, T, C, H, _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(s0),
+                    _ptr(gy), _ptr(gsT), _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu), _ptr(gs0), _ptr(ws), n))
+            gu = torch.sum(gu, 0).reshape(u.shape)
+        return (None, None, None, None, gr.to(r.dtype), gk.to(r.dtype), gv.to(r.dtype), gw.to(r.dtype), gu.to(u.dtype), gs0, None)
 
 
 class RWKVKernelOperator:
@@ -197,6 +237,14 @@ class RWKVKernelOperator:
             init_state, state_map = self._resolve_state(B, r, init_state, state_map)
             for x in (r, k, v, w, u):
                 assert x.is_contiguous()
+            leaves = (r, k, v, w, u) + ((init_state,) if init_state is not None else ())
+            if torch.is_grad_enabled() and any(x.requires_grad for x in leaves):
+                # gradients through the state (not in the reference): one fp32 state per batch row
+                assert state_map is None and (init_state is None or init_state.shape[0] == B), \
+                    "gradients through the state need one init_state row per batch row and no state_map"
+                assert init_state is None or init_state.dtype == torch.float32, \
+                    "gradients through the state need an fp32 init_state"
+                return _WKV6State.apply(B, T, C, H, r, k, v, w, u, init_state, self.algo)
             return _forward_with_state(B, T, C, H, state_map, r, k, v, w, u, init_state, self.algo)
         o = _WKV6.apply(B, T, C, H, r, k, v, w, u, self.algo)
         return o, None

@@ -357,6 +357,85 @@ def test_fused_group_norm_gate_on_a_fallback_pair(op, oracle):
     check_close("out", out, want, torch.bfloat16)
 
 
+# Gradients through the state (an extension of the reference's stateful call): loss =
+# sum(y*gy) + sum(S_T*gS) with S_0 given; checked against the float64 adjoint-form oracle (itself
+# pinned by torch.autograd through the python loop).
+def _state_grad_case(op, oracle, B, T, H, seed, dtype, algo, with_s0=True, with_gs=True, wild=False):
+    N = 64
+    ins = oracle.make_inputs(B, T, H, N, seed, with_state=True)
+    if wild:
+        ins[3][B - 1, T // 3:T // 3 + 20, 5:25] = 6.0
+    odt = out_dtype(dtype)
+    dev, ref = cast_inputs(ins[:5], dtype)
+    gy_dev, gy_ref = cast_inputs(ins[5:6], odt)
+    s0 = ins[6].float() * 3 if with_s0 else None
+    gS = torch.randn(B, H, N, N, generator=torch.Generator().manual_seed(seed)) if with_gs else None
+    leaves = [x.clone().requires_grad_(True) for x in dev]
+    s0_dev = s0.cuda().requires_grad_(True) if with_s0 else None
+    op.algo = algo
+    y, sT = op(*leaves, return_state=True, init_state=s0_dev)
+    assert sT.dtype == torch.float32 and y.requires_grad
+    loss = (y.float() * gy_dev[0].float()).sum()
+    if with_gs:
+        loss = loss + (sT * gS.cuda()).sum()
+    got = torch.autograd.grad(loss, leaves + ([s0_dev] if with_s0 else []))
+    torch.cuda.synchronize()
+    want = oracle.backward_state_c(*ref, gy_ref[0], N, None if s0 is None else to_np(s0), None if gS is None else to_np(gS))
+    y_ref, sT_ref = oracle.forward_c(*ref, N, None if s0 is None else to_np(s0))
+    check_close("y", y.detach(), y_ref, odt)
+    check_close("sT", sT.detach(), sT_ref, odt)
+    names = "gr gk gv gw gu".split() + (["gs0"] if with_s0 else [])
+    for name, g, gr in zip(names, got, want):
+        check_close(name, to_np(g).reshape(gr.shape), gr, odt, is_grad=True)
+    if not with_s0:
+        assert float(got[3][:, 0].abs().max()) == 0.0      # zero initial state: the first decay reaches nothing
+    if not with_gs:
+        assert float(got[3][:, -1].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dt,T", [("f32", 37), ("f32", 1), ("bf16", 50), ("f16", 16)])
+def test_state_gradients_scan(op, oracle, dt, T):
+    _state_grad_case(op, oracle, 2, T, 2, 80 + T, DTYPES[dt], SCAN)
+
+
+@pytest.mark.parametrize("B,T,H", [(2, 64, 2), (2, 150, 1), (1, 512, 3)])
+def test_state_gradients_chunk_bf16(op, oracle, B, T, H):
+    _state_grad_case(op, oracle, B, T, H, 85 + T, torch.bfloat16, CHUNK)
+
+
+def test_state_gradients_one_sided(op, oracle):
+    _state_grad_case(op, oracle, 2, 96, 2, 91, torch.bfloat16, CHUNK, with_s0=False, with_gs=True)
+    _state_grad_case(op, oracle, 2, 96, 2, 92, torch.bfloat16, CHUNK, with_s0=True, with_gs=False)
+    _state_grad_case(op, oracle, 2, 40, 2, 93, torch.float32, SCAN, with_s0=False, with_gs=True)
+    _state_grad_case(op, oracle, 2, 40, 2, 94, torch.float32, SCAN, with_s0=True, with_gs=False)
+
+
+def test_state_gradients_on_a_fallback_pair(op, oracle):
+    _state_grad_case(op, oracle, 2, 128, 2, 95, torch.bfloat16, CHUNK, wild=True)
+
+
+def test_backpropagation_over_two_pieces_equals_one_piece(op):
+    # the property the state gradient exists for: a sequence cut in two, the state and its gradient
+    # handed across the cut, gives the gradients of the uncut sequence (fp32, exact kernels)
+    from oracle import wkv6_ref
+    B, T, H, N, cut = 2, 96, 2, 64, 40
+    ins = wkv6_ref.make_inputs(B, T, H, N, 96)
+    r, k, v, w, u, gy = (x.float().cuda() for x in ins[:6])
+    op.algo = SCAN
+    whole = [x.clone().requires_grad_(True) for x in (r, k, v, w, u)]
+    y, _ = op(*whole)
+    g_whole = torch.autograd.grad((y * gy).sum(), whole)
+    parts = [x.clone().requires_grad_(True) for x in (r, k, v, w, u)]
+    a = [x[:, :cut].contiguous() for x in parts[:4]] + [parts[4]]
+    b = [x[:, cut:].contiguous() for x in parts[:4]] + [parts[4]]
+    ya, sa = op(*a, return_state=True)
+    yb, _ = op(*b, return_state=True, init_state=sa)
+    g_parts = torch.autograd.grad((torch.cat([ya, yb], 1) * gy).sum(), parts)
+    for name, x, z in zip("gr gk gv gw gu".split(), g_parts, g_whole):
+        err = float((x - z).abs().max()) / max(1e-12, float(z.abs().max()))
+        assert err <= 2e-5, (name, err)
+
+
 def test_chunk_matches_scan_on_padding_mask(op, oracle):
     B, T, H, N = 1, 96, 1, 64
     ins = oracle.make_inputs(B, T, H, N, 54)

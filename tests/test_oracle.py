@@ -214,3 +214,28 @@ def test_group_norm_gate_is_a_per_head_layer_norm(oracle):
     flat = np.full((1, 1, N), 2.5)
     out = oracle.group_norm_gate_np(flat, np.ones_like(flat), np.ones((1, N)), np.full((1, N), 0.25), N)
     assert np.abs(out - 0.25).max() < 1e-12
+
+
+def test_state_gradients_vs_autograd(oracle):
+    # gradient into the initial state and from the final state: the adjoint-form C oracle against
+    # torch.autograd through the python loop (float64), for  L = sum(y*gy) + sum(S_T*gS)
+    B, T, H, N = 2, 11, 2, 64
+    ins = oracle.make_inputs(B, T, H, N, 21, with_state=True)
+    r, k, v, w, u, gy = (x.double() for x in ins[:6])
+    s0 = ins[6].double()
+    gS = torch.randn(B, H, N, N, generator=torch.Generator().manual_seed(3), dtype=torch.float64)
+    leaves = [x.clone().requires_grad_(True) for x in (r, k, v, w, u, s0)]
+    y, sT = oracle.loop_torch(*leaves[:5], N, init_state=leaves[5])
+    want = torch.autograd.grad((y * gy).sum() + (sT * gS).sum(), leaves)
+    got = oracle.backward_state_c(*(x.numpy() for x in (r, k, v, w, u, gy)), N, s0.numpy(), gS.numpy())
+    for name, a, b in zip("gr gk gv gw gu gs0".split(), got, want):
+        b = b.numpy().reshape(a.shape)
+        assert np.abs(a - b).max() <= 1e-10 * max(1.0, np.abs(b).max()), name
+    # with a state the first and last decay do receive a gradient
+    assert np.abs(got[3][:, 0]).max() > 0 and np.abs(got[3][:, -1]).max() > 0
+    # without states it is the stateless backward
+    plain = oracle.backward_c(*(x.numpy() for x in (r, k, v, w, u, gy)), N)
+    again = oracle.backward_state_c(*(x.numpy() for x in (r, k, v, w, u, gy)), N)
+    for a, b in zip(plain, again[:5]):
+        assert np.array_equal(a, b)
+    assert np.abs(again[3][:, 0]).max() == 0 and np.abs(again[3][:, -1]).max() == 0
