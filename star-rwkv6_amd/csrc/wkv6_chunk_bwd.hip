@@ -2,7 +2,7 @@
 // the notation are in wkv6_chunk_fwd.hip.
 //
 // Phase 1 (only when the forward pass did not leave its chunk states behind) sweeps the chunks in
-// time order and writes the state at every chunk start to the workspace (fp32,
+// time order and writes the state at every chunk start to the workspace (bf16,
 // [b][h][chunk][j][i]); phase 2 sweeps them in reverse order with the reverse state G in MFMA
 // accumulators.  G is kept twice, once with rows j / columns i (for gv) and once transposed (for
 // gk), so that it can be fed back to the MFMAs as an operand without leaving the registers; the
@@ -20,21 +20,20 @@
 //   gw_t[j]  = -exp(w_t[j]) ( E[j] + sum_{m<t} (Q_m - P_m) - P_t ),  E[j] = sum_i S0[j][i] G_new[j][i]
 // (the last line is the flow balance across decay step t, anchored at the exact tile-boundary term E).
 //
-// Workgroup: one per (batch, head), 8 + 4 NG waves in four-wave roles (one wave of each role per SIMD):
+// Workgroup: one per (batch, head), 12 waves in four-wave roles (one wave of each role per SIMD):
 //   loader/producer (wave p <-> tile p, lane = channel): brings the raw r, k, w, v, gy rows of a
 //       chunk from global memory straight into LDS tiles two items ahead, and one item ahead turns
-//       r, k, w into the bf16 tiles R~, K~, exp(-c_t) plus g and the diagonal sum r u k;
-//   gv role (wave q <-> value columns 16q..): reverse state with rows j, produces gv;
-//   NG consumer groups (wave q <-> key columns 16q..): reverse state with rows i, produce gr, gk,
-//       gw, gu.  With NG = 2 both groups advance G through every tile (4 MFMAs and a scaling) but
-//       share out the expensive per-tile work: group 0 takes tiles 3 and 1, group 1 tiles 2 and 0.
+//       r, k, w into the bf16 tiles R~, K~, exp(-c_t) plus g and the diagonal sum r u k; the same
+//       waves then run the gv role (wave q <-> value columns 16q..): reverse state with rows j,
+//       produces gv;
+//   two consumer groups (wave q <-> key columns 16q..): reverse state with rows i, produce gr, gk,
+//       gw, gu.  Both groups advance G through every tile (4 MFMAs and a scaling) but share out the
+//       expensive per-tile work: group 0 takes tiles 3 and 1, group 1 tiles 2 and 0.
 // All tiles are stored once, [token][channel]; v and gy are consumed as they came from memory.
 #include "wkv6_mfma.h"
 #include "wkv6_kernels.h"
 #include "wkv6_scan_body.h"
 
-#include <stdlib.h>
-#include <type_traits>
 
 namespace wkv6 {
 
@@ -84,9 +83,9 @@ struct BwdArgs {
 };
 
 // ------------------------------------------------------------------------------------------
-// Consumer group GRP of NG: gr, gk, gw, gu.
+// Consumer group GRP of two: gr, gk, gw, gu.
 // ------------------------------------------------------------------------------------------
-template <bool kSweepStates, bool kRagged, int NG, int GRP>
+template <bool kSweepStates, bool kRagged, int GRP>
 __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *smem, const int *s_wild, int b, int h, int q, int lane)
 {
     const int T = a.T, H = a.H;
@@ -97,7 +96,7 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     const int nchunk = (T + CL - 1) / CL;
     // chunk states: bf16 [chunk][j][i] in the first half of this workgroup's workspace slice
     bf16_t *ck = reinterpret_cast<bf16_t *>(a.ckpt + (int64_t)(b * H + h) * nchunk * (kN * kN));
-    auto mine = [](int p) { return NG == 1 || (p & 1) == (GRP ^ 1); };   // group 0: tiles 3, 1; group 1: tiles 2, 0
+    auto mine = [](int p) { return (p & 1) == (GRP ^ 1); };   // group 0: tiles 3, 1; group 1: tiles 2, 0
     int item = 0;
     WKV6_STAMP_DECL;
     if (kSweepStates) {
@@ -216,7 +215,7 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
         if (!kSweepStates) load_state(c > 0 ? c - 1 : 0, Sraw);
 #pragma unroll
         for (int p = 0; p < 3; ++p) {
-            if (NG == 2 && GRP == 1 && p == 2) continue;   // group 1 needs the states of tiles 0 and 2 only
+            if (GRP == 1 && p == 2) continue;   // group 1 needs the states of tiles 0 and 2 only
             const s16x4 kq = tile_frag_tok(kt, 16 * q, 16 * p, l16, g);
             const float gq = gg[p * kN + col];
 #pragma unroll
@@ -375,11 +374,11 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     }
     // gu: fold the four lane groups (different tokens, same channel), then the consumer groups
     gu_acc = sum_rows(gu_acc);
-    if (NG == 2 && GRP == 1 && g == 0) reinterpret_cast<float *>(smem + BwdLds::kGu)[col] = gu_acc;
+    if (GRP == 1 && g == 0) reinterpret_cast<float *>(smem + BwdLds::kGu)[col] = gu_acc;
     __threadfence_block();
     __syncthreads();
     if (GRP == 0 && g == 0 && !*s_wild) {   // (the exact second pass writes gu itself)
-        if (NG == 2) gu_acc += reinterpret_cast<const float *>(smem + BwdLds::kGu)[col];
+        gu_acc += reinterpret_cast<const float *>(smem + BwdLds::kGu)[col];
         store1(a.gu + (int64_t)b * C + h * kN + col, gu_acc);
     }
 }
@@ -449,30 +448,10 @@ __device__ __forceinline__ void bwd_gv_chunk(GvState &st, const BwdArgs &a, cons
     }
 }
 
-template <bool kSweepStates, bool kRagged>
-__device__ __forceinline__ void bwd_gv(const BwdArgs &a, unsigned char *smem, int b, int h, int q, int lane)
-{
-    const int T = a.T, H = a.H;
-    const int64_t C = (int64_t)H * kN;
-    const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
-    const int nchunk = (T + CL - 1) / CL;
-    GvState st;
-    st.init(a.gsT ? a.gsT + (int64_t)(b * H + h) * (kN * kN) : nullptr, 16 * q + (lane & 15), lane >> 4);
-    int item = 0;
-    if (kSweepStates)
-        for (; item < nchunk; ++item) __syncthreads();
-    for (int c = nchunk - 1; c >= 0; --c, ++item) {
-        __syncthreads();
-        bwd_gv_chunk<kRagged>(st, a, smem, a.gv + base, (uint32_t)C * 2u, c, item, q, lane);
-    }
-    __threadfence_block();
-    __syncthreads();
-}
-
 // ------------------------------------------------------------------------------------------
 // Loader / producer: wave p <-> tile p of every chunk, lane = channel.
 // ------------------------------------------------------------------------------------------
-template <bool kSweepStates, bool kRagged, bool kAlsoGv>
+template <bool kSweepStates, bool kRagged>
 __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *smem, int *s_wild, int b, int h, int p, int lane)
 {
     const int T = a.T, H = a.H;
@@ -595,7 +574,7 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     };
     // item `it` is loaded during iteration it-2 (or the prologue) and prepared during iteration it-1
     GvState gvst;
-    if (kAlsoGv) gvst.init(a.gsT ? a.gsT + (int64_t)(b * H + h) * (kN * kN) : nullptr, 16 * p + (lane & 15), lane >> 4);
+    gvst.init(a.gsT ? a.gsT + (int64_t)(b * H + h) * (kN * kN) : nullptr, 16 * p + (lane & 15), lane >> 4);
     WKV6_STAMP_DECL;
     issue_loads(0);
     wait_younger(nitem > 1 ? issue_loads(1) : 0);
@@ -610,14 +589,14 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
         if (it + 1 < nitem) {
             WKV6_STAMP();
             // (with a ragged tail the number of gv stores issued is not fixed: wait for everything older)
-            const int gv_stores = (kAlsoGv && !kRagged && it >= 1 && item_full(it - 1)) ? 16 : 0;
+            const int gv_stores = (!kRagged && it >= 1 && item_full(it - 1)) ? 16 : 0;
             wait_younger(younger + gv_stores);
             WKV6_STAMP();
             prepare(it + 1);
             WKV6_STAMP();
         }
         // the gv role, on the waves the operand preparation leaves partly idle
-        if (kAlsoGv && item_full(it)) bwd_gv_chunk<kRagged>(gvst, a, smem, a.gv + base, rowbytes, item_chunk(it), it, p, lane);
+        if (item_full(it)) bwd_gv_chunk<kRagged>(gvst, a, smem, a.gv + base, rowbytes, item_chunk(it), it, p, lane);
         WKV6_STAMP();
     }
     wait_loads<0>();
@@ -625,17 +604,12 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     __syncthreads();
 }
 
-// Wave layouts (four waves per role, one of each role per SIMD):
-//   kLayout 0: 16 waves = loader/producer | gv | consumer group 0 | consumer group 1
-//   kLayout 1: 12 waves = loader/producer + gv | consumer group 0 | consumer group 1
-//   kLayout 2: 12 waves = loader/producer | gv | one consumer group doing every tile
-template <int kLayout> struct BwdLayout {
-    static constexpr int kWaves = kLayout == 0 ? 16 : 12;
-    static constexpr int kGroups = kLayout == 2 ? 1 : 2;
-};
+// Wave layout: 12 waves, four per role, one wave of each role per SIMD:
+//   loader/producer + gv | consumer group 0 (tiles 3, 1) | consumer group 1 (tiles 2, 0)
+constexpr int kBwdWaves = 12;
 
-template <bool kSweepStates, bool kRagged, int kLayout>
-__global__ __launch_bounds__(BwdLayout<kLayout>::kWaves * 64) void chunk_bwd_kernel(BwdArgs a)
+template <bool kSweepStates, bool kRagged>
+__global__ __launch_bounds__(kBwdWaves * 64) void chunk_bwd_kernel(BwdArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_wild;
@@ -649,25 +623,13 @@ __global__ __launch_bounds__(BwdLayout<kLayout>::kWaves * 64) void chunk_bwd_ker
 #endif
     __syncthreads();
 
-    constexpr int NG = BwdLayout<kLayout>::kGroups;
     const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int role = wave >> 2, q = wave & 3;
-    if (kLayout == 0) {
-        if (role == 0) bwd_producer<kSweepStates, kRagged, false>(a, smem, &s_wild, b, h, q, lane);
-        else if (role == 1) bwd_gv<kSweepStates, kRagged>(a, smem, b, h, q, lane);
-        else if (role == 2) bwd_consumer<kSweepStates, kRagged, NG, 0>(a, smem, &s_wild, b, h, q, lane);
-        else bwd_consumer<kSweepStates, kRagged, NG, NG - 1>(a, smem, &s_wild, b, h, q, lane);
-    } else if (kLayout == 1) {
-        if (role == 0) bwd_producer<kSweepStates, kRagged, true>(a, smem, &s_wild, b, h, q, lane);
-        else if (role == 1) bwd_consumer<kSweepStates, kRagged, NG, 0>(a, smem, &s_wild, b, h, q, lane);
-        else bwd_consumer<kSweepStates, kRagged, NG, NG - 1>(a, smem, &s_wild, b, h, q, lane);
-    } else {
-        if (role == 0) bwd_producer<kSweepStates, kRagged, false>(a, smem, &s_wild, b, h, q, lane);
-        else if (role == 1) bwd_gv<kSweepStates, kRagged>(a, smem, b, h, q, lane);
-        else bwd_consumer<kSweepStates, kRagged, NG, 0>(a, smem, &s_wild, b, h, q, lane);
-    }
+    if (role == 0) bwd_producer<kSweepStates, kRagged>(a, smem, &s_wild, b, h, q, lane);
+    else if (role == 1) bwd_consumer<kSweepStates, kRagged, 0>(a, smem, &s_wild, b, h, q, lane);
+    else bwd_consumer<kSweepStates, kRagged, 1>(a, smem, &s_wild, b, h, q, lane);
 #ifdef WKV6_TIMING
     if (threadIdx.x == 0) a.dbg[16 * 256 + 2 * blockIdx.x + 1] = __builtin_readcyclecounter();
 #endif
@@ -758,26 +720,15 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
     a.gu_sum = states_ready ? (bf16_t *)gu_sum : nullptr;
     a.arrivals = reinterpret_cast<int *>(reinterpret_cast<char *>(workspace) + chunk_backward_workspace_bytes(B, T, H));
     a.dbg = reinterpret_cast<long long *>((float *)workspace + (size_t)(B * H) * ((T + CL - 1) / CL) * kN * kN + 1024);
-    auto launch = [&](auto kern, int waves) -> hipError_t {
+    auto launch = [&](auto kern) -> hipError_t {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(waves * 64), lds, st, a);
+        hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(kBwdWaves * 64), lds, st, a);
         return hipGetLastError();
     };
     const bool ragged = (T % CL) != 0;   // the last chunk has tokens past the end
-    auto run = [&](auto layout_tag) -> hipError_t {
-        constexpr int kLayout = decltype(layout_tag)::value;
-        constexpr int nw = BwdLayout<kLayout>::kWaves;
-        if (states_ready) return ragged ? launch(chunk_bwd_kernel<false, true, kLayout>, nw) : launch(chunk_bwd_kernel<false, false, kLayout>, nw);
-        return ragged ? launch(chunk_bwd_kernel<true, true, kLayout>, nw) : launch(chunk_bwd_kernel<true, false, kLayout>, nw);
-    };
-#ifdef WKV6_DEV_LAYOUTS
-    const char *env = getenv("WKV6_BWD_LAYOUT");
-    const int layout = env ? atoi(env) : 1;
-    if (layout == 0) return run(std::integral_constant<int, 0>());
-    if (layout == 2) return run(std::integral_constant<int, 2>());
-#endif
-    return run(std::integral_constant<int, 1>());
+    if (states_ready) return ragged ? launch(chunk_bwd_kernel<false, true>) : launch(chunk_bwd_kernel<false, false>);
+    return ragged ? launch(chunk_bwd_kernel<true, true>) : launch(chunk_bwd_kernel<true, false>);
 }
 
 }  // namespace wkv6

@@ -68,16 +68,9 @@ __device__ __forceinline__ uint32_t ystage_off(int t, int ch) {
 #define WKV6_FSTAMP_DECL do { } while (0)
 #endif
 
-// Wave layout.  kFwdHalves: producer waves per tile (1 or 2).  kFwdGroups: consumer groups; with 2
-// both carry the state and each produces y for every other tile, with 1 one group does every tile.
-#ifndef WKV6_FWD_HALVES
-#define WKV6_FWD_HALVES 1
-#endif
-#ifndef WKV6_FWD_GROUPS
-#define WKV6_FWD_GROUPS 2
-#endif
-constexpr int kFwdHalves = WKV6_FWD_HALVES, kFwdGroups = WKV6_FWD_GROUPS;
-constexpr int kFwdThreads = 4 * (kFwdHalves + kFwdGroups) * 64;
+// Wave layout: 12 waves, four per role, one wave of each role per SIMD:
+//   loader/producer (wave p <-> tile p) | consumer group 0 (y of tiles 0, 2) | consumer group 1 (tiles 1, 3)
+constexpr int kFwdThreads = 12 * 64;
 
 struct FwdArgs {
     long long *dbg;
@@ -101,7 +94,7 @@ struct FwdArgs {
 // Consumer group GRP of two: both groups carry the state through every tile (4 MFMAs and a
 // scaling), group 0 produces y for tiles 0 and 2, group 1 for tiles 1 and 3.
 // ------------------------------------------------------------------------------------------
-template <typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse, int NG, int GRP>
+template <typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse, int GRP>
 __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned char *smem, int q, int lane)
 {
     const int T = a.T, H = a.H;
@@ -173,7 +166,7 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
                 f32x4 U[4];
 #pragma unroll
                 for (int m = 0; m < 4; ++m) U[m] = mfma16(tile_frag_tok(kt, 16 * m, 16 * p, l16, g), vf, (f32x4){0.f, 0.f, 0.f, 0.f});
-                if (NG == 1 || (p & 1) == GRP) {
+                if ((p & 1) == GRP) {
                     const int row = 16 * p + l16;
                     const bf16x8 rf0 = tile_frag_ch(rt, row, 0, g), rf1 = tile_frag_ch(rt, row, 1, g);
                     const bf16x8 kf0 = tile_frag_ch(kt, row, 0, g), kf1 = tile_frag_ch(kt, row, 1, g);
@@ -236,16 +229,14 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
 }
 
 // ------------------------------------------------------------------------------------------
-// Loader / producer, lane = channel.  kHalves = 1: wave p <-> tile p of every chunk.  kHalves = 2:
-// wave 2p+hf <-> tokens 8hf..8hf+7 of tile p; the second-half wave redoes the first half's exp(w)
-// to get its starting decay.
+// Loader / producer, lane = channel: wave p <-> tile p of every chunk.
 // ------------------------------------------------------------------------------------------
-template <bool kRagged, bool kMulti, bool kFuse, int kHalves>
+template <bool kRagged, bool kMulti, bool kFuse>
 __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *smem, int *s_wild, int pw, int lane)
 {
-    constexpr int NT = 16 / kHalves;   // tokens per wave and chunk
+    constexpr int NT = 16;   // tokens per wave and chunk
     const int T = a.T, H = a.H;
-    const int p = kHalves == 2 ? pw >> 1 : pw, hf = kHalves == 2 ? pw & 1 : 0;
+    const int p = pw;
     const int ch = lane;
     const int64_t C = (int64_t)H * kN;
     const int nchunk = (T + CL - 1) / CL;
@@ -271,24 +262,16 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
     point_loads();
     // Rows past the end of the sequence are fetched from row T-1 (valid memory); the operand
     // preparation turns them into r = k = 0, w = -inf (decay 1), and the v rows only ever meet zero
-    // operands.  Each wave loads what it reads itself (with kHalves = 2 the second-half wave also
-    // the first half's w rows), so its own vmcnt covers its inputs; v is picked up by the consumers
-    // a barrier later.
-    static_assert(!kFuse || kHalves == 1, "the fused output stage is written for one producer wave per tile");
-    constexpr int kLoads = (kHalves == 2 ? 5 : 8) + (kFuse ? 2 : 0);   // per chunk and wave
+    // operands.  Each wave loads what it reads itself, so its own vmcnt covers its inputs; v is
+    // picked up by the consumers a barrier later.
+    constexpr int kLoads = 8 + (kFuse ? 2 : 0);   // per chunk and wave
     constexpr int kLoads0 = kLoads + (kFuse ? 2 : 0);                  // wave 0 also brings the norm's scale and offset
     auto issue_loads = [&](int it) {   // visit `it` = the load stream's current (pair, chunk)
         const int tb = ld_c * CL + 16 * p;
         const uint32_t rkw = lds0 + FwdLds::kRawRKW + (it & 1) * 3 * kTileBytes + 16 * p * kTileRow;
         const uint32_t vv = lds0 + FwdLds::kRawV + (it % 3) * kTileBytes + 16 * p * kTileRow;
-        if (kHalves == 2) {
-            // (the first-half wave loads its w block twice, which keeps the count uniform)
-            const int t_first = tb + lrow;
-            load_rows8_to_lds(wb, (uint32_t)(kRagged ? min(t_first, T - 1) : t_first) * rowbytes + lpiece, rkw + 2 * kTileBytes);
-        }
 #pragma unroll
-        for (int x = 0; x < 2 / kHalves; ++x) {
-            const int blk = kHalves == 2 ? hf : x;
+        for (int blk = 0; blk < 2; ++blk) {
             const int t = tb + 8 * blk + lrow;
             const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes + lpiece;
             load_rows8_to_lds(wb, o, rkw + 2 * kTileBytes + 8 * blk * kTileRow);
@@ -363,27 +346,16 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
         const unsigned char *raw = smem + FwdLds::kRawRKW + (it & 1) * 3 * kTileBytes;
         unsigned char *op = smem + FwdLds::kOp + (it & 1) * FwdLds::kOpBytes;
         const int tb = pp_c * CL + 16 * p;
-        const int e0 = 8 * hf;   // first token of this wave inside the tile
         // exponents are kept in base 2 (one v_exp_f32 each, no extra scaling multiply)
         float cs2 = 0.f, pa = 1.f;
-        if (kHalves == 2 && hf) {
-            // decay accumulated over the first half of the tile
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                uint32_t rw = *reinterpret_cast<const uint16_t *>(raw + 2 * kTileBytes + choff[e] + e * kTileRow);
-                if (kRagged && tb + e >= T) rw = 0xff80u;
-                cs2 += exp2_fast(fmaf(bf16_bits_to_float(rw), kLog2e, kLog2Log2e));
-            }
-            pa = exp2_fast(-cs2);
-        }
         float fr[NT], fk[NT], fw[NT];
 #pragma unroll
         for (int e = 0; e < NT; ++e) {
-            const uint32_t o = choff[e & 7] + (e0 + e) * kTileRow;
+            const uint32_t o = choff[e & 7] + e * kTileRow;
             uint32_t ra = *reinterpret_cast<const uint16_t *>(raw + o);
             uint32_t rk = *reinterpret_cast<const uint16_t *>(raw + kTileBytes + o);
             uint32_t rw = *reinterpret_cast<const uint16_t *>(raw + 2 * kTileBytes + o);
-            if (kRagged && tb + e0 + e >= T) { ra = 0u; rk = 0u; rw = 0xff80u; }
+            if (kRagged && tb + e >= T) { ra = 0u; rk = 0u; rw = 0xff80u; }
             fr[e] = bf16_bits_to_float(ra); fk[e] = bf16_bits_to_float(rk); fw[e] = bf16_bits_to_float(rw);
         }
         float xr[NT], xk[NT], pr[NT];
@@ -399,27 +371,19 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
 #pragma unroll
         for (int e = 0; e < NT; e += 2) {
             const uint32_t pr2 = pack_bf16x2(xr[e], xr[e + 1]), pk2 = pack_bf16x2(xk[e], xk[e + 1]);
-            const uint32_t o0 = choff[e & 7] + (e0 + e) * kTileRow, o1 = choff[(e + 1) & 7] + (e0 + e + 1) * kTileRow;
+            const uint32_t o0 = choff[e & 7] + e * kTileRow, o1 = choff[(e + 1) & 7] + (e + 1) * kTileRow;
             *reinterpret_cast<uint16_t *>(op + FwdLds::kOpRt + o0) = (uint16_t)pr2;
             *reinterpret_cast<uint16_t *>(op + FwdLds::kOpRt + o1) = (uint16_t)(pr2 >> 16);
             *reinterpret_cast<uint16_t *>(op + FwdLds::kOpKt + o0) = (uint16_t)pk2;
             *reinterpret_cast<uint16_t *>(op + FwdLds::kOpKt + o1) = (uint16_t)(pk2 >> 16);
         }
-        if (kHalves == 1 || hf) {
-            // the whole tile's decay: g, and the range check of exp(+c)
-            if (__builtin_amdgcn_ballot_w64(!(cs2 <= kWildLimit * kLog2e)) != 0ull) {
-                if (lane == 0) s_wild[pp_n] = 1;
-            }
-            reinterpret_cast<float *>(op + FwdLds::kOpG)[p * kN + ch] = pa;
+        // the whole tile's decay: g, and the range check of exp(+c)
+        if (__builtin_amdgcn_ballot_w64(!(cs2 <= kWildLimit * kLog2e)) != 0ull) {
+            if (lane == 0) s_wild[pp_n] = 1;
         }
-        float *ruk = reinterpret_cast<float *>(op + FwdLds::kOpRuk) + 16 * p + e0;
-        if constexpr (kHalves == 2) {
-            const float tot = transpose_reduce8(pr, lane);
-            if ((lane & 7) == 0) ruk[(lane >> 3) & 7] = tot;
-        } else {
-            const float tot = transpose_reduce16(pr, lane);
-            if ((lane & 3) == 0) ruk[(lane >> 2) & 15] = tot;
-        }
+        reinterpret_cast<float *>(op + FwdLds::kOpG)[p * kN + ch] = pa;
+        const float tot = transpose_reduce16(pr, lane);
+        if ((lane & 3) == 0) reinterpret_cast<float *>(op + FwdLds::kOpRuk)[16 * p + ((lane >> 2) & 15)] = tot;
         if (++pp_c == nchunk && kMulti) {   // the next preparation opens the next pair: its head's u
             pp_c = 0; ++pp_n;
             if (pp_n < n_my) {
@@ -502,9 +466,9 @@ __global__ __launch_bounds__(kFwdThreads) void chunk_fwd_kernel(FwdArgs a)
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int role = wave >> 2, q = wave & 3;
-    if (role < kFwdHalves) fwd_producer<kRagged, kMulti, kFuse, kFwdHalves>(a, smem, s_wild, wave, lane);
-    else if (kFwdGroups == 1 || role == kFwdHalves) fwd_consumer<Ts, kSave, kRagged, kMulti, kFuse, kFwdGroups, 0>(a, smem, q, lane);
-    else fwd_consumer<Ts, kSave, kRagged, kMulti, kFuse, kFwdGroups, 1>(a, smem, q, lane);
+    if (role == 0) fwd_producer<kRagged, kMulti, kFuse>(a, smem, s_wild, wave, lane);
+    else if (role == 1) fwd_consumer<Ts, kSave, kRagged, kMulti, kFuse, 0>(a, smem, q, lane);
+    else fwd_consumer<Ts, kSave, kRagged, kMulti, kFuse, 1>(a, smem, q, lane);
     // exact second pass for every pair of this workgroup that had a tile leave the representable range
     __threadfence_block();   // workgroup scope is enough (and a device-scope fence would write back the L2)
     __syncthreads();

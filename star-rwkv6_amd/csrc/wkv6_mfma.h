@@ -152,20 +152,6 @@ __device__ __forceinline__ float transpose_reduce16(const float (&p)[16], int la
     return x;
 }
 
-// same for 8 per-lane values; lane l receives the total of value (l>>3)&7
-__device__ __forceinline__ float transpose_reduce8(const float (&p)[8], int lane) {
-    float x4[4], x2[2];
-    const bool b5 = lane & 32, b4 = lane & 16, b3 = lane & 8;
-#pragma unroll
-    for (int a = 0; a < 4; ++a) x4[a] = (b5 ? p[a + 4] : p[a]) + __shfl_xor(b5 ? p[a] : p[a + 4], 32);
-#pragma unroll
-    for (int a = 0; a < 2; ++a) x2[a] = (b4 ? x4[a + 2] : x4[a]) + __shfl_xor(b4 ? x4[a] : x4[a + 2], 16);
-    float x = (b3 ? x2[1] : x2[0]) + __shfl_xor(b3 ? x2[0] : x2[1], 8);
-    x += __shfl_xor(x, 4);
-    x += __shfl_xor(x, 2);
-    x += __shfl_xor(x, 1);
-    return x;
-}
 
 // Writes row-major [token][channel] bf16 with 4-byte stores: lanes 2c and 2c+1 swap one value so
 // that the even lane stores (x[c], x[c+1]) of an even token row and the odd lane those of the
