@@ -75,6 +75,22 @@ __device__ __forceinline__ void store1(float *p, float a) { *p = a; }
 __device__ __forceinline__ void store1(bf16_t *p, float a) {
     *reinterpret_cast<uint16_t *>(p) = (uint16_t)pack_bf16x2(a, 0.f);
 }
+// four consecutive elements as fp32, one vector load
+__device__ __forceinline__ void load4(const float *p, float (&o)[4]) {
+    const float4 x = *reinterpret_cast<const float4 *>(p);
+    o[0] = x.x; o[1] = x.y; o[2] = x.z; o[3] = x.w;
+}
+__device__ __forceinline__ void load4(const bf16_t *p, float (&o)[4]) {
+    const uint2 x = *reinterpret_cast<const uint2 *>(p);
+    o[0] = __uint_as_float(x.x << 16); o[1] = __uint_as_float(x.x & 0xffff0000u);
+    o[2] = __uint_as_float(x.y << 16); o[3] = __uint_as_float(x.y & 0xffff0000u);
+}
+__device__ __forceinline__ void load4(const f16_t *p, float (&o)[4]) {
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    const h4 x = *reinterpret_cast<const h4 *>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = (float)x[i];
+}
 __device__ __forceinline__ float load1(const float *p) { return *p; }
 __device__ __forceinline__ float load1(const bf16_t *p) {
     return bf16_bits_to_float(*reinterpret_cast<const uint16_t *>(p));

@@ -29,6 +29,71 @@ __global__ __launch_bounds__(256) void scan_fwd_kernel(int T, int H,
     scan_fwd_body<Tin, Tout, Ts>(lds, blockIdx.x / H, blockIdx.x % H, T, H, r, k, v, w, u, s0, map, y, sT);
 }
 
+// One timestep (T = 1: the decode step of a served model).  Nothing is carried inside the kernel, so
+// a pair needs no workgroup: one wave per (batch, head), four pairs per workgroup, no LDS, no
+// barrier.  Lane l owns value columns 4 (l & 15) .. +3 of key rows 16 (l >> 4) .. +15: the state
+// streams through as sixteen 16-byte loads and stores per lane, all issued at once, and y is
+// folded over the four row groups with two wavefront shuffles per value.
+template <typename Tin, typename Tout, typename Ts>
+__global__ __launch_bounds__(256) void step_fwd_kernel(int npairs, int H,
+        const Tin *__restrict__ r, const Tin *__restrict__ k, const Tin *__restrict__ v,
+        const Tin *__restrict__ w, const Tin *__restrict__ u,
+        const Ts *__restrict__ s0, const int64_t *__restrict__ map,
+        Tout *__restrict__ y, Ts *__restrict__ sT)
+{
+    const int lane = threadIdx.x & 63;
+    const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (pair >= npairs) return;
+    const int b = pair / H, h = pair - b * H;
+    const int i4 = (lane & 15) * 4, j0 = (lane >> 4) * 16;
+    const int64_t tok = (int64_t)pair * kN;   // T = 1: (b, 0, h*64) is element pair*64 of a (B,1,C) tensor
+    float S[16][4];
+    if (s0) {
+        const int64_t row = map ? map[b] : (int64_t)b;
+        const Ts *p = s0 + ((row * H + h) * kN + j0) * kN + i4;
+#pragma unroll
+        for (int jj = 0; jj < 16; ++jj) load4(p + jj * kN, S[jj]);
+    } else {
+#pragma unroll
+        for (int jj = 0; jj < 16; ++jj) S[jj][0] = S[jj][1] = S[jj][2] = S[jj][3] = 0.f;
+    }
+    Raw8<Tin> rr[2], rk[2], rw[2], ru[2];
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+        rr[x].load(r + tok + j0 + 8 * x); rk[x].load(k + tok + j0 + 8 * x);
+        rw[x].load(w + tok + j0 + 8 * x); ru[x].load(u + h * kN + j0 + 8 * x);
+    }
+    float vv[4];
+    load4(v + tok + i4, vv);
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+        float fr[8], fk[8], fw[8], fu[8];
+        rr[x].to_float(fr); rk[x].to_float(fk); rw[x].to_float(fw); ru[x].to_float(fu);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float d = decay_from_raw(fw[e]), uk = fu[e] * fk[e];
+            float (&Sj)[4] = S[8 * x + e];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                acc[c] = fmaf(fr[e], fmaf(uk, vv[c], Sj[c]), acc[c]);
+                Sj[c] = fmaf(Sj[c], d, fk[e] * vv[c]);
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        acc[c] += __shfl_xor(acc[c], 16);
+        acc[c] += __shfl_xor(acc[c], 32);
+    }
+    if (lane < 16) store4(y + tok + i4, acc[0], acc[1], acc[2], acc[3]);
+    if (sT) {
+        Ts *p = sT + ((int64_t)pair * kN + j0) * kN + i4;
+#pragma unroll
+        for (int jj = 0; jj < 16; ++jj) store4(p + jj * kN, S[jj][0], S[jj][1], S[jj][2], S[jj][3]);
+    }
+}
+
 template <typename Tin, typename Tout>
 __global__ __launch_bounds__(256) void scan_bwd_a_kernel(int T, int H,
         const Tin *__restrict__ r, const Tin *__restrict__ k, const Tin *__restrict__ v,
@@ -70,6 +135,12 @@ static hipError_t launch_fwd(hipStream_t st, int64_t B, int64_t T, int64_t H, co
                              const void *v, const void *w, const void *u, const void *s0, const int64_t *map,
                              void *y, void *sT)
 {
+    if (T == 1) {
+        hipLaunchKernelGGL((step_fwd_kernel<Tin, Tout, Ts>), dim3((unsigned)((B * H + 3) / 4)), dim3(256), 0, st, (int)(B * H), (int)H,
+                           (const Tin *)r, (const Tin *)k, (const Tin *)v, (const Tin *)w, (const Tin *)u,
+                           (const Ts *)s0, map, (Tout *)y, (Ts *)sT);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL((scan_fwd_kernel<Tin, Tout, Ts>), dim3((unsigned)(B * H)), dim3(256), 0, st, (int)T, (int)H,
                        (const Tin *)r, (const Tin *)k, (const Tin *)v, (const Tin *)w, (const Tin *)u,
                        (const Ts *)s0, map, (Tout *)y, (Ts *)sT);
