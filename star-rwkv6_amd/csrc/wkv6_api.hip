@@ -103,6 +103,10 @@ int wkv6_forward_gn_gate(void *stream, int dtype, int state_dtype,
     if (!(gn_eps >= 0.f)) return WKV6_ERR_ARG;
     if (state_dtype != out_type(dtype) && state_dtype != WKV6_F32) return WKV6_ERR_ARG;
     if (!chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;   // bf16 tensors only
+    if (T == 1)   // a decode step: the single-timestep kernel
+        return finish(wkv6::step_forward_fused((hipStream_t)stream, state_dtype, B, H, r, k, v, w, u,
+                                               has_init_state ? s : nullptr, has_init_state ? state_map : nullptr,
+                                               gate, gn_scale, gn_offset, gn_eps, out, ys));
     return finish(wkv6::chunk_forward_fused((hipStream_t)stream, state_dtype, B, T, H, r, k, v, w, u,
                                             has_init_state ? s : nullptr, has_init_state ? state_map : nullptr,
                                             gate, gn_scale, gn_offset, gn_eps, out, ys));

@@ -17,6 +17,12 @@ hipError_t scan_backward(hipStream_t st, int dtype, int64_t B, int64_t T, int64_
                          const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace);
 
+// one timestep (T = 1) with the layer's output stage fused in (bf16 tensors), see chunk_forward_fused
+hipError_t step_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64_t H,
+                              const void *r, const void *k, const void *v, const void *w, const void *u,
+                              const void *s0, const int64_t *map, const void *gate, const float *gn_scale,
+                              const float *gn_offset, float gn_eps, void *out, void *sT);
+
 // with gradients through the state: S_0 = s0 (null = 0), G_T = gsT (null = 0), gs0 = dL/dS_0 (may be null);
 // states are fp32 (B,H,64,64) [key][value]
 size_t scan_backward_state_workspace_bytes(int64_t B, int64_t T, int64_t C);

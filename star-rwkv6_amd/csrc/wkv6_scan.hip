@@ -34,12 +34,15 @@ __global__ __launch_bounds__(256) void scan_fwd_kernel(int T, int H,
 // barrier.  Lane l owns value columns 4 (l & 15) .. +3 of key rows 16 (l >> 4) .. +15: the state
 // streams through as sixteen 16-byte loads and stores per lane, all issued at once, and y is
 // folded over the four row groups with two wavefront shuffles per value.
-template <typename Tin, typename Tout, typename Ts>
+// kFuse: y is replaced by (layer_norm(y over the head's 64 channels, eps) * gn_scale + gn_offset) * gate,
+// the model's next two steps (the 64 values of a head sit in 16 lanes of the wave).
+template <typename Tin, typename Tout, typename Ts, bool kFuse>
 __global__ __launch_bounds__(256) void step_fwd_kernel(int npairs, int H,
         const Tin *__restrict__ r, const Tin *__restrict__ k, const Tin *__restrict__ v,
         const Tin *__restrict__ w, const Tin *__restrict__ u,
         const Ts *__restrict__ s0, const int64_t *__restrict__ map,
-        Tout *__restrict__ y, Ts *__restrict__ sT)
+        Tout *__restrict__ y, Ts *__restrict__ sT,
+        const Tin *__restrict__ gate, const float *__restrict__ gn_scale, const float *__restrict__ gn_offset, float gn_eps)
 {
     const int lane = threadIdx.x & 63;
     const int pair = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -85,6 +88,25 @@ __global__ __launch_bounds__(256) void step_fwd_kernel(int npairs, int H,
     for (int c = 0; c < 4; ++c) {
         acc[c] += __shfl_xor(acc[c], 16);
         acc[c] += __shfl_xor(acc[c], 32);
+    }
+    if (kFuse) {
+        // every lane holds the y of its 4 columns; fold mean and variance over the 16 column groups
+        float sum = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+#pragma unroll
+        for (int m = 8; m >= 1; m >>= 1) sum += __shfl_xor(sum, m);
+        const float mu = sum * (1.f / kN);
+        float d[4], sq = 0.f;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) { d[c] = acc[c] - mu; sq = fmaf(d[c], d[c], sq); }
+#pragma unroll
+        for (int m = 8; m >= 1; m >>= 1) sq += __shfl_xor(sq, m);
+        const float rstd = __builtin_amdgcn_rsqf(sq * (1.f / kN) + gn_eps);
+        float gt[4], sc[4], of[4];
+        load4(gate + tok + i4, gt);
+        load4(gn_scale + h * kN + i4, sc);
+        load4(gn_offset + h * kN + i4, of);
+#pragma unroll
+        for (int c = 0; c < 4; ++c) acc[c] = fmaf(d[c] * rstd, sc[c], of[c]) * gt[c];
     }
     if (lane < 16) store4(y + tok + i4, acc[0], acc[1], acc[2], acc[3]);
     if (sT) {
@@ -136,9 +158,9 @@ static hipError_t launch_fwd(hipStream_t st, int64_t B, int64_t T, int64_t H, co
                              void *y, void *sT)
 {
     if (T == 1) {
-        hipLaunchKernelGGL((step_fwd_kernel<Tin, Tout, Ts>), dim3((unsigned)((B * H + 3) / 4)), dim3(256), 0, st, (int)(B * H), (int)H,
+        hipLaunchKernelGGL((step_fwd_kernel<Tin, Tout, Ts, false>), dim3((unsigned)((B * H + 3) / 4)), dim3(256), 0, st, (int)(B * H), (int)H,
                            (const Tin *)r, (const Tin *)k, (const Tin *)v, (const Tin *)w, (const Tin *)u,
-                           (const Ts *)s0, map, (Tout *)y, (Ts *)sT);
+                           (const Ts *)s0, map, (Tout *)y, (Ts *)sT, (const Tin *)nullptr, (const float *)nullptr, (const float *)nullptr, 0.f);
         return hipGetLastError();
     }
     hipLaunchKernelGGL((scan_fwd_kernel<Tin, Tout, Ts>), dim3((unsigned)(B * H)), dim3(256), 0, st, (int)T, (int)H,
@@ -159,6 +181,24 @@ hipError_t scan_forward(hipStream_t st, int dtype, int state_dtype, int64_t B, i
         return sf32 ? launch_fwd<bf16_t, bf16_t, float>(st, B, T, H, r, k, v, w, u, s0, map, y, sT)
                     : launch_fwd<bf16_t, bf16_t, bf16_t>(st, B, T, H, r, k, v, w, u, s0, map, y, sT);
     }
+}
+
+// single timestep with the fused output stage (bf16 tensors)
+hipError_t step_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64_t H,
+                              const void *r, const void *k, const void *v, const void *w, const void *u,
+                              const void *s0, const int64_t *map, const void *gate, const float *gn_scale,
+                              const float *gn_offset, float gn_eps, void *out, void *sT)
+{
+    const dim3 grid((unsigned)((B * H + 3) / 4)), block(256);
+    if (state_dtype == kF32)
+        hipLaunchKernelGGL((step_fwd_kernel<bf16_t, bf16_t, float, true>), grid, block, 0, st, (int)(B * H), (int)H,
+                           (const bf16_t *)r, (const bf16_t *)k, (const bf16_t *)v, (const bf16_t *)w, (const bf16_t *)u,
+                           (const float *)s0, map, (bf16_t *)out, (float *)sT, (const bf16_t *)gate, gn_scale, gn_offset, gn_eps);
+    else
+        hipLaunchKernelGGL((step_fwd_kernel<bf16_t, bf16_t, bf16_t, true>), grid, block, 0, st, (int)(B * H), (int)H,
+                           (const bf16_t *)r, (const bf16_t *)k, (const bf16_t *)v, (const bf16_t *)w, (const bf16_t *)u,
+                           (const bf16_t *)s0, map, (bf16_t *)out, (bf16_t *)sT, (const bf16_t *)gate, gn_scale, gn_offset, gn_eps);
+    return hipGetLastError();
 }
 
 template <typename Tin, typename Tout>
