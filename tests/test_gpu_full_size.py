@@ -101,3 +101,55 @@ def test_config5_prefill_then_decode(op, oracle):
     y_one, s_one = op(r, k, v, w, u, return_state=True, init_state=h0)
     assert rel_inf(to_np(y_all), to_np(y_one)) <= 1e-2
     assert rel_inf(to_np(s), to_np(s_one)) <= 1e-2
+
+
+def test_config5_prefill_with_fused_output_stage(op):
+    # B=64 T=512 C=2048: the fused group norm + gate against the same two steps applied on the GPU to
+    # the unfused kernel's own y (both normalise the bf16-rounded y, so they agree to output rounding),
+    # and the carried state is the unfused one bit for bit
+    import torch.nn.functional as F
+    from oracle import wkv6_ref
+    B, T, H, N = 64, 512, 32, 64
+    print("config 5 prefill, fused output stage", flush=True)
+    ins = wkv6_ref.make_inputs(B, T, H, N, 3, with_state=True)
+    r, k, v, w, u = (x.to(torch.bfloat16).cuda().contiguous() for x in ins[:5])
+    s0 = ins[6].float().cuda()
+    g = torch.Generator().manual_seed(9)
+    gate = torch.randn(B, T, H * N, generator=g).to(torch.bfloat16).cuda()
+    scale, offset = (torch.rand(H, N, generator=g) + 0.5).cuda(), (torch.randn(H, N, generator=g) * 0.3).cuda()
+    op.algo = AUTO
+    y, sT = op(r, k, v, w, u, return_state=True, init_state=s0)
+    out, sT2 = op.forward_gn_gate(r, k, v, w, u, gate, scale, offset, 64e-5, return_state=True, init_state=s0)
+    torch.cuda.synchronize()
+    assert torch.equal(sT, sT2)
+    x = F.layer_norm(y.float().reshape(B, T, H, N), (N,), None, None, 64e-5)
+    want = ((x * scale + offset).reshape(B, T, H * N) * gate.float())
+    err = float((out.float() - want).abs().max()) / float(want.abs().max())
+    assert err <= 1e-2, err
+    assert bool(torch.isfinite(out.float()).all())
+
+
+def test_config2_state_gradients_across_a_cut(op):
+    # B=8 C=2048 at T=1024 cut into 512 + 512: with the state and its gradient handed across the cut
+    # the chunked bf16 kernels give the gradients of the uncut call (to bf16 rounding of y and the
+    # state's bf16 operands)
+    from oracle import wkv6_ref
+    B, T, H, N, cut = 8, 1024, 32, 64, 512
+    print("config 2 size, state gradients across a cut", flush=True)
+    ins = wkv6_ref.make_inputs(B, T, H, N, 4)
+    r, k, v, w, u, gy = (x.to(torch.bfloat16).cuda().contiguous() for x in ins[:6])
+    op.algo = AUTO
+    whole = [x.clone().requires_grad_(True) for x in (r, k, v, w, u)]
+    y, _ = op(*whole)
+    g_whole = torch.autograd.grad((y.float() * gy.float()).sum(), whole)
+    parts = [x.clone().requires_grad_(True) for x in (r, k, v, w, u)]
+    a = [x[:, :cut].contiguous() for x in parts[:4]] + [parts[4]]
+    b = [x[:, cut:].contiguous() for x in parts[:4]] + [parts[4]]
+    ya, sa = op(*a, return_state=True)
+    yb, _ = op(*b, return_state=True, init_state=sa)
+    g_parts = torch.autograd.grad((torch.cat([ya, yb], 1).float() * gy.float()).sum(), parts)
+    torch.cuda.synchronize()
+    for name, x, z in zip("gr gk gv gw gu".split(), g_parts, g_whole):
+        assert bool(torch.isfinite(x.float()).all())
+        err = float((x.float() - z.float()).abs().max()) / float(z.float().abs().max())
+        assert err <= 1e-2, (name, err)
