@@ -129,6 +129,26 @@ def bench_stateful(a):
         st, _native.BF16, _native.F32, B, Tp, C, H, 1, None, P(pre[0]), P(pre[1]), P(pre[2]), P(pre[3]), P(u), P(h0),
         P(gate), P(gn_scale), P(gn_offset), 64e-5, P(yp), P(sa))), 20)
 
+    # one long sequence alone on the chip (B=1, T=4096): as one pass, and as time segments side by
+    # side (what the optional forward workspace enables)
+    T1 = 4096
+    g1 = torch.Generator().manual_seed(a.seed + 1)
+    solo = [torch.randn(1, T1, C, generator=g1).to(torch.bfloat16).to(dev) for _ in range(3)]
+    solo.append((torch.rand(1, T1, C, generator=g1) * 7 - 6).to(torch.bfloat16).to(dev))
+    solo = [solo[0], solo[1], solo[2], solo[3]]
+    y_solo = torch.empty(1, T1, C, dtype=torch.bfloat16, device=dev)
+    s_solo, s_solo_out = h0[:1].contiguous(), torch.empty_like(h0[:1])
+    n_ws = int(lib.wkv6_forward_workspace_bytes(_native.BF16, _native.ALGO_AUTO, 1, T1, C, H))
+    ws = torch.empty(max(n_ws, 16), dtype=torch.uint8, device=dev)
+
+    def solo_call(use_ws):
+        _native.check(lib.wkv6_forward_with_state_ex(st, _native.BF16, _native.F32, _native.ALGO_AUTO, 1, T1, C, H, 1, None,
+                                                     P(solo[0]), P(solo[1]), P(solo[2]), P(solo[3]), P(u), P(s_solo), P(y_solo),
+                                                     P(s_solo_out), P(ws) if use_ws else None, n_ws if use_ws else 0))
+
+    solo_one_ms = timed(lambda: solo_call(False), 20)
+    solo_seg_ms = timed(lambda: solo_call(True), 20) if n_ws else None
+
     def two_steps():
         call(one, 1, y1, sa, sb); call(one, 1, y1, sb, sa)
 
@@ -139,6 +159,7 @@ def bench_stateful(a):
         "config": {"workload": "c5: prefill T=512 then T=1 decode steps with carried state"},
         "prefill_Mtokens_per_s": B * Tp / (pre_ms * 1e-3) / 1e6, "prefill_ms": pre_ms,
         "prefill_with_group_norm_and_gate_ms": fused_ms,
+        "single_sequence_prefill": {"B": 1, "T": T1, "one_pass_ms": solo_one_ms, "in_time_segments_ms": solo_seg_ms},
         "decode_steps_per_s": 1.0 / (dec_ms * 1e-3), "decode_us_per_step": dec_ms * 1e3,
         "decode_state_GBps": state_bytes / (dec_ms * 1e-3) / 1e9,
         "decode_frac_of_hbm_peak": state_bytes / (dec_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,

@@ -52,15 +52,19 @@ int wkv6_last_status(void) { return g_last_status; }
 int wkv6_last_hip_error(void) { return g_last_hip_error; }
 
 size_t wkv6_forward_workspace_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
-    (void)dtype; (void)algo; (void)B; (void)T; (void)C; (void)H;
-    return 0;
+    if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
+    const bool chunk = (algo == WKV6_ALGO_CHUNK && chunk_possible(dtype, T, C)) ||
+                       (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
+    // optional: with it, a long sequence of few (batch, head) pairs runs as time segments side by side
+    return chunk ? wkv6::chunk_forward_segments_workspace_bytes(B, T, H) : 0;
 }
 
 static int forward_impl(void *stream, int dtype, int state_dtype, int algo,
                         int64_t B, int64_t T, int64_t C, int64_t H,
                         int has_init_state, const int64_t *state_map,
                         const void *r, const void *k, const void *v, const void *w, const void *u,
-                        const void *s, void *y, void *ys, void *saved) {
+                        const void *s, void *y, void *ys, void *saved,
+                        void *workspace = nullptr, size_t workspace_bytes = 0) {
     int rc = check_shape(dtype, B, T, C, H);
     if (rc != WKV6_OK) return rc;
     if (!r || !k || !v || !w || !u || !y) return WKV6_ERR_ARG;
@@ -76,6 +80,11 @@ static int forward_impl(void *stream, int dtype, int state_dtype, int algo,
                        (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
     if (!chunk)
         return finish(wkv6::scan_forward(st, dtype, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys));
+    if (!saved && workspace && aligned16(workspace)) {
+        const size_t need = wkv6::chunk_forward_segments_workspace_bytes(B, T, H);
+        if (need > 0 && workspace_bytes >= need)
+            return finish(wkv6::chunk_forward_segments_run(st, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys, workspace));
+    }
     return finish(wkv6::chunk_forward(st, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys, saved));
 }
 
@@ -84,9 +93,8 @@ int wkv6_forward_with_state_ex(void *stream, int dtype, int state_dtype, int alg
                                int has_init_state, const int64_t *state_map,
                                const void *r, const void *k, const void *v, const void *w, const void *u,
                                const void *s, void *y, void *ys, void *workspace, size_t workspace_bytes) {
-    (void)workspace; (void)workspace_bytes;
     return forward_impl(stream, dtype, state_dtype, algo, B, T, C, H, has_init_state, state_map, r, k, v, w, u, s, y, ys,
-                        nullptr);
+                        nullptr, workspace, workspace_bytes);
 }
 
 int wkv6_forward_gn_gate(void *stream, int dtype, int state_dtype,

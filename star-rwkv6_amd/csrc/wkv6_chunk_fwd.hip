@@ -76,6 +76,8 @@ struct FwdArgs {
     long long *dbg;
     int T, H;
     int nitems;      // B * H (batch, head) pairs; with kMulti a workgroup takes every gridDim.x-th of them
+    int split;       // 1, 2 or 4 workgroups per pair, each with the consumer waves of 4 / split column slices
+    float *dsum;     // null, or [4 tiles][pairs][64]: per pair, log2(e) * sum of exp(w) over the tokens of tile p of every chunk
     const bf16_t *r, *k, *v, *w, *u;
     const void *s0;
     const int64_t *map;
@@ -95,14 +97,14 @@ struct FwdArgs {
 // scaling), group 0 produces y for tiles 0 and 2, group 1 for tiles 1 and 3.
 // ------------------------------------------------------------------------------------------
 template <typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse, int GRP>
-__device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned char *smem, int q, int lane)
+__device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned char *smem, int bh0, int q, int lane)
 {
     const int T = a.T, H = a.H;
     const int g = lane >> 4, l16 = lane & 15;
     const int64_t C = (int64_t)H * kN;
     const int nchunk = (T + CL - 1) / CL;
     const int stride = (int)gridDim.x;
-    const int n_my = kMulti ? (a.nitems - (int)blockIdx.x + stride - 1) / stride : 1;
+    const int n_my = kMulti ? (a.nitems - bh0 + stride - 1) / stride : 1;
     const Ts *s0 = reinterpret_cast<const Ts *>(a.s0);
     // initial state of a (batch, head) pair as stored (converted when the pair starts)
     Ts Sraw[16];
@@ -115,10 +117,10 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) Sraw[4 * m + rr] = p[(16 * m + 4 * g + rr) * kN];
     };
-    if (s0 != nullptr) request_state((int)blockIdx.x);
+    if (s0 != nullptr) request_state(bh0);
     WKV6_FSTAMP_DECL;
     int it = 0;   // chunk visits of this workgroup so far: picks the LDS buffers
-    for (int n = 0, bh = (int)blockIdx.x; n < n_my; ++n, bh += stride) {
+    for (int n = 0, bh = bh0; n < n_my; ++n, bh += stride) {
         const int b = bh / H, h = bh - b * H;
         const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
         f32x4 S[4];
@@ -166,7 +168,7 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
                 f32x4 U[4];
 #pragma unroll
                 for (int m = 0; m < 4; ++m) U[m] = mfma16(tile_frag_tok(kt, 16 * m, 16 * p, l16, g), vf, (f32x4){0.f, 0.f, 0.f, 0.f});
-                if ((p & 1) == GRP) {
+                if ((p & 1) == GRP && (kFuse || a.y != nullptr)) {   // (no y wanted: a pass that only builds the state)
                     const int row = 16 * p + l16;
                     const bf16x8 rf0 = tile_frag_ch(rt, row, 0, g), rf1 = tile_frag_ch(rt, row, 1, g);
                     const bf16x8 kf0 = tile_frag_ch(kt, row, 0, g), kf1 = tile_frag_ch(kt, row, 1, g);
@@ -232,7 +234,7 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
 // Loader / producer, lane = channel: wave p <-> tile p of every chunk.
 // ------------------------------------------------------------------------------------------
 template <bool kRagged, bool kMulti, bool kFuse>
-__device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *smem, int *s_wild, int pw, int lane)
+__device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *smem, int *s_wild, int bh0, int part, int pw, int lane)
 {
     constexpr int NT = 16;   // tokens per wave and chunk
     const int T = a.T, H = a.H;
@@ -241,7 +243,7 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
     const int64_t C = (int64_t)H * kN;
     const int nchunk = (T + CL - 1) / CL;
     const int stride = (int)gridDim.x;
-    const int n_my = kMulti ? (a.nitems - (int)blockIdx.x + stride - 1) / stride : 1;
+    const int n_my = kMulti ? (a.nitems - bh0 + stride - 1) / stride : 1;
     const int nvisit = n_my * nchunk;   // chunk visits of this workgroup, pair after pair
     const uint32_t rowbytes = (uint32_t)C * 2u;
     const uint32_t lds0 = lds_address(smem);
@@ -250,7 +252,7 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
     const uint32_t lpiece = (uint32_t)(((lane & 7) ^ lrow) << 4);
     // The load stream and the preparation stream each walk the visits in order; `ld_*` / `pp_*` are
     // the (pair, chunk) the next load / preparation belongs to.
-    int ld_c = 0, ld_bh = (int)blockIdx.x, ld_h = 0;
+    int ld_c = 0, ld_bh = bh0, ld_h = 0;
     const bf16_t *rb, *kb_, *vb, *wb, *gb = nullptr;   // uniform: this pair's first row (gb: gate, fused output stage)
     auto point_loads = [&]() {
         const int b = ld_bh / H, h = ld_bh - b * H;
@@ -304,7 +306,7 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
     // Fused output stage for the chunk the consumers staged during the previous visit; wave p takes
     // tile p, lane = channel:  out = ((y - mean) * rstd * gn_scale + gn_offset) * gate, mean and
     // variance over the head's 64 channels of a token (two passes, like a layer norm).
-    int fl_c = 0, fl_bh = (int)blockIdx.x;
+    int fl_c = 0, fl_bh = bh0;
     bf16_t *ob = nullptr;
     auto point_output = [&]() {
         const int b = fl_bh / H, h = fl_bh - b * H;
@@ -339,8 +341,9 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
         }
         if (++fl_c == nchunk && kMulti) { fl_c = 0; fl_bh += stride; if (fl_bh < a.nitems) point_output(); }
     };
-    int pp_c = 0, pp_n = 0, pp_h = (int)blockIdx.x % H;
+    int pp_c = 0, pp_n = 0, pp_h = bh0 % H;
     float uc = load1(a.u + pp_h * kN + ch);
+    float dacc = 0.f;   // base-2 decay exponent summed over this wave's tiles of the current pair
     const float kLog2Log2e = 0.5287663729448977f;   // log2(log2(e)): exp(w) log2(e) = 2^(w log2(e) + this)
     auto prepare = [&](int it) {   // visit `it` = the preparation stream's current (pair, chunk)
         const unsigned char *raw = smem + FwdLds::kRawRKW + (it & 1) * 3 * kTileBytes;
@@ -381,13 +384,18 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
         if (__builtin_amdgcn_ballot_w64(!(cs2 <= kWildLimit * kLog2e)) != 0ull) {
             if (lane == 0) s_wild[pp_n] = 1;
         }
+        dacc += cs2;
         reinterpret_cast<float *>(op + FwdLds::kOpG)[p * kN + ch] = pa;
         const float tot = transpose_reduce16(pr, lane);
         if ((lane & 3) == 0) reinterpret_cast<float *>(op + FwdLds::kOpRuk)[16 * p + ((lane >> 2) & 15)] = tot;
+        if (pp_c + 1 == nchunk && a.dsum != nullptr && part == 0) {   // the pair's total decay, this wave's tiles
+            a.dsum[((int64_t)p * a.nitems + (bh0 + pp_n * stride)) * kN + ch] = dacc;
+            dacc = 0.f;
+        }
         if (++pp_c == nchunk && kMulti) {   // the next preparation opens the next pair: its head's u
             pp_c = 0; ++pp_n;
             if (pp_n < n_my) {
-                pp_h = ((int)blockIdx.x + pp_n * stride) % H;
+                pp_h = (bh0 + pp_n * stride) % H;
                 uc = load1(a.u + pp_h * kN + ch);
             }
         }
@@ -465,18 +473,28 @@ __global__ __launch_bounds__(kFwdThreads) void chunk_fwd_kernel(FwdArgs a)
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int role = wave >> 2, q = wave & 3;
-    if (role == 0) fwd_producer<kRagged, kMulti, kFuse>(a, smem, s_wild, wave, lane);
-    else if (role == 1) fwd_consumer<Ts, kSave, kRagged, kMulti, kFuse, 0>(a, smem, q, lane);
-    else fwd_consumer<Ts, kSave, kRagged, kMulti, kFuse, 1>(a, smem, q, lane);
+    // With fewer pairs than compute units a pair is shared by `split` workgroups: the value columns of
+    // the state are independent of each other, so each workgroup carries the consumer waves of its
+    // 4 / split column slices (and repeats the operand preparation, which does not depend on them).
+    const int split = kMulti || kFuse ? 1 : a.split;
+    const int bh0 = (int)blockIdx.x / split, part = (int)blockIdx.x - bh0 * split;
+    const int nq = 4 / split;   // consumer waves per group
+    if (wave < 4) {
+        fwd_producer<kRagged, kMulti, kFuse>(a, smem, s_wild, bh0, part, wave, lane);
+    } else {
+        const int cw = wave - 4, grp = cw / nq, q = part * nq + (cw - grp * nq);
+        if (grp == 0) fwd_consumer<Ts, kSave, kRagged, kMulti, kFuse, 0>(a, smem, bh0, q, lane);
+        else fwd_consumer<Ts, kSave, kRagged, kMulti, kFuse, 1>(a, smem, bh0, q, lane);
+    }
     // exact second pass for every pair of this workgroup that had a tile leave the representable range
+    // (workgroups sharing a pair all see the same flags and all redo the whole pair: the same values)
     __threadfence_block();   // workgroup scope is enough (and a device-scope fence would write back the L2)
     __syncthreads();
     const int stride = (int)gridDim.x;
-    const int n_my = kMulti ? (a.nitems - (int)blockIdx.x + stride - 1) / stride : 1;
+    const int n_my = kMulti ? (a.nitems - bh0 + stride - 1) / stride : 1;
     for (int n = 0; n < n_my; ++n) {
         if (!s_wild[n]) continue;   // uniform over the workgroup
-        const int bh = (int)blockIdx.x + n * stride;
+        const int bh = bh0 + n * stride;
         __syncthreads();
         scan_fwd_body<bf16_t, bf16_t, Ts>(*reinterpret_cast<ScanFwdLds *>(smem), bh / a.H, bh % a.H, a.T, a.H, a.r, a.k, a.v, a.w, a.u,
                                           reinterpret_cast<const Ts *>(a.s0), a.map, kFuse ? a.out : a.y, reinterpret_cast<Ts *>(a.sT));
@@ -507,7 +525,8 @@ static hipError_t launch_fwd(hipStream_t st, const FwdArgs &a, unsigned grid) {
     const size_t lds = kFuse ? FwdLds::kBytesFused : FwdLds::kBytes;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kFwdThreads), lds, st, a);
+    const int split = kMulti || kFuse ? 1 : a.split;
+    hipLaunchKernelGGL(kern, dim3(grid * split), dim3((4 + 8 / split) * 64), lds, st, a);
     return hipGetLastError();
 }
 template <typename Ts, bool kSave, bool kRagged, bool kFuse>
@@ -526,24 +545,26 @@ static hipError_t launch_fwd_fused(hipStream_t st, const FwdArgs &a, bool ragged
 
 // One workgroup per pair while they all fit on the chip at once; beyond that one workgroup per
 // compute unit (more only if a workgroup would otherwise get more pairs than it keeps flags for).
-static unsigned forward_grid(int64_t pairs, bool *multi) {
+static unsigned forward_grid(int64_t pairs, bool *multi, int *split) {
     const int64_t cus = compute_units();
     *multi = pairs > cus;
+    *split = pairs * 4 <= cus ? 4 : pairs * 2 <= cus ? 2 : 1;
     return (unsigned)(!*multi ? pairs : (pairs + cus * kMaxPairsPerWorkgroup - 1) / (cus * kMaxPairsPerWorkgroup) * cus);
 }
 
 hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u,
-                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states)
+                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states, float *dsum)
 {
     FwdArgs a = {};
+    a.dsum = dsum;
     a.T = (int)T; a.H = (int)H; a.nitems = (int)(B * H);
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
     a.s0 = s0; a.map = map; a.y = (bf16_t *)y; a.sT = sT; a.ckpt = (float *)saved_states;
     a.arrivals = saved_states ? reinterpret_cast<int *>(reinterpret_cast<char *>(saved_states) + chunk_backward_workspace_bytes(B, T, H)) : nullptr;
     a.dbg = saved_states ? reinterpret_cast<long long *>((float *)saved_states + (size_t)(B * H) * ((T + CL - 1) / CL) * kN * kN + 1024) : nullptr;
     bool multi;
-    const unsigned grid = forward_grid(B * H, &multi);
+    const unsigned grid = forward_grid(B * H, &multi, &a.split);
     const bool save = saved_states != nullptr, ragged = (T % CL) != 0;
     return state_dtype == kF32 ? launch_fwd<float>(st, a, save, ragged, multi, grid)
                                : launch_fwd<bf16_t>(st, a, save, ragged, multi, grid);
@@ -560,10 +581,97 @@ hipError_t chunk_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64
     a.s0 = s0; a.map = map; a.sT = sT;
     a.gate = (const bf16_t *)gate; a.gn_scale = gn_scale; a.gn_offset = gn_offset; a.gn_eps = gn_eps; a.out = (bf16_t *)out;
     bool multi;
-    const unsigned grid = forward_grid(B * H, &multi);
+    const unsigned grid = forward_grid(B * H, &multi, &a.split);
+    a.split = 1;   // the output stage needs a chunk's whole rows in one workgroup
     const bool ragged = (T % CL) != 0;
     return state_dtype == kF32 ? launch_fwd_fused<float>(st, a, ragged, multi, grid)
                                : launch_fwd_fused<bf16_t>(st, a, ragged, multi, grid);
+}
+
+// ------------------------------------------------------------------------------------------
+// Long sequences, few pairs: time cut into segments that run side by side.
+//
+// With fewer (batch, head) pairs than half the compute units most of the chip would idle while each
+// pair walks its sequence alone.  The map from a segment's incoming state to its outgoing state is
+// affine, S_out = D o S_in + U with D[j] = exp(-sum_t exp(w_t[j])) over the segment and U the state
+// the segment builds from zero, so: (A) every segment runs from a zero state (all segments at once;
+// a (B,T,C) tensor cut into P equal segments IS a (B*P, T/P, C) tensor; no y in this pass) and leaves
+// U and, from the producer waves, the exponent of D; (B) a tiny kernel chains the P affine maps per pair,
+// leaving each segment's true incoming state where its U was (and the final state); (C) every
+// segment runs again from its true state and writes y.  Twice the forward work on P times the
+// workgroups.
+// ------------------------------------------------------------------------------------------
+template <typename Ts>
+__global__ __launch_bounds__(256) void segment_chain_kernel(int P, int H, const Ts *__restrict__ s0, const int64_t *__restrict__ map,
+                                                            const float *__restrict__ dsum, float *__restrict__ states, Ts *__restrict__ sT)
+{
+    // one workgroup per (batch, head); thread: key row j = tid >> 2, value columns 16 (tid & 3) .. +15.
+    // states[(b*P + seg), h] holds U on entry and the segment's incoming state on exit.
+    const int b = blockIdx.x / H, h = blockIdx.x - b * H;
+    const int j = threadIdx.x >> 2, i0 = (threadIdx.x & 3) * 16;
+    float S[16];
+    if (s0) {
+        const int64_t row = map ? map[b] : (int64_t)b;
+        const Ts *p = s0 + ((row * H + h) * kN + j) * kN + i0;
+#pragma unroll
+        for (int e = 0; e < 16; e += 4) { float x[4]; load4(p + e, x); S[e] = x[0]; S[e + 1] = x[1]; S[e + 2] = x[2]; S[e + 3] = x[3]; }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) S[e] = 0.f;
+    }
+    for (int seg = 0; seg < P; ++seg) {
+        const int64_t vrow = (int64_t)b * P + seg;
+        float *u = states + ((vrow * H + h) * kN + j) * kN + i0;
+        const int64_t vp = vrow * H + h, np = (int64_t)gridDim.x * P;   // this segment's pair, pairs of all segments
+        const float d = exp2_fast(-((dsum[vp * kN + j] + dsum[(np + vp) * kN + j]) + (dsum[(2 * np + vp) * kN + j] + dsum[(3 * np + vp) * kN + j])));
+#pragma unroll
+        for (int e = 0; e < 16; e += 4) {
+            const float4 x = *reinterpret_cast<const float4 *>(u + e);
+            *reinterpret_cast<float4 *>(u + e) = make_float4(S[e], S[e + 1], S[e + 2], S[e + 3]);
+            S[e] = fmaf(S[e], d, x.x); S[e + 1] = fmaf(S[e + 1], d, x.y);
+            S[e + 2] = fmaf(S[e + 2], d, x.z); S[e + 3] = fmaf(S[e + 3], d, x.w);
+        }
+    }
+    if (sT) {
+        Ts *p = sT + (((int64_t)b * H + h) * kN + j) * kN + i0;
+#pragma unroll
+        for (int e = 0; e < 16; e += 4) store4(p + e, S[e], S[e + 1], S[e + 2], S[e + 3]);
+    }
+}
+
+// Number of segments for this shape (1 = not worth it / not possible): the pairs times the segments
+// should still fit the chip once, a segment is a whole number of chunks and at least four of them.
+int chunk_forward_segments(int64_t B, int64_t T, int64_t H) {
+    const int64_t pairs = B * H, cus = compute_units();
+    // (two passes over T / P tokens and two more launches against one pass over T: nothing to gain
+    // below four segments or on short sequences)
+    if (T < 2048) return 1;
+    for (int P = 8; P >= 4; P >>= 1)
+        if (pairs * P <= cus && T % (P * CL) == 0) return P;
+    return 1;
+}
+size_t chunk_forward_segments_workspace_bytes(int64_t B, int64_t T, int64_t H) {
+    const int P = chunk_forward_segments(B, T, H);
+    return P <= 1 ? 0 : (size_t)(B * P * H) * (kN * kN + 4 * kN) * sizeof(float);
+}
+
+hipError_t chunk_forward_segments_run(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
+                                      const void *r, const void *k, const void *v, const void *w, const void *u,
+                                      const void *s0, const int64_t *map, void *y, void *sT, void *workspace)
+{
+    const int P = chunk_forward_segments(B, T, H);
+    const int64_t L = T / P, rows = B * P;
+    float *states = (float *)workspace, *dsum = states + rows * H * kN * kN;
+    hipError_t e = chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, nullptr, nullptr, nullptr, states, nullptr, dsum);
+    if (e != hipSuccess) return e;
+    if (state_dtype == kF32)
+        hipLaunchKernelGGL(segment_chain_kernel<float>, dim3((unsigned)(B * H)), dim3(256), 0, st, P, (int)H,
+                           (const float *)s0, map, (const float *)dsum, states, (float *)sT);
+    else
+        hipLaunchKernelGGL(segment_chain_kernel<bf16_t>, dim3((unsigned)(B * H)), dim3(256), 0, st, P, (int)H,
+                           (const bf16_t *)s0, map, (const float *)dsum, states, (bf16_t *)sT);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    return chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, states, nullptr, y, nullptr, nullptr);
 }
 
 }  // namespace wkv6

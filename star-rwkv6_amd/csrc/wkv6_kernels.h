@@ -34,7 +34,16 @@ hipError_t scan_backward_state(hipStream_t st, int dtype, int64_t B, int64_t T, 
 // --- chunk-parallel MFMA form, bf16 tensors only (wkv6_chunk.hip) ---
 hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u,
-                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states);
+                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states,
+                         float *dsum = nullptr);   // dsum: see chunk_forward_segments_run
+
+// Few pairs, long sequence: the forward as P time segments side by side (two passes joined by the
+// affine map of a segment's state).  chunk_forward_segments = P for the shape (1 = does not apply).
+int chunk_forward_segments(int64_t B, int64_t T, int64_t H);
+size_t chunk_forward_segments_workspace_bytes(int64_t B, int64_t T, int64_t H);
+hipError_t chunk_forward_segments_run(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
+                                      const void *r, const void *k, const void *v, const void *w, const void *u,
+                                      const void *s0, const int64_t *map, void *y, void *sT, void *workspace);
 
 // forward with the layer's output stage fused in: out = (group_norm_head(y) * gn_scale + gn_offset) * gate
 hipError_t chunk_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,

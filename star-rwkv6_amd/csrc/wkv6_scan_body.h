@@ -134,7 +134,7 @@ __device__ __forceinline__ void scan_fwd_body(ScanFwdLds &L, int b, int h, int T
                     const float4 c = *reinterpret_cast<const float4 *>(&s_part[qq][t][c4]);
                     a.x += c.x; a.y += c.y; a.z += c.z; a.w += c.w;
                 }
-                store4(y + base + (int64_t)(t0 + t) * C + c4, a.x, a.y, a.z, a.w);
+                if (y) store4(y + base + (int64_t)(t0 + t) * C + c4, a.x, a.y, a.z, a.w);
             }
         }
         // the next tile's LDS writes touch s_r/s_k/s_v/s_d/s_ruk only, all readers of which are

@@ -110,10 +110,13 @@ def _forward_with_state(B, T, C, H, state_map, r, k, v, w, u, init_state, algo=_
         y = torch.empty((B, T, C), device=r.device, dtype=odt)
         ys = torch.empty((B, H, N, N), device=r.device, dtype=sdt)
         with torch.cuda.device(r.device):
+            # optional workspace: lets a long sequence of few (batch, head) pairs run as time segments
+            n = lib.wkv6_forward_workspace_bytes(_DTYPE_CODE[r.dtype], algo, B, T, C, H)
+            ws = torch.empty(int(n), device=r.device, dtype=torch.uint8) if n else None
             _native.check(lib.wkv6_forward_with_state_ex(
                 _stream(), _DTYPE_CODE[r.dtype], _DTYPE_CODE[sdt], algo, B, T, C, H,
                 int(init_state is not None), _ptr(state_map),
-                _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(init_state), _ptr(y), _ptr(ys), None, 0))
+                _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(init_state), _ptr(y), _ptr(ys), _ptr(ws), n))
     return y, ys
 
 

@@ -445,6 +445,43 @@ def test_backpropagation_over_two_pieces_equals_one_piece(op):
         assert err <= 2e-5, (name, err)
 
 
+# Few pairs, long sequence: with the optional forward workspace the sequence runs as time segments
+# side by side (two passes joined by the affine state map of a segment).
+@pytest.mark.parametrize("B,T,H,sdt", [(1, 2048, 2, torch.float32), (2, 2304, 1, torch.bfloat16), (3, 4096, 5, torch.float32), (12, 2048, 4, torch.float32)])
+def test_forward_in_time_segments(op, oracle, B, T, H, sdt):
+    from rwkv_kernel import _native
+    N = 64
+    lib = _native.load()
+    assert lib.wkv6_forward_workspace_bytes(_native.BF16, CHUNK, B, T, H * N, H) > 0
+    assert lib.wkv6_forward_workspace_bytes(_native.BF16, CHUNK, 8, 1024, 2048, 32) == 0    # fills the chip as it is
+    assert lib.wkv6_forward_workspace_bytes(_native.BF16, CHUNK, B, T + 64, H * N, H) == 0  # no equal segments
+    ins = oracle.make_inputs(B, T, H, N, 60 + B, with_state=True)
+    dev, ref = cast_inputs(ins[:5], torch.bfloat16)
+    kinds = min(2, B)
+    s_dev, s_ref = cast_inputs([ins[6][:kinds]], sdt)
+    smap = [(b + 1) % kinds for b in range(B)]
+    op.algo = CHUNK
+    y, sT = op(*dev, return_state=True, init_state=s_dev[0], state_map=smap)
+    torch.cuda.synchronize()
+    y_ref, sT_ref = oracle.forward_c(*ref, N, s_ref[0], smap)
+    check_close("y", y, y_ref, torch.bfloat16)
+    check_close("sT", sT, sT_ref, torch.bfloat16)
+    # a segment that leaves the chunked form's range is redone exactly in both passes
+    ins[3][0, T // 2 + 30:T // 2 + 50, 20:40] = 6.0
+    dev2, ref2 = cast_inputs(ins[:5], torch.bfloat16)
+    y2, sT2 = op(*dev2, return_state=True, init_state=s_dev[0], state_map=smap)
+    y2_ref, sT2_ref = oracle.forward_c(*ref2, N, s_ref[0], smap)
+    check_close("y with an exact segment", y2, y2_ref, torch.bfloat16)
+    check_close("sT with an exact segment", sT2, sT2_ref, torch.bfloat16)
+    # and from a zero state, against the same call without the workspace (the torch flavour's
+    # stateless forward does not pass one)
+    y0, s0T = op(*dev, return_state=True)
+    y1, _ = op(*dev)
+    torch.cuda.synchronize()
+    check_close("y vs one pass", y0, to_np(y1).astype(np.float64), torch.bfloat16)
+    check_close("sT zero", s0T, oracle.forward_c(*ref, N)[1], torch.bfloat16)
+
+
 def test_chunk_matches_scan_on_padding_mask(op, oracle):
     B, T, H, N = 1, 96, 1, 64
     ins = oracle.make_inputs(B, T, H, N, 54)
