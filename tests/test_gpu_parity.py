@@ -290,7 +290,7 @@ def test_chunk_falls_back_on_extreme_decay(op, oracle):
 # More (batch, head) pairs than the chip has compute units: a forward workgroup then runs several
 # pairs back to back through one pipeline (the state, the head's u, the saved states and the
 # fallback flag all switch at the pair boundaries).
-@pytest.mark.parametrize("B,T,H", [(75, 64, 4), (43, 150, 7), (300, 32, 1)])
+@pytest.mark.parametrize("B,T,H", [(75, 64, 4), (43, 150, 7), (300, 32, 1), (1100, 16, 8)])   # the last: more than 32 pairs per compute unit
 def test_chunk_many_pairs_fwd_bwd_bf16(op, oracle, B, T, H):
     _case(op, oracle, B, T, H, 90 + T, torch.bfloat16, CHUNK)
 
