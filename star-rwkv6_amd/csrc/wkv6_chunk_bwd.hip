@@ -42,14 +42,15 @@ constexpr int CL = 64;   // tokens per chunk
 
 // LDS map of the backward kernel (byte offsets into the dynamic block); "item" = one chunk visit
 struct BwdLds {
-    static constexpr int kRawRK = 0;                                   // [item & 1][r, k] raw tiles
-    static constexpr int kRawW = kRawRK + 2 * 2 * kTileBytes;          // [item % 3] raw w tiles
+    static constexpr int kRawRK = 0;                                   // [item % 3][r, k] raw tiles, turned into R~, K~ in place
+    static constexpr int kRawW = kRawRK + 3 * 2 * kTileBytes;          // [item % 3] raw w tiles
     static constexpr int kRawVG = kRawW + 3 * kTileBytes;              // [item % 3][v, gy] raw tiles
     static constexpr int kOp = kRawVG + 3 * 2 * kTileBytes;            // [item & 1] operand blocks
-    static constexpr int kOpRt = 0, kOpKt = kTileBytes, kOpFr = 2 * kTileBytes;   // R~, K~, exp(-c_t) tiles
-    static constexpr int kOpG = 3 * kTileBytes, kOpRuk = kOpG + 4 * kN * 4;       // g[4][64], ruk[64] (fp32)
+    static constexpr int kOpFr = 0;                                               // exp(-c_t) tile
+    static constexpr int kOpG = kTileBytes, kOpRuk = kOpG + 4 * kN * 4;           // g[4][64], ruk[64] (fp32)
     static constexpr int kOpBytes = kOpRuk + CL * 4;
-    static constexpr int kVgy = kOp + 2 * kOpBytes;                    // [8 consumer waves][16] fp32: <v_t, gy_t>
+    static constexpr int kState = kOp + 2 * kOpBytes;                  // [item & 1] saved forward state of the chunk, bf16 [j][i] as a tile
+    static constexpr int kVgy = kState + 2 * kTileBytes;                    // [8 consumer waves][16] fp32: <v_t, gy_t>
     static constexpr int kGu = kVgy + 8 * 16 * 4;                      // [64] fp32: gu partial of consumer group 1
     static constexpr int kBytes = kGu + kN * 4;
 };
@@ -111,7 +112,7 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
             __syncthreads();
             if (GRP != 0) continue;
             const unsigned char *op = smem + BwdLds::kOp + (item & 1) * BwdLds::kOpBytes;
-            const unsigned char *kt = op + BwdLds::kOpKt;
+            const unsigned char *kt = smem + BwdLds::kRawRK + (item % 3) * 2 * kTileBytes + kTileBytes;
             const float *gg = reinterpret_cast<const float *>(op + BwdLds::kOpG);
             const unsigned char *vt = smem + BwdLds::kRawVG + (item % 3) * 2 * kTileBytes;
             bf16_t *dst = ck + (int64_t)c * (kN * kN) + col * kN;
@@ -145,10 +146,11 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     float gu_acc = 0.f;
     bf16_t *gr_h = a.gr + base, *gk_h = a.gk + base, *gw_h = a.gw + base;
     const uint32_t rowbytes = (uint32_t)C * 2u;
-    // Checkpointed forward state as loaded (packed bf16), requested one visit ahead.  A wave's loads
-    // and stores complete in program order, so this load is not reported complete before the
-    // gradient stores issued ahead of it have reached the L2; the request therefore goes out as early
-    // in the visit as the registers allow, and the wait for it comes at the very end.
+    // Saved forward state of a chunk as packed bf16: Sraw[m] = S^T[i = 16m + 4g .. +3][j = col].  With
+    // the states left by the forward pass it comes out of LDS, where the producer waves put the
+    // chunk's block (the consumer waves then issue no global load at all: their loads would queue
+    // behind their own gradient stores, and a wave's memory operations complete in program order);
+    // with kSweepStates this kernel wrote the states itself a moment ago and reads them back here.
     uint2 Sraw[4];
     auto load_state = [&](int c, uint2 (&dst)[4]) {
         if ((WKV6_ABLATE & 2) && T > 0) { dst[0] = dst[1] = dst[2] = dst[3] = make_uint2(0u, 0u); return; }
@@ -157,10 +159,7 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
         for (int m = 0; m < 4; ++m) dst[m] = *reinterpret_cast<const uint2 *>(src + 16 * m + 4 * g);
     };
     // One chunk visit.  All four tiles are always processed (tokens past the end were prepared as
-    // r = k = 0, decay 1, so they leave both states alone and contribute nothing), which keeps the
-    // body free of branches that change the number of memory operations: the wait for the
-    // prefetched state of the next visit (the fake use at the end) is then counted exactly instead
-    // of draining this wave's stores every chunk.
+    // r = k = 0, decay 1, so they leave both states alone and contribute nothing).
     // gr, gk, gw of the 4 tokens from `tfirst` on, channel col, as packed pairs {gr01, gk01, gw01, gr23, gk23, gw23}
     auto store_tile = [&](int tfirst, const uint32_t (&pk)[6]) {
 #pragma unroll
@@ -180,20 +179,28 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
         WKV6_STAMP();
         __syncthreads();
         WKV6_STAMP();
-        // with kSweepStates the checkpoints were written by this kernel a moment ago: read them
-        // here; otherwise the load was issued two visits ago
-        if (kSweepStates) load_state(c, Sraw);
+        if (kSweepStates) {
+            load_state(c, Sraw);
+        } else {
+            // row j = col of the state tile: values i = 32h + 4g .. +3 and 32h + 16 + 4g .. +3 per read pair
+            const unsigned char *stt = smem + BwdLds::kState + (item & 1) * kTileBytes;
+            const u32x4 lo = __builtin_bit_cast(u32x4, tile_frag_ch(stt, col, 0, g)), hi = __builtin_bit_cast(u32x4, tile_frag_ch(stt, col, 1, g));
+            Sraw[0] = make_uint2(lo[0], lo[1]); Sraw[1] = make_uint2(lo[2], lo[3]);
+            Sraw[2] = make_uint2(hi[0], hi[1]); Sraw[3] = make_uint2(hi[2], hi[3]);
+        }
         // Uniform block offsets of this item.  They pass through fresh_s() before every tile, which
         // keeps the compiler from forming (block + lane offset) for all tiles at once and holding
         // two dozen address registers across the chunk.
         int op_off = BwdLds::kOp + (item & 1) * BwdLds::kOpBytes;
+        int rk_off = BwdLds::kRawRK + (item % 3) * 2 * kTileBytes;
         int vg_off = BwdLds::kRawVG + (item % 3) * 2 * kTileBytes;
         int w_off = BwdLds::kRawW + (item % 3) * kTileBytes;
         const unsigned char *rt, *kt, *fr, *vt, *gyt, *wt;
         const float *gg;
         auto fresh_pointers = [&]() {
             op_off = fresh_s(op_off); vg_off = fresh_s(vg_off); w_off = fresh_s(w_off);
-            rt = smem + op_off + BwdLds::kOpRt; kt = smem + op_off + BwdLds::kOpKt; fr = smem + op_off + BwdLds::kOpFr;
+            rk_off = fresh_s(rk_off);
+            rt = smem + rk_off; kt = smem + rk_off + kTileBytes; fr = smem + op_off + BwdLds::kOpFr;
             gg = reinterpret_cast<const float *>(smem + op_off + BwdLds::kOpG);
             vt = smem + vg_off; gyt = vt + kTileBytes; wt = smem + w_off;
         };
@@ -210,9 +217,6 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
             SopL[0] = make_bf16x8(Sraw[0].x, Sraw[0].y, Sraw[1].x, Sraw[1].y);
             SopH[0] = make_bf16x8(Sraw[2].x, Sraw[2].y, Sraw[3].x, Sraw[3].y);
         }
-        // the registers of the packed state are free again: request the next visit's (chunk 0
-        // fetches itself once more, unused)
-        if (!kSweepStates) load_state(c > 0 ? c - 1 : 0, Sraw);
 #pragma unroll
         for (int p = 0; p < 3; ++p) {
             if (GRP == 1 && p == 2) continue;   // group 1 needs the states of tiles 0 and 2 only
@@ -355,17 +359,8 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
             WKV6_STAMP();
             __builtin_amdgcn_sched_barrier(0);
         }
-        // fake use of the next visit's state: the wait for its loads lands here, after this visit's
-        // stores in program order and with their number known
-        if (!kSweepStates) asm volatile("" : "+v"(Sraw[0]), "+v"(Sraw[1]), "+v"(Sraw[2]), "+v"(Sraw[3]));
         ++item;
     };
-    if (!kSweepStates && nchunk > 0) {
-        load_state(nchunk - 1, Sraw);
-        // have the first state arrive here: a wait for it inside the loop would be sized for this
-        // path (nothing younger in flight) and drain the stores on every visit
-        asm volatile("" : "+v"(Sraw[0]), "+v"(Sraw[1]), "+v"(Sraw[2]), "+v"(Sraw[3]));
-    }
     for (int c = nchunk - 1; c >= 0; --c) visit(c, Sraw);
     if (a.gs0 && GRP == 0) {   // the reverse state has arrived at t = 0: dL/dS_0
 #pragma unroll
@@ -406,7 +401,7 @@ __device__ __forceinline__ void bwd_gv_chunk(GvState &st, const BwdArgs &a, cons
     const int col = 16 * q + l16;
     f32x4 (&Gi)[4] = st.Gi;
     const unsigned char *op = smem + BwdLds::kOp + (item & 1) * BwdLds::kOpBytes;
-    const unsigned char *rt = op + BwdLds::kOpRt, *kt = op + BwdLds::kOpKt;
+    const unsigned char *rt = smem + BwdLds::kRawRK + (item % 3) * 2 * kTileBytes, *kt = rt + kTileBytes;
     const float *gg_ = reinterpret_cast<const float *>(op + BwdLds::kOpG);
     const float *ruk = reinterpret_cast<const float *>(op + BwdLds::kOpRuk);
     const unsigned char *gyt = smem + BwdLds::kRawVG + (item % 3) * 2 * kTileBytes + kTileBytes;
@@ -477,7 +472,7 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
         if ((WKV6_ABLATE & 1) && T > 0) return 0;
         const int tb = item_chunk(it) * CL + 16 * p;
         const bool full = item_full(it);
-        const uint32_t rk = lds0 + BwdLds::kRawRK + (it & 1) * 2 * kTileBytes + 16 * p * kTileRow;
+        const uint32_t rk = lds0 + BwdLds::kRawRK + (it % 3) * 2 * kTileBytes + 16 * p * kTileRow;
         const uint32_t ww = lds0 + BwdLds::kRawW + (it % 3) * kTileBytes + 16 * p * kTileRow;
         const uint32_t vg = lds0 + BwdLds::kRawVG + (it % 3) * 2 * kTileBytes + 16 * p * kTileRow;
 #pragma unroll
@@ -494,18 +489,38 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
         }
         return full ? 10 : 6;
     };
+    // The saved forward state of item `it` (phase 2 with the states left by the forward pass): the
+    // chunk's 64x64 bf16 block [j][i] is a tile with j in the place of the token; wave p brings rows
+    // 16p..16p+15.  It is requested ONE item ahead (two slots), ahead of the tile loads in the queue,
+    // and awaited at the end of the visit, behind the gv stores issued in between -- the consumer
+    // waves, which would otherwise load it behind their own gradient stores and wait for those to
+    // reach the L2, then have no load to wait for at all.
+    const bf16_t *ckb = reinterpret_cast<const bf16_t *>(a.ckpt + (int64_t)(b * H + h) * nchunk * (kN * kN));
+    auto issue_state = [&](int it) {
+        const bf16_t *src = ckb + (int64_t)item_chunk(it) * (kN * kN);
+        const uint32_t dst = lds0 + BwdLds::kState + (it & 1) * kTileBytes + 16 * p * kTileRow;
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+            load_rows8_to_lds(src, (uint32_t)((16 * p + 8 * hf + lrow) * kTileRow) + lpiece, dst + 8 * hf * kTileRow);
+    };
     // Waits for this wave's tile loads of one item.  `n` = operations issued after them: the loads
     // of the following item and, with the gv role on this wave, the 16 gv stores of the chunk
     // visit in between (memory operations of a wave complete in program order; the stores are left
     // in flight -- waiting for them costs more than a microsecond per chunk under load).
     auto wait_younger = [&](int n) {
         if ((WKV6_ABLATE & 1) && T > 0) return;
-        switch (n) {
+        switch (n) {   // tile loads {0, 6, 10} + state loads {0, 2} + gv stores {0, 16}
+        case 28: wait_loads<28>(); break;
         case 26: wait_loads<26>(); break;
+        case 24: wait_loads<24>(); break;
         case 22: wait_loads<22>(); break;
+        case 18: wait_loads<18>(); break;
         case 16: wait_loads<16>(); break;
+        case 12: wait_loads<12>(); break;
         case 10: wait_loads<10>(); break;
+        case 8: wait_loads<8>(); break;
         case 6: wait_loads<6>(); break;
+        case 2: wait_loads<2>(); break;
         default: wait_loads<0>(); break;
         }
     };
@@ -519,11 +534,12 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
         const bool full = item_full(it);
         // lane addresses of the 8 swizzle phases in the three blocks this item uses (the row and tensor
         // offsets on top of them are instruction immediates)
-        const unsigned char *a_rk[8], *a_w[8];
+        unsigned char *a_rk[8];
+        const unsigned char *a_w[8];
         unsigned char *a_op[8];
 #pragma unroll
         for (int sw = 0; sw < 8; ++sw) {
-            a_rk[sw] = smem + (BwdLds::kRawRK + (it & 1) * 2 * kTileBytes + choff[sw]);
+            a_rk[sw] = smem + (BwdLds::kRawRK + (it % 3) * 2 * kTileBytes + choff[sw]);
             a_w[sw] = smem + (BwdLds::kRawW + (it % 3) * kTileBytes + choff[sw]);
             a_op[sw] = smem + (BwdLds::kOp + (it & 1) * BwdLds::kOpBytes + choff[sw]);
         }
@@ -558,10 +574,12 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
             const uint32_t pr2 = pack_bf16x2(xr[e], xr[e + 1]), pk2 = pack_bf16x2(xk[e], xk[e + 1]);
             const uint32_t pf2 = pack_bf16x2(fa[e], fa[e + 1]);
             unsigned char *o0 = a_op[e & 7] + e * kTileRow, *o1 = a_op[(e + 1) & 7] + (e + 1) * kTileRow;
-            *reinterpret_cast<uint16_t *>(o0 + BwdLds::kOpRt) = (uint16_t)pr2;
-            *reinterpret_cast<uint16_t *>(o1 + BwdLds::kOpRt) = (uint16_t)(pr2 >> 16);
-            *reinterpret_cast<uint16_t *>(o0 + BwdLds::kOpKt) = (uint16_t)pk2;
-            *reinterpret_cast<uint16_t *>(o1 + BwdLds::kOpKt) = (uint16_t)(pk2 >> 16);
+            unsigned char *q0 = a_rk[e & 7] + e * kTileRow, *q1 = a_rk[(e + 1) & 7] + (e + 1) * kTileRow;
+            // R~ and K~ take the place of the raw r and k this lane read above
+            *reinterpret_cast<uint16_t *>(q0) = (uint16_t)pr2;
+            *reinterpret_cast<uint16_t *>(q1) = (uint16_t)(pr2 >> 16);
+            *reinterpret_cast<uint16_t *>(q0 + kTileBytes) = (uint16_t)pk2;
+            *reinterpret_cast<uint16_t *>(q1 + kTileBytes) = (uint16_t)(pk2 >> 16);
             *reinterpret_cast<uint16_t *>(o0 + BwdLds::kOpFr) = (uint16_t)pf2;
             *reinterpret_cast<uint16_t *>(o1 + BwdLds::kOpFr) = (uint16_t)(pf2 >> 16);
         }
@@ -576,6 +594,8 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     GvState gvst;
     gvst.init(a.gsT ? a.gsT + (int64_t)(b * H + h) * (kN * kN) : nullptr, 16 * p + (lane & 15), lane >> 4);
     WKV6_STAMP_DECL;
+    constexpr bool kStatesByLoad = !kSweepStates;   // (with kSweepStates the consumers read the states this kernel wrote itself)
+    if (kStatesByLoad && nitem > 0) issue_state(0);
     issue_loads(0);
     wait_younger(nitem > 1 ? issue_loads(1) : 0);
     prepare(0);
@@ -583,20 +603,24 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
         WKV6_STAMP();
         __syncthreads();
         WKV6_STAMP();
-        // free again: the raw r, k block of item `it` (read by this wave's prepare before the barrier)
-        // and the raw w, v, gy blocks of item it-1 (read by the other roles before the barrier)
+        // free again: the r, k block of item it-1 and the raw w, v, gy blocks of item it-1 (read by the
+        // other roles before the barrier), and the state tile of item it-1
+        const int state_loads = (kStatesByLoad && it + 1 < nitem) ? 2 : 0;
+        if (state_loads) issue_state(it + 1);
         const int younger = it + 2 < nitem ? issue_loads(it + 2) : 0;
         if (it + 1 < nitem) {
             WKV6_STAMP();
             // (with a ragged tail the number of gv stores issued is not fixed: wait for everything older)
             const int gv_stores = (!kRagged && it >= 1 && item_full(it - 1)) ? 16 : 0;
-            wait_younger(younger + gv_stores);
+            wait_younger(younger + state_loads + gv_stores);
             WKV6_STAMP();
             prepare(it + 1);
             WKV6_STAMP();
         }
         // the gv role, on the waves the operand preparation leaves partly idle
         if (item_full(it)) bwd_gv_chunk<kRagged>(gvst, a, smem, a.gv + base, rowbytes, item_chunk(it), it, p, lane);
+        // the next item's state has to be in LDS when the consumers pass the barrier
+        if (state_loads) wait_younger(younger + ((!kRagged && item_full(it)) ? 16 : 0));
         WKV6_STAMP();
     }
     wait_loads<0>();
