@@ -22,8 +22,9 @@
 //
 // Workgroup: one per (batch, head), 12 waves in four-wave roles (one wave of each role per SIMD):
 //   loader/producer (wave p <-> tile p, lane = channel): brings the raw r, k, w, v, gy rows of a
-//       chunk from global memory straight into LDS tiles two items ahead, and one item ahead turns
-//       r, k, w into the bf16 tiles R~, K~, exp(-c_t) plus g and the diagonal sum r u k; the same
+//       chunk from global memory straight into LDS tiles two items ahead (and the chunk's saved
+//       forward state one item ahead), and one item ahead turns r, k, w into the bf16 tiles R~, K~
+//       (written over the raw r, k), exp(-c_t) plus g and the diagonal sum r u k; the same
 //       waves then run the gv role (wave q <-> value columns 16q..): reverse state with rows j,
 //       produces gv;
 //   two consumer groups (wave q <-> key columns 16q..): reverse state with rows i, produce gr, gk,
@@ -119,7 +120,16 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
 #pragma unroll
             for (int m = 0; m < 4; ++m)
                 *reinterpret_cast<uint2 *>(dst + 16 * m + 4 * g) = make_uint2(pack_bf16x2(S[m][0], S[m][1]), pack_bf16x2(S[m][2], S[m][3]));
-            if (c + 1 == nchunk) continue;   // the state after the last chunk is never used
+            if (c + 1 == nchunk) {
+                // The state after the last chunk is never used.  The last chunk's own state is what
+                // phase 2 starts with: it goes straight into the LDS state tile of the next item
+                // (the producer waves load the tiles of all later items from the workspace).
+                unsigned char *stt = smem + BwdLds::kState + ((item + 1) & 1) * kTileBytes;
+#pragma unroll
+                for (int m = 0; m < 4; ++m)
+                    *reinterpret_cast<uint2 *>(stt + tile_off(col, 16 * m + 4 * g)) = make_uint2(pack_bf16x2(S[m][0], S[m][1]), pack_bf16x2(S[m][2], S[m][3]));
+                continue;
+            }
 #pragma unroll 1
             for (int p = 0; p < 4; ++p) {
                 const s16x4 kq = tile_frag_tok(kt, 16 * q, 16 * p, l16, g);
@@ -146,18 +156,12 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     float gu_acc = 0.f;
     bf16_t *gr_h = a.gr + base, *gk_h = a.gk + base, *gw_h = a.gw + base;
     const uint32_t rowbytes = (uint32_t)C * 2u;
-    // Saved forward state of a chunk as packed bf16: Sraw[m] = S^T[i = 16m + 4g .. +3][j = col].  With
-    // the states left by the forward pass it comes out of LDS, where the producer waves put the
-    // chunk's block (the consumer waves then issue no global load at all: their loads would queue
-    // behind their own gradient stores, and a wave's memory operations complete in program order);
-    // with kSweepStates this kernel wrote the states itself a moment ago and reads them back here.
+    // Saved forward state of a chunk as packed bf16: Sraw[m] = S^T[i = 16m + 4g .. +3][j = col].  It
+    // comes out of LDS, where the producer waves put the chunk's block from the workspace (written
+    // by the forward pass, or by phase 1 above).  The consumer waves issue no global load at all:
+    // their loads would queue behind their own gradient stores, and a wave's memory operations
+    // complete in program order.
     uint2 Sraw[4];
-    auto load_state = [&](int c, uint2 (&dst)[4]) {
-        if ((WKV6_ABLATE & 2) && T > 0) { dst[0] = dst[1] = dst[2] = dst[3] = make_uint2(0u, 0u); return; }
-        const bf16_t *src = ck + (int64_t)c * (kN * kN) + col * kN;
-#pragma unroll
-        for (int m = 0; m < 4; ++m) dst[m] = *reinterpret_cast<const uint2 *>(src + 16 * m + 4 * g);
-    };
     // One chunk visit.  All four tiles are always processed (tokens past the end were prepared as
     // r = k = 0, decay 1, so they leave both states alone and contribute nothing).
     // gr, gk, gw of the 4 tokens from `tfirst` on, channel col, as packed pairs {gr01, gk01, gw01, gr23, gk23, gw23}
@@ -179,14 +183,13 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
         WKV6_STAMP();
         __syncthreads();
         WKV6_STAMP();
-        if (kSweepStates) {
-            load_state(c, Sraw);
-        } else {
+        {
             // row j = col of the state tile: values i = 32h + 4g .. +3 and 32h + 16 + 4g .. +3 per read pair
             const unsigned char *stt = smem + BwdLds::kState + (item & 1) * kTileBytes;
             const u32x4 lo = __builtin_bit_cast(u32x4, tile_frag_ch(stt, col, 0, g)), hi = __builtin_bit_cast(u32x4, tile_frag_ch(stt, col, 1, g));
             Sraw[0] = make_uint2(lo[0], lo[1]); Sraw[1] = make_uint2(lo[2], lo[3]);
             Sraw[2] = make_uint2(hi[0], hi[1]); Sraw[3] = make_uint2(hi[2], hi[3]);
+            if ((WKV6_ABLATE & 2) && T > 0) Sraw[0] = Sraw[1] = Sraw[2] = Sraw[3] = make_uint2(0u, 0u);
         }
         // Uniform block offsets of this item.  They pass through fresh_s() before every tile, which
         // keeps the compiler from forming (block + lane offset) for all tiles at once and holding
@@ -594,8 +597,10 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     GvState gvst;
     gvst.init(a.gsT ? a.gsT + (int64_t)(b * H + h) * (kN * kN) : nullptr, 16 * p + (lane & 15), lane >> 4);
     WKV6_STAMP_DECL;
-    constexpr bool kStatesByLoad = !kSweepStates;   // (with kSweepStates the consumers read the states this kernel wrote itself)
-    if (kStatesByLoad && nitem > 0) issue_state(0);
+    // phase 2 items get their chunk's saved state loaded one item ahead -- except, with kSweepStates,
+    // the first of them, whose state the consumers hand over through LDS at the end of phase 1
+    auto state_by_load = [&](int it) { return it < nitem && item_full(it) && !(kSweepStates && it == nchunk); };
+    if (state_by_load(0)) issue_state(0);
     issue_loads(0);
     wait_younger(nitem > 1 ? issue_loads(1) : 0);
     prepare(0);
@@ -605,7 +610,7 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
         WKV6_STAMP();
         // free again: the r, k block of item it-1 and the raw w, v, gy blocks of item it-1 (read by the
         // other roles before the barrier), and the state tile of item it-1
-        const int state_loads = (kStatesByLoad && it + 1 < nitem) ? 2 : 0;
+        const int state_loads = state_by_load(it + 1) ? 2 : 0;
         if (state_loads) issue_state(it + 1);
         const int younger = it + 2 < nitem ? issue_loads(it + 2) : 0;
         if (it + 1 < nitem) {
