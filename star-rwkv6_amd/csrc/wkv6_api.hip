@@ -120,12 +120,28 @@ int wkv6_forward_gn_gate(void *stream, int dtype, int state_dtype,
                                             gate, gn_scale, gn_offset, gn_eps, out, ys));
 }
 
+// Size of the part of the saved block that the kernels of one pass use (chunk states, arrival
+// counters; sized so that the guarded per-timestep pass of the backward can use the same buffer).
+static size_t saved_base_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
+    const size_t ws = wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H), sv = wkv6::chunk_saved_bytes(B, T, H);
+    return ((ws > sv ? ws : sv) + 255) & ~(size_t)255;
+}
+// Segments the training pair of this shape runs in (1: one piece).  A (B,T,C) tensor cut into P
+// segments is handled as a (B*P, T/P, C) tensor, so the base part is sized for that shape.
+static int train_segments(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
+    const bool chunk = (algo == WKV6_ALGO_CHUNK && chunk_possible(dtype, T, C)) ||
+                       (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
+    return chunk ? wkv6::chunk_train_segments(B, T, H) : 1;
+}
+
 size_t wkv6_saved_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
     if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
     const bool chunk = (algo == WKV6_ALGO_CHUNK && chunk_possible(dtype, T, C)) ||
                        (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
-    // sized so that the guarded per-timestep pass of the backward can use the same buffer
     if (!chunk) return 0;
+    const int P = train_segments(dtype, algo, B, T, C, H);
+    if (P > 1)
+        return saved_base_bytes(dtype, WKV6_ALGO_CHUNK, B * P, T / P, C, H) + wkv6::train_segments_layout(B, T, H, nullptr).bytes;
     const size_t ws = wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H), sv = wkv6::chunk_saved_bytes(B, T, H);
     return ws > sv ? ws : sv;
 }
@@ -135,6 +151,14 @@ int wkv6_forward_save(void *stream, int dtype, int algo, int64_t B, int64_t T, i
                       void *y, void *saved, size_t saved_bytes) {
     const size_t need = wkv6_saved_bytes(dtype, algo, B, T, C, H);
     if (need > 0 && (!saved || saved_bytes < need || !aligned16(saved))) return WKV6_ERR_WORKSPACE;
+    if (need > 0 && train_segments(dtype, algo, B, T, C, H) > 1) {
+        // few pairs, long sequence: time segments side by side
+        const int P = train_segments(dtype, algo, B, T, C, H);
+        if (!r || !k || !v || !w || !u || !y) return WKV6_ERR_ARG;
+        if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(y)) return WKV6_ERR_ARG;
+        char *extra = reinterpret_cast<char *>(saved) + saved_base_bytes(dtype, WKV6_ALGO_CHUNK, B * P, T / P, C, H);
+        return finish(wkv6::chunk_forward_save_segments((hipStream_t)stream, B, T, H, r, k, v, w, u, y, saved, extra));
+    }
     return forward_impl(stream, dtype, out_type(dtype), algo, B, T, C, H, 0, nullptr, r, k, v, w, u, nullptr, y, nullptr,
                         need > 0 ? saved : nullptr);
 }
@@ -176,6 +200,20 @@ size_t wkv6_backward_workspace_bytes(int dtype, int64_t B, int64_t T, int64_t C,
     return wkv6_backward_workspace_bytes_ex(dtype, WKV6_ALGO_AUTO, B, T, C, H);
 }
 
+// backward_saved / backward_saved_sum of a shape whose training pair runs in time segments
+static int backward_segments_impl(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                                  const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                                  void *gr, void *gk, void *gv, void *gw, void *gu, void *gu_sum, void *saved, size_t saved_bytes) {
+    if (!r || !k || !v || !w || !u || !gy || !gr || !gk || !gv || !gw || !gu) return WKV6_ERR_ARG;
+    if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(gy) || !aligned16(gr) ||
+        !aligned16(gk) || !aligned16(gv) || !aligned16(gw)) return WKV6_ERR_ARG;
+    if (!saved || saved_bytes < wkv6_saved_bytes(dtype, algo, B, T, C, H) || !aligned16(saved)) return WKV6_ERR_WORKSPACE;
+    const int P = train_segments(dtype, algo, B, T, C, H);
+    char *extra = reinterpret_cast<char *>(saved) + saved_base_bytes(dtype, WKV6_ALGO_CHUNK, B * P, T / P, C, H);
+    return finish(wkv6::chunk_backward_saved_segments((hipStream_t)stream, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, gu_sum,
+                                                      saved, extra));
+}
+
 static int backward_impl(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, size_t workspace_bytes,
@@ -213,6 +251,9 @@ int wkv6_backward_saved(void *stream, int dtype, int algo, int64_t B, int64_t T,
                         void *gr, void *gk, void *gv, void *gw, void *gu, void *saved, size_t saved_bytes) {
     // `saved` doubles as the workspace: the guarded per-timestep pass only runs when the chunked
     // results (and with them the saved states) are discarded anyway
+    if (check_shape(dtype, B, T, C, H) == WKV6_OK && algo >= WKV6_ALGO_AUTO && algo <= WKV6_ALGO_CHUNK &&
+        train_segments(dtype, algo, B, T, C, H) > 1)
+        return backward_segments_impl(stream, dtype, algo, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, nullptr, saved, saved_bytes);
     return backward_impl(stream, dtype, algo, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, saved, saved_bytes,
                          wkv6_saved_bytes(dtype, algo, B, T, C, H) > 0);
 }
@@ -222,6 +263,9 @@ int wkv6_backward_saved_sum(void *stream, int dtype, int algo, int64_t B, int64_
                             void *gr, void *gk, void *gv, void *gw, void *gu, void *gu_sum,
                             void *saved, size_t saved_bytes) {
     if (!gu_sum) return WKV6_ERR_ARG;
+    if (check_shape(dtype, B, T, C, H) == WKV6_OK && algo >= WKV6_ALGO_AUTO && algo <= WKV6_ALGO_CHUNK &&
+        train_segments(dtype, algo, B, T, C, H) > 1)
+        return backward_segments_impl(stream, dtype, algo, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, gu_sum, saved, saved_bytes);
     const size_t need = wkv6_saved_bytes(dtype, algo, B, T, C, H);
     if (need > 0 && saved_bytes < need) return WKV6_ERR_WORKSPACE;
     return backward_impl(stream, dtype, algo, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, saved, saved_bytes,

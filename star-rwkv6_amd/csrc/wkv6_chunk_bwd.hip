@@ -600,6 +600,10 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     // phase 2 items get their chunk's saved state loaded one item ahead -- except, with kSweepStates,
     // the first of them, whose state the consumers hand over through LDS at the end of phase 1
     auto state_by_load = [&](int it) { return it < nitem && item_full(it) && !(kSweepStates && it == nchunk); };
+    // gv stores an item's visit leaves in flight behind the loads issued before them.  The chunk with
+    // the ragged tail issues anything from 0 to 16 (a store whose lanes are all past the end is
+    // skipped): counting none for it makes the waits behind it wait for everything older.
+    auto gv_stores = [&](int it) { return !item_full(it) ? 0 : (kRagged && item_chunk(it) == nchunk - 1) ? 0 : 16; };
     if (state_by_load(0)) issue_state(0);
     issue_loads(0);
     wait_younger(nitem > 1 ? issue_loads(1) : 0);
@@ -615,9 +619,7 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
         const int younger = it + 2 < nitem ? issue_loads(it + 2) : 0;
         if (it + 1 < nitem) {
             WKV6_STAMP();
-            // (with a ragged tail the number of gv stores issued is not fixed: wait for everything older)
-            const int gv_stores = (!kRagged && it >= 1 && item_full(it - 1)) ? 16 : 0;
-            wait_younger(younger + state_loads + gv_stores);
+            wait_younger(younger + state_loads + (it >= 1 ? gv_stores(it - 1) : 0));
             WKV6_STAMP();
             prepare(it + 1);
             WKV6_STAMP();
@@ -625,7 +627,7 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
         // the gv role, on the waves the operand preparation leaves partly idle
         if (item_full(it)) bwd_gv_chunk<kRagged>(gvst, a, smem, a.gv + base, rowbytes, item_chunk(it), it, p, lane);
         // the next item's state has to be in LDS when the consumers pass the barrier
-        if (state_loads) wait_younger(younger + ((!kRagged && item_full(it)) ? 16 : 0));
+        if (state_loads) wait_younger(younger + gv_stores(it));
         WKV6_STAMP();
     }
     wait_loads<0>();
@@ -758,6 +760,44 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
     const bool ragged = (T % CL) != 0;   // the last chunk has tokens past the end
     if (states_ready) return ragged ? launch(chunk_bwd_kernel<false, true>) : launch(chunk_bwd_kernel<false, false>);
     return ragged ? launch(chunk_bwd_kernel<true, true>) : launch(chunk_bwd_kernel<true, false>);
+}
+
+// Training pair in time segments, last step: gu of a batch row = sum over its segments; the decay
+// gradient at the first and the last token of a sequence is zero by definition
+// (rwkv_kernels.cu:381,406), where the kernels, given explicit states, leave rounding residue.
+__global__ void segments_finish_kernel(int P, int64_t T, int C, const bf16_t *__restrict__ gu_rows,
+                                       bf16_t *__restrict__ gu, bf16_t *__restrict__ gw)
+{
+    const int c = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
+    if (c >= C) return;
+    float acc = 0.f;
+    for (int p = 0; p < P; ++p) acc += load1(gu_rows + ((int64_t)b * P + p) * C + c);
+    store1(gu + (int64_t)b * C + c, acc);
+    store1(gw + (int64_t)b * T * C + c, 0.f);
+    store1(gw + ((int64_t)b * T + T - 1) * C + c, 0.f);
+}
+
+hipError_t chunk_backward_saved_segments(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                                         const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                                         void *gr, void *gk, void *gv, void *gw, void *gu, void *gu_sum,
+                                         void *saved, void *extra)
+{
+    const TrainSegments s = train_segments_layout(B, T, H, extra);
+    const int64_t L = T / s.P, rows = B * s.P;
+    // (1) what each segment alone sends back into its incoming state (its other results are redone in (3))
+    hipError_t e = chunk_backward(st, rows, L, H, r, k, v, w, u, gy, gr, gk, gv, gw, s.gu_rows, saved, true, nullptr,
+                                  s.states, nullptr, s.gstates);
+    if (e != hipSuccess) return e;
+    // (2) chained backwards in time: the gradient arriving at the end of every segment
+    if ((e = segment_chain_reverse(st, s.P, B, H, s.dsum, s.gstates)) != hipSuccess) return e;
+    // (3) every segment again, between its true incoming state and its true arriving gradient
+    e = chunk_backward(st, rows, L, H, r, k, v, w, u, gy, gr, gk, gv, gw, s.gu_rows, saved, true, gu_sum,
+                       s.states, s.gstates, nullptr);
+    if (e != hipSuccess) return e;
+    const int C = (int)(H * kN);
+    hipLaunchKernelGGL(segments_finish_kernel, dim3((unsigned)((C + 255) / 256), (unsigned)B), dim3(256), 0, st,
+                       s.P, T, C, (const bf16_t *)s.gu_rows, (bf16_t *)gu, (bf16_t *)gw);
+    return hipGetLastError();
 }
 
 }  // namespace wkv6

@@ -601,7 +601,10 @@ hipError_t chunk_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64
 // segment runs again from its true state and writes y.  Twice the forward work on P times the
 // workgroups.
 // ------------------------------------------------------------------------------------------
-template <typename Ts>
+// kReverse: the same chain walked from the last segment to the first, which is what the reverse
+// state of the backward pass obeys (the gradient arriving at the end of segment p is what segment
+// p + 1 sends into its incoming state: its own contribution plus D_{p+1} times what arrives at its end).
+template <typename Ts, bool kReverse = false>
 __global__ __launch_bounds__(256) void segment_chain_kernel(int P, int H, const Ts *__restrict__ s0, const int64_t *__restrict__ map,
                                                             const float *__restrict__ dsum, float *__restrict__ states, Ts *__restrict__ sT)
 {
@@ -619,7 +622,8 @@ __global__ __launch_bounds__(256) void segment_chain_kernel(int P, int H, const 
 #pragma unroll
         for (int e = 0; e < 16; ++e) S[e] = 0.f;
     }
-    for (int seg = 0; seg < P; ++seg) {
+    for (int n = 0; n < P; ++n) {
+        const int seg = kReverse ? P - 1 - n : n;
         const int64_t vrow = (int64_t)b * P + seg;
         float *u = states + ((vrow * H + h) * kN + j) * kN + i0;
         const int64_t vp = vrow * H + h, np = (int64_t)gridDim.x * P;   // this segment's pair, pairs of all segments
@@ -672,6 +676,51 @@ hipError_t chunk_forward_segments_run(hipStream_t st, int state_dtype, int64_t B
                            (const bf16_t *)s0, map, (const float *)dsum, states, (bf16_t *)sT);
     if ((e = hipGetLastError()) != hipSuccess) return e;
     return chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, states, nullptr, y, nullptr, nullptr);
+}
+
+hipError_t segment_chain_reverse(hipStream_t st, int P, int64_t B, int64_t H, const float *dsum, float *states) {
+    hipLaunchKernelGGL((segment_chain_kernel<float, true>), dim3((unsigned)(B * H)), dim3(256), 0, st, P, (int)H,
+                       (const float *)nullptr, (const int64_t *)nullptr, dsum, states, (float *)nullptr);
+    return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------
+// The same for the training pair (saving forward, backward from the saved states): the forward
+// keeps every segment's incoming state and decay exponents for the backward, whose reverse state
+// is chained the same way (see chunk_backward_saved_segments).
+// ------------------------------------------------------------------------------------------
+int chunk_train_segments(int64_t B, int64_t T, int64_t H) {
+    const int64_t pairs = B * H, cus = compute_units();
+    // (1.7 forward and 2 backward passes over T / P tokens against one of each over T: pays from P = 4)
+    if (T < 2048) return 1;
+    for (int P = 16; P >= 4; P >>= 1)
+        if (pairs * P <= cus && T % (P * CL) == 0 && T / P >= 4 * CL) return P;
+    return 1;
+}
+TrainSegments train_segments_layout(int64_t B, int64_t T, int64_t H, void *extra) {
+    TrainSegments s;
+    s.P = chunk_train_segments(B, T, H);
+    const size_t pairs = (size_t)(B * s.P * H);
+    s.states = reinterpret_cast<float *>(extra);
+    s.dsum = s.states + pairs * kN * kN;
+    s.gstates = s.dsum + pairs * 4 * kN;
+    s.gu_rows = s.gstates + pairs * kN * kN;
+    s.bytes = (pairs * (2 * kN * kN + 4 * kN) + (size_t)(B * s.P * H) * kN) * sizeof(float);   // (gu rows: room for fp32)
+    return s;
+}
+
+hipError_t chunk_forward_save_segments(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                                       const void *r, const void *k, const void *v, const void *w, const void *u,
+                                       void *y, void *saved, void *extra)
+{
+    const TrainSegments s = train_segments_layout(B, T, H, extra);
+    const int64_t L = T / s.P, rows = B * s.P;
+    hipError_t e = chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, nullptr, nullptr, nullptr, s.states, nullptr, s.dsum);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(segment_chain_kernel<float>, dim3((unsigned)(B * H)), dim3(256), 0, st, s.P, (int)H,
+                       (const float *)nullptr, (const int64_t *)nullptr, (const float *)s.dsum, s.states, (float *)nullptr);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    return chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, s.states, nullptr, y, nullptr, saved);
 }
 
 }  // namespace wkv6

@@ -45,6 +45,28 @@ hipError_t chunk_forward_segments_run(hipStream_t st, int state_dtype, int64_t B
                                       const void *r, const void *k, const void *v, const void *w, const void *u,
                                       const void *s0, const int64_t *map, void *y, void *sT, void *workspace);
 
+// The training pair of a long sequence of few pairs as P time segments side by side.  The saving
+// forward leaves, behind the saved chunk states (`extra`), every segment's incoming state and decay
+// exponents; the backward chains its reverse state through the same affine maps (two passes each).
+struct TrainSegments {
+    int P;              // segments per sequence (1: does not apply)
+    float *states;      // [B*P][H][64][64] state entering each segment
+    float *dsum;        // decay exponents of each segment (as chunk_forward leaves them)
+    float *gstates;     // [B*P][H][64][64] gradient arriving at the end of each segment
+    void *gu_rows;      // [B*P][C] gu of each segment
+    size_t bytes;       // size of the block
+};
+int chunk_train_segments(int64_t B, int64_t T, int64_t H);
+TrainSegments train_segments_layout(int64_t B, int64_t T, int64_t H, void *extra);
+hipError_t segment_chain_reverse(hipStream_t st, int P, int64_t B, int64_t H, const float *dsum, float *states);
+hipError_t chunk_forward_save_segments(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                                       const void *r, const void *k, const void *v, const void *w, const void *u,
+                                       void *y, void *saved, void *extra);
+hipError_t chunk_backward_saved_segments(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                                         const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                                         void *gr, void *gk, void *gv, void *gw, void *gu, void *gu_sum,
+                                         void *saved, void *extra);
+
 // forward with the layer's output stage fused in: out = (group_norm_head(y) * gn_scale + gn_offset) * gate
 hipError_t chunk_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                                const void *r, const void *k, const void *v, const void *w, const void *u,

@@ -59,8 +59,11 @@ class _WKV6(torch.autograd.Function):
                                                         _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(y),
                                                         _ptr(saved), nsave))
                 else:
+                    # optional workspace: a long sequence of few (batch, head) pairs runs as time segments
+                    n = lib.wkv6_forward_workspace_bytes(code, algo, B, T, C, H)
+                    ws = torch.empty(int(n), device=r.device, dtype=torch.uint8) if n else None
                     _native.check(lib.wkv6_forward_ex(_stream(), code, algo, B, T, C, H,
-                                                      _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(y), None, 0))
+                                                      _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(y), _ptr(ws), n))
             ctx.saved_states = saved
             ctx.save_for_backward(r, k, v, w, u)
             return y
@@ -138,7 +141,6 @@ class _WKV6State(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, gy, gsT):
-        lib = _native.load()
         B, T, C, H = ctx.dims
         r, k, v, w, u = ctx.saved_tensors[:5]
         s0 = ctx.saved_tensors[5] if ctx.has_s0 else None
@@ -146,18 +148,26 @@ class _WKV6State(torch.autograd.Function):
             odt = _out_dtype(r.dtype)
             gy = torch.zeros((B, T, C), device=r.device, dtype=odt) if gy is None else gy.to(odt).contiguous()
             gsT = None if gsT is None else gsT.float().contiguous()
-            gr, gk, gv, gw = (torch.empty((B, T, C), device=r.device, dtype=odt) for _ in range(4))
-            gu = torch.empty((B, C), device=r.device, dtype=odt)
-            gs0 = torch.empty((B, H, C // H, C // H), device=r.device, dtype=torch.float32) if ctx.has_s0 else None
-            code = _DTYPE_CODE[r.dtype]
-            with torch.cuda.device(r.device):
-                n = lib.wkv6_backward_with_state_workspace_bytes(code, ctx.algo, B, T, C, H)
-                ws = torch.empty(max(int(n), 16), device=r.device, dtype=torch.uint8)
-                _native.check(lib.wkv6_backward_with_state(
-                    _stream(), code, ctx.algo, B, T, C, H, _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(s0),
-                    _ptr(gy), _ptr(gsT), _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu), _ptr(gs0), _ptr(ws), n))
+            gr, gk, gv, gw, gu, gs0 = _backward_with_state(B, T, C, H, r, k, v, w, u, s0, gy, gsT, ctx.algo, ctx.has_s0)
             gu = torch.sum(gu, 0).reshape(u.shape)
         return (None, None, None, None, gr.to(r.dtype), gk.to(r.dtype), gv.to(r.dtype), gw.to(r.dtype), gu.to(u.dtype), gs0, None)
+
+
+def _backward_with_state(B, T, C, H, r, k, v, w, u, s0, gy, gsT, algo, want_gs0):
+    """gr, gk, gv, gw, per-row gu (B, C), dL/dS_0 or None, through wkv6_backward_with_state."""
+    lib = _native.load()
+    odt = _out_dtype(r.dtype)
+    gr, gk, gv, gw = (torch.empty((B, T, C), device=r.device, dtype=odt) for _ in range(4))
+    gu = torch.empty((B, C), device=r.device, dtype=odt)
+    gs0 = torch.empty((B, H, C // H, C // H), device=r.device, dtype=torch.float32) if want_gs0 else None
+    code = _DTYPE_CODE[r.dtype]
+    with torch.cuda.device(r.device):
+        n = lib.wkv6_backward_with_state_workspace_bytes(code, algo, B, T, C, H)
+        ws = torch.empty(max(int(n), 16), device=r.device, dtype=torch.uint8)
+        _native.check(lib.wkv6_backward_with_state(
+            _stream(), code, algo, B, T, C, H, _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(s0),
+            _ptr(gy), _ptr(gsT), _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu), _ptr(gs0), _ptr(ws), n))
+    return gr, gk, gv, gw, gu, gs0
 
 
 class RWKVKernelOperator:

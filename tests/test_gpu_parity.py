@@ -482,6 +482,22 @@ def test_forward_in_time_segments(op, oracle, B, T, H, sdt):
     check_close("sT zero", s0T, oracle.forward_c(*ref, N)[1], torch.bfloat16)
 
 
+@pytest.mark.parametrize("B,T,H,P", [(1, 2048, 2, 8), (2, 4096, 1, 16), (3, 3072, 5, 8), (1, 8192, 20, 8)])
+def test_training_pair_in_time_segments(op, oracle, B, T, H, P):
+    """Few pairs, long sequence: forward_save + backward_saved_sum run the sequence as P segments side
+    by side (joined by the affine state map and, for the reverse state, its transpose); against the
+    oracle over the whole sequence."""
+    from rwkv_kernel import _native
+
+    lib = _native.load()
+    C = H * 64
+    whole = lib.wkv6_backward_workspace_bytes_ex(_native.BF16, CHUNK, B, T, C, H)
+    assert lib.wkv6_saved_bytes(_native.BF16, CHUNK, B, T, C, H) >= whole + B * P * H * 2 * 64 * 64 * 4   # segment states
+    _, grads = _case(op, oracle, B, T, H, 90 + H, torch.bfloat16, CHUNK)
+    gw = grads[3]
+    assert float(gw[:, 0].abs().max()) == 0.0 and float(gw[:, -1].abs().max()) == 0.0
+
+
 def test_chunk_matches_scan_on_padding_mask(op, oracle):
     B, T, H, N = 1, 96, 1, 64
     ins = oracle.make_inputs(B, T, H, N, 54)
