@@ -498,6 +498,23 @@ def test_training_pair_in_time_segments(op, oracle, B, T, H, P):
     assert float(gw[:, 0].abs().max()) == 0.0 and float(gw[:, -1].abs().max()) == 0.0
 
 
+def test_training_pair_in_time_segments_with_fallback_segments(op, oracle):
+    # segments whose decay the tile scaling cannot represent are redone by the exact per-timestep
+    # code in every pass (forward passes, both backward passes); decay exactly 0 and exactly 1
+    # across segment boundaries
+    B, T, H, N = 1, 2048, 3, 64          # 8 segments of 256 tokens
+    ins = oracle.make_inputs(B, T, H, N, 97)
+    ins[3][0, 700:720, 70:90] = 6.0      # inside segment 2, head 1
+    ins[3][0, 1279:1282, 130:140] = 20.0  # decay 0 around the boundary of segments 4 and 5, head 2
+    ins[3][0, 250:260] = -1e9            # decay 1 across the boundary of segments 0 and 1
+    dev, ref = cast_inputs(ins[:5], torch.bfloat16)
+    gy_dev, gy_ref = cast_inputs(ins[5:6], torch.bfloat16)
+    y, grads = _run_fwd_bwd(op, dev + gy_dev, CHUNK)
+    check_close("y", y, oracle.forward_c(*ref, N)[0], torch.bfloat16)
+    for name, g, gr in zip("gr gk gv gw gu".split(), grads, oracle.backward_c(*ref, gy_ref[0], N)):
+        check_close(name, to_np(g).reshape(gr.shape), gr, torch.bfloat16, is_grad=True)
+
+
 def test_chunk_matches_scan_on_padding_mask(op, oracle):
     B, T, H, N = 1, 96, 1, 64
     ins = oracle.make_inputs(B, T, H, N, 54)
