@@ -202,7 +202,7 @@ def main():
     a = parse()
     if a.gpus != 1:
         print("bench.py: this build measures ONE GPU; --gpus %d is not supported "
-              "(the operator needs no cross-GPU exchange; see DESIGN.md)" % a.gpus, file=sys.stderr)
+              "(every (batch, head) pair is independent: more GPUs split B or H with no exchange)" % a.gpus, file=sys.stderr)
         sys.exit(2)
     import torch
     from oracle import wkv6_ref
