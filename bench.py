@@ -27,6 +27,7 @@ WORKLOADS = {
     "c2": (8, 1024, 32, "bf16"),   # RWKV6-1.6B layer shape: the configuration the metric is quoted on
     "c3": (4, 4096, 64, "bf16"),   # RWKV6-7B layer shape
     "c1": (2, 128, 4, "f32"),
+    "long1": (1, 8192, 32, "bf16"),   # one long sequence per GPU (fine-tuning): 32 pairs, runs as time segments
 }
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (separate runs), scaled
