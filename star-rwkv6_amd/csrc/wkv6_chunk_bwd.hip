@@ -784,9 +784,10 @@ hipError_t chunk_backward_saved_segments(hipStream_t st, int64_t B, int64_t T, i
 {
     const TrainSegments s = train_segments_layout(B, T, H, extra);
     const int64_t L = T / s.P, rows = B * s.P;
-    // (1) what each segment alone sends back into its incoming state (its other results are redone in (3))
-    hipError_t e = chunk_backward(st, rows, L, H, r, k, v, w, u, gy, gr, gk, gv, gw, s.gu_rows, saved, true, nullptr,
-                                  s.states, nullptr, s.gstates);
+    // (1) What each segment alone sends back into its incoming state: G_0 = sum_t (prod_{s<t} d_s) r_t^T gy_t.
+    // That is the state the FORWARD recurrence builds from zero over the segment read back to front
+    // with r in the place of k and gy in the place of v, so the forward kernel's state-only pass does it.
+    hipError_t e = chunk_forward(st, kF32, rows, L, H, r, r, gy, w, u, nullptr, nullptr, nullptr, s.gstates, nullptr, nullptr, true);
     if (e != hipSuccess) return e;
     // (2) chained backwards in time: the gradient arriving at the end of every segment
     if ((e = segment_chain_reverse(st, s.P, B, H, s.dsum, s.gstates)) != hipSuccess) return e;

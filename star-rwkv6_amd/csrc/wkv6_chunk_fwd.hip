@@ -77,6 +77,7 @@ struct FwdArgs {
     int T, H;
     int nitems;      // B * H (batch, head) pairs; with kMulti a workgroup takes every gridDim.x-th of them
     int split;       // 1, 2 or 4 workgroups per pair, each with the consumer waves of 4 / split column slices
+    int reverse;     // 1: the time axis is read back to front (row T-1-t in the place of row t); T a multiple of 64
     float *dsum;     // null, or [4 tiles][pairs][64]: per pair, log2(e) * sum of exp(w) over the tokens of tile p of every chunk
     const bf16_t *r, *k, *v, *w, *u;
     const void *s0;
@@ -275,7 +276,7 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
             const int t = tb + 8 * blk + lrow;
-            const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes + lpiece;
+            const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : a.reverse ? T - 1 - t : t) * rowbytes + lpiece;
             load_rows8_to_lds(wb, o, rkw + 2 * kTileBytes + 8 * blk * kTileRow);
             load_rows8_to_lds(rb, o, rkw + 8 * blk * kTileRow);
             load_rows8_to_lds(kb_, o, rkw + kTileBytes + 8 * blk * kTileRow);
@@ -497,7 +498,7 @@ __global__ __launch_bounds__(kFwdThreads) void chunk_fwd_kernel(FwdArgs a)
         const int bh = bh0 + n * stride;
         __syncthreads();
         scan_fwd_body<bf16_t, bf16_t, Ts>(*reinterpret_cast<ScanFwdLds *>(smem), bh / a.H, bh % a.H, a.T, a.H, a.r, a.k, a.v, a.w, a.u,
-                                          reinterpret_cast<const Ts *>(a.s0), a.map, kFuse ? a.out : a.y, reinterpret_cast<Ts *>(a.sT));
+                                          reinterpret_cast<const Ts *>(a.s0), a.map, kFuse ? a.out : a.y, reinterpret_cast<Ts *>(a.sT), a.reverse != 0);
         if (kFuse) {
             __threadfence_block();
             __syncthreads();
@@ -554,10 +555,11 @@ static unsigned forward_grid(int64_t pairs, bool *multi, int *split) {
 
 hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u,
-                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states, float *dsum)
+                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states, float *dsum, bool reverse)
 {
     FwdArgs a = {};
     a.dsum = dsum;
+    a.reverse = reverse && (T % CL) == 0;
     a.T = (int)T; a.H = (int)H; a.nitems = (int)(B * H);
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
     a.s0 = s0; a.map = map; a.y = (bf16_t *)y; a.sT = sT; a.ckpt = (float *)saved_states;

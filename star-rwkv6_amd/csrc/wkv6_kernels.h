@@ -35,7 +35,8 @@ hipError_t scan_backward_state(hipStream_t st, int dtype, int64_t B, int64_t T, 
 hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u,
                          const void *s0, const int64_t *map, void *y, void *sT, void *saved_states,
-                         float *dsum = nullptr);   // dsum: see chunk_forward_segments_run
+                         float *dsum = nullptr,    // dsum: see chunk_forward_segments_run
+                         bool reverse = false);    // the time axis read back to front (T a multiple of 64, no y)
 
 // Few pairs, long sequence: the forward as P time segments side by side (two passes joined by the
 // affine map of a segment's state).  chunk_forward_segments = P for the shape (1 = does not apply).

@@ -40,7 +40,7 @@ __device__ __forceinline__ void scan_fwd_body(ScanFwdLds &L, int b, int h, int T
         const Tin *__restrict__ r, const Tin *__restrict__ k, const Tin *__restrict__ v,
         const Tin *__restrict__ w, const Tin *__restrict__ u,
         const Ts *__restrict__ s0, const int64_t *__restrict__ map,
-        Tout *__restrict__ y, Ts *__restrict__ sT)
+        Tout *__restrict__ y, Ts *__restrict__ sT, bool reverse = false)   // reverse: timestep t reads row T-1-t (no y then)
 {
     auto &s_r = L.s_r; auto &s_k = L.s_k; auto &s_d = L.s_d; auto &s_v = L.s_v;
     auto &s_part = L.s_part; auto &s_ruk = L.s_ruk; auto &s_u = L.s_u;
@@ -73,7 +73,7 @@ __device__ __forceinline__ void scan_fwd_body(ScanFwdLds &L, int b, int h, int T
 
     auto prefetch = [&](int t0) {
         const int t = t0 + st;
-        if (t < T) { ra.load(pa + (int64_t)t * C); rb.load(pb + (int64_t)t * C); }
+        if (t < T) { const int64_t row = reverse ? T - 1 - t : t; ra.load(pa + row * C); rb.load(pb + row * C); }
         else { ra.zero(); rb.zero(); }
     };
     prefetch(0);
