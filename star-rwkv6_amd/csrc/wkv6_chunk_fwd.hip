@@ -606,43 +606,52 @@ hipError_t chunk_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64
 // kReverse: the same chain walked from the last segment to the first, which is what the reverse
 // state of the backward pass obeys (the gradient arriving at the end of segment p is what segment
 // p + 1 sends into its incoming state: its own contribution plus D_{p+1} times what arrives at its end).
-template <typename Ts, bool kReverse = false>
-__global__ __launch_bounds__(256) void segment_chain_kernel(int P, int H, const Ts *__restrict__ s0, const int64_t *__restrict__ map,
+template <typename Ts, bool kReverse, int P>
+__global__ __launch_bounds__(256) void segment_chain_kernel(int H, const Ts *__restrict__ s0, const int64_t *__restrict__ map,
                                                             const float *__restrict__ dsum, float *__restrict__ states, Ts *__restrict__ sT)
 {
-    // one workgroup per (batch, head); thread: key row j = tid >> 2, value columns 16 (tid & 3) .. +15.
-    // states[(b*P + seg), h] holds U on entry and the segment's incoming state on exit.
-    const int b = blockIdx.x / H, h = blockIdx.x - b * H;
-    const int j = threadIdx.x >> 2, i0 = (threadIdx.x & 3) * 16;
-    float S[16];
+    // Thread: four value columns i0..i0+3 of one key row j of one (batch, head): 1024 threads per pair,
+    // gridDim.x * 256 = B * H * 1024.  states[(b*P + seg), h] holds U on entry and the segment's
+    // incoming state on exit.  All P loads are issued before the chain is walked (their addresses do
+    // not depend on it): the kernel takes about two memory round trips instead of 2 P.
+    const int e = blockIdx.x * 256 + threadIdx.x;
+    const int i0 = (e & 15) * 4, j = (e >> 4) & 63, bh = e >> 10;
+    const int b = bh / H, h = bh - b * H;
+    const int64_t np = (int64_t)(gridDim.x >> 2) * P;   // pairs of all segments
+    auto pair_of_step = [&](int n) { return ((int64_t)b * P + (kReverse ? P - 1 - n : n)) * H + h; };   // step n of the walk
+    float4 x[P];
+    float d[P];
+#pragma unroll
+    for (int n = 0; n < P; ++n) {
+        const int64_t vp = pair_of_step(n);
+        x[n] = *reinterpret_cast<const float4 *>(states + (vp * kN + j) * kN + i0);
+        d[n] = (dsum[vp * kN + j] + dsum[(np + vp) * kN + j]) + (dsum[(2 * np + vp) * kN + j] + dsum[(3 * np + vp) * kN + j]);
+    }
+    float S[4] = {0.f, 0.f, 0.f, 0.f};
     if (s0) {
         const int64_t row = map ? map[b] : (int64_t)b;
-        const Ts *p = s0 + ((row * H + h) * kN + j) * kN + i0;
-#pragma unroll
-        for (int e = 0; e < 16; e += 4) { float x[4]; load4(p + e, x); S[e] = x[0]; S[e + 1] = x[1]; S[e + 2] = x[2]; S[e + 3] = x[3]; }
-    } else {
-#pragma unroll
-        for (int e = 0; e < 16; ++e) S[e] = 0.f;
+        load4(s0 + ((row * H + h) * kN + j) * kN + i0, S);
     }
+#pragma unroll
     for (int n = 0; n < P; ++n) {
-        const int seg = kReverse ? P - 1 - n : n;
-        const int64_t vrow = (int64_t)b * P + seg;
-        float *u = states + ((vrow * H + h) * kN + j) * kN + i0;
-        const int64_t vp = vrow * H + h, np = (int64_t)gridDim.x * P;   // this segment's pair, pairs of all segments
-        const float d = exp2_fast(-((dsum[vp * kN + j] + dsum[(np + vp) * kN + j]) + (dsum[(2 * np + vp) * kN + j] + dsum[(3 * np + vp) * kN + j])));
-#pragma unroll
-        for (int e = 0; e < 16; e += 4) {
-            const float4 x = *reinterpret_cast<const float4 *>(u + e);
-            *reinterpret_cast<float4 *>(u + e) = make_float4(S[e], S[e + 1], S[e + 2], S[e + 3]);
-            S[e] = fmaf(S[e], d, x.x); S[e + 1] = fmaf(S[e + 1], d, x.y);
-            S[e + 2] = fmaf(S[e + 2], d, x.z); S[e + 3] = fmaf(S[e + 3], d, x.w);
-        }
+        const float dd = exp2_fast(-d[n]);
+        *reinterpret_cast<float4 *>(states + (pair_of_step(n) * kN + j) * kN + i0) = make_float4(S[0], S[1], S[2], S[3]);
+        S[0] = fmaf(S[0], dd, x[n].x); S[1] = fmaf(S[1], dd, x[n].y); S[2] = fmaf(S[2], dd, x[n].z); S[3] = fmaf(S[3], dd, x[n].w);
     }
-    if (sT) {
-        Ts *p = sT + (((int64_t)b * H + h) * kN + j) * kN + i0;
-#pragma unroll
-        for (int e = 0; e < 16; e += 4) store4(p + e, S[e], S[e + 1], S[e + 2], S[e + 3]);
+    if (sT) store4(sT + (((int64_t)b * H + h) * kN + j) * kN + i0, S[0], S[1], S[2], S[3]);
+}
+template <typename Ts, bool kReverse>
+static hipError_t launch_chain(hipStream_t st, int P, int64_t B, int64_t H, const Ts *s0, const int64_t *map,
+                               const float *dsum, float *states, Ts *sT)
+{
+    const dim3 grid((unsigned)(B * H * 4)), block(256);
+    switch (P) {
+    case 4: hipLaunchKernelGGL((segment_chain_kernel<Ts, kReverse, 4>), grid, block, 0, st, (int)H, s0, map, dsum, states, sT); break;
+    case 8: hipLaunchKernelGGL((segment_chain_kernel<Ts, kReverse, 8>), grid, block, 0, st, (int)H, s0, map, dsum, states, sT); break;
+    case 16: hipLaunchKernelGGL((segment_chain_kernel<Ts, kReverse, 16>), grid, block, 0, st, (int)H, s0, map, dsum, states, sT); break;
+    default: return hipErrorInvalidValue;
     }
+    return hipGetLastError();
 }
 
 // Number of segments for this shape (1 = not worth it / not possible): the pairs times the segments
@@ -670,20 +679,14 @@ hipError_t chunk_forward_segments_run(hipStream_t st, int state_dtype, int64_t B
     float *states = (float *)workspace, *dsum = states + rows * H * kN * kN;
     hipError_t e = chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, nullptr, nullptr, nullptr, states, nullptr, dsum);
     if (e != hipSuccess) return e;
-    if (state_dtype == kF32)
-        hipLaunchKernelGGL(segment_chain_kernel<float>, dim3((unsigned)(B * H)), dim3(256), 0, st, P, (int)H,
-                           (const float *)s0, map, (const float *)dsum, states, (float *)sT);
-    else
-        hipLaunchKernelGGL(segment_chain_kernel<bf16_t>, dim3((unsigned)(B * H)), dim3(256), 0, st, P, (int)H,
-                           (const bf16_t *)s0, map, (const float *)dsum, states, (bf16_t *)sT);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
+    e = state_dtype == kF32 ? launch_chain<float, false>(st, P, B, H, (const float *)s0, map, dsum, states, (float *)sT)
+                            : launch_chain<bf16_t, false>(st, P, B, H, (const bf16_t *)s0, map, dsum, states, (bf16_t *)sT);
+    if (e != hipSuccess) return e;
     return chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, states, nullptr, y, nullptr, nullptr);
 }
 
 hipError_t segment_chain_reverse(hipStream_t st, int P, int64_t B, int64_t H, const float *dsum, float *states) {
-    hipLaunchKernelGGL((segment_chain_kernel<float, true>), dim3((unsigned)(B * H)), dim3(256), 0, st, P, (int)H,
-                       (const float *)nullptr, (const int64_t *)nullptr, dsum, states, (float *)nullptr);
-    return hipGetLastError();
+    return launch_chain<float, true>(st, P, B, H, nullptr, nullptr, dsum, states, nullptr);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -719,9 +722,7 @@ hipError_t chunk_forward_save_segments(hipStream_t st, int64_t B, int64_t T, int
     const int64_t L = T / s.P, rows = B * s.P;
     hipError_t e = chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, nullptr, nullptr, nullptr, s.states, nullptr, s.dsum);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(segment_chain_kernel<float>, dim3((unsigned)(B * H)), dim3(256), 0, st, s.P, (int)H,
-                       (const float *)nullptr, (const int64_t *)nullptr, (const float *)s.dsum, s.states, (float *)nullptr);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
+    if ((e = launch_chain<float, false>(st, s.P, B, H, nullptr, nullptr, s.dsum, s.states, nullptr)) != hipSuccess) return e;
     return chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, s.states, nullptr, y, nullptr, saved);
 }
 
