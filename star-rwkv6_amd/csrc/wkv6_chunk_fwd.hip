@@ -661,8 +661,8 @@ int chunk_forward_segments(int64_t B, int64_t T, int64_t H) {
     // (two passes over T / P tokens and two more launches against one pass over T: nothing to gain
     // below four segments or on short sequences)
     if (T < 2048) return 1;
-    for (int P = 8; P >= 4; P >>= 1)
-        if (pairs * P <= cus && T % (P * CL) == 0) return P;
+    for (int P = 16; P >= 4; P >>= 1)
+        if (pairs * P <= cus && T % (P * CL) == 0 && T / P >= 4 * CL) return P;
     return 1;
 }
 size_t chunk_forward_segments_workspace_bytes(int64_t B, int64_t T, int64_t H) {
