@@ -646,6 +646,7 @@ static hipError_t launch_chain(hipStream_t st, int P, int64_t B, int64_t H, cons
 {
     const dim3 grid((unsigned)(B * H * 4)), block(256);
     switch (P) {
+    case 2: hipLaunchKernelGGL((segment_chain_kernel<Ts, kReverse, 2>), grid, block, 0, st, (int)H, s0, map, dsum, states, sT); break;
     case 4: hipLaunchKernelGGL((segment_chain_kernel<Ts, kReverse, 4>), grid, block, 0, st, (int)H, s0, map, dsum, states, sT); break;
     case 8: hipLaunchKernelGGL((segment_chain_kernel<Ts, kReverse, 8>), grid, block, 0, st, (int)H, s0, map, dsum, states, sT); break;
     case 16: hipLaunchKernelGGL((segment_chain_kernel<Ts, kReverse, 16>), grid, block, 0, st, (int)H, s0, map, dsum, states, sT); break;
@@ -696,9 +697,10 @@ hipError_t segment_chain_reverse(hipStream_t st, int P, int64_t B, int64_t H, co
 // ------------------------------------------------------------------------------------------
 int chunk_train_segments(int64_t B, int64_t T, int64_t H) {
     const int64_t pairs = B * H, cus = compute_units();
-    // (1.7 forward and 2 backward passes over T / P tokens against one of each over T: pays from P = 4)
+    // (two state-only passes at 0.7 of a forward each on top of the forward and the backward: 1.5
+    // times the work on P times the workgroups, and three small kernels)
     if (T < 2048) return 1;
-    for (int P = 16; P >= 4; P >>= 1)
+    for (int P = 16; P >= 2; P >>= 1)
         if (pairs * P <= cus && T % (P * CL) == 0 && T / P >= 4 * CL) return P;
     return 1;
 }
