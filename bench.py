@@ -319,7 +319,7 @@ def main():
         "roofline": {
             "bound": "hbm", "kernel": "wkv6_%s (%s)" % ("backward" if dom == "bwd" else "forward", algo_used),
             "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get((a.workload, algo_used, dom)),
+            "traffic": None if a.plain_pair else MEASURED_TRAFFIC_BYTES.get((a.workload, algo_used, dom)),
             "algorithmic_bytes": dom_bytes, "avg_ms": dom_ms,
         },
         "fwd_bwd": {

@@ -1,10 +1,10 @@
 // WKV6 backward in chunk-parallel form for gfx950 (bf16 MFMA, fp32 states); the forward kernel and
 // the notation are in wkv6_chunk_fwd.hip.
 //
-// Phase 1 (only when the forward pass did not leave its chunk states behind) sweeps the chunks in
-// time order and writes the state at every chunk start to the workspace (bf16,
-// [b][h][chunk][j][i]); phase 2 sweeps them in reverse order with the reverse state G in MFMA
-// accumulators.  G is kept twice, once with rows j / columns i (for gv) and once transposed (for
+// The forward state at every chunk start comes from the workspace (bf16, [b][h][chunk][j][i]), left
+// there by the saving forward pass -- or, when the caller has none, by a state-only pass of the
+// forward kernel that chunk_backward() runs first.  The kernel sweeps the chunks in reverse order
+// with the reverse state G in MFMA accumulators.  G is kept twice, once with rows j / columns i (for gv) and once transposed (for
 // gk), so that it can be fed back to the MFMAs as an operand without leaving the registers; the
 // forward state at the tile starts of a chunk is recomputed from the checkpoint and held as packed
 // bf16 operands.
@@ -87,7 +87,7 @@ struct BwdArgs {
 // ------------------------------------------------------------------------------------------
 // Consumer group GRP of two: gr, gk, gw, gu.
 // ------------------------------------------------------------------------------------------
-template <bool kSweepStates, bool kRagged, int GRP>
+template <bool kRagged, int GRP>
 __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *smem, const int *s_wild, int b, int h, int q, int lane)
 {
     const int T = a.T, H = a.H;
@@ -101,50 +101,6 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     auto mine = [](int p) { return (p & 1) == (GRP ^ 1); };   // group 0: tiles 3, 1; group 1: tiles 2, 0
     int item = 0;
     WKV6_STAMP_DECL;
-    if (kSweepStates) {
-        // phase 1: S^T (rows i, column j = col), checkpoint at every chunk start; group 0 only
-        f32x4 S[4];
-#pragma unroll
-        for (int m = 0; m < 4; ++m) {
-            S[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
-            if (a.s0) S[m] = *reinterpret_cast<const f32x4 *>(a.s0 + (int64_t)(b * H + h) * (kN * kN) + col * kN + 16 * m + 4 * g);
-        }
-        for (int c = 0; c < nchunk; ++c, ++item) {
-            __syncthreads();
-            if (GRP != 0) continue;
-            const unsigned char *op = smem + BwdLds::kOp + (item & 1) * BwdLds::kOpBytes;
-            const unsigned char *kt = smem + BwdLds::kRawRK + (item % 3) * 2 * kTileBytes + kTileBytes;
-            const float *gg = reinterpret_cast<const float *>(op + BwdLds::kOpG);
-            const unsigned char *vt = smem + BwdLds::kRawVG + (item % 3) * 2 * kTileBytes;
-            bf16_t *dst = ck + (int64_t)c * (kN * kN) + col * kN;
-#pragma unroll
-            for (int m = 0; m < 4; ++m)
-                *reinterpret_cast<uint2 *>(dst + 16 * m + 4 * g) = make_uint2(pack_bf16x2(S[m][0], S[m][1]), pack_bf16x2(S[m][2], S[m][3]));
-            if (c + 1 == nchunk) {
-                // The state after the last chunk is never used.  The last chunk's own state is what
-                // phase 2 starts with: it goes straight into the LDS state tile of the next item
-                // (the producer waves load the tiles of all later items from the workspace).
-                unsigned char *stt = smem + BwdLds::kState + ((item + 1) & 1) * kTileBytes;
-#pragma unroll
-                for (int m = 0; m < 4; ++m)
-                    *reinterpret_cast<uint2 *>(stt + tile_off(col, 16 * m + 4 * g)) = make_uint2(pack_bf16x2(S[m][0], S[m][1]), pack_bf16x2(S[m][2], S[m][3]));
-                continue;
-            }
-#pragma unroll 1
-            for (int p = 0; p < 4; ++p) {
-                const s16x4 kq = tile_frag_tok(kt, 16 * q, 16 * p, l16, g);
-                const float gq = gg[p * kN + col];
-#pragma unroll
-                for (int m = 0; m < 4; ++m) S[m] = mfma16(tile_frag_tok(vt, 16 * m, 16 * p, l16, g), kq, S[m]);
-                settle(S[0], S[1], S[2], S[3]);
-#pragma unroll
-                for (int m = 0; m < 4; ++m) { S[m][0] *= gq; S[m][1] *= gq; S[m][2] *= gq; S[m][3] *= gq; }
-            }
-        }
-        // the checkpoints are read back by other waves too: have them in memory before the next barrier
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-    // phase 2
     float *vgyw = reinterpret_cast<float *>(smem + BwdLds::kVgy) + (4 * GRP + q) * 16;
     f32x4 Gj[4];   // reverse state, rows i, column j = col (the copy with rows j lives in the gv waves)
 #pragma unroll
@@ -157,8 +113,8 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     bf16_t *gr_h = a.gr + base, *gk_h = a.gk + base, *gw_h = a.gw + base;
     const uint32_t rowbytes = (uint32_t)C * 2u;
     // Saved forward state of a chunk as packed bf16: Sraw[m] = S^T[i = 16m + 4g .. +3][j = col].  It
-    // comes out of LDS, where the producer waves put the chunk's block from the workspace (written
-    // by the forward pass, or by phase 1 above).  The consumer waves issue no global load at all:
+    // comes out of LDS, where the producer waves put the chunk's block from the workspace.  The
+    // consumer waves issue no global load at all:
     // their loads would queue behind their own gradient stores, and a wave's memory operations
     // complete in program order.
     uint2 Sraw[4];
@@ -394,7 +350,7 @@ struct GvState {
             for (int rr = 0; rr < 4; ++rr) Gi[m][rr] = gsT ? gsT[(16 * m + 4 * g + rr) * kN + col] : 0.f;
     }
 };
-// the tiles of chunk c (phase 2 item `item`), last to first
+// the tiles of chunk c (chunk visit `item`), last to first
 template <bool kRagged>
 __device__ __forceinline__ void bwd_gv_chunk(GvState &st, const BwdArgs &a, const unsigned char *smem, bf16_t *gv_h,
                                              uint32_t rowbytes, int c, int item, int q, int lane)
@@ -449,7 +405,7 @@ __device__ __forceinline__ void bwd_gv_chunk(GvState &st, const BwdArgs &a, cons
 // ------------------------------------------------------------------------------------------
 // Loader / producer: wave p <-> tile p of every chunk, lane = channel.
 // ------------------------------------------------------------------------------------------
-template <bool kSweepStates, bool kRagged>
+template <bool kRagged>
 __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *smem, int *s_wild, int b, int h, int p, int lane)
 {
     const int T = a.T, H = a.H;
@@ -457,14 +413,12 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     const int64_t C = (int64_t)H * kN;
     const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
     const int nchunk = (T + CL - 1) / CL;
-    const int nitem = kSweepStates ? 2 * nchunk : nchunk;   // [phase 1 chunks 0..n-1] then phase 2 chunks n-1..0
+    const int nitem = nchunk;   // item = chunk visit: chunks n-1 .. 0
     const float uc = load1(a.u + h * kN + ch);
     const bf16_t *rb = a.r + base, *kb_ = a.k + base, *vb = a.v + base, *wb = a.w + base, *gb = a.gy + base;   // uniform
     const uint32_t rowbytes = (uint32_t)C * 2u;
     const uint32_t lds0 = lds_address(smem);
-    // item -> (chunk, full): phase 1 items need only k, v, w
-    auto item_chunk = [&](int it) { return kSweepStates ? (it < nchunk ? it : 2 * nchunk - 1 - it) : nchunk - 1 - it; };
-    auto item_full = [&](int it) { return kSweepStates ? it >= nchunk : true; };
+    auto item_chunk = [&](int it) { return nchunk - 1 - it; };
     // this lane's part of an 8-row block load: row (lane >> 3), 16-byte piece swizzled with the row
     const int lrow = lane >> 3;
     const uint32_t lpiece = (uint32_t)(((lane & 7) ^ lrow) << 4);
@@ -474,7 +428,6 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     auto issue_loads = [&](int it) -> int {
         if ((WKV6_ABLATE & 1) && T > 0) return 0;
         const int tb = item_chunk(it) * CL + 16 * p;
-        const bool full = item_full(it);
         const uint32_t rk = lds0 + BwdLds::kRawRK + (it % 3) * 2 * kTileBytes + 16 * p * kTileRow;
         const uint32_t ww = lds0 + BwdLds::kRawW + (it % 3) * kTileBytes + 16 * p * kTileRow;
         const uint32_t vg = lds0 + BwdLds::kRawVG + (it % 3) * 2 * kTileBytes + 16 * p * kTileRow;
@@ -485,14 +438,12 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
             load_rows8_to_lds(kb_, o, rk + kTileBytes + 8 * hf * kTileRow);
             load_rows8_to_lds(wb, o, ww + 8 * hf * kTileRow);
             load_rows8_to_lds(vb, o, vg + 8 * hf * kTileRow);
-            if (full) {
-                load_rows8_to_lds(rb, o, rk + 8 * hf * kTileRow);
-                load_rows8_to_lds(gb, o, vg + kTileBytes + 8 * hf * kTileRow);
-            }
+            load_rows8_to_lds(rb, o, rk + 8 * hf * kTileRow);
+            load_rows8_to_lds(gb, o, vg + kTileBytes + 8 * hf * kTileRow);
         }
-        return full ? 10 : 6;
+        return 10;
     };
-    // The saved forward state of item `it` (phase 2 with the states left by the forward pass): the
+    // The saved forward state of item `it`: the
     // chunk's 64x64 bf16 block [j][i] is a tile with j in the place of the token; wave p brings rows
     // 16p..16p+15.  It is requested ONE item ahead (two slots), ahead of the tile loads in the queue,
     // and awaited at the end of the visit, behind the gv stores issued in between -- the consumer
@@ -534,7 +485,6 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     const float kLog2Log2e = 0.5287663729448977f;   // log2(log2(e)): exp(w) log2(e) = 2^(w log2(e) + this)
     auto prepare = [&](int it) {
         const int tb = item_chunk(it) * CL + 16 * p;
-        const bool full = item_full(it);
         // lane addresses of the 8 swizzle phases in the three blocks this item uses (the row and tensor
         // offsets on top of them are instruction immediates)
         unsigned char *a_rk[8];
@@ -552,7 +502,6 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
             uint32_t ra = *reinterpret_cast<const uint16_t *>(a_rk[e & 7] + e * kTileRow);
             uint32_t rk = *reinterpret_cast<const uint16_t *>(a_rk[e & 7] + kTileBytes + e * kTileRow);
             uint32_t rw = *reinterpret_cast<const uint16_t *>(a_w[e & 7] + e * kTileRow);
-            if (!full) ra = 0u;   // r is not loaded for the phase 1 items
             if (kRagged && tb + e >= T) { ra = 0u; rk = 0u; rw = 0xff80u; }
             fr[e] = bf16_bits_to_float(ra); fk[e] = bf16_bits_to_float(rk); fw[e] = bf16_bits_to_float(rw);
         }
@@ -588,22 +537,19 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
         }
         unsigned char *op = smem + BwdLds::kOp + (it & 1) * BwdLds::kOpBytes;
         reinterpret_cast<float *>(op + BwdLds::kOpG)[p * kN + ch] = pa;
-        if (full) {
-            const float tr = transpose_reduce16(pr, lane);
-            if ((lane & 3) == 0) reinterpret_cast<float *>(op + BwdLds::kOpRuk)[16 * p + ((lane >> 2) & 15)] = tr;
-        }
+        const float tr = transpose_reduce16(pr, lane);
+        if ((lane & 3) == 0) reinterpret_cast<float *>(op + BwdLds::kOpRuk)[16 * p + ((lane >> 2) & 15)] = tr;
     };
     // item `it` is loaded during iteration it-2 (or the prologue) and prepared during iteration it-1
     GvState gvst;
     gvst.init(a.gsT ? a.gsT + (int64_t)(b * H + h) * (kN * kN) : nullptr, 16 * p + (lane & 15), lane >> 4);
     WKV6_STAMP_DECL;
-    // phase 2 items get their chunk's saved state loaded one item ahead -- except, with kSweepStates,
-    // the first of them, whose state the consumers hand over through LDS at the end of phase 1
-    auto state_by_load = [&](int it) { return it < nitem && item_full(it) && !(kSweepStates && it == nchunk); };
+    // every item's saved state is loaded one item ahead
+    auto state_by_load = [&](int it) { return it < nitem; };
     // gv stores an item's visit leaves in flight behind the loads issued before them.  The chunk with
     // the ragged tail issues anything from 0 to 16 (a store whose lanes are all past the end is
     // skipped): counting none for it makes the waits behind it wait for everything older.
-    auto gv_stores = [&](int it) { return !item_full(it) ? 0 : (kRagged && item_chunk(it) == nchunk - 1) ? 0 : 16; };
+    auto gv_stores = [&](int it) { return (kRagged && item_chunk(it) == nchunk - 1) ? 0 : 16; };
     if (state_by_load(0)) issue_state(0);
     issue_loads(0);
     wait_younger(nitem > 1 ? issue_loads(1) : 0);
@@ -625,7 +571,7 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
             WKV6_STAMP();
         }
         // the gv role, on the waves the operand preparation leaves partly idle
-        if (item_full(it)) bwd_gv_chunk<kRagged>(gvst, a, smem, a.gv + base, rowbytes, item_chunk(it), it, p, lane);
+        bwd_gv_chunk<kRagged>(gvst, a, smem, a.gv + base, rowbytes, item_chunk(it), it, p, lane);
         // the next item's state has to be in LDS when the consumers pass the barrier
         if (state_loads) wait_younger(younger + gv_stores(it));
         WKV6_STAMP();
@@ -639,7 +585,7 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
 //   loader/producer + gv | consumer group 0 (tiles 3, 1) | consumer group 1 (tiles 2, 0)
 constexpr int kBwdWaves = 12;
 
-template <bool kSweepStates, bool kRagged>
+template <bool kRagged>
 __global__ __launch_bounds__(kBwdWaves * 64) void chunk_bwd_kernel(BwdArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -658,9 +604,9 @@ __global__ __launch_bounds__(kBwdWaves * 64) void chunk_bwd_kernel(BwdArgs a)
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int role = wave >> 2, q = wave & 3;
-    if (role == 0) bwd_producer<kSweepStates, kRagged>(a, smem, &s_wild, b, h, q, lane);
-    else if (role == 1) bwd_consumer<kSweepStates, kRagged, 0>(a, smem, &s_wild, b, h, q, lane);
-    else bwd_consumer<kSweepStates, kRagged, 1>(a, smem, &s_wild, b, h, q, lane);
+    if (role == 0) bwd_producer<kRagged>(a, smem, &s_wild, b, h, q, lane);
+    else if (role == 1) bwd_consumer<kRagged, 0>(a, smem, &s_wild, b, h, q, lane);
+    else bwd_consumer<kRagged, 1>(a, smem, &s_wild, b, h, q, lane);
 #ifdef WKV6_TIMING
     if (threadIdx.x == 0) a.dbg[16 * 256 + 2 * blockIdx.x + 1] = __builtin_readcyclecounter();
 #endif
@@ -758,8 +704,13 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
         return hipGetLastError();
     };
     const bool ragged = (T % CL) != 0;   // the last chunk has tokens past the end
-    if (states_ready) return ragged ? launch(chunk_bwd_kernel<false, true>) : launch(chunk_bwd_kernel<false, false>);
-    return ragged ? launch(chunk_bwd_kernel<true, true>) : launch(chunk_bwd_kernel<true, false>);
+    if (!states_ready) {
+        // No states from a saving forward: the forward kernel's state-only pass (no y) leaves them in
+        // the workspace first.
+        hipError_t e = chunk_forward(st, kF32, B, T, H, r, k, v, w, u, s0, nullptr, nullptr, nullptr, workspace, nullptr, false, false);
+        if (e != hipSuccess) return e;
+    }
+    return ragged ? launch(chunk_bwd_kernel<true>) : launch(chunk_bwd_kernel<false>);
 }
 
 // Training pair in time segments, last step: gu of a batch row = sum over its segments; the decay

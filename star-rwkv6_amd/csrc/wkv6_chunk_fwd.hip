@@ -135,7 +135,7 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
             for (int m = 0; m < 4; ++m) S[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
         }
         bf16_t *y_h = a.y + base;
-        if (kSave && GRP == 0 && b == 0 && q == 0 && lane == 0) a.arrivals[h] = 0;
+        if (kSave && GRP == 0 && b == 0 && q == 0 && lane == 0 && a.arrivals) a.arrivals[h] = 0;
         for (int c = 0; c < nchunk; ++c, ++it) {
             WKV6_FSTAMP();
             if (kSave && GRP == 0) {
@@ -555,7 +555,8 @@ static unsigned forward_grid(int64_t pairs, bool *multi, int *split) {
 
 hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u,
-                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states, float *dsum, bool reverse)
+                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states, float *dsum, bool reverse,
+                         bool counters)
 {
     FwdArgs a = {};
     a.dsum = dsum;
@@ -563,7 +564,7 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
     a.T = (int)T; a.H = (int)H; a.nitems = (int)(B * H);
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
     a.s0 = s0; a.map = map; a.y = (bf16_t *)y; a.sT = sT; a.ckpt = (float *)saved_states;
-    a.arrivals = saved_states ? reinterpret_cast<int *>(reinterpret_cast<char *>(saved_states) + chunk_backward_workspace_bytes(B, T, H)) : nullptr;
+    a.arrivals = saved_states && counters ? reinterpret_cast<int *>(reinterpret_cast<char *>(saved_states) + chunk_backward_workspace_bytes(B, T, H)) : nullptr;
     a.dbg = saved_states ? reinterpret_cast<long long *>((float *)saved_states + (size_t)(B * H) * ((T + CL - 1) / CL) * kN * kN + 1024) : nullptr;
     bool multi;
     const unsigned grid = forward_grid(B * H, &multi, &a.split);

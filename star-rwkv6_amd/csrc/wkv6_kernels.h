@@ -36,7 +36,8 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
                          const void *r, const void *k, const void *v, const void *w, const void *u,
                          const void *s0, const int64_t *map, void *y, void *sT, void *saved_states,
                          float *dsum = nullptr,    // dsum: see chunk_forward_segments_run
-                         bool reverse = false);    // the time axis read back to front (T a multiple of 64, no y)
+                         bool reverse = false,     // the time axis read back to front (T a multiple of 64, no y)
+                         bool counters = true);    // saved_states ends with the per-head counters of the fused gu sum (zeroed here)
 
 // Few pairs, long sequence: the forward as P time segments side by side (two passes joined by the
 // affine map of a segment's state).  chunk_forward_segments = P for the shape (1 = does not apply).
