@@ -86,7 +86,9 @@ int wkv6_forward_with_state_ex(void *stream, int dtype, int state_dtype, int alg
 /* Optional workspace of wkv6_forward_ex / wkv6_forward_with_state_ex (0 = none useful).  Where it is
  * non-zero -- a long bf16 sequence with so few (batch, head) pairs that most of the chip would idle --
  * passing that many bytes lets the forward run as time segments side by side (same results to
- * rounding); without it the call works as always. */
+ * rounding); without it the call works as always.  Batches need T to divide into equal segments
+ * of whole 64-token chunks; a single sequence (B = 1) may have any length if its final state is
+ * fp32 or not asked for. */
 size_t wkv6_forward_workspace_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H);
 
 /* Forward (inference) with the layer's output stage fused in; y itself is not written:

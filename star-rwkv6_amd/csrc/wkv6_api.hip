@@ -82,7 +82,10 @@ static int forward_impl(void *stream, int dtype, int state_dtype, int algo,
         return finish(wkv6::scan_forward(st, dtype, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys));
     if (!saved && workspace && aligned16(workspace)) {
         const size_t need = wkv6::chunk_forward_segments_workspace_bytes(B, T, H);
-        if (need > 0 && workspace_bytes >= need)
+        // (tokens left over behind the equal segments are run from an fp32 state: possible when the
+        // final state is fp32 or not wanted)
+        const bool remainder_ok = wkv6::chunk_forward_segments_remainder(B, T, H) == 0 || state_dtype == WKV6_F32 || !ys;
+        if (need > 0 && workspace_bytes >= need && remainder_ok)
             return finish(wkv6::chunk_forward_segments_run(st, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys, workspace));
     }
     return finish(wkv6::chunk_forward(st, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys, saved));

@@ -609,7 +609,8 @@ hipError_t chunk_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64
 // p + 1 sends into its incoming state: its own contribution plus D_{p+1} times what arrives at its end).
 template <typename Ts, bool kReverse, int P>
 __global__ __launch_bounds__(256) void segment_chain_kernel(int H, const Ts *__restrict__ s0, const int64_t *__restrict__ map,
-                                                            const float *__restrict__ dsum, float *__restrict__ states, Ts *__restrict__ sT)
+                                                            const float *__restrict__ dsum, float *__restrict__ states, Ts *__restrict__ sT,
+                                                            float *__restrict__ sT32)   // the final state: as Ts and / or as fp32 (either may be null)
 {
     // Thread: four value columns i0..i0+3 of one key row j of one (batch, head): 1024 threads per pair,
     // gridDim.x * 256 = B * H * 1024.  states[(b*P + seg), h] holds U on entry and the segment's
@@ -640,51 +641,77 @@ __global__ __launch_bounds__(256) void segment_chain_kernel(int H, const Ts *__r
         S[0] = fmaf(S[0], dd, x[n].x); S[1] = fmaf(S[1], dd, x[n].y); S[2] = fmaf(S[2], dd, x[n].z); S[3] = fmaf(S[3], dd, x[n].w);
     }
     if (sT) store4(sT + (((int64_t)b * H + h) * kN + j) * kN + i0, S[0], S[1], S[2], S[3]);
+    if (sT32) store4(sT32 + (((int64_t)b * H + h) * kN + j) * kN + i0, S[0], S[1], S[2], S[3]);
 }
 template <typename Ts, bool kReverse>
 static hipError_t launch_chain(hipStream_t st, int P, int64_t B, int64_t H, const Ts *s0, const int64_t *map,
-                               const float *dsum, float *states, Ts *sT)
+                               const float *dsum, float *states, Ts *sT, float *sT32 = nullptr)
 {
     const dim3 grid((unsigned)(B * H * 4)), block(256);
     switch (P) {
-    case 2: hipLaunchKernelGGL((segment_chain_kernel<Ts, kReverse, 2>), grid, block, 0, st, (int)H, s0, map, dsum, states, sT); break;
-    case 4: hipLaunchKernelGGL((segment_chain_kernel<Ts, kReverse, 4>), grid, block, 0, st, (int)H, s0, map, dsum, states, sT); break;
-    case 8: hipLaunchKernelGGL((segment_chain_kernel<Ts, kReverse, 8>), grid, block, 0, st, (int)H, s0, map, dsum, states, sT); break;
-    case 16: hipLaunchKernelGGL((segment_chain_kernel<Ts, kReverse, 16>), grid, block, 0, st, (int)H, s0, map, dsum, states, sT); break;
+    case 2: hipLaunchKernelGGL((segment_chain_kernel<Ts, kReverse, 2>), grid, block, 0, st, (int)H, s0, map, dsum, states, sT, sT32); break;
+    case 4: hipLaunchKernelGGL((segment_chain_kernel<Ts, kReverse, 4>), grid, block, 0, st, (int)H, s0, map, dsum, states, sT, sT32); break;
+    case 8: hipLaunchKernelGGL((segment_chain_kernel<Ts, kReverse, 8>), grid, block, 0, st, (int)H, s0, map, dsum, states, sT, sT32); break;
+    case 16: hipLaunchKernelGGL((segment_chain_kernel<Ts, kReverse, 16>), grid, block, 0, st, (int)H, s0, map, dsum, states, sT, sT32); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
 }
 
-// Number of segments for this shape (1 = not worth it / not possible): the pairs times the segments
-// should still fit the chip once, a segment is a whole number of chunks and at least four of them.
-int chunk_forward_segments(int64_t B, int64_t T, int64_t H) {
+// Number of segments for this shape (1 = not worth it / not possible) and their length: the pairs
+// times the segments should still fit the chip once, a segment is a whole number of chunks and at
+// least four of them.  A single sequence need not divide evenly: what is left over behind the P
+// segments (less than P chunks) follows as an ordinary pass from the state the segments end in.
+// (With B > 1 the first P * L tokens of every batch row are not one contiguous (B*P, L, C) tensor.)
+static int forward_segments_plan(int64_t B, int64_t T, int64_t H, int64_t *L) {
     const int64_t pairs = B * H, cus = compute_units();
     // (two passes over T / P tokens and two more launches against one pass over T: nothing to gain
     // below four segments or on short sequences)
     if (T < 2048) return 1;
-    for (int P = 16; P >= 4; P >>= 1)
-        if (pairs * P <= cus && T % (P * CL) == 0 && T / P >= 4 * CL) return P;
+    for (int P = 16; P >= 4; P >>= 1) {
+        const int64_t l = T / P / CL * CL;
+        if (pairs * P > cus || l < 4 * CL) continue;
+        if (P * l != T && B != 1) continue;
+        *L = l;
+        return P;
+    }
     return 1;
+}
+int chunk_forward_segments(int64_t B, int64_t T, int64_t H) {
+    int64_t L;
+    return forward_segments_plan(B, T, H, &L);
+}
+int64_t chunk_forward_segments_remainder(int64_t B, int64_t T, int64_t H) {
+    int64_t L = 0;
+    const int P = forward_segments_plan(B, T, H, &L);
+    return P <= 1 ? 0 : T - P * L;
 }
 size_t chunk_forward_segments_workspace_bytes(int64_t B, int64_t T, int64_t H) {
     const int P = chunk_forward_segments(B, T, H);
-    return P <= 1 ? 0 : (size_t)(B * P * H) * (kN * kN + 4 * kN) * sizeof(float);
+    // per segment and pair a state and the decay exponents; per pair the state the segments end in
+    return P <= 1 ? 0 : ((size_t)(B * P * H) * (kN * kN + 4 * kN) + (size_t)(B * H) * kN * kN) * sizeof(float);
 }
 
+// A remainder needs fp32 states at the boundary or no final state (see the API layer's check).
 hipError_t chunk_forward_segments_run(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                                       const void *r, const void *k, const void *v, const void *w, const void *u,
                                       const void *s0, const int64_t *map, void *y, void *sT, void *workspace)
 {
-    const int P = chunk_forward_segments(B, T, H);
-    const int64_t L = T / P, rows = B * P;
-    float *states = (float *)workspace, *dsum = states + rows * H * kN * kN;
+    int64_t L = 0;
+    const int P = forward_segments_plan(B, T, H, &L);
+    const int64_t rows = B * P, rem = T - P * L;
+    float *states = (float *)workspace, *dsum = states + rows * H * kN * kN, *mid = dsum + rows * H * 4 * kN;
     hipError_t e = chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, nullptr, nullptr, nullptr, states, nullptr, dsum);
     if (e != hipSuccess) return e;
-    e = state_dtype == kF32 ? launch_chain<float, false>(st, P, B, H, (const float *)s0, map, dsum, states, (float *)sT)
-                            : launch_chain<bf16_t, false>(st, P, B, H, (const bf16_t *)s0, map, dsum, states, (bf16_t *)sT);
+    void *end_state = rem ? nullptr : sT;   // with a remainder the segments end in `mid`
+    e = state_dtype == kF32 ? launch_chain<float, false>(st, P, B, H, (const float *)s0, map, dsum, states, (float *)end_state, rem ? mid : nullptr)
+                            : launch_chain<bf16_t, false>(st, P, B, H, (const bf16_t *)s0, map, dsum, states, (bf16_t *)end_state, rem ? mid : nullptr);
     if (e != hipSuccess) return e;
-    return chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, states, nullptr, y, nullptr, nullptr);
+    e = chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, states, nullptr, y, nullptr, nullptr);
+    if (e != hipSuccess || rem == 0) return e;
+    const int64_t off = P * L * H * kN;   // (B == 1) elements in front of the remainder
+    auto at = [&](const void *p) { return (const void *)((const bf16_t *)p + off); };
+    return chunk_forward(st, kF32, B, rem, H, at(r), at(k), at(v), at(w), u, mid, nullptr, (bf16_t *)y + off, sT, nullptr);
 }
 
 hipError_t segment_chain_reverse(hipStream_t st, int P, int64_t B, int64_t H, const float *dsum, float *states) {

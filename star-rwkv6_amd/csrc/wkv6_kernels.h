@@ -42,6 +42,7 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
 // Few pairs, long sequence: the forward as P time segments side by side (two passes joined by the
 // affine map of a segment's state).  chunk_forward_segments = P for the shape (1 = does not apply).
 int chunk_forward_segments(int64_t B, int64_t T, int64_t H);
+int64_t chunk_forward_segments_remainder(int64_t B, int64_t T, int64_t H);   // tokens behind the P equal segments (single sequence only)
 size_t chunk_forward_segments_workspace_bytes(int64_t B, int64_t T, int64_t H);
 hipError_t chunk_forward_segments_run(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                                       const void *r, const void *k, const void *v, const void *w, const void *u,

@@ -447,14 +447,16 @@ def test_backpropagation_over_two_pieces_equals_one_piece(op):
 
 # Few pairs, long sequence: with the optional forward workspace the sequence runs as time segments
 # side by side (two passes joined by the affine state map of a segment).
-@pytest.mark.parametrize("B,T,H,sdt", [(1, 2048, 2, torch.float32), (2, 2304, 1, torch.bfloat16), (3, 4096, 5, torch.float32), (12, 2048, 4, torch.float32)])
+@pytest.mark.parametrize("B,T,H,sdt", [(1, 2048, 2, torch.float32), (2, 2304, 1, torch.bfloat16), (3, 4096, 5, torch.float32), (12, 2048, 4, torch.float32),
+                                       (1, 5000, 2, torch.float32), (1, 3000, 3, torch.bfloat16)])   # single sequences that leave a remainder
 def test_forward_in_time_segments(op, oracle, B, T, H, sdt):
     from rwkv_kernel import _native
     N = 64
     lib = _native.load()
     assert lib.wkv6_forward_workspace_bytes(_native.BF16, CHUNK, B, T, H * N, H) > 0
     assert lib.wkv6_forward_workspace_bytes(_native.BF16, CHUNK, 8, 1024, 2048, 32) == 0    # fills the chip as it is
-    assert lib.wkv6_forward_workspace_bytes(_native.BF16, CHUNK, B, T + 64, H * N, H) == 0  # no equal segments
+    # no equal segments: only a single sequence can leave a remainder behind them
+    assert (lib.wkv6_forward_workspace_bytes(_native.BF16, CHUNK, B, T + 64, H * N, H) > 0) == (B == 1)
     ins = oracle.make_inputs(B, T, H, N, 60 + B, with_state=True)
     dev, ref = cast_inputs(ins[:5], torch.bfloat16)
     kinds = min(2, B)
@@ -473,8 +475,7 @@ def test_forward_in_time_segments(op, oracle, B, T, H, sdt):
     y2_ref, sT2_ref = oracle.forward_c(*ref2, N, s_ref[0], smap)
     check_close("y with an exact segment", y2, y2_ref, torch.bfloat16)
     check_close("sT with an exact segment", sT2, sT2_ref, torch.bfloat16)
-    # and from a zero state, against the same call without the workspace (the torch flavour's
-    # stateless forward does not pass one)
+    # and from a zero state, with and without a final state
     y0, s0T = op(*dev, return_state=True)
     y1, _ = op(*dev)
     torch.cuda.synchronize()
