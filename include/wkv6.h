@@ -106,6 +106,15 @@ int wkv6_forward_gn_gate(void *stream, int dtype, int state_dtype,
                          const void *r, const void *k, const void *v, const void *w, const void *u,
                          const void *s, const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
                          void *out, void *ys);
+/* Same with the optional workspace of wkv6_forward_workspace_bytes(dtype, WKV6_ALGO_CHUNK, ...): a long
+ * sequence of few (batch, head) pairs then runs as time segments side by side.  No counterpart in the
+ * reference. */
+int wkv6_forward_gn_gate_ex(void *stream, int dtype, int state_dtype,
+                            int64_t B, int64_t T, int64_t C, int64_t H,
+                            int has_init_state, const int64_t *state_map,
+                            const void *r, const void *k, const void *v, const void *w, const void *u,
+                            const void *s, const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
+                            void *out, void *ys, void *workspace, size_t workspace_bytes);
 
 /* Backward of the stateless forward: gr,gk,gv,gw (B,T,C) and gu (B,C), all in the output type.
  * Replaces backward_{bf16,fp16,fp32}(B,T,C,H,r,k,v,w,u,gy,gr,gk,gv,gw,gu),

@@ -106,6 +106,16 @@ int wkv6_forward_gn_gate(void *stream, int dtype, int state_dtype,
                          const void *r, const void *k, const void *v, const void *w, const void *u,
                          const void *s, const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
                          void *out, void *ys) {
+    return wkv6_forward_gn_gate_ex(stream, dtype, state_dtype, B, T, C, H, has_init_state, state_map, r, k, v, w, u, s,
+                                   gate, gn_scale, gn_offset, gn_eps, out, ys, nullptr, 0);
+}
+
+int wkv6_forward_gn_gate_ex(void *stream, int dtype, int state_dtype,
+                            int64_t B, int64_t T, int64_t C, int64_t H,
+                            int has_init_state, const int64_t *state_map,
+                            const void *r, const void *k, const void *v, const void *w, const void *u,
+                            const void *s, const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
+                            void *out, void *ys, void *workspace, size_t workspace_bytes) {
     int rc = check_shape(dtype, B, T, C, H);
     if (rc != WKV6_OK) return rc;
     if (!r || !k || !v || !w || !u || !gate || !gn_scale || !gn_offset || !out) return WKV6_ERR_ARG;
@@ -118,6 +128,14 @@ int wkv6_forward_gn_gate(void *stream, int dtype, int state_dtype,
         return finish(wkv6::step_forward_fused((hipStream_t)stream, state_dtype, B, H, r, k, v, w, u,
                                                has_init_state ? s : nullptr, has_init_state ? state_map : nullptr,
                                                gate, gn_scale, gn_offset, gn_eps, out, ys));
+    if (workspace && aligned16(workspace)) {   // optional: few pairs, long sequence -> time segments side by side
+        const size_t need = wkv6::chunk_forward_segments_workspace_bytes(B, T, H);
+        const bool remainder_ok = wkv6::chunk_forward_segments_remainder(B, T, H) == 0 || state_dtype == WKV6_F32 || !ys;
+        if (need > 0 && workspace_bytes >= need && remainder_ok)
+            return finish(wkv6::chunk_forward_segments_run((hipStream_t)stream, state_dtype, B, T, H, r, k, v, w, u,
+                                                           has_init_state ? s : nullptr, has_init_state ? state_map : nullptr,
+                                                           out, ys, workspace, gate, gn_scale, gn_offset, gn_eps));
+    }
     return finish(wkv6::chunk_forward_fused((hipStream_t)stream, state_dtype, B, T, H, r, k, v, w, u,
                                             has_init_state ? s : nullptr, has_init_state ? state_map : nullptr,
                                             gate, gn_scale, gn_offset, gn_eps, out, ys));

@@ -693,9 +693,11 @@ size_t chunk_forward_segments_workspace_bytes(int64_t B, int64_t T, int64_t H) {
 }
 
 // A remainder needs fp32 states at the boundary or no final state (see the API layer's check).
+// With `gate` the passes that produce output run the fused output stage (y = out then).
 hipError_t chunk_forward_segments_run(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                                       const void *r, const void *k, const void *v, const void *w, const void *u,
-                                      const void *s0, const int64_t *map, void *y, void *sT, void *workspace)
+                                      const void *s0, const int64_t *map, void *y, void *sT, void *workspace,
+                                      const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps)
 {
     int64_t L = 0;
     const int P = forward_segments_plan(B, T, H, &L);
@@ -707,10 +709,14 @@ hipError_t chunk_forward_segments_run(hipStream_t st, int state_dtype, int64_t B
     e = state_dtype == kF32 ? launch_chain<float, false>(st, P, B, H, (const float *)s0, map, dsum, states, (float *)end_state, rem ? mid : nullptr)
                             : launch_chain<bf16_t, false>(st, P, B, H, (const bf16_t *)s0, map, dsum, states, (bf16_t *)end_state, rem ? mid : nullptr);
     if (e != hipSuccess) return e;
-    e = chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, states, nullptr, y, nullptr, nullptr);
+    e = gate ? chunk_forward_fused(st, kF32, rows, L, H, r, k, v, w, u, states, nullptr, gate, gn_scale, gn_offset, gn_eps, y, nullptr)
+             : chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, states, nullptr, y, nullptr, nullptr);
     if (e != hipSuccess || rem == 0) return e;
     const int64_t off = P * L * H * kN;   // (B == 1) elements in front of the remainder
     auto at = [&](const void *p) { return (const void *)((const bf16_t *)p + off); };
+    if (gate)
+        return chunk_forward_fused(st, kF32, B, rem, H, at(r), at(k), at(v), at(w), u, mid, nullptr, at(gate), gn_scale, gn_offset, gn_eps,
+                                   (bf16_t *)y + off, sT);
     return chunk_forward(st, kF32, B, rem, H, at(r), at(k), at(v), at(w), u, mid, nullptr, (bf16_t *)y + off, sT, nullptr);
 }
 

@@ -46,7 +46,9 @@ int64_t chunk_forward_segments_remainder(int64_t B, int64_t T, int64_t H);   // 
 size_t chunk_forward_segments_workspace_bytes(int64_t B, int64_t T, int64_t H);
 hipError_t chunk_forward_segments_run(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                                       const void *r, const void *k, const void *v, const void *w, const void *u,
-                                      const void *s0, const int64_t *map, void *y, void *sT, void *workspace);
+                                      const void *s0, const int64_t *map, void *y, void *sT, void *workspace,
+                                      const void *gate = nullptr, const float *gn_scale = nullptr,
+                                      const float *gn_offset = nullptr, float gn_eps = 0.f);
 
 // The training pair of a long sequence of few pairs as P time segments side by side.  The saving
 // forward leaves, behind the saved chunk states (`extra`), every segment's incoming state and decay

@@ -284,9 +284,12 @@ class RWKVKernelOperator:
             out = torch.empty_like(r)
             ys = torch.empty((B, H, N, N), device=r.device, dtype=sdt) if return_state else None
             with torch.cuda.device(r.device):
-                _native.check(lib.wkv6_forward_gn_gate(
+                # optional workspace: a long sequence of few (batch, head) pairs runs as time segments
+                n = lib.wkv6_forward_workspace_bytes(_DTYPE_CODE[r.dtype], _native.ALGO_CHUNK, B, T, C, H)
+                ws = torch.empty(int(n), device=r.device, dtype=torch.uint8) if n else None
+                _native.check(lib.wkv6_forward_gn_gate_ex(
                     _stream(), _DTYPE_CODE[r.dtype], _DTYPE_CODE[sdt], B, T, C, H,
                     int(init_state is not None), _ptr(state_map),
                     _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(init_state), _ptr(gate), _ptr(sc), _ptr(of),
-                    float(epsilon), _ptr(out), _ptr(ys)))
+                    float(epsilon), _ptr(out), _ptr(ys), _ptr(ws), n))
         return out, ys

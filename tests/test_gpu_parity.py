@@ -331,7 +331,8 @@ def test_chunk_many_pairs_fall_back_pair_by_pair(op, oracle):
 # relative to the largest reference value (the kernel normalises the bf16-rounded y, as a caller
 # would).
 @pytest.mark.parametrize("B,T,H,with_state", [(2, 64, 2, False), (3, 150, 2, True), (1, 1000, 3, False),
-                                              (70, 96, 4, True), (1, 16, 1, False), (5, 1, 3, True), (2, 1, 2, False)])
+                                              (70, 96, 4, True), (1, 16, 1, False), (5, 1, 3, True), (2, 1, 2, False),
+                                              (1, 2600, 2, True), (2, 2048, 3, False)])   # the last two: in time segments
 def test_fused_group_norm_gate(op, oracle, B, T, H, with_state):
     N = 64
     ins = oracle.make_inputs(B, T, H, N, 70 + T, with_state=True)
