@@ -611,13 +611,14 @@ def test_fused_gu_batch_sum(op, oracle, B, T, H, dt):
 
 
 @pytest.mark.gpu
-def test_training_pair_replays_in_a_hip_graph(op, oracle):
+@pytest.mark.parametrize("B,T,H", [(2, 256, 4), (1, 2048, 3)])   # the second: seven launches (time segments)
+def test_training_pair_replays_in_a_hip_graph(op, oracle, B, T, H):
     """forward_save + backward_saved_sum captured once into a graph (the library allocates nothing
     and only enqueues on the given stream), replayed several times with eager work and
     synchronisations in between; every replay must reproduce the eager results bit for bit."""
     from rwkv_kernel import _native
     lib = _native.load()
-    B, T, H, N = 2, 256, 4, 64
+    N = 64
     C = H * N
     r, k, v, w, u, gy = (x.to(torch.bfloat16).cuda().contiguous() for x in oracle.make_inputs(B, T, H, N, 21))
     n = lib.wkv6_saved_bytes(_native.BF16, _native.ALGO_AUTO, B, T, C, H)
