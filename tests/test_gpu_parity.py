@@ -449,7 +449,7 @@ def test_backpropagation_over_two_pieces_equals_one_piece(op):
 # Few pairs, long sequence: with the optional forward workspace the sequence runs as time segments
 # side by side (two passes joined by the affine state map of a segment).
 @pytest.mark.parametrize("B,T,H,sdt", [(1, 2048, 2, torch.float32), (2, 2304, 1, torch.bfloat16), (3, 4096, 5, torch.float32), (12, 2048, 4, torch.float32),
-                                       (1, 5000, 2, torch.float32), (1, 3000, 3, torch.bfloat16)])   # single sequences that leave a remainder
+                                       (1, 5000, 2, torch.float32), (1, 3000, 3, torch.bfloat16), (1, 4097, 2, torch.float32)])   # single sequences that leave a remainder (the last: of one token)
 def test_forward_in_time_segments(op, oracle, B, T, H, sdt):
     from rwkv_kernel import _native
     N = 64
