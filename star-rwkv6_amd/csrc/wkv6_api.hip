@@ -297,7 +297,13 @@ size_t wkv6_backward_with_state_workspace_bytes(int dtype, int algo, int64_t B, 
     if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
     size_t need = wkv6::scan_backward_state_workspace_bytes(B, T, C);
     const size_t c = wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H);
-    return c > need ? c : need;
+    if (c > need) need = c;
+    const int P = train_segments(dtype, algo, B, T, C, H);   // few pairs, long sequence: time segments side by side
+    if (P > 1) {
+        const size_t seg = saved_base_bytes(dtype, WKV6_ALGO_CHUNK, B * P, T / P, C, H) + wkv6::train_segments_layout(B, T, H, nullptr).bytes;
+        if (seg > need) need = seg;
+    }
+    return need;
 }
 
 int wkv6_backward_with_state(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
@@ -319,6 +325,12 @@ int wkv6_backward_with_state(void *stream, int dtype, int algo, int64_t B, int64
     const bool chunk = algo == WKV6_ALGO_CHUNK || (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
     if (!chunk)
         return finish(wkv6::scan_backward_state(st, dtype, B, T, H, r, k, v, w, u, s0, gy, gsT, gr, gk, gv, gw, gu, gs0, workspace));
+    const int P = train_segments(dtype, algo, B, T, C, H);
+    if (P > 1) {
+        char *extra = reinterpret_cast<char *>(workspace) + saved_base_bytes(dtype, WKV6_ALGO_CHUNK, B * P, T / P, C, H);
+        return finish(wkv6::chunk_backward_state_segments(st, B, T, H, r, k, v, w, u, s0, gy, gsT, gr, gk, gv, gw, gu, gs0,
+                                                          workspace, extra));
+    }
     return finish(wkv6::chunk_backward(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace, false, nullptr,
                                        s0, gsT, gs0));
 }

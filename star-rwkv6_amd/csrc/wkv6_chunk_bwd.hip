@@ -717,15 +717,15 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
 // gradient at the first and the last token of a sequence is zero by definition
 // (rwkv_kernels.cu:381,406), where the kernels, given explicit states, leave rounding residue.
 __global__ void segments_finish_kernel(int P, int64_t T, int C, const bf16_t *__restrict__ gu_rows,
-                                       bf16_t *__restrict__ gu, bf16_t *__restrict__ gw)
+                                       bf16_t *__restrict__ gu, bf16_t *__restrict__ gw, bool zero_first, bool zero_last)
 {
     const int c = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
     if (c >= C) return;
     float acc = 0.f;
     for (int p = 0; p < P; ++p) acc += load1(gu_rows + ((int64_t)b * P + p) * C + c);
     store1(gu + (int64_t)b * C + c, acc);
-    store1(gw + (int64_t)b * T * C + c, 0.f);
-    store1(gw + ((int64_t)b * T + T - 1) * C + c, 0.f);
+    if (zero_first) store1(gw + (int64_t)b * T * C + c, 0.f);
+    if (zero_last) store1(gw + ((int64_t)b * T + T - 1) * C + c, 0.f);
 }
 
 hipError_t chunk_backward_saved_segments(hipStream_t st, int64_t B, int64_t T, int64_t H,
@@ -748,7 +748,36 @@ hipError_t chunk_backward_saved_segments(hipStream_t st, int64_t B, int64_t T, i
     if (e != hipSuccess) return e;
     const int C = (int)(H * kN);
     hipLaunchKernelGGL(segments_finish_kernel, dim3((unsigned)((C + 255) / 256), (unsigned)B), dim3(256), 0, st,
-                       s.P, T, C, (const bf16_t *)s.gu_rows, (bf16_t *)gu, (bf16_t *)gw);
+                       s.P, T, C, (const bf16_t *)s.gu_rows, (bf16_t *)gu, (bf16_t *)gw, true, true);
+    return hipGetLastError();
+}
+
+// The same with an initial state, a gradient arriving at the final state and dL/dS_0 wanted
+// (wkv6_backward_with_state): nothing was saved by a forward pass, so the segments' incoming
+// states and the chunk states are rebuilt first (state-only passes of the forward kernel).
+hipError_t chunk_backward_state_segments(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                                         const void *r, const void *k, const void *v, const void *w, const void *u,
+                                         const float *s0, const void *gy, const float *gsT,
+                                         void *gr, void *gk, void *gv, void *gw, void *gu, float *gs0,
+                                         void *saved, void *extra)
+{
+    const TrainSegments s = train_segments_layout(B, T, H, extra);
+    const int64_t L = T / s.P, rows = B * s.P;
+    hipError_t e = chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, nullptr, nullptr, nullptr, s.states, nullptr, s.dsum);
+    if (e != hipSuccess) return e;
+    if ((e = segment_chain_forward(st, s.P, B, H, s.dsum, s.states, s0)) != hipSuccess) return e;
+    e = chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, s.states, nullptr, nullptr, nullptr, saved, nullptr, false, false);
+    if (e != hipSuccess) return e;
+    e = chunk_forward(st, kF32, rows, L, H, r, r, gy, w, u, nullptr, nullptr, nullptr, s.gstates, nullptr, nullptr, true);
+    if (e != hipSuccess) return e;
+    if ((e = segment_chain_reverse(st, s.P, B, H, s.dsum, s.gstates, gsT, gs0)) != hipSuccess) return e;
+    e = chunk_backward(st, rows, L, H, r, k, v, w, u, gy, gr, gk, gv, gw, s.gu_rows, saved, true, nullptr,
+                       s.states, s.gstates, nullptr);
+    if (e != hipSuccess) return e;
+    const int C = (int)(H * kN);
+    // (the decay gradient at an end of the sequence is zero by definition only where no state / no gradient comes in)
+    hipLaunchKernelGGL(segments_finish_kernel, dim3((unsigned)((C + 255) / 256), (unsigned)B), dim3(256), 0, st,
+                       s.P, T, C, (const bf16_t *)s.gu_rows, (bf16_t *)gu, (bf16_t *)gw, s0 == nullptr, gsT == nullptr);
     return hipGetLastError();
 }
 

@@ -720,8 +720,12 @@ hipError_t chunk_forward_segments_run(hipStream_t st, int state_dtype, int64_t B
     return chunk_forward(st, kF32, B, rem, H, at(r), at(k), at(v), at(w), u, mid, nullptr, (bf16_t *)y + off, sT, nullptr);
 }
 
-hipError_t segment_chain_reverse(hipStream_t st, int P, int64_t B, int64_t H, const float *dsum, float *states) {
-    return launch_chain<float, true>(st, P, B, H, nullptr, nullptr, dsum, states, nullptr);
+hipError_t segment_chain_reverse(hipStream_t st, int P, int64_t B, int64_t H, const float *dsum, float *states,
+                                 const float *arriving, float *leaving) {
+    return launch_chain<float, true>(st, P, B, H, arriving, nullptr, dsum, states, leaving);
+}
+hipError_t segment_chain_forward(hipStream_t st, int P, int64_t B, int64_t H, const float *dsum, float *states, const float *s0) {
+    return launch_chain<float, false>(st, P, B, H, s0, nullptr, dsum, states, nullptr);
 }
 
 // ------------------------------------------------------------------------------------------

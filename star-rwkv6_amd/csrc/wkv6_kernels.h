@@ -63,7 +63,17 @@ struct TrainSegments {
 };
 int chunk_train_segments(int64_t B, int64_t T, int64_t H);
 TrainSegments train_segments_layout(int64_t B, int64_t T, int64_t H, void *extra);
-hipError_t segment_chain_reverse(hipStream_t st, int P, int64_t B, int64_t H, const float *dsum, float *states);
+// states[(b*P + seg), h]: on entry what each segment builds alone, on exit what enters it (forward: the
+// state, from s0 or zero; reverse: the gradient arriving at its end, from `arriving` or zero, and
+// `leaving` receives what leaves the first segment, dL/dS_0).
+hipError_t segment_chain_forward(hipStream_t st, int P, int64_t B, int64_t H, const float *dsum, float *states, const float *s0);
+hipError_t segment_chain_reverse(hipStream_t st, int P, int64_t B, int64_t H, const float *dsum, float *states,
+                                 const float *arriving = nullptr, float *leaving = nullptr);
+hipError_t chunk_backward_state_segments(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                                         const void *r, const void *k, const void *v, const void *w, const void *u,
+                                         const float *s0, const void *gy, const float *gsT,
+                                         void *gr, void *gk, void *gv, void *gw, void *gu, float *gs0,
+                                         void *saved, void *extra);
 hipError_t chunk_forward_save_segments(hipStream_t st, int64_t B, int64_t T, int64_t H,
                                        const void *r, const void *k, const void *v, const void *w, const void *u,
                                        void *y, void *saved, void *extra);

@@ -420,6 +420,17 @@ def test_state_gradients_one_sided(op, oracle):
     _state_grad_case(op, oracle, 2, 40, 2, 94, torch.float32, SCAN, with_s0=True, with_gs=False)
 
 
+@pytest.mark.parametrize("with_s0,with_gs", [(True, True), (False, True), (True, False), (False, False)])
+def test_state_gradients_in_time_segments(op, oracle, with_s0, with_gs):
+    # few pairs, long sequence: wkv6_backward_with_state rebuilds the segments' states, chains the
+    # reverse state from the arriving gradient and returns what leaves the first segment as dL/dS_0
+    _state_grad_case(op, oracle, 1, 2048, 3, 98, torch.bfloat16, CHUNK, with_s0=with_s0, with_gs=with_gs)
+
+
+def test_state_gradients_in_time_segments_with_a_fallback_segment(op, oracle):
+    _state_grad_case(op, oracle, 2, 2048, 1, 99, torch.bfloat16, CHUNK, wild=True)
+
+
 def test_state_gradients_on_a_fallback_pair(op, oracle):
     _state_grad_case(op, oracle, 2, 128, 2, 95, torch.bfloat16, CHUNK, wild=True)
 
