@@ -205,6 +205,14 @@ int wkv6_forward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64
     return wkv6_forward_ex(stream, dtype, WKV6_ALGO_AUTO, B, T, C, H, r, k, v, w, u, y, nullptr, 0);
 }
 
+// Workspace of a backward without saved states that runs in time segments (0: it does not): the
+// saved-states block of the (B*P, T/P, C) shape, then the segments' states.
+static size_t segments_workspace_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
+    const int P = train_segments(dtype, algo, B, T, C, H);
+    if (P <= 1) return 0;
+    return saved_base_bytes(dtype, WKV6_ALGO_CHUNK, B * P, T / P, C, H) + wkv6::train_segments_layout(B, T, H, nullptr).bytes;
+}
+
 size_t wkv6_backward_workspace_bytes_ex(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
     if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
     // The per-timestep path keeps one fp32 per element (P), the chunked path one fp32 state per
@@ -213,6 +221,9 @@ size_t wkv6_backward_workspace_bytes_ex(int dtype, int algo, int64_t B, int64_t 
     if (algo == WKV6_ALGO_CHUNK || (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C))) {
         const size_t c = wkv6::chunk_backward_workspace_bytes(B, T, H);
         if (c > need) need = c;
+        // few pairs, long sequence: the backward runs in time segments and keeps their states here
+        const size_t seg = segments_workspace_bytes(dtype, algo, B, T, C, H);
+        if (seg > need) need = seg;
     }
     return need;
 }
@@ -256,6 +267,12 @@ static int backward_impl(void *stream, int dtype, int algo, int64_t B, int64_t T
         if (rc == WKV6_OK && gu_sum) rc = finish(wkv6::sum_over_batch(st, out_type(dtype), B, C, gu, gu_sum));
         return rc;
     }
+    if (!states_ready && train_segments(dtype, algo, B, T, C, H) > 1) {
+        const int P = train_segments(dtype, algo, B, T, C, H);
+        char *extra = reinterpret_cast<char *>(workspace) + saved_base_bytes(dtype, WKV6_ALGO_CHUNK, B * P, T / P, C, H);
+        return finish(wkv6::chunk_backward_state_segments(st, B, T, H, r, k, v, w, u, nullptr, gy, nullptr, gr, gk, gv, gw, gu, nullptr,
+                                                          workspace, extra));
+    }
     return finish(wkv6::chunk_backward(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace, states_ready,
                                        states_ready ? gu_sum : nullptr));
 }
@@ -298,12 +315,7 @@ size_t wkv6_backward_with_state_workspace_bytes(int dtype, int algo, int64_t B, 
     size_t need = wkv6::scan_backward_state_workspace_bytes(B, T, C);
     const size_t c = wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H);
     if (c > need) need = c;
-    const int P = train_segments(dtype, algo, B, T, C, H);   // few pairs, long sequence: time segments side by side
-    if (P > 1) {
-        const size_t seg = saved_base_bytes(dtype, WKV6_ALGO_CHUNK, B * P, T / P, C, H) + wkv6::train_segments_layout(B, T, H, nullptr).bytes;
-        if (seg > need) need = seg;
-    }
-    return need;
+    return need;   // (includes the segments' states where the backward runs in time segments)
 }
 
 int wkv6_backward_with_state(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
