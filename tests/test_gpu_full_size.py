@@ -1,4 +1,4 @@
-"""Parity at the benchmark's full shapes (BASELINE configs 2, 3 and 5), against the float64 C
+"""Parity at the benchmark's full shapes (B8 T1024 C2048, B4 T4096 C4096, B64 C2048 stateful, B1 T8192), against the float64 C
 oracle where it finishes in seconds and through size-independent properties beyond that."""
 import numpy as np
 import pytest

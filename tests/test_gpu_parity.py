@@ -53,7 +53,7 @@ def _case(op, oracle, B, T, H, seed, dtype, algo, strict=False):
 
 @pytest.mark.parametrize("seed", [0, 1, 2])
 def test_config1_forward_fp32(op, oracle, seed):
-    # BASELINE config 1: fp32, B=2 T=128 H=4 N=64; max-abs(y) <= 1e-4
+    # the fp32 correctness shape: B=2 T=128 H=4 N=64; max-abs(y) <= 1e-4
     _case(op, oracle, 2, 128, 4, seed, torch.float32, SCAN, strict=True)
 
 
