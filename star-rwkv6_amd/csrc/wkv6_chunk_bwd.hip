@@ -696,7 +696,10 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
     a.B = (int)B;
     a.gu_sum = states_ready ? (bf16_t *)gu_sum : nullptr;
     a.arrivals = reinterpret_cast<int *>(reinterpret_cast<char *>(workspace) + chunk_backward_workspace_bytes(B, T, H));
+    a.dbg = nullptr;
+#ifdef WKV6_TIMING   // development builds only: cycle stamps behind the workspace (the caller makes room)
     a.dbg = reinterpret_cast<long long *>((float *)workspace + (size_t)(B * H) * ((T + CL - 1) / CL) * kN * kN + 1024);
+#endif
     auto launch = [&](auto kern) -> hipError_t {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
