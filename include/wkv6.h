@@ -144,7 +144,7 @@ size_t wkv6_backward_workspace_bytes_ex(int dtype, int algo, int64_t B, int64_t 
  * the state at every 64-token chunk start, as bf16), and the backward that consumes it and therefore
  * skips its own forward state sweep.  `saved` is caller-owned device memory of wkv6_saved_bytes()
  * bytes (0 = this path saves nothing; pass NULL), must be left untouched between the two calls,
- * and serves the backward as its workspace too.  A long sequence (T >= 2048) of so few (batch, head)
+ * and serves the backward as its workspace too.  A long sequence (T >= 1024) of so few (batch, head)
  * pairs that they fill at most half of the compute units runs as 2, 4, 8 or 16 time segments side by
  * side in both calls (same results to rounding); wkv6_saved_bytes() includes what that keeps.
  * No counterpart in the reference, whose backward

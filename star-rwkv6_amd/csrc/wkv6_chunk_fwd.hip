@@ -669,7 +669,7 @@ static int forward_segments_plan(int64_t B, int64_t T, int64_t H, int64_t *L) {
     const int64_t pairs = B * H, cus = compute_units();
     // (two passes over T / P tokens and two more launches against one pass over T: nothing to gain
     // below four segments or on short sequences)
-    if (T < 2048) return 1;
+    if (T < 1024) return 1;
     for (int P = 16; P >= 4; P >>= 1) {
         const int64_t l = T / P / CL * CL;
         if (pairs * P > cus || l < 4 * CL) continue;
@@ -739,9 +739,9 @@ int chunk_train_segments(int64_t B, int64_t T, int64_t H) {
     const int64_t pairs = B * H, cus = compute_units();
     // (two state-only passes at 0.7 of a forward each on top of the forward and the backward: 1.5
     // times the work on P times the workgroups, and three small kernels)
-    if (T < 2048) return 1;
+    if (T < 1024) return 1;
     for (int P = 16; P >= 2; P >>= 1)
-        if (pairs * P <= cus && T % (P * CL) == 0 && T / P >= 4 * CL) return P;
+        if (pairs * P <= cus && T % (P * CL) == 0 && T / P >= 4 * CL && (T >= 2048 || P >= 4)) return P;
     return 1;
 }
 TrainSegments train_segments_layout(int64_t B, int64_t T, int64_t H, void *extra) {

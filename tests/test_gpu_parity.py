@@ -495,7 +495,8 @@ def test_forward_in_time_segments(op, oracle, B, T, H, sdt):
     check_close("sT zero", s0T, oracle.forward_c(*ref, N)[1], torch.bfloat16)
 
 
-@pytest.mark.parametrize("B,T,H,P", [(1, 2048, 2, 8), (2, 4096, 1, 16), (3, 3072, 5, 8), (1, 8192, 20, 8), (13, 2048, 5, 2)])
+@pytest.mark.parametrize("B,T,H,P", [(1, 2048, 2, 8), (2, 4096, 1, 16), (3, 3072, 5, 8), (1, 8192, 20, 8), (13, 2048, 5, 2),
+                                     (2, 1024, 3, 4), (1, 1536, 2, 4)])
 def test_training_pair_in_time_segments(op, oracle, B, T, H, P):
     """Few pairs, long sequence: forward_save + backward_saved_sum run the sequence as P segments side
     by side (joined by the affine state map and, for the reverse state, its transpose); against the
