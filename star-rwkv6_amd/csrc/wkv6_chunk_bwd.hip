@@ -35,6 +35,8 @@
 #include "wkv6_kernels.h"
 #include "wkv6_scan_body.h"
 
+#include <type_traits>
+
 
 namespace wkv6 {
 
@@ -57,21 +59,7 @@ struct BwdLds {
 };
 static_assert(BwdLds::kBytes <= 160 * 1024, "LDS block of the backward kernel");
 
-// development aid (-DWKV6_TIMING): cycle stamps of workgroup 0, 256 slots per wave, behind the workspace
-#ifdef WKV6_TIMING
-#define WKV6_STAMP() do { if (blockIdx.x == 0 && lane == 0 && dbg_n < 250) a.dbg[(threadIdx.x >> 6) * 256 + dbg_n++] = __builtin_readcyclecounter(); } while (0)
-#define WKV6_STAMP_DECL int dbg_n = 0
-#else
-#define WKV6_STAMP() do { } while (0)
-#define WKV6_STAMP_DECL do { } while (0)
-#endif
-
-#ifndef WKV6_ABLATE
-#define WKV6_ABLATE 0   // timing experiments only: 1 no tile loads, 2 no state loads, 4 no gr/gk/gw stores, 8 no gv stores
-#endif
-
 struct BwdArgs {
-    long long *dbg;
     int T, H;
     const bf16_t *r, *k, *v, *w, *u, *gy;
     bf16_t *gr, *gk, *gv, *gw, *gu;
@@ -100,7 +88,6 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     bf16_t *ck = reinterpret_cast<bf16_t *>(a.ckpt + (int64_t)(b * H + h) * nchunk * (kN * kN));
     auto mine = [](int p) { return (p & 1) == (GRP ^ 1); };   // group 0: tiles 3, 1; group 1: tiles 2, 0
     int item = 0;
-    WKV6_STAMP_DECL;
     float *vgyw = reinterpret_cast<float *>(smem + BwdLds::kVgy) + (4 * GRP + q) * 16;
     f32x4 Gj[4];   // reverse state, rows i, column j = col (the copy with rows j lives in the gv waves)
 #pragma unroll
@@ -126,7 +113,6 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
         for (int hh = 0; hh < 2; ++hh) {
             const int t = tfirst + 2 * hh;
             const uint32_t o = (uint32_t)t * rowbytes + 2u * (uint32_t)col;
-            if ((WKV6_ABLATE & 4) && T > 0) continue;
             if (!kRagged || t < T) {
                 st16_lo(gr_h, o, pk[3 * hh]); st16_lo(gk_h, o, pk[3 * hh + 1]); st16_lo(gw_h, o, pk[3 * hh + 2]);
             }
@@ -136,16 +122,13 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
         }
     };
     auto visit = [&](int c, uint2 (&Sraw)[4]) {
-        WKV6_STAMP();
         __syncthreads();
-        WKV6_STAMP();
         {
             // row j = col of the state tile: values i = 32h + 4g .. +3 and 32h + 16 + 4g .. +3 per read pair
             const unsigned char *stt = smem + BwdLds::kState + (item & 1) * kTileBytes;
             const u32x4 lo = __builtin_bit_cast(u32x4, tile_frag_ch(stt, col, 0, g)), hi = __builtin_bit_cast(u32x4, tile_frag_ch(stt, col, 1, g));
             Sraw[0] = make_uint2(lo[0], lo[1]); Sraw[1] = make_uint2(lo[2], lo[3]);
             Sraw[2] = make_uint2(hi[0], hi[1]); Sraw[3] = make_uint2(hi[2], hi[3]);
-            if ((WKV6_ABLATE & 2) && T > 0) Sraw[0] = Sraw[1] = Sraw[2] = Sraw[3] = make_uint2(0u, 0u);
         }
         // Uniform block offsets of this item.  They pass through fresh_s() before every tile, which
         // keeps the compiler from forming (block + lane offset) for all tiles at once and holding
@@ -188,7 +171,6 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
             for (int m = 0; m < 4; ++m) { S[m][0] *= gq; S[m][1] *= gq; S[m][2] *= gq; S[m][3] *= gq; }
             if (mine(p + 1)) { SopL[p + 1] = acc_as_operand(S[0], S[1]); SopH[p + 1] = acc_as_operand(S[2], S[3]); }
         }
-        WKV6_STAMP();
         __builtin_amdgcn_sched_barrier(0);   // keep the scheduler from interleaving the tiles (register pressure)
 #pragma unroll
         for (int p = 3; p >= 0; --p) {
@@ -206,7 +188,6 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
                     Gj[m][0] = fmaf(Gj[m][0], gq, Upd[m][0]); Gj[m][1] = fmaf(Gj[m][1], gq, Upd[m][1]);
                     Gj[m][2] = fmaf(Gj[m][2], gq, Upd[m][2]); Gj[m][3] = fmaf(Gj[m][3], gq, Upd[m][3]);
                 }
-                WKV6_STAMP();
                 __builtin_amdgcn_sched_barrier(0);
                 continue;
             }
@@ -251,7 +232,6 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
 #pragma unroll
             for (int m = 0; m < 4; ++m) Gj[m] = mfma16(tile_frag_tok(gyt, 16 * m, 16 * p, l16, g), rtq, Gj[m]);
             settle(X, W, Gj);   // all read by VALU code from here on
-            WKV6_STAMP();
             __builtin_amdgcn_sched_barrier(0);
             // tile-boundary term E[j] = sum_i S0[j][i] G_new[j][i]
             float E;
@@ -315,7 +295,6 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
             const uint32_t packed[6] = {pack_bf16x2(gro[0], gro[1]), pack_bf16x2(gko[0], gko[1]), pack_bf16x2(gwo[0], gwo[1]),
                                         pack_bf16x2(gro[2], gro[3]), pack_bf16x2(gko[2], gko[3]), pack_bf16x2(gwo[2], gwo[3])};
             store_tile(t0 + tk, packed);
-            WKV6_STAMP();
             __builtin_amdgcn_sched_barrier(0);
         }
         ++item;
@@ -396,7 +375,6 @@ __device__ __forceinline__ void bwd_gv_chunk(GvState &st, const BwdArgs &a, cons
 #pragma unroll
         for (int rr = 0; rr < 4; ++rr) {
             const int t = t0 + tk + rr;
-            if ((WKV6_ABLATE & 8) && T > 0) continue;
             if (!kRagged || t < T) st16(gv_h, (uint32_t)t * rowbytes + 2u * (uint32_t)col, GV[rr]);
         }
     }
@@ -426,7 +404,6 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     // turns them into r = k = 0, w = -inf (decay 1), and the v, gy rows only ever meet zero operands.
     // Returns the number of loads.
     auto issue_loads = [&](int it) -> int {
-        if ((WKV6_ABLATE & 1) && T > 0) return 0;
         const int tb = item_chunk(it) * CL + 16 * p;
         const uint32_t rk = lds0 + BwdLds::kRawRK + (it % 3) * 2 * kTileBytes + 16 * p * kTileRow;
         const uint32_t ww = lds0 + BwdLds::kRawW + (it % 3) * kTileBytes + 16 * p * kTileRow;
@@ -462,7 +439,6 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     // visit in between (memory operations of a wave complete in program order; the stores are left
     // in flight -- waiting for them costs more than a microsecond per chunk under load).
     auto wait_younger = [&](int n) {
-        if ((WKV6_ABLATE & 1) && T > 0) return;
         switch (n) {   // tile loads {0, 6, 10} + state loads {0, 2} + gv stores {0, 16}
         case 28: wait_loads<28>(); break;
         case 26: wait_loads<26>(); break;
@@ -543,7 +519,6 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     // item `it` is loaded during iteration it-2 (or the prologue) and prepared during iteration it-1
     GvState gvst;
     gvst.init(a.gsT ? a.gsT + (int64_t)(b * H + h) * (kN * kN) : nullptr, 16 * p + (lane & 15), lane >> 4);
-    WKV6_STAMP_DECL;
     // every item's saved state is loaded one item ahead
     auto state_by_load = [&](int it) { return it < nitem; };
     // gv stores an item's visit leaves in flight behind the loads issued before them.  The chunk with
@@ -555,26 +530,20 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     wait_younger(nitem > 1 ? issue_loads(1) : 0);
     prepare(0);
     for (int it = 0; it < nitem; ++it) {
-        WKV6_STAMP();
         __syncthreads();
-        WKV6_STAMP();
         // free again: the r, k block of item it-1 and the raw w, v, gy blocks of item it-1 (read by the
         // other roles before the barrier), and the state tile of item it-1
         const int state_loads = state_by_load(it + 1) ? 2 : 0;
         if (state_loads) issue_state(it + 1);
         const int younger = it + 2 < nitem ? issue_loads(it + 2) : 0;
         if (it + 1 < nitem) {
-            WKV6_STAMP();
             wait_younger(younger + state_loads + (it >= 1 ? gv_stores(it - 1) : 0));
-            WKV6_STAMP();
             prepare(it + 1);
-            WKV6_STAMP();
         }
         // the gv role, on the waves the operand preparation leaves partly idle
         bwd_gv_chunk<kRagged>(gvst, a, smem, a.gv + base, rowbytes, item_chunk(it), it, p, lane);
         // the next item's state has to be in LDS when the consumers pass the barrier
         if (state_loads) wait_younger(younger + gv_stores(it));
-        WKV6_STAMP();
     }
     wait_loads<0>();
     __threadfence_block();
@@ -594,10 +563,6 @@ __global__ __launch_bounds__(kBwdWaves * 64) void chunk_bwd_kernel(BwdArgs a)
     static_assert(sizeof(ScanBwdALds) <= BwdLds::kBytes && sizeof(ScanBwdBLds) <= BwdLds::kBytes,
                   "the exact second pass reuses the LDS block");
     if (threadIdx.x == 0) s_wild = 0;
-    if (WKV6_ABLATE & 1) for (int i = threadIdx.x; i < BwdLds::kBytes / 4; i += blockDim.x) reinterpret_cast<uint32_t *>(smem)[i] = 0u;
-#ifdef WKV6_TIMING
-    if (threadIdx.x == 0) a.dbg[16 * 256 + 2 * blockIdx.x] = __builtin_readcyclecounter();
-#endif
     __syncthreads();
 
     const int b = blockIdx.x / a.H, h = blockIdx.x % a.H;
@@ -607,9 +572,6 @@ __global__ __launch_bounds__(kBwdWaves * 64) void chunk_bwd_kernel(BwdArgs a)
     if (role == 0) bwd_producer<kRagged>(a, smem, &s_wild, b, h, q, lane);
     else if (role == 1) bwd_consumer<kRagged, 0>(a, smem, &s_wild, b, h, q, lane);
     else bwd_consumer<kRagged, 1>(a, smem, &s_wild, b, h, q, lane);
-#ifdef WKV6_TIMING
-    if (threadIdx.x == 0) a.dbg[16 * 256 + 2 * blockIdx.x + 1] = __builtin_readcyclecounter();
-#endif
     // exact second pass for this (b, h) if any of its tiles left the representable range; the
     // workgroup's own slice of the state workspace (nchunk x 64 x 64 floats = T' x 64) holds P
     if (s_wild) {
@@ -696,12 +658,9 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
     a.B = (int)B;
     a.gu_sum = states_ready ? (bf16_t *)gu_sum : nullptr;
     a.arrivals = reinterpret_cast<int *>(reinterpret_cast<char *>(workspace) + chunk_backward_workspace_bytes(B, T, H));
-    a.dbg = nullptr;
-#ifdef WKV6_TIMING   // development builds only: cycle stamps behind the workspace (the caller makes room)
-    a.dbg = reinterpret_cast<long long *>((float *)workspace + (size_t)(B * H) * ((T + CL - 1) / CL) * kN * kN + 1024);
-#endif
-    auto launch = [&](auto kern) -> hipError_t {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    auto launch = [&](auto ragged_tag) -> hipError_t {
+        constexpr auto kern = chunk_bwd_kernel<decltype(ragged_tag)::value>;
+        hipError_t e = allow_dynamic_lds<kern>((int)lds);
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(kBwdWaves * 64), lds, st, a);
         return hipGetLastError();
@@ -713,7 +672,7 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
         hipError_t e = chunk_forward(st, kF32, B, T, H, r, k, v, w, u, s0, nullptr, nullptr, nullptr, workspace, nullptr, false, false);
         if (e != hipSuccess) return e;
     }
-    return ragged ? launch(chunk_bwd_kernel<true>) : launch(chunk_bwd_kernel<false>);
+    return ragged ? launch(std::true_type{}) : launch(std::false_type{});
 }
 
 // Training pair in time segments, last step: gu of a batch row = sum over its segments; the decay

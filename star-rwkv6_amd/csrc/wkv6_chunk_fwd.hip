@@ -59,21 +59,11 @@ __device__ __forceinline__ uint32_t ystage_off(int t, int ch) {
     return ((uint32_t)t << 7) + (((((uint32_t)ch >> 4) ^ ((uint32_t)t >> 2)) & 3u) << 5) + (((uint32_t)ch & 15u) << 1);
 }
 
-// development aid (-DWKV6_TIMING): cycle stamps of workgroup 0, 256 slots per wave, behind the workspace
-#ifdef WKV6_TIMING
-#define WKV6_FSTAMP() do { if (blockIdx.x == 0 && lane == 0 && dbg_n < 250) a.dbg[(threadIdx.x >> 6) * 256 + dbg_n++] = __builtin_readcyclecounter(); } while (0)
-#define WKV6_FSTAMP_DECL int dbg_n = 0
-#else
-#define WKV6_FSTAMP() do { } while (0)
-#define WKV6_FSTAMP_DECL do { } while (0)
-#endif
-
 // Wave layout: 12 waves, four per role, one wave of each role per SIMD:
 //   loader/producer (wave p <-> tile p) | consumer group 0 (y of tiles 0, 2) | consumer group 1 (tiles 1, 3)
 constexpr int kFwdThreads = 12 * 64;
 
 struct FwdArgs {
-    long long *dbg;
     int T, H;
     int nitems;      // B * H (batch, head) pairs; with kMulti a workgroup takes every gridDim.x-th of them
     int split;       // 1, 2 or 4 workgroups per pair, each with the consumer waves of 4 / split column slices
@@ -119,7 +109,6 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
             for (int rr = 0; rr < 4; ++rr) Sraw[4 * m + rr] = p[(16 * m + 4 * g + rr) * kN];
     };
     if (s0 != nullptr) request_state(bh0);
-    WKV6_FSTAMP_DECL;
     int it = 0;   // chunk visits of this workgroup so far: picks the LDS buffers
     for (int n = 0, bh = bh0; n < n_my; ++n, bh += stride) {
         const int b = bh / H, h = bh - b * H;
@@ -137,7 +126,6 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
         bf16_t *y_h = a.y + base;
         if (kSave && GRP == 0 && b == 0 && q == 0 && lane == 0 && a.arrivals) a.arrivals[h] = 0;
         for (int c = 0; c < nchunk; ++c, ++it) {
-            WKV6_FSTAMP();
             if (kSave && GRP == 0) {
                 // bf16 [chunk][j][i], in the first half of this pair's slice of the workspace
                 bf16_t *dst = reinterpret_cast<bf16_t *>(a.ckpt + (int64_t)bh * nchunk * (kN * kN)) + (int64_t)c * (kN * kN) + 16 * q + l16;
@@ -146,9 +134,7 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
 #pragma unroll
                     for (int rr = 0; rr < 4; ++rr) store1(dst + (16 * m + 4 * g + rr) * kN, S[m][rr]);
             }
-            WKV6_FSTAMP();
             __syncthreads();
-            WKV6_FSTAMP();
             // the next pair's initial state is requested one chunk visit ahead of its use
             if (kMulti && s0 != nullptr && c == nchunk - 1 && n + 1 < n_my) request_state(bh + stride);
             // Tokens past the end were prepared as r = k = 0, decay 1: their tiles leave the state alone,
@@ -216,7 +202,6 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
                     S[m][0] = (S[m][0] + U[m][0]) * gg.x; S[m][1] = (S[m][1] + U[m][1]) * gg.y;
                     S[m][2] = (S[m][2] + U[m][2]) * gg.z; S[m][3] = (S[m][3] + U[m][3]) * gg.w;
                 }
-                WKV6_FSTAMP();
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -401,16 +386,13 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
             }
         }
     };
-    WKV6_FSTAMP_DECL;
     // visit `it` is loaded during visit it-2 (or the prologue), prepared during visit it-1
     issue_loads(0);
     if (nvisit > 1) issue_loads(1);
     wait_visit_loads(nvisit > 1, false);
     prepare(0);
     for (int it = 0; it < nvisit; ++it) {
-        WKV6_FSTAMP();
         __syncthreads();
-        WKV6_FSTAMP();
         // the raw r, k, w block of visit `it` (read by this wave's prepare(it) before the barrier) and the
         // raw v block of visit it-1 (read by the consumers before the barrier) are free again.
         // The output stage's 16 stores go out behind the loads and are not waited for: a wave's
@@ -421,12 +403,9 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
         if (outputs && kRagged) output_stage(it - 1);
         if (it + 2 < nvisit) issue_loads(it + 2);
         if (outputs && !kRagged) output_stage(it - 1);
-        WKV6_FSTAMP();
         if (it + 1 < nvisit) {
             wait_visit_loads(it + 2 < nvisit, outputs && !kRagged);
-            WKV6_FSTAMP();
             prepare(it + 1);
-            WKV6_FSTAMP();
         }
     }
     if (kFuse) {
@@ -522,9 +501,9 @@ static int compute_units() {
 
 template <typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse>
 static hipError_t launch_fwd(hipStream_t st, const FwdArgs &a, unsigned grid) {
-    auto kern = chunk_fwd_kernel<Ts, kSave, kRagged, kMulti, kFuse>;
+    constexpr auto kern = chunk_fwd_kernel<Ts, kSave, kRagged, kMulti, kFuse>;
     const size_t lds = kFuse ? FwdLds::kBytesFused : FwdLds::kBytes;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = allow_dynamic_lds<kern>((int)lds);
     if (e != hipSuccess) return e;
     const int split = kMulti || kFuse ? 1 : a.split;
     hipLaunchKernelGGL(kern, dim3(grid * split), dim3((4 + 8 / split) * 64), lds, st, a);
@@ -565,9 +544,6 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
     a.s0 = s0; a.map = map; a.y = (bf16_t *)y; a.sT = sT; a.ckpt = (float *)saved_states;
     a.arrivals = saved_states && counters ? reinterpret_cast<int *>(reinterpret_cast<char *>(saved_states) + chunk_backward_workspace_bytes(B, T, H)) : nullptr;
-#ifdef WKV6_TIMING   // development builds only: cycle stamps behind the saved states (the caller makes room)
-    a.dbg = saved_states ? reinterpret_cast<long long *>((float *)saved_states + (size_t)(B * H) * ((T + CL - 1) / CL) * kN * kN + 1024) : nullptr;
-#endif
     bool multi;
     const unsigned grid = forward_grid(B * H, &multi, &a.split);
     const bool save = saved_states != nullptr, ragged = (T % CL) != 0;

@@ -4,7 +4,24 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace wkv6 {
+
+// Raises kernel Kern's dynamic-LDS limit to `bytes`, once per device (the setting is idempotent and
+// per device; the flags below only save the runtime call on later launches).
+template <auto Kern>
+inline hipError_t allow_dynamic_lds(int bytes) {
+    static std::atomic<bool> done[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const bool known = dev >= 0 && dev < 64;
+    if (known && done[dev].load(std::memory_order_acquire)) return hipSuccess;
+    e = hipFuncSetAttribute(reinterpret_cast<const void *>(Kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess && known) done[dev].store(true, std::memory_order_release);
+    return e;
+}
 
 enum { kBF16 = 0, kF16 = 1, kF32 = 2 };  // same numbering as the public header
 

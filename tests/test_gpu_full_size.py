@@ -48,9 +48,10 @@ def test_config2_full_size_vs_oracle(op, oracle):
 
 
 def test_config3_long_sequence(op, oracle):
-    # B=4 T=4096 C=4096 H=64 bf16.  Oracle on one batch row (rows are independent; gu is checked on
-    # that row's partial), plus properties over the full tensor: finite, gw endpoints exactly zero,
-    # and the two device algorithms agree with each other everywhere.
+    # B=4 T=4096 C=4096 H=64 bf16.  Oracle on one batch row (rows are independent) for y, gr, gk, gv,
+    # gw; gu, the one quantity reduced over all B x T = 16384 tokens, against its float64 closed form
+    # sum_{b,t} r k <v, gy> over all four rows; plus properties over the full tensor: finite, gw
+    # end points exactly zero, and the two device algorithms agree with each other everywhere.
     B, T, H, N = 4, 4096, 64, 64
     print("config 3 full size", flush=True)
     ins = oracle.make_inputs(B, T, H, N, 1)
@@ -67,7 +68,12 @@ def test_config3_long_sequence(op, oracle):
     g_ref = oracle.backward_c(*row, gyr[0][:1], N)
     for name, g, gr in zip("gr gk gv gw".split(), grads[:4], g_ref[:4]):
         check_close(name + " row0", g[:1], gr, torch.bfloat16, is_grad=True)
+    rr, kk, vv = (x.reshape(B, T, H, N) for x in ref[:3])
+    vg = np.einsum("bthi,bthi->bth", vv, gyr[0].reshape(B, T, H, N))
+    gu_ref = np.einsum("bthj,bthj,bth->hj", rr, kk, vg)
+    check_close("gu (closed form over all rows)", to_np(grads[4]).reshape(H, N), gu_ref, torch.bfloat16, is_grad=True)
     y2, grads2 = _fwd_bwd(op, dev, gyd[0], SCAN)
+    check_close("gu scan (closed form over all rows)", to_np(grads2[4]).reshape(H, N), gu_ref, torch.bfloat16, is_grad=True)
     for name, a, b in zip("y gr gk gv gw gu".split(), [y] + grads, [y2] + grads2):
         e = rel_inf(to_np(a), to_np(b))
         assert e <= 1e-2, "%s: chunked vs scan rel-inf %.3e" % (name, e)

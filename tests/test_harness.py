@@ -138,3 +138,67 @@ def test_inference_forward_uses_the_fused_output_stage():
     scale = float(want.abs().max())
     assert float((fused - want).abs().max()) <= 5e-2 * scale
     assert float((fused - unfused.detach()).abs().max()) <= 3e-2 * scale
+
+
+@pytest.mark.gpu
+def test_config4_full_size_train_step(oracle):
+    """Configuration 4 at its real size through the torch binding: 24 layers, d_model 2048, 32 heads
+    of 64, FFN 7168, vocabulary 65536 (rwkv6_model.py:261-276), 8 x 1024 uniform random token ids,
+    bf16 autocast, next-token cross entropy, forward + backward + AdamW.  Loss and every gradient
+    are finite, and what one mid-stack layer's operator call saw -- r, k, v, w, u coming in, gy
+    arriving -- reproduces that call's y and five gradients against the float64 oracle (one batch
+    row for the (B,T,C) tensors, the closed form over all rows for gu) within 1e-2."""
+    import numpy as np
+    from _util import check_close, to_np
+    from rwkv_kernel import RWKVKernelOperator
+
+    dev = torch.device("cuda:0")
+    B, T, N = 8, 1024, 64
+    H = hz.CONFIG4["hidden_size"] // N
+    print("config 4 full size", flush=True)
+    op = RWKVKernelOperator(N, T)
+    layer, rec = hz.CONFIG4["num_layers"] // 2, {}
+
+    class Recording:
+        """The operator, keeping the tensors of its call number `layer` (0-based)."""
+        calls = 0
+
+        def __call__(self, r, k, v, w, u):
+            mine = self.calls == layer
+            self.calls += 1
+            if mine:
+                for name, x in zip("rkvwu", (r, k, v, w, u)):
+                    x.retain_grad()
+                    rec[name] = x
+            y, s = op(r, k, v, w, u)
+            if mine:
+                rec["y"] = y.detach()
+                y.register_hook(lambda g: rec.__setitem__("gy", g.detach().clone()))
+            return y, s
+
+    torch.manual_seed(11)
+    with torch.device(dev):
+        recorder = Recording()
+        model = hz.RWKV6(recorder, **hz.CONFIG4)
+    opt = torch.optim.AdamW(model.parameters(), lr=1e-4, fused=True)
+    ids = torch.randint(0, hz.CONFIG4["vocabulary_size"], (B, T + 1), device=dev)
+    loss = float(hz.train_step(model, opt, ids, torch.bfloat16))
+    torch.cuda.synchronize()
+    assert np.isfinite(loss) and abs(loss - np.log(hz.CONFIG4["vocabulary_size"])) < 2.0, loss
+    for n, p in model.named_parameters():
+        assert p.grad is not None and bool(torch.isfinite(p.grad).all()), n
+        assert bool(torch.isfinite(p).all()), n
+    assert recorder.calls == hz.CONFIG4["num_layers"] and set(rec) == set("rkvwu") | {"y", "gy"}
+    assert rec["r"].dtype == torch.bfloat16 and tuple(rec["r"].shape) == (B, T, H * N)
+
+    row = 3
+    ins = [to_np(rec[n][row:row + 1]) for n in "rkvw"] + [to_np(rec["u"])]
+    gy = to_np(rec["gy"][row:row + 1])
+    y_ref, _ = oracle.forward_c(*ins, N)
+    check_close("y", rec["y"][row:row + 1], y_ref, torch.bfloat16)
+    g_ref = oracle.backward_c(*ins, gy, N)
+    for name, leaf, want in zip("gr gk gv gw".split(), "rkvw", g_ref[:4]):
+        check_close(name, rec[leaf].grad[row:row + 1], want, torch.bfloat16, is_grad=True)
+    r4, k4, v4, g4 = (to_np(rec[n]).reshape(B, T, H, N) for n in ("r", "k", "v", "gy"))
+    gu_ref = np.einsum("bthj,bthj,bth->hj", r4, k4, np.einsum("bthi,bthi->bth", v4, g4))
+    check_close("gu", to_np(rec["u"].grad).reshape(H, N), gu_ref, torch.bfloat16, is_grad=True)
