@@ -3,7 +3,9 @@
  * time-mixing operator.  Plain pointers and sizes only; every pointer (state_map and workspace
  * included) is a DEVICE pointer to a row-major contiguous, 16-byte aligned array; all work is
  * enqueued on `stream` (a hipStream_t, may be NULL = default stream) and the calls return
- * without synchronising.  The library keeps no mutable state: calls are re-entrant.
+ * without synchronising.  Calls are re-entrant: what the library keeps between calls are per-device
+ * caches of things that do not change (compute-unit count, kernel attributes already set, the
+ * address of its scratch array); the one exception is wkv6_backward_static, see there.
  *
  * Each entry point names the reference interface it replaces (paths relative to the
  * reference tree infiy-quine/STAR-RWKV6).
@@ -42,7 +44,7 @@ enum {
 
 /* Algorithm selector for the *_ex entry points. */
 enum {
-    WKV6_ALGO_AUTO = 0,  /* library picks: chunked MFMA path for bf16/f16 when T allows, else scan */
+    WKV6_ALGO_AUTO = 0,  /* library picks: chunked MFMA path for bf16 tensors with T >= 32, else scan  */
     WKV6_ALGO_SCAN = 1,  /* per-timestep fp32 recurrence, state in VGPRs                       */
     WKV6_ALGO_CHUNK = 2  /* chunk-parallel form, bf16 MFMA for the dense intra-chunk products; bf16
                             tensors only.  A workgroup whose (batch, head) pair has a 16-token tile
@@ -128,6 +130,24 @@ int wkv6_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int6
                   void *gr, void *gk, void *gv, void *gw, void *gu,
                   void *workspace, size_t workspace_bytes);
 size_t wkv6_backward_workspace_bytes(int dtype, int64_t B, int64_t T, int64_t C, int64_t H);
+
+/* wkv6_backward without a workspace argument and without any allocation: the workspace is a
+ * fixed array in device memory that belongs to the library (WKV6_STATIC_SCRATCH_BYTES, present on
+ * every GPU the library is used on from the first such call until the process ends).  No
+ * counterpart in the reference; it is for callers that cannot allocate device memory at the
+ * point of the call -- code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc -- and neither the library nor anything it calls allocates or frees memory here (the
+ * first call on a device looks the array's address up once).  Shapes whose
+ * wkv6_backward_workspace_bytes() exceeds WKV6_STATIC_SCRATCH_BYTES are refused with
+ * WKV6_ERR_WORKSPACE (the benchmark shape B=8 T=1024 C=2048 needs exactly that much).  All calls
+ * on one GPU share the one array: two calls whose kernels overlap in time on the same GPU
+ * (different streams, different host threads) race -- serialise them.  Same results as
+ * wkv6_backward. */
+#define WKV6_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
+int wkv6_backward_static(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
+                         const void *r, const void *k, const void *v, const void *w, const void *u,
+                         const void *gy,
+                         void *gr, void *gk, void *gv, void *gw, void *gu);
 
 /* Same two calls with the algorithm forced (tests and benchmarks compare the two paths). */
 int wkv6_forward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,

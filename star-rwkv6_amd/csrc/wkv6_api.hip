@@ -4,7 +4,31 @@
 
 #include <string.h>
 
+#include <atomic>
+
+// Workspace of wkv6_backward_static: device memory the library owns, one copy per GPU.  In host
+// code the name below is only a handle for hipGetSymbolAddress; the address that kernels, copies and
+// memsets take is looked up per device (static_scratch()).
+static __device__ __align__(256) unsigned char scratch[WKV6_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+// Device address of `scratch` on the current device (null on failure, *err says why); looked up on
+// the first call per device.
+void *static_scratch(hipError_t *err) {
+    static std::atomic<void *> ptr[64];
+    int dev = 0;
+    *err = hipGetDevice(&dev);
+    if (*err != hipSuccess) return nullptr;
+    if (dev < 0 || dev >= 64) { *err = hipErrorInvalidDevice; return nullptr; }
+    void *p = ptr[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        *err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (*err != hipSuccess) return nullptr;
+        ptr[dev].store(p, std::memory_order_release);
+    }
+    return p;
+}
 
 // Shapes the chunked MFMA kernels take; everything else runs the per-timestep kernels.
 // (the chunked kernels index one batch row with 32-bit element offsets)
@@ -352,6 +376,20 @@ int wkv6_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int6
                   void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, size_t workspace_bytes) {
     return wkv6_backward_ex(stream, dtype, WKV6_ALGO_AUTO, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu,
                             workspace, workspace_bytes);
+}
+
+int wkv6_backward_static(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
+                         const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                         void *gr, void *gk, void *gv, void *gw, void *gu) {
+    const int rc = check_shape(dtype, B, T, C, H);
+    if (rc != WKV6_OK) return rc;
+    const size_t need = wkv6_backward_workspace_bytes(dtype, B, T, C, H);
+    if (need > WKV6_STATIC_SCRATCH_BYTES) return WKV6_ERR_WORKSPACE;   // larger than the library's own array
+    hipError_t e = hipSuccess;
+    void *ws = static_scratch(&e);
+    if (ws == nullptr) return finish(e);
+    // (the workspace needs no initial contents; what the last call left in it is overwritten)
+    return wkv6_backward(stream, dtype, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, ws, WKV6_STATIC_SCRATCH_BYTES);
 }
 
 // ---- XLA custom-call surface ------------------------------------------------------------

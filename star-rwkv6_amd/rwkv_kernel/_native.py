@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(_PKG, "lib", "libwkv6_gfx950.so")
 
 BF16, F16, F32 = 0, 1, 2
 ALGO_AUTO, ALGO_SCAN, ALGO_CHUNK = 0, 1, 2
+STATIC_SCRATCH_BYTES = 64 << 20   # WKV6_STATIC_SCRATCH_BYTES
 
 _i64, _int, _p, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
 
@@ -27,6 +28,7 @@ SIGNATURES = {
     "wkv6_forward_gn_gate_ex": (_int, [_p, _int, _int] + [_i64] * 4 + [_int, _p] + [_p] * 9 + [ctypes.c_float, _p, _p] + [_p, _sz]),
     "wkv6_backward": (_int, [_p, _int] + [_i64] * 4 + [_p] * 11 + [_p, _sz]),
     "wkv6_backward_workspace_bytes": (_sz, [_int] + [_i64] * 4),
+    "wkv6_backward_static": (_int, [_p, _int] + [_i64] * 4 + [_p] * 11),
     "wkv6_forward_ex": (_int, [_p, _int, _int] + [_i64] * 4 + [_p] * 6 + [_p, _sz]),
     "wkv6_backward_ex": (_int, [_p, _int, _int] + [_i64] * 4 + [_p] * 11 + [_p, _sz]),
     "wkv6_backward_workspace_bytes_ex": (_sz, [_int, _int] + [_i64] * 4),
