@@ -239,3 +239,33 @@ def test_state_gradients_vs_autograd(oracle):
     for a, b in zip(plain, again[:5]):
         assert np.array_equal(a, b)
     assert np.abs(again[3][:, 0]).max() == 0 and np.abs(again[3][:, -1]).max() == 0
+
+
+def test_state_layout_is_the_transpose_of_the_cuda_indexing(oracle):
+    # The oracle (and the library) keep a state as [key j][value i] like the python-loop flavour,
+    # ops_rwkv_kernal.py:85-91.  The reference's CUDA kernels index it the other way round: thread i
+    # owns VALUE channel i (v = _v[t], rwkv_kernels.cu:129), its float state[j] runs over the KEY
+    # channels (:131-156), and a stored state is read and written at offset i*N + j (:177-189), i.e.
+    # s[b,h,value,key].  Restated below with exactly that indexing; the two must agree through a
+    # transpose of the last two axes, for the incoming and for the returned state.
+    B, T, H, N = 2, 9, 2, 4
+    r, k, v, w, u, _ = _rand(B, T, H, N, 5, oracle)
+    s_vk = np.random.default_rng(5).normal(size=(B, H, N, N)) * 0.3     # [value i][key j]
+    y = np.zeros((B, T, H * N))
+    ys_vk = np.zeros_like(s_vk)
+    for b in range(B):
+        for h in range(H):
+            for i in range(N):                                          # thread i
+                state = s_vk[b, h, i].copy()                            # state[j] = _s[... + i*N + j]
+                for t in range(T):
+                    c = slice(h * N, (h + 1) * N)
+                    x = k[b, t, c] * v[b, t, h * N + i]                 # x[j] = k_[j] * v
+                    y[b, t, h * N + i] = (r[b, t, c] * (u[h] * x + state)).sum()
+                    state = state * np.exp(-np.exp(w[b, t, c])) + x
+                ys_vk[b, h, i] = state                                  # _ys[... + i*N + j] = state[j]
+    y_o, s_o = oracle.forward_c(r, k, v, w, u, N, init_state=np.swapaxes(s_vk, -1, -2))
+    np.testing.assert_allclose(y_o, y, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(s_o, np.swapaxes(ys_vk, -1, -2), rtol=1e-12, atol=1e-12)
+    # and it is a real difference: feeding the CUDA-indexed state untransposed gives another y
+    y_wrong, _ = oracle.forward_c(r, k, v, w, u, N, init_state=s_vk)
+    assert np.abs(y_wrong - y).max() > 1e-2
