@@ -92,7 +92,12 @@ class TimeMix(nn.Module):
         xw = x + x_shift * self.dense_xw(x_mix)
         xg = x + x_shift * self.dense_xg(x_mix)
         r, k, v, w, g = self.dense_r(xr), self.dense_k(xk), self.dense_v(xv), self.dense_w(xw), F.silu(self.dense_g(xg))
-        if mask is not None:   # rwkv6_model.py:149-152: padded tokens neither write nor decay the state
+        if mask is not None:
+            # Padded tokens neither write to the state nor decay it.  rwkv6_model.py:149-152 sets
+            # w = -1e9 there (decay 1) and multiplies xk by the mask -- after k has already been
+            # computed from xk (:148), so in the reference as committed k stays unmasked and a padded
+            # token still writes k v^T into the state.  The evident intent is implemented here: k is
+            # masked.  (A deliberate deviation; the operator itself is not involved.)
             m = mask.to(x.dtype)[..., None]
             k = k * m
             w = w * m + (1 - m) * -1e9

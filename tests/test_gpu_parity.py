@@ -224,6 +224,58 @@ def test_xla_custom_call_targets(op, oracle):
     assert lib.wkv6_last_status() == 1
 
 
+@pytest.mark.parametrize("B,T,H", [(2, 256, 2), (8, 1024, 32)])
+def test_xla_custom_call_targets_bf16(op, oracle, B, T, H):
+    # What a JAX caller reaches: bf16 tensors through the three custom-call targets, where the
+    # library's own choice is the chunked MFMA kernels and wkv_backward has to rebuild the chunk
+    # states itself; the state_map buffer is built the way the jax flavour ships it, as (value, 0)
+    # int32 pairs.  At the benchmark size too.
+    from rwkv_kernel import _native
+
+    lib = _native.load()
+    N = 64
+    C = H * N
+    print("custom-call targets bf16 B%d T%d H%d" % (B, T, H), flush=True)
+    ins = oracle.make_inputs(B, T, H, N, 77, with_state=True)
+    dev, ref = cast_inputs(ins[:5], torch.bfloat16)
+    gyd, gyr = cast_inputs(ins[5:6], torch.bfloat16)
+    stream = torch.cuda.current_stream().cuda_stream
+    bf = dict(dtype=torch.bfloat16, device="cuda")
+    desc = lambda S: _native.create_descriptor(B, T, C, H, S, _native.BF16, _native.BF16)
+
+    def call(fn, bufs, d):
+        arr = (ctypes.c_void_p * len(bufs))(*[b.data_ptr() for b in bufs])
+        fn(stream, arr, d, len(d))
+        torch.cuda.synchronize()
+        assert lib.wkv6_last_status() == 0
+
+    y = torch.empty(B, T, C, **bf)
+    call(lib.wkv_forward, dev + [y], desc(False))
+    y_ref, _ = oracle.forward_c(*ref, N)
+    check_close("y", y, y_ref, torch.bfloat16)
+
+    outs = [torch.empty(B, T, C, **bf) for _ in range(4)] + [torch.empty(B, C, **bf)]
+    ws = torch.empty(lib.wkv6_backward_workspace_bytes(_native.BF16, B, T, C, H), dtype=torch.uint8, device="cuda")
+    call(lib.wkv_backward, dev + gyd + outs + [ws], desc(False))
+    g_ref = oracle.backward_c(*ref, gyr[0], N)
+    for name, g, gr in zip("gr gk gv gw".split(), outs, g_ref):
+        check_close(name, g, gr, torch.bfloat16, is_grad=True)
+    check_close("gu", to_np(outs[4]).sum(0).reshape(H, N), g_ref[4], torch.bfloat16, is_grad=True)
+
+    # one state per batch row, rows permuted by the map; bf16 state = the output type
+    s0 = ins[6].to(torch.bfloat16).cuda()
+    perm = torch.randperm(B, generator=torch.Generator().manual_seed(3))
+    m32 = perm.to(torch.int32)
+    pairs = torch.stack([m32, torch.zeros_like(m32)], -1).reshape(2 * B).cuda()   # little endian int64
+    ys = torch.empty(B, H, N, N, **bf)
+    call(lib.wkv_forward_with_state, [pairs] + dev + [s0, y, ys], desc(True))
+    y_ref, s_ref = oracle.forward_c(*ref, N, to_np(s0), perm.numpy())
+    check_close("y with state", y, y_ref, torch.bfloat16)
+    check_close("ys", ys, s_ref, torch.bfloat16)
+    call(lib.wkv_forward_with_state, dev + [y, ys], desc(False))
+    check_close("ys from zero", ys, oracle.forward_c(*ref, N)[1], torch.bfloat16)
+
+
 # ---------------------------------------------------------------------------------------------
 # chunk-parallel MFMA path (bf16 tensors)
 # ---------------------------------------------------------------------------------------------

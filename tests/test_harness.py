@@ -57,7 +57,8 @@ def test_time_mix_follows_the_reference_layer():
     y, _ = op(r, k, v, w, tm.time_faaaa)
     ref = tm.dense_o(tm.group_norm(y) * g)
     assert torch.allclose(tm(x), ref, atol=1e-5)
-    # a padded position (rwkv6_model.py:149-152) gets k = 0 and w = -1e9: same call, masked operands
+    # a padded position gets w = -1e9 (rwkv6_model.py:152) and k = 0 (what :151 means to do; the
+    # reference masks xk after k was computed from it): same call, masked operands
     mask = torch.ones(2, 16, dtype=torch.bool); mask[:, 5] = False
     m = mask.float()[..., None]
     y_m, _ = op(r, k * m, v, w * m + (1 - m) * -1e9, tm.time_faaaa)
