@@ -1,7 +1,7 @@
 // WKV6 backward in chunk-parallel form for gfx950 (bf16 MFMA, fp32 states); the forward kernel and
 // the notation are in wkv6_chunk_fwd.hip.
 //
-// The forward state at every chunk start comes from the workspace (bf16, [b][h][chunk][j][i]), left
+// The forward state at every chunk start comes from the workspace (bf16, transposed: [b][h][chunk][i][j]), left
 // there by the saving forward pass -- or, when the caller has none, by a state-only pass of the
 // forward kernel that chunk_backward() runs first.  The kernel sweeps the chunks in reverse order
 // with the reverse state G in MFMA accumulators.  G is kept twice, once with rows j / columns i (for gv) and once transposed (for
@@ -52,7 +52,7 @@ struct BwdLds {
     static constexpr int kOpFr = 0;                                               // exp(-c_t) tile
     static constexpr int kOpG = kTileBytes, kOpRuk = kOpG + 4 * kN * 4;           // g[4][64], ruk[64] (fp32)
     static constexpr int kOpBytes = kOpRuk + CL * 4;
-    static constexpr int kState = kOp + 2 * kOpBytes;                  // [item & 1] saved forward state of the chunk, bf16 [j][i] as a tile
+    static constexpr int kState = kOp + 2 * kOpBytes;                  // [item & 1] saved forward state of the chunk, bf16 [i][j] (transposed) as a tile
     static constexpr int kVgy = kState + 2 * kTileBytes;                    // [8 consumer waves][16] fp32: <v_t, gy_t>
     static constexpr int kGu = kVgy + 8 * 16 * 4;                      // [64] fp32: gu partial of consumer group 1
     static constexpr int kBytes = kGu + kN * 4;
@@ -84,8 +84,6 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     const int64_t C = (int64_t)H * kN;
     const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
     const int nchunk = (T + CL - 1) / CL;
-    // chunk states: bf16 [chunk][j][i] in the first half of this workgroup's workspace slice
-    bf16_t *ck = reinterpret_cast<bf16_t *>(a.ckpt + (int64_t)(b * H + h) * nchunk * (kN * kN));
     auto mine = [](int p) { return (p & 1) == (GRP ^ 1); };   // group 0: tiles 3, 1; group 1: tiles 2, 0
     int item = 0;
     float *vgyw = reinterpret_cast<float *>(smem + BwdLds::kVgy) + (4 * GRP + q) * 16;
@@ -124,11 +122,13 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     auto visit = [&](int c, uint2 (&Sraw)[4]) {
         __syncthreads();
         {
-            // row j = col of the state tile: values i = 32h + 4g .. +3 and 32h + 16 + 4g .. +3 per read pair
+            // the tile holds the state transposed (rows i, channels j): S^T[16m + 4g + e][col], e < 4, per read
             const unsigned char *stt = smem + BwdLds::kState + (item & 1) * kTileBytes;
-            const u32x4 lo = __builtin_bit_cast(u32x4, tile_frag_ch(stt, col, 0, g)), hi = __builtin_bit_cast(u32x4, tile_frag_ch(stt, col, 1, g));
-            Sraw[0] = make_uint2(lo[0], lo[1]); Sraw[1] = make_uint2(lo[2], lo[3]);
-            Sraw[2] = make_uint2(hi[0], hi[1]); Sraw[3] = make_uint2(hi[2], hi[3]);
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                const u32x2 x = __builtin_bit_cast(u32x2, tile_frag_tok(stt, 16 * q, 16 * m, l16, g));
+                Sraw[m] = make_uint2(x[0], x[1]);
+            }
         }
         // Uniform block offsets of this item.  They pass through fresh_s() before every tile, which
         // keeps the compiler from forming (block + lane offset) for all tiles at once and holding
@@ -336,7 +336,6 @@ __device__ __forceinline__ void bwd_gv_chunk(GvState &st, const BwdArgs &a, cons
 {
     const int T = a.T;
     const int g = lane >> 4, l16 = lane & 15;
-    const int col = 16 * q + l16;
     f32x4 (&Gi)[4] = st.Gi;
     const unsigned char *op = smem + BwdLds::kOp + (item & 1) * BwdLds::kOpBytes;
     const unsigned char *rt = smem + BwdLds::kRawRK + (item % 3) * 2 * kTileBytes, *kt = rt + kTileBytes;
@@ -346,7 +345,7 @@ __device__ __forceinline__ void bwd_gv_chunk(GvState &st, const BwdArgs &a, cons
     const int t0 = c * CL;
 #pragma unroll 1
     for (int pp = 3; pp >= 0; --pp) {
-        const int row = 16 * pp + l16, tk = 16 * pp + 4 * g;
+        const int row = 16 * pp + l16;
         const bf16x8 rf0 = tile_frag_ch(rt, row, 0, g), rf1 = tile_frag_ch(rt, row, 1, g);
         const bf16x8 kf0 = tile_frag_ch(kt, row, 0, g), kf1 = tile_frag_ch(kt, row, 1, g);
         const s16x4 gyq = tile_frag_tok(gyt, 16 * q, 16 * pp, l16, g);
@@ -364,18 +363,21 @@ __device__ __forceinline__ void bwd_gv_chunk(GvState &st, const BwdArgs &a, cons
             const float4 gg = *reinterpret_cast<const float4 *>(&gg_[pp * kN + 16 * m + 4 * g]);
             Gi[m][0] *= gg.x; Gi[m][1] *= gg.y; Gi[m][2] *= gg.z; Gi[m][3] *= gg.w;
         }
+        // the products are formed transposed (accumulator rows i = 4g + r, column s = l16): a lane holds
+        // four neighbouring channels of one token and writes them with one 8-byte store
         f32x4 GV = {0.f, 0.f, 0.f, 0.f};
-        GV = mfma16(pack4(A), gyq, GV);
+        GV = mfma16(gyq, pack4(A), GV);
         chain_gap(GV);
-        GV = mfma32(kf0, acc_as_operand(Gi[0], Gi[1]), GV);
-        GV = mfma32(kf1, acc_as_operand(Gi[2], Gi[3]), GV);
+        GV = mfma32(acc_as_operand(Gi[0], Gi[1]), kf0, GV);
+        GV = mfma32(acc_as_operand(Gi[2], Gi[3]), kf1, GV);
 #pragma unroll
         for (int m = 0; m < 4; ++m) Gi[m] = mfma16(tile_frag_tok(rt, 16 * m, 16 * pp, l16, g), gyq, Gi[m]);
         settle(GV, Gi);
-#pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-            const int t = t0 + tk + rr;
-            if (!kRagged || t < T) st16(gv_h, (uint32_t)t * rowbytes + 2u * (uint32_t)col, GV[rr]);
+        {
+            const int t = t0 + row;   // channels 16q + 4g .. +3 of this token
+            if (!kRagged || t < T)
+                *reinterpret_cast<uint2 *>(reinterpret_cast<char *>(gv_h) + ((uint32_t)t * rowbytes + 2u * (uint32_t)(16 * q + 4 * g))) =
+                    make_uint2(pack_bf16x2(GV[0], GV[1]), pack_bf16x2(GV[2], GV[3]));
         }
     }
 }
@@ -421,7 +423,7 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
         return 10;
     };
     // The saved forward state of item `it`: the
-    // chunk's 64x64 bf16 block [j][i] is a tile with j in the place of the token; wave p brings rows
+    // chunk's 64x64 bf16 block [i][j] is a tile with i in the place of the token; wave p brings rows
     // 16p..16p+15.  It is requested ONE item ahead (two slots), ahead of the tile loads in the queue,
     // and awaited at the end of the visit, behind the gv stores issued in between -- the consumer
     // waves, which would otherwise load it behind their own gradient stores and wait for those to
@@ -435,21 +437,17 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
             load_rows8_to_lds(src, (uint32_t)((16 * p + 8 * hf + lrow) * kTileRow) + lpiece, dst + 8 * hf * kTileRow);
     };
     // Waits for this wave's tile loads of one item.  `n` = operations issued after them: the loads
-    // of the following item and, with the gv role on this wave, the 16 gv stores of the chunk
+    // of the following item and, with the gv role on this wave, the 4 gv stores of the chunk
     // visit in between (memory operations of a wave complete in program order; the stores are left
     // in flight -- waiting for them costs more than a microsecond per chunk under load).
     auto wait_younger = [&](int n) {
-        switch (n) {   // tile loads {0, 6, 10} + state loads {0, 2} + gv stores {0, 16}
-        case 28: wait_loads<28>(); break;
-        case 26: wait_loads<26>(); break;
-        case 24: wait_loads<24>(); break;
-        case 22: wait_loads<22>(); break;
-        case 18: wait_loads<18>(); break;
+        switch (n) {   // tile loads {0, 10} + state loads {0, 2} + gv stores {0, 4}
         case 16: wait_loads<16>(); break;
+        case 14: wait_loads<14>(); break;
         case 12: wait_loads<12>(); break;
         case 10: wait_loads<10>(); break;
-        case 8: wait_loads<8>(); break;
         case 6: wait_loads<6>(); break;
+        case 4: wait_loads<4>(); break;
         case 2: wait_loads<2>(); break;
         default: wait_loads<0>(); break;
         }
@@ -522,9 +520,9 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     // every item's saved state is loaded one item ahead
     auto state_by_load = [&](int it) { return it < nitem; };
     // gv stores an item's visit leaves in flight behind the loads issued before them.  The chunk with
-    // the ragged tail issues anything from 0 to 16 (a store whose lanes are all past the end is
+    // the ragged tail issues anything from 0 to 4 (a store whose lanes are all past the end is
     // skipped): counting none for it makes the waits behind it wait for everything older.
-    auto gv_stores = [&](int it) { return (kRagged && item_chunk(it) == nchunk - 1) ? 0 : 16; };
+    auto gv_stores = [&](int it) { return (kRagged && item_chunk(it) == nchunk - 1) ? 0 : 4; };
     if (state_by_load(0)) issue_state(0);
     issue_loads(0);
     wait_younger(nitem > 1 ? issue_loads(1) : 0);

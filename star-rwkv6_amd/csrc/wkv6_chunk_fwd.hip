@@ -126,15 +126,18 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
         bf16_t *y_h = a.y + base;
         if (kSave && GRP == 0 && b == 0 && q == 0 && lane == 0 && a.arrivals) a.arrivals[h] = 0;
         for (int c = 0; c < nchunk; ++c, ++it) {
+            __syncthreads();
             if (kSave && GRP == 0) {
-                // bf16 [chunk][j][i], in the first half of this pair's slice of the workspace
-                bf16_t *dst = reinterpret_cast<bf16_t *>(a.ckpt + (int64_t)bh * nchunk * (kN * kN)) + (int64_t)c * (kN * kN) + 16 * q + l16;
+                // The state at the chunk start goes to the workspace transposed, bf16 [chunk][i][j] in the
+                // first half of this pair's slice: a lane's four rows j = 16m + 4g .. +3 of its column i are
+                // eight contiguous bytes there, so a chunk takes four stores per lane.  They are issued behind
+                // the barrier (the state registers do not change before the end of tile 0) and queue while
+                // the other waves already work on the chunk.
+                char *dst = reinterpret_cast<char *>(a.ckpt + (int64_t)bh * nchunk * (kN * kN)) + (int64_t)c * (kN * kN * 2) + (16 * q + l16) * (kN * 2) + 8 * g;
 #pragma unroll
                 for (int m = 0; m < 4; ++m)
-#pragma unroll
-                    for (int rr = 0; rr < 4; ++rr) store1(dst + (16 * m + 4 * g + rr) * kN, S[m][rr]);
+                    *reinterpret_cast<uint2 *>(dst + 32 * m) = make_uint2(pack_bf16x2(S[m][0], S[m][1]), pack_bf16x2(S[m][2], S[m][3]));
             }
-            __syncthreads();
             // the next pair's initial state is requested one chunk visit ahead of its use
             if (kMulti && s0 != nullptr && c == nchunk - 1 && n + 1 < n_my) request_state(bh + stride);
             // Tokens past the end were prepared as r = k = 0, decay 1: their tiles leave the state alone,
@@ -165,18 +168,27 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
                     AT = mfma32(kf0, rf0, AT);
                     AT = mfma32(kf1, rf1, AT);
                     // Y = R~ S
+                    // Without the fused output stage the products are formed transposed (the operands change
+                    // places): accumulator rows i = 4g + r, column t = l16, so that a lane holds four
+                    // neighbouring channels of one token and writes them with one 8-byte store.
                     f32x4 Y = {0.f, 0.f, 0.f, 0.f};
-                    Y = mfma32(rf0, acc_as_operand(S[0], S[1]), Y);
-                    Y = mfma32(rf1, acc_as_operand(S[2], S[3]), Y);
+                    if (kFuse) {
+                        Y = mfma32(rf0, acc_as_operand(S[0], S[1]), Y);
+                        Y = mfma32(rf1, acc_as_operand(S[2], S[3]), Y);
+                    } else {
+                        Y = mfma32(acc_as_operand(S[0], S[1]), rf0, Y);
+                        Y = mfma32(acc_as_operand(S[2], S[3]), rf1, Y);
+                    }
                     settle(AT);
 #pragma unroll
                     for (int rr = 0; rr < 4; ++rr) {
                         const int s = 4 * g + rr;
                         AT[rr] = (l16 > s) ? AT[rr] : ((l16 == s) ? rukv : 0.f);
                     }
-                    // Y += A V : the masked A^T accumulator IS the A operand (row t = l16, k-slots s = 4g+r)
+                    // Y += A V : the masked A^T accumulator IS the operand holding A (token t = l16, k-slots s = 4g+r)
                     chain_gap(Y);
-                    Y = mfma16(make_s16x4(pack_bf16x2(AT[0], AT[1]), pack_bf16x2(AT[2], AT[3])), vf, Y);
+                    const s16x4 aop = make_s16x4(pack_bf16x2(AT[0], AT[1]), pack_bf16x2(AT[2], AT[3]));
+                    Y = kFuse ? mfma16(aop, vf, Y) : mfma16(vf, aop, Y);
                     settle(Y);
                     if (kFuse) {
                         unsigned char *ys = const_cast<unsigned char *>(smem) + FwdLds::kYStage + (it & 1) * kTileBytes;
@@ -187,11 +199,10 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
                         *reinterpret_cast<uint16_t *>(ys + ystage_off(tk + 2, chn)) = (uint16_t)y23;
                         *reinterpret_cast<uint16_t *>(ys + ystage_off(tk + 3, chn)) = (uint16_t)(y23 >> 16);
                     } else {
-#pragma unroll
-                        for (int rr = 0; rr < 4; ++rr) {
-                            const int t = t0 + 16 * p + 4 * g + rr;
-                            if (!kRagged || t < T) st16(y_h, (uint32_t)t * (uint32_t)C * 2u + 2u * (uint32_t)(16 * q + l16), Y[rr]);
-                        }
+                        const int t = t0 + 16 * p + l16;   // channels 16q + 4g .. +3 of this token
+                        if (!kRagged || t < T)
+                            *reinterpret_cast<uint2 *>(reinterpret_cast<char *>(y_h) + ((uint32_t)t * (uint32_t)C * 2u + 2u * (uint32_t)(16 * q + 4 * g))) =
+                                make_uint2(pack_bf16x2(Y[0], Y[1]), pack_bf16x2(Y[2], Y[3]));
                     }
                 }
                 // S <- diag(g) (S + U)
