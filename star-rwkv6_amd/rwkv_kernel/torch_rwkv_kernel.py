@@ -26,6 +26,25 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+_STAGGER = 256   # bytes
+
+
+def _staggered(count, shape, dtype, device, first=1):
+    """`count` tensors of one shape out of ONE allocation, the k-th starting (first + k) * 256 bytes
+    past where a tensor of its own would start.  A workgroup of the kernels walks all (B,T,C) tensors
+    of a call row by row in step; torch's allocator hands out large blocks on 2 MiB boundaries, and
+    tensors whose bases agree modulo 4 KiB keep sending those streams to the same memory channel at
+    the same moment (about 5 % of the training pair at B8 T1024 C2048).  The tensors are views of
+    the common block, which lives as long as any of them."""
+    n = 1
+    for d in shape:
+        n *= d
+    es = torch.empty((), dtype=dtype).element_size()
+    step = (n * es + _STAGGER - 1) // _STAGGER * _STAGGER + _STAGGER
+    block = torch.empty(count * step + first * _STAGGER, dtype=torch.uint8, device=device)
+    return [block[first * _STAGGER + i * step: first * _STAGGER + i * step + n * es].view(dtype).view(shape) for i in range(count)]
+
+
 def _ptr(t):
     return None if t is None else t.data_ptr()
 
@@ -48,13 +67,13 @@ class _WKV6(torch.autograd.Function):
             ctx.dims = (B, T, C, H)
             ctx.algo = algo
             code = _DTYPE_CODE[r.dtype]
-            y = torch.empty((B, T, C), device=r.device, dtype=_out_dtype(r.dtype))
+            (y,) = _staggered(1, (B, T, C), _out_dtype(r.dtype), r.device, first=5)
             saved = None
             with torch.cuda.device(r.device):
                 need_grad = any(ctx.needs_input_grad[4:9])
                 nsave = lib.wkv6_saved_bytes(code, algo, B, T, C, H) if need_grad else 0
                 if nsave:
-                    saved = torch.empty(nsave, dtype=torch.uint8, device=r.device)
+                    (saved,) = _staggered(1, (nsave,), torch.uint8, r.device, first=6)
                     _native.check(lib.wkv6_forward_save(_stream(), code, algo, B, T, C, H,
                                                         _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(y),
                                                         _ptr(saved), nsave))
@@ -78,7 +97,7 @@ class _WKV6(torch.autograd.Function):
             odt = _out_dtype(r.dtype)
             assert gy.dtype in (torch.bfloat16, torch.float32) and gy.dtype == odt
             gy = gy.contiguous()
-            gr, gk, gv, gw = (torch.empty((B, T, C), device=gy.device, dtype=odt) for _ in range(4))
+            gr, gk, gv, gw = _staggered(4, (B, T, C), odt, gy.device, first=7)
             gu = torch.empty((B, C), device=gy.device, dtype=odt)
             code = _DTYPE_CODE[r.dtype]
             args = (_ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(gy), _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu))
@@ -110,7 +129,7 @@ def _forward_with_state(B, T, C, H, state_map, r, k, v, w, u, init_state, algo=_
         odt = _out_dtype(r.dtype)
         sdt = init_state.dtype if init_state is not None else (state_dtype or odt)
         N = C // H
-        y = torch.empty((B, T, C), device=r.device, dtype=odt)
+        (y,) = _staggered(1, (B, T, C), odt, r.device, first=5)
         ys = torch.empty((B, H, N, N), device=r.device, dtype=sdt)
         with torch.cuda.device(r.device):
             # optional workspace: lets a long sequence of few (batch, head) pairs run as time segments
@@ -157,7 +176,7 @@ def _backward_with_state(B, T, C, H, r, k, v, w, u, s0, gy, gsT, algo, want_gs0)
     """gr, gk, gv, gw, per-row gu (B, C), dL/dS_0 or None, through wkv6_backward_with_state."""
     lib = _native.load()
     odt = _out_dtype(r.dtype)
-    gr, gk, gv, gw = (torch.empty((B, T, C), device=r.device, dtype=odt) for _ in range(4))
+    gr, gk, gv, gw = _staggered(4, (B, T, C), odt, r.device, first=7)
     gu = torch.empty((B, C), device=r.device, dtype=odt)
     gs0 = torch.empty((B, H, C // H, C // H), device=r.device, dtype=torch.float32) if want_gs0 else None
     code = _DTYPE_CODE[r.dtype]
