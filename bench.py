@@ -27,6 +27,7 @@ WORKLOADS = {
     "c2": (8, 1024, 32, "bf16"),   # RWKV6-1.6B layer shape: the configuration the metric is quoted on
     "c3": (4, 4096, 64, "bf16"),   # RWKV6-7B layer shape
     "c1": (2, 128, 4, "f32"),
+    "c2_f16": (8, 1024, 32, "f16"),   # the c2 shape with fp16 tensors: y, gy and the gradients are fp32
     "long1": (1, 8192, 32, "bf16"),   # one long sequence per GPU (fine-tuning): 32 pairs, runs as time segments
 }
 
@@ -252,9 +253,11 @@ def main():
     B, T, H, dt_name = WORKLOADS[a.workload]
     N = 64
     C = H * N
-    dtype = {"bf16": torch.bfloat16, "f32": torch.float32}[dt_name]
-    code = {"bf16": _native.BF16, "f32": _native.F32}[dt_name]
-    es = 2 if dt_name == "bf16" else 4
+    dtype = {"bf16": torch.bfloat16, "f32": torch.float32, "f16": torch.float16}[dt_name]
+    odtype = torch.float32 if dt_name == "f16" else dtype   # fp16 tensors: fp32 outputs (and upstream gradient)
+    code = {"bf16": _native.BF16, "f32": _native.F32, "f16": _native.F16}[dt_name]
+    es = 4 if dt_name == "f32" else 2                       # bytes per input element
+    eo = 2 if dt_name == "bf16" else 4                      # bytes per output element
     algo = {"auto": _native.ALGO_AUTO, "scan": _native.ALGO_SCAN, "chunk": _native.ALGO_CHUNK}[a.algo]
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -264,7 +267,7 @@ def main():
     # step, and tensors whose bases agree modulo 4 KiB send all those streams to the same memory
     # channel at the same time (which costs about 5 % at this size; torch's own allocator returns
     # 2 MiB-aligned blocks).  The torch flavour carves the tensors it allocates itself the same way.
-    nbytes = B * T * C * es
+    nbytes = B * T * C * max(es, eo)
     slot = (nbytes + (2 << 20) - 1) // (2 << 20) * (2 << 20) + (2 << 20)
     nsave = 0 if a.plain_pair else lib.wkv6_saved_bytes(code, algo, B, T, C, H)
     pool = torch.empty(11 * slot + nsave + (2 << 20), dtype=torch.uint8, device=dev)
@@ -274,17 +277,19 @@ def main():
         o = first + i * slot + i * a.stagger
         return pool[o:o + nb]
 
-    def big(i, src=None):
-        t = carve(i).view(dtype).view(B, T, C)
+    def big(i, src=None, dt=None):
+        dt = dt or dtype
+        t = carve(i, B * T * C * torch.empty((), dtype=dt).element_size()).view(dt).view(B, T, C)
         if src is not None:
-            t.copy_(src.to(dtype))
+            t.copy_(src.to(dt))
         return t
 
     ins = synthetic_inputs(B, T, H, N, a.seed)
-    r, k, v, w, gy = (big(i, ins[j]) for i, j in enumerate((0, 1, 2, 3, 5)))
+    r, k, v, w = (big(i, ins[i]) for i in range(4))
+    gy = big(4, ins[5], odtype)
     u = ins[4].to(dtype).to(dev).contiguous()
-    y, gr, gk, gv, gw = (big(5 + i) for i in range(5))
-    gu_part = torch.empty(B, C, dtype=dtype, device=dev)
+    y, gr, gk, gv, gw = (big(5 + i, None, odtype) for i in range(5))
+    gu_part = torch.empty(B, C, dtype=odtype, device=dev)
     fws_bytes = lib.wkv6_forward_workspace_bytes(code, algo, B, T, C, H)
     bws_bytes = lib.wkv6_backward_workspace_bytes_ex(code, algo, B, T, C, H)
     fws = torch.empty(max(fws_bytes, 16), dtype=torch.uint8, device=dev)
@@ -305,7 +310,7 @@ def main():
             _native.check(lib.wkv6_forward_ex(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(y),
                                               P(fws), fws_bytes))
 
-    gu_sum = torch.empty(C, dtype=dtype, device=dev)
+    gu_sum = torch.empty(C, dtype=odtype, device=dev)
 
     def bwd_call():
         if nsave:   # the batch sum of gu comes out of the same launch
@@ -354,8 +359,8 @@ def main():
     copy_gbs = 2 * src.numel() / (c_avg * 1e-3) / 1e9
     del src, dst
 
-    bytes_fwd = 5 * B * T * C * es + C * es
-    bytes_bwd = 9 * B * T * C * es + 2 * C * es
+    bytes_fwd = B * T * C * (4 * es + eo) + C * es                # r, k, v, w in, y out
+    bytes_bwd = B * T * C * (4 * es + eo + 4 * eo) + C * (es + eo)   # r, k, v, w, gy in, four gradients out
     bytes_step = bytes_fwd + bytes_bwd
     dom = "bwd" if b_avg >= f_avg else "fwd"
     dom_bytes, dom_ms = (bytes_bwd, b_avg) if dom == "bwd" else (bytes_fwd, f_avg)

@@ -35,6 +35,14 @@ void *static_scratch(hipError_t *err) {
 bool chunk_possible(int dtype, int64_t T, int64_t C) { return dtype == WKV6_BF16 && T * C < (1LL << 31); }
 bool chunk_eligible(int dtype, int64_t T, int64_t C) { return chunk_possible(dtype, T, C) && T >= 32; }
 
+// The training pair (wkv6_forward_save / wkv6_backward_saved*) also runs fp16 tensors on the chunked
+// kernels: r, k, w are unpacked exactly, v and gy go through bf16 copies kept behind the saved states.
+bool train_chunk(int dtype, int algo, int64_t T, int64_t C) {
+    if (dtype != WKV6_BF16 && dtype != WKV6_F16) return false;
+    if (T * C >= (1LL << 31)) return false;
+    return algo == WKV6_ALGO_CHUNK || (algo == WKV6_ALGO_AUTO && T >= 32);
+}
+
 thread_local int g_last_status = WKV6_OK;
 thread_local int g_last_hip_error = 0;
 
@@ -179,8 +187,19 @@ static int train_segments(int dtype, int algo, int64_t B, int64_t T, int64_t C, 
     return chunk ? wkv6::chunk_train_segments(B, T, H) : 1;
 }
 
+// fp16 training pair: the bf16 copies of v and gy sit behind the base part of the saved block
+static size_t f16_stage_offset(int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
+    const size_t ws = wkv6::scan_backward_workspace_bytes(B, T, C), cw = wkv6::chunk_backward_workspace_bytes(B, T, H),
+                 sv = wkv6::chunk_saved_bytes(B, T, H);
+    const size_t m = ws > cw ? (ws > sv ? ws : sv) : (cw > sv ? cw : sv);
+    (void)algo;
+    return (m + 255) & ~(size_t)255;
+}
+
 size_t wkv6_saved_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
     if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
+    if (dtype == WKV6_F16)
+        return train_chunk(dtype, algo, T, C) ? f16_stage_offset(algo, B, T, C, H) + 2 * (size_t)(B * T * C) * 2 : 0;
     const bool chunk = (algo == WKV6_ALGO_CHUNK && chunk_possible(dtype, T, C)) ||
                        (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
     if (!chunk) return 0;
@@ -196,6 +215,15 @@ int wkv6_forward_save(void *stream, int dtype, int algo, int64_t B, int64_t T, i
                       void *y, void *saved, size_t saved_bytes) {
     const size_t need = wkv6_saved_bytes(dtype, algo, B, T, C, H);
     if (need > 0 && (!saved || saved_bytes < need || !aligned16(saved))) return WKV6_ERR_WORKSPACE;
+    if (need > 0 && dtype == WKV6_F16) {
+        if (algo < WKV6_ALGO_AUTO || algo > WKV6_ALGO_CHUNK) return WKV6_ERR_ARG;
+        if (!r || !k || !v || !w || !u || !y) return WKV6_ERR_ARG;
+        if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(y)) return WKV6_ERR_ARG;
+        void *v_bf16 = reinterpret_cast<char *>(saved) + f16_stage_offset(algo, B, T, C, H);
+        hipError_t e = wkv6::convert_to_bf16((hipStream_t)stream, wkv6::kF16, v, v_bf16, B * T * C);
+        if (e != hipSuccess) return finish(e);
+        return finish(wkv6::chunk_forward_save_f16((hipStream_t)stream, B, T, H, r, k, v, v_bf16, w, u, y, saved));
+    }
     if (need > 0 && train_segments(dtype, algo, B, T, C, H) > 1) {
         // few pairs, long sequence: time segments side by side
         const int P = train_segments(dtype, algo, B, T, C, H);
@@ -308,11 +336,31 @@ int wkv6_backward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, in
                          workspace_bytes, false);
 }
 
+// fp16 training pair, backward: gy (fp32) gets its bf16 copy next to the one of v the forward left
+static int backward_saved_f16(void *stream, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
+                              const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                              void *gr, void *gk, void *gv, void *gw, void *gu, void *gu_sum, void *saved, size_t saved_bytes) {
+    if (!r || !k || !v || !w || !u || !gy || !gr || !gk || !gv || !gw || !gu) return WKV6_ERR_ARG;
+    if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(gy) || !aligned16(gr) ||
+        !aligned16(gk) || !aligned16(gv) || !aligned16(gw)) return WKV6_ERR_ARG;
+    if (!saved || saved_bytes < wkv6_saved_bytes(WKV6_F16, algo, B, T, C, H) || !aligned16(saved)) return WKV6_ERR_WORKSPACE;
+    char *v_bf16 = reinterpret_cast<char *>(saved) + f16_stage_offset(algo, B, T, C, H);
+    char *gy_bf16 = v_bf16 + (size_t)(B * T * C) * 2;
+    hipStream_t st = (hipStream_t)stream;
+    hipError_t e = wkv6::convert_to_bf16(st, wkv6::kF32, gy, gy_bf16, B * T * C);
+    if (e != hipSuccess) return finish(e);
+    return finish(wkv6::chunk_backward(st, B, T, H, r, k, v_bf16, w, u, gy_bf16, gr, gk, gv, gw, gu, saved, true, gu_sum,
+                                       nullptr, nullptr, nullptr, wkv6::kF16, v, gy));
+}
+
 int wkv6_backward_saved(void *stream, int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H,
                         const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
                         void *gr, void *gk, void *gv, void *gw, void *gu, void *saved, size_t saved_bytes) {
     // `saved` doubles as the workspace: the guarded per-timestep pass only runs when the chunked
     // results (and with them the saved states) are discarded anyway
+    if (check_shape(dtype, B, T, C, H) == WKV6_OK && algo >= WKV6_ALGO_AUTO && algo <= WKV6_ALGO_CHUNK &&
+        dtype == WKV6_F16 && train_chunk(dtype, algo, T, C))
+        return backward_saved_f16(stream, algo, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, nullptr, saved, saved_bytes);
     if (check_shape(dtype, B, T, C, H) == WKV6_OK && algo >= WKV6_ALGO_AUTO && algo <= WKV6_ALGO_CHUNK &&
         train_segments(dtype, algo, B, T, C, H) > 1)
         return backward_segments_impl(stream, dtype, algo, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, nullptr, saved, saved_bytes);
@@ -325,6 +373,9 @@ int wkv6_backward_saved_sum(void *stream, int dtype, int algo, int64_t B, int64_
                             void *gr, void *gk, void *gv, void *gw, void *gu, void *gu_sum,
                             void *saved, size_t saved_bytes) {
     if (!gu_sum) return WKV6_ERR_ARG;
+    if (check_shape(dtype, B, T, C, H) == WKV6_OK && algo >= WKV6_ALGO_AUTO && algo <= WKV6_ALGO_CHUNK &&
+        dtype == WKV6_F16 && train_chunk(dtype, algo, T, C))
+        return backward_saved_f16(stream, algo, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, gu_sum, saved, saved_bytes);
     if (check_shape(dtype, B, T, C, H) == WKV6_OK && algo >= WKV6_ALGO_AUTO && algo <= WKV6_ALGO_CHUNK &&
         train_segments(dtype, algo, B, T, C, H) > 1)
         return backward_segments_impl(stream, dtype, algo, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, gu_sum, saved, saved_bytes);

@@ -61,8 +61,9 @@ static_assert(BwdLds::kBytes <= 160 * 1024, "LDS block of the backward kernel");
 
 struct BwdArgs {
     int T, H;
-    const bf16_t *r, *k, *v, *w, *u, *gy;
-    bf16_t *gr, *gk, *gv, *gw, *gu;
+    const bf16_t *r, *k, *v, *w, *u, *gy;   // 16-bit elements: bf16, or fp16 with v and gy bf16 copies (see OutOf)
+    const void *v_orig, *gy_orig;           // v and gy as the caller holds them (read by the exact per-timestep pass)
+    bf16_t *gr, *gk, *gv, *gw, *gu;         // elements of the output type (bf16, or fp32 for fp16 tensors)
     bf16_t *gu_sum;   // null, or C elements: receives the sum of gu over the batch
     int *arrivals;    // per head: workgroups that have delivered their gu partial (zero on entry)
     int B;
@@ -75,7 +76,7 @@ struct BwdArgs {
 // ------------------------------------------------------------------------------------------
 // Consumer group GRP of two: gr, gk, gw, gu.
 // ------------------------------------------------------------------------------------------
-template <bool kRagged, int GRP>
+template <typename Tin, bool kRagged, int GRP>
 __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *smem, const int *s_wild, int b, int h, int q, int lane)
 {
     const int T = a.T, H = a.H;
@@ -93,10 +94,11 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
         Gj[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
         if (a.gsT) Gj[m] = *reinterpret_cast<const f32x4 *>(a.gsT + (int64_t)(b * H + h) * (kN * kN) + col * kN + 16 * m + 4 * g);
     }
-    const float uj = load1(a.u + h * kN + col);
+    typedef typename OutOf<Tin>::type Tout;
+    const float uj = load1(reinterpret_cast<const Tin *>(a.u) + h * kN + col);
     float gu_acc = 0.f;
-    bf16_t *gr_h = a.gr + base, *gk_h = a.gk + base, *gw_h = a.gw + base;
-    const uint32_t rowbytes = (uint32_t)C * 2u;
+    Tout *gr_h = reinterpret_cast<Tout *>(a.gr) + base, *gk_h = reinterpret_cast<Tout *>(a.gk) + base, *gw_h = reinterpret_cast<Tout *>(a.gw) + base;
+    const uint32_t rowbytes = (uint32_t)C * (uint32_t)sizeof(Tout);
     // Saved forward state of a chunk as packed bf16: Sraw[m] = S^T[i = 16m + 4g .. +3][j = col].  It
     // comes out of LDS, where the producer waves put the chunk's block from the workspace.  The
     // consumer waves issue no global load at all:
@@ -105,17 +107,32 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     uint2 Sraw[4];
     // One chunk visit.  All four tiles are always processed (tokens past the end were prepared as
     // r = k = 0, decay 1, so they leave both states alone and contribute nothing).
-    // gr, gk, gw of the 4 tokens from `tfirst` on, channel col, as packed pairs {gr01, gk01, gw01, gr23, gk23, gw23}
-    auto store_tile = [&](int tfirst, const uint32_t (&pk)[6]) {
+    // gr, gk, gw of the 4 tokens from `tfirst` on, channel col (bf16 outputs: two tokens share one conversion per tensor)
+    auto store_tile = [&](int tfirst, const float (&gro)[4], const float (&gko)[4], const float (&gwo)[4]) {
+        if constexpr (sizeof(Tout) == 2) {
+            const uint32_t pk[6] = {pack_bf16x2(gro[0], gro[1]), pack_bf16x2(gko[0], gko[1]), pack_bf16x2(gwo[0], gwo[1]),
+                                    pack_bf16x2(gro[2], gro[3]), pack_bf16x2(gko[2], gko[3]), pack_bf16x2(gwo[2], gwo[3])};
 #pragma unroll
-        for (int hh = 0; hh < 2; ++hh) {
-            const int t = tfirst + 2 * hh;
-            const uint32_t o = (uint32_t)t * rowbytes + 2u * (uint32_t)col;
-            if (!kRagged || t < T) {
-                st16_lo(gr_h, o, pk[3 * hh]); st16_lo(gk_h, o, pk[3 * hh + 1]); st16_lo(gw_h, o, pk[3 * hh + 2]);
+            for (int hh = 0; hh < 2; ++hh) {
+                const int t = tfirst + 2 * hh;
+                const uint32_t o = (uint32_t)t * rowbytes + 2u * (uint32_t)col;
+                if (!kRagged || t < T) {
+                    st16_lo(gr_h, o, pk[3 * hh]); st16_lo(gk_h, o, pk[3 * hh + 1]); st16_lo(gw_h, o, pk[3 * hh + 2]);
+                }
+                if (!kRagged || t + 1 < T) {
+                    st16_hi(gr_h, o + rowbytes, pk[3 * hh]); st16_hi(gk_h, o + rowbytes, pk[3 * hh + 1]); st16_hi(gw_h, o + rowbytes, pk[3 * hh + 2]);
+                }
             }
-            if (!kRagged || t + 1 < T) {
-                st16_hi(gr_h, o + rowbytes, pk[3 * hh]); st16_hi(gk_h, o + rowbytes, pk[3 * hh + 1]); st16_hi(gw_h, o + rowbytes, pk[3 * hh + 2]);
+        } else {
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) {
+                const int t = tfirst + rr;
+                const uint32_t o = (uint32_t)t * rowbytes + 4u * (uint32_t)col;
+                if (!kRagged || t < T) {
+                    *reinterpret_cast<float *>(reinterpret_cast<char *>(gr_h) + o) = gro[rr];
+                    *reinterpret_cast<float *>(reinterpret_cast<char *>(gk_h) + o) = gko[rr];
+                    *reinterpret_cast<float *>(reinterpret_cast<char *>(gw_h) + o) = gwo[rr];
+                }
             }
         }
     };
@@ -254,7 +271,7 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
                 a_[0] = a4[0]; a_[1] = a4[1]; a_[2] = a4[2]; a_[3] = a4[3];
                 unpack4(tile_frag_tok(fr, 16 * q, 16 * p + 4, l16, g), nx);   // rows tk+4..: only the first is used
                 a_[4] = (g == 3) ? gq : nx[0];                                  // a_16 = g
-                unpack4(tile_frag_tok(wt, 16 * q, 16 * p, l16, g), w_);
+                unpack4_in<Tin>(tile_frag_tok(wt, 16 * q, 16 * p, l16, g), w_);   // (the raw tile: the input type)
                 unpack4(rtq, rt_); unpack4(ktq, kt_);
             }
             const float4 vg4 = *reinterpret_cast<const float4 *>(&vgyw[4 * g]);
@@ -291,10 +308,7 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
                 for (int rr = 0; rr < 4; ++rr)
                     if ((t0 + tk + rr == 0 && !a.s0) || (t0 + tk + rr == T - 1 && !a.gsT)) gwo[rr] = 0.f;
             }
-            // two tokens share one conversion per tensor
-            const uint32_t packed[6] = {pack_bf16x2(gro[0], gro[1]), pack_bf16x2(gko[0], gko[1]), pack_bf16x2(gwo[0], gwo[1]),
-                                        pack_bf16x2(gro[2], gro[3]), pack_bf16x2(gko[2], gko[3]), pack_bf16x2(gwo[2], gwo[3])};
-            store_tile(t0 + tk, packed);
+            store_tile(t0 + tk, gro, gko, gwo);
             __builtin_amdgcn_sched_barrier(0);
         }
         ++item;
@@ -312,7 +326,7 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     __syncthreads();
     if (GRP == 0 && g == 0 && !*s_wild) {   // (the exact second pass writes gu itself)
         gu_acc += reinterpret_cast<const float *>(smem + BwdLds::kGu)[col];
-        store1(a.gu + (int64_t)b * C + h * kN + col, gu_acc);
+        store1(reinterpret_cast<Tout *>(a.gu) + (int64_t)b * C + h * kN + col, gu_acc);
     }
 }
 
@@ -330,9 +344,9 @@ struct GvState {
     }
 };
 // the tiles of chunk c (chunk visit `item`), last to first
-template <bool kRagged>
-__device__ __forceinline__ void bwd_gv_chunk(GvState &st, const BwdArgs &a, const unsigned char *smem, bf16_t *gv_h,
-                                             uint32_t rowbytes, int c, int item, int q, int lane)
+template <typename Tout, bool kRagged>
+__device__ __forceinline__ void bwd_gv_chunk(GvState &st, const BwdArgs &a, const unsigned char *smem, Tout *gv_h,
+                                             uint32_t rowelems, int c, int item, int q, int lane)
 {
     const int T = a.T;
     const int g = lane >> 4, l16 = lane & 15;
@@ -375,9 +389,7 @@ __device__ __forceinline__ void bwd_gv_chunk(GvState &st, const BwdArgs &a, cons
         settle(GV, Gi);
         {
             const int t = t0 + row;   // channels 16q + 4g .. +3 of this token
-            if (!kRagged || t < T)
-                *reinterpret_cast<uint2 *>(reinterpret_cast<char *>(gv_h) + ((uint32_t)t * rowbytes + 2u * (uint32_t)(16 * q + 4 * g))) =
-                    make_uint2(pack_bf16x2(GV[0], GV[1]), pack_bf16x2(GV[2], GV[3]));
+            if (!kRagged || t < T) store4(gv_h + ((uint32_t)t * rowelems + (uint32_t)(16 * q + 4 * g)), GV[0], GV[1], GV[2], GV[3]);
         }
     }
 }
@@ -385,7 +397,7 @@ __device__ __forceinline__ void bwd_gv_chunk(GvState &st, const BwdArgs &a, cons
 // ------------------------------------------------------------------------------------------
 // Loader / producer: wave p <-> tile p of every chunk, lane = channel.
 // ------------------------------------------------------------------------------------------
-template <bool kRagged>
+template <typename Tin, bool kRagged>
 __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *smem, int *s_wild, int b, int h, int p, int lane)
 {
     const int T = a.T, H = a.H;
@@ -394,7 +406,8 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
     const int nchunk = (T + CL - 1) / CL;
     const int nitem = nchunk;   // item = chunk visit: chunks n-1 .. 0
-    const float uc = load1(a.u + h * kN + ch);
+    typedef typename OutOf<Tin>::type Tout;
+    const float uc = load1(reinterpret_cast<const Tin *>(a.u) + h * kN + ch);
     const bf16_t *rb = a.r + base, *kb_ = a.k + base, *vb = a.v + base, *wb = a.w + base, *gb = a.gy + base;   // uniform
     const uint32_t rowbytes = (uint32_t)C * 2u;
     const uint32_t lds0 = lds_address(smem);
@@ -476,8 +489,8 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
             uint32_t ra = *reinterpret_cast<const uint16_t *>(a_rk[e & 7] + e * kTileRow);
             uint32_t rk = *reinterpret_cast<const uint16_t *>(a_rk[e & 7] + kTileBytes + e * kTileRow);
             uint32_t rw = *reinterpret_cast<const uint16_t *>(a_w[e & 7] + e * kTileRow);
-            if (kRagged && tb + e >= T) { ra = 0u; rk = 0u; rw = 0xff80u; }
-            fr[e] = bf16_bits_to_float(ra); fk[e] = bf16_bits_to_float(rk); fw[e] = bf16_bits_to_float(rw);
+            if (kRagged && tb + e >= T) { ra = 0u; rk = 0u; rw = neg_inf_bits<Tin>(); }
+            fr[e] = in_bits_to_float<Tin>(ra); fk[e] = in_bits_to_float<Tin>(rk); fw[e] = in_bits_to_float<Tin>(rw);
         }
         // exponents are kept in base 2 (one v_exp_f32 each, no extra scaling multiply)
         float xr[16], xk[16], pr[16], fa[16];
@@ -539,7 +552,7 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
             prepare(it + 1);
         }
         // the gv role, on the waves the operand preparation leaves partly idle
-        bwd_gv_chunk<kRagged>(gvst, a, smem, a.gv + base, rowbytes, item_chunk(it), it, p, lane);
+        bwd_gv_chunk<Tout, kRagged>(gvst, a, smem, reinterpret_cast<Tout *>(a.gv) + base, (uint32_t)C, item_chunk(it), it, p, lane);
         // the next item's state has to be in LDS when the consumers pass the barrier
         if (state_loads) wait_younger(younger + gv_stores(it));
     }
@@ -552,7 +565,7 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
 //   loader/producer + gv | consumer group 0 (tiles 3, 1) | consumer group 1 (tiles 2, 0)
 constexpr int kBwdWaves = 12;
 
-template <bool kRagged>
+template <typename Tin, bool kRagged>
 __global__ __launch_bounds__(kBwdWaves * 64) void chunk_bwd_kernel(BwdArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -567,9 +580,10 @@ __global__ __launch_bounds__(kBwdWaves * 64) void chunk_bwd_kernel(BwdArgs a)
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int role = wave >> 2, q = wave & 3;
-    if (role == 0) bwd_producer<kRagged>(a, smem, &s_wild, b, h, q, lane);
-    else if (role == 1) bwd_consumer<kRagged, 0>(a, smem, &s_wild, b, h, q, lane);
-    else bwd_consumer<kRagged, 1>(a, smem, &s_wild, b, h, q, lane);
+    typedef typename OutOf<Tin>::type Tout;
+    if (role == 0) bwd_producer<Tin, kRagged>(a, smem, &s_wild, b, h, q, lane);
+    else if (role == 1) bwd_consumer<Tin, kRagged, 0>(a, smem, &s_wild, b, h, q, lane);
+    else bwd_consumer<Tin, kRagged, 1>(a, smem, &s_wild, b, h, q, lane);
     // exact second pass for this (b, h) if any of its tiles left the representable range; the
     // workgroup's own slice of the state workspace (nchunk x 64 x 64 floats = T' x 64) holds P
     if (s_wild) {
@@ -579,12 +593,15 @@ __global__ __launch_bounds__(kBwdWaves * 64) void chunk_bwd_kernel(BwdArgs a)
         const float *s0p = a.s0 ? a.s0 + so : nullptr, *gsTp = a.gsT ? a.gsT + so : nullptr;
         const bool states = a.s0 || a.gsT || a.gs0;
         __syncthreads();
-        scan_bwd_a_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdALds *>(smem), b, h, a.T, a.H, a.r, a.k, a.v, a.w, a.u, a.gy, a.gr, a.gu, ck, kN,
-                                        s0p, gsTp, states ? s_ft : nullptr);
+        auto in = [](const void *p) { return reinterpret_cast<const Tin *>(p); };
+        auto out = [](void *p) { return reinterpret_cast<Tout *>(p); };
+        const Tout *gyp = reinterpret_cast<const Tout *>(a.gy_orig);
+        scan_bwd_a_body<Tin, Tout>(*reinterpret_cast<ScanBwdALds *>(smem), b, h, a.T, a.H, in(a.r), in(a.k), in(a.v_orig), in(a.w), in(a.u), gyp,
+                                   out(a.gr), out(a.gu), ck, kN, s0p, gsTp, states ? s_ft : nullptr);
         __threadfence_block();
         __syncthreads();
-        scan_bwd_b_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdBLds *>(smem), b, h, a.T, a.H, a.r, a.k, a.v, a.w, a.u, a.gy, ck, kN, a.gk, a.gv, a.gw,
-                                        gsTp, states ? s_ft : nullptr, a.gs0 ? a.gs0 + so : nullptr, a.s0 == nullptr);
+        scan_bwd_b_body<Tin, Tout>(*reinterpret_cast<ScanBwdBLds *>(smem), b, h, a.T, a.H, in(a.r), in(a.k), in(a.v_orig), in(a.w), in(a.u), gyp, ck, kN,
+                                   out(a.gk), out(a.gv), out(a.gw), gsTp, states ? s_ft : nullptr, a.gs0 ? a.gs0 + so : nullptr, a.s0 == nullptr);
     }
     // Fused batch sum of gu (what the caller otherwise does with one more kernel): the workgroup that
     // is the last of its head to deliver adds up the B partials.  The partials travel as written-
@@ -598,7 +615,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void chunk_bwd_kernel(BwdArgs a)
         __syncthreads();
         const int tid = threadIdx.x;
         if (tid < kN) {          // wave 0
-            const float part = load1(a.gu + (int64_t)b * C + h * kN + tid);
+            const float part = load1(reinterpret_cast<const Tout *>(a.gu) + (int64_t)b * C + h * kN + tid);
             __hip_atomic_store(a.ckpt + (int64_t)(b * a.H + h) * slice + slice / 2 + tid, part, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             if (tid == 0)
@@ -609,7 +626,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void chunk_bwd_kernel(BwdArgs a)
             float acc = 0.f;
             for (int bb = 0; bb < a.B; ++bb)
                 acc += __hip_atomic_load(a.ckpt + (int64_t)(bb * a.H + h) * slice + slice / 2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            store1(a.gu_sum + h * kN + tid, acc);
+            store1(reinterpret_cast<Tout *>(a.gu_sum) + h * kN + tid, acc);
             if (tid == 0) __hip_atomic_store(a.arrivals + h, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // armed again
         }
     }
@@ -643,10 +660,12 @@ hipError_t sum_over_batch(hipStream_t st, int out_dtype, int64_t B, int64_t C, c
 hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
                           const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
                           void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, bool states_ready,
-                          void *gu_sum, const float *s0, const float *gsT, float *gs0)
+                          void *gu_sum, const float *s0, const float *gsT, float *gs0,
+                          int in_dtype, const void *v_orig, const void *gy_orig)
 {
     const size_t lds = BwdLds::kBytes;
     BwdArgs a;
+    a.v_orig = v_orig ? v_orig : v; a.gy_orig = gy_orig ? gy_orig : gy;
     a.s0 = s0; a.gsT = gsT; a.gs0 = gs0;
     a.T = (int)T; a.H = (int)H;
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w;
@@ -656,12 +675,17 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
     a.B = (int)B;
     a.gu_sum = states_ready ? (bf16_t *)gu_sum : nullptr;
     a.arrivals = reinterpret_cast<int *>(reinterpret_cast<char *>(workspace) + chunk_backward_workspace_bytes(B, T, H));
-    auto launch = [&](auto ragged_tag) -> hipError_t {
-        constexpr auto kern = chunk_bwd_kernel<decltype(ragged_tag)::value>;
+    auto launch_as = [&](auto in_tag, auto ragged_tag) -> hipError_t {
+        constexpr auto kern = chunk_bwd_kernel<decltype(in_tag), decltype(ragged_tag)::value>;
         hipError_t e = allow_dynamic_lds<kern>((int)lds);
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(kBwdWaves * 64), lds, st, a);
         return hipGetLastError();
+    };
+    auto launch = [&](auto ragged_tag) -> hipError_t {
+        // fp16 tensors (fp32 gradients): only with saved states, v and gy as bf16 copies plus the originals
+        if (in_dtype == kF16) return states_ready && v_orig && gy_orig ? launch_as(f16_t{}, ragged_tag) : hipErrorInvalidValue;
+        return launch_as(bf16_t{}, ragged_tag);
     };
     const bool ragged = (T % CL) != 0;   // the last chunk has tokens past the end
     if (!states_ready) {

@@ -69,7 +69,8 @@ struct FwdArgs {
     int split;       // 1, 2 or 4 workgroups per pair, each with the consumer waves of 4 / split column slices
     int reverse;     // 1: the time axis is read back to front (row T-1-t in the place of row t); T a multiple of 64
     float *dsum;     // null, or [4 tiles][pairs][64]: per pair, log2(e) * sum of exp(w) over the tokens of tile p of every chunk
-    const bf16_t *r, *k, *v, *w, *u;
+    const bf16_t *r, *k, *v, *w, *u;   // 16-bit elements: bf16, or fp16 with v a bf16 copy (see OutOf)
+    const void *v_orig;                // v as the caller holds it (the exact per-timestep pass reads this one)
     const void *s0;
     const int64_t *map;
     bf16_t *y;
@@ -87,7 +88,7 @@ struct FwdArgs {
 // Consumer group GRP of two: both groups carry the state through every tile (4 MFMAs and a
 // scaling), group 0 produces y for tiles 0 and 2, group 1 for tiles 1 and 3.
 // ------------------------------------------------------------------------------------------
-template <typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse, int GRP>
+template <typename Tin, typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse, int GRP>
 __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned char *smem, int bh0, int q, int lane)
 {
     const int T = a.T, H = a.H;
@@ -123,7 +124,8 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
 #pragma unroll
             for (int m = 0; m < 4; ++m) S[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
         }
-        bf16_t *y_h = a.y + base;
+        typedef typename OutOf<Tin>::type Tout;
+        Tout *y_h = reinterpret_cast<Tout *>(a.y) + base;
         if (kSave && GRP == 0 && b == 0 && q == 0 && lane == 0 && a.arrivals) a.arrivals[h] = 0;
         for (int c = 0; c < nchunk; ++c, ++it) {
             __syncthreads();
@@ -200,9 +202,7 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
                         *reinterpret_cast<uint16_t *>(ys + ystage_off(tk + 3, chn)) = (uint16_t)(y23 >> 16);
                     } else {
                         const int t = t0 + 16 * p + l16;   // channels 16q + 4g .. +3 of this token
-                        if (!kRagged || t < T)
-                            *reinterpret_cast<uint2 *>(reinterpret_cast<char *>(y_h) + ((uint32_t)t * (uint32_t)C * 2u + 2u * (uint32_t)(16 * q + 4 * g))) =
-                                make_uint2(pack_bf16x2(Y[0], Y[1]), pack_bf16x2(Y[2], Y[3]));
+                        if (!kRagged || t < T) store4(y_h + ((uint32_t)t * (uint32_t)C + (uint32_t)(16 * q + 4 * g)), Y[0], Y[1], Y[2], Y[3]);
                     }
                 }
                 // S <- diag(g) (S + U)
@@ -230,7 +230,7 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
 // ------------------------------------------------------------------------------------------
 // Loader / producer, lane = channel: wave p <-> tile p of every chunk.
 // ------------------------------------------------------------------------------------------
-template <bool kRagged, bool kMulti, bool kFuse>
+template <typename Tin, bool kRagged, bool kMulti, bool kFuse>
 __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *smem, int *s_wild, int bh0, int part, int pw, int lane)
 {
     constexpr int NT = 16;   // tokens per wave and chunk
@@ -339,7 +339,7 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
         if (++fl_c == nchunk && kMulti) { fl_c = 0; fl_bh += stride; if (fl_bh < a.nitems) point_output(); }
     };
     int pp_c = 0, pp_n = 0, pp_h = bh0 % H;
-    float uc = load1(a.u + pp_h * kN + ch);
+    float uc = load1(reinterpret_cast<const Tin *>(a.u) + pp_h * kN + ch);
     float dacc = 0.f;   // base-2 decay exponent summed over this wave's tiles of the current pair
     const float kLog2Log2e = 0.5287663729448977f;   // log2(log2(e)): exp(w) log2(e) = 2^(w log2(e) + this)
     auto prepare = [&](int it) {   // visit `it` = the preparation stream's current (pair, chunk)
@@ -355,8 +355,8 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
             uint32_t ra = *reinterpret_cast<const uint16_t *>(raw + o);
             uint32_t rk = *reinterpret_cast<const uint16_t *>(raw + kTileBytes + o);
             uint32_t rw = *reinterpret_cast<const uint16_t *>(raw + 2 * kTileBytes + o);
-            if (kRagged && tb + e >= T) { ra = 0u; rk = 0u; rw = 0xff80u; }
-            fr[e] = bf16_bits_to_float(ra); fk[e] = bf16_bits_to_float(rk); fw[e] = bf16_bits_to_float(rw);
+            if (kRagged && tb + e >= T) { ra = 0u; rk = 0u; rw = neg_inf_bits<Tin>(); }
+            fr[e] = in_bits_to_float<Tin>(ra); fk[e] = in_bits_to_float<Tin>(rk); fw[e] = in_bits_to_float<Tin>(rw);
         }
         float xr[NT], xk[NT], pr[NT];
 #pragma unroll
@@ -393,7 +393,7 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
             pp_c = 0; ++pp_n;
             if (pp_n < n_my) {
                 pp_h = (bh0 + pp_n * stride) % H;
-                uc = load1(a.u + pp_h * kN + ch);
+                uc = load1(reinterpret_cast<const Tin *>(a.u) + pp_h * kN + ch);
             }
         }
     };
@@ -453,7 +453,7 @@ __device__ __forceinline__ void output_stage_in_place(const FwdArgs &a, int bh) 
     }
 }
 
-template <typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse>
+template <typename Tin, typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse>
 __global__ __launch_bounds__(kFwdThreads) void chunk_fwd_kernel(FwdArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -471,11 +471,11 @@ __global__ __launch_bounds__(kFwdThreads) void chunk_fwd_kernel(FwdArgs a)
     const int bh0 = (int)blockIdx.x / split, part = (int)blockIdx.x - bh0 * split;
     const int nq = 4 / split;   // consumer waves per group
     if (wave < 4) {
-        fwd_producer<kRagged, kMulti, kFuse>(a, smem, s_wild, bh0, part, wave, lane);
+        fwd_producer<Tin, kRagged, kMulti, kFuse>(a, smem, s_wild, bh0, part, wave, lane);
     } else {
         const int cw = wave - 4, grp = cw / nq, q = part * nq + (cw - grp * nq);
-        if (grp == 0) fwd_consumer<Ts, kSave, kRagged, kMulti, kFuse, 0>(a, smem, bh0, q, lane);
-        else fwd_consumer<Ts, kSave, kRagged, kMulti, kFuse, 1>(a, smem, bh0, q, lane);
+        if (grp == 0) fwd_consumer<Tin, Ts, kSave, kRagged, kMulti, kFuse, 0>(a, smem, bh0, q, lane);
+        else fwd_consumer<Tin, Ts, kSave, kRagged, kMulti, kFuse, 1>(a, smem, bh0, q, lane);
     }
     // exact second pass for every pair of this workgroup that had a tile leave the representable range
     // (workgroups sharing a pair all see the same flags and all redo the whole pair: the same values)
@@ -487,8 +487,10 @@ __global__ __launch_bounds__(kFwdThreads) void chunk_fwd_kernel(FwdArgs a)
         if (!s_wild[n]) continue;   // uniform over the workgroup
         const int bh = bh0 + n * stride;
         __syncthreads();
-        scan_fwd_body<bf16_t, bf16_t, Ts>(*reinterpret_cast<ScanFwdLds *>(smem), bh / a.H, bh % a.H, a.T, a.H, a.r, a.k, a.v, a.w, a.u,
-                                          reinterpret_cast<const Ts *>(a.s0), a.map, kFuse ? a.out : a.y, reinterpret_cast<Ts *>(a.sT), a.reverse != 0);
+        typedef typename OutOf<Tin>::type Tout;
+        auto in = [](const void *p) { return reinterpret_cast<const Tin *>(p); };
+        scan_fwd_body<Tin, Tout, Ts>(*reinterpret_cast<ScanFwdLds *>(smem), bh / a.H, bh % a.H, a.T, a.H, in(a.r), in(a.k), in(a.v_orig), in(a.w), in(a.u),
+                                     reinterpret_cast<const Ts *>(a.s0), a.map, reinterpret_cast<Tout *>(kFuse ? a.out : a.y), reinterpret_cast<Ts *>(a.sT), a.reverse != 0);
         if (kFuse) {
             __threadfence_block();
             __syncthreads();
@@ -510,9 +512,9 @@ static int compute_units() {
     return cached[dev];
 }
 
-template <typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse>
+template <typename Tin, typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse>
 static hipError_t launch_fwd(hipStream_t st, const FwdArgs &a, unsigned grid) {
-    constexpr auto kern = chunk_fwd_kernel<Ts, kSave, kRagged, kMulti, kFuse>;
+    constexpr auto kern = chunk_fwd_kernel<Tin, Ts, kSave, kRagged, kMulti, kFuse>;
     const size_t lds = kFuse ? FwdLds::kBytesFused : FwdLds::kBytes;
     hipError_t e = allow_dynamic_lds<kern>((int)lds);
     if (e != hipSuccess) return e;
@@ -520,18 +522,18 @@ static hipError_t launch_fwd(hipStream_t st, const FwdArgs &a, unsigned grid) {
     hipLaunchKernelGGL(kern, dim3(grid * split), dim3((4 + 8 / split) * 64), lds, st, a);
     return hipGetLastError();
 }
-template <typename Ts, bool kSave, bool kRagged, bool kFuse>
+template <typename Tin, typename Ts, bool kSave, bool kRagged, bool kFuse>
 static hipError_t launch_fwd(hipStream_t st, const FwdArgs &a, bool multi, unsigned grid) {
-    return multi ? launch_fwd<Ts, kSave, kRagged, true, kFuse>(st, a, grid) : launch_fwd<Ts, kSave, kRagged, false, kFuse>(st, a, grid);
+    return multi ? launch_fwd<Tin, Ts, kSave, kRagged, true, kFuse>(st, a, grid) : launch_fwd<Tin, Ts, kSave, kRagged, false, kFuse>(st, a, grid);
 }
 template <typename Ts>
 static hipError_t launch_fwd(hipStream_t st, const FwdArgs &a, bool save, bool ragged, bool multi, unsigned grid) {
-    if (save) return ragged ? launch_fwd<Ts, true, true, false>(st, a, multi, grid) : launch_fwd<Ts, true, false, false>(st, a, multi, grid);
-    return ragged ? launch_fwd<Ts, false, true, false>(st, a, multi, grid) : launch_fwd<Ts, false, false, false>(st, a, multi, grid);
+    if (save) return ragged ? launch_fwd<bf16_t, Ts, true, true, false>(st, a, multi, grid) : launch_fwd<bf16_t, Ts, true, false, false>(st, a, multi, grid);
+    return ragged ? launch_fwd<bf16_t, Ts, false, true, false>(st, a, multi, grid) : launch_fwd<bf16_t, Ts, false, false, false>(st, a, multi, grid);
 }
 template <typename Ts>
 static hipError_t launch_fwd_fused(hipStream_t st, const FwdArgs &a, bool ragged, bool multi, unsigned grid) {
-    return ragged ? launch_fwd<Ts, false, true, true>(st, a, multi, grid) : launch_fwd<Ts, false, false, true>(st, a, multi, grid);
+    return ragged ? launch_fwd<bf16_t, Ts, false, true, true>(st, a, multi, grid) : launch_fwd<bf16_t, Ts, false, false, true>(st, a, multi, grid);
 }
 
 // One workgroup per pair while they all fit on the chip at once; beyond that one workgroup per
@@ -553,6 +555,7 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
     a.reverse = reverse && (T % CL) == 0;
     a.T = (int)T; a.H = (int)H; a.nitems = (int)(B * H);
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
+    a.v_orig = v;
     a.s0 = s0; a.map = map; a.y = (bf16_t *)y; a.sT = sT; a.ckpt = (float *)saved_states;
     a.arrivals = saved_states && counters ? reinterpret_cast<int *>(reinterpret_cast<char *>(saved_states) + chunk_backward_workspace_bytes(B, T, H)) : nullptr;
     bool multi;
@@ -560,6 +563,45 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
     const bool save = saved_states != nullptr, ragged = (T % CL) != 0;
     return state_dtype == kF32 ? launch_fwd<float>(st, a, save, ragged, multi, grid)
                                : launch_fwd<bf16_t>(st, a, save, ragged, multi, grid);
+}
+
+// bf16 copy of an fp16 or fp32 tensor (n a multiple of 8 elements, 16-byte aligned): what the MFMAs take as v and gy
+template <typename Tsrc>
+__global__ __launch_bounds__(256) void to_bf16_kernel(const Tsrc *__restrict__ src, bf16_t *__restrict__ dst, int64_t n8)
+{
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)gridDim.x * 256) {
+        Raw8<Tsrc> x;
+        x.load(src + 8 * i);
+        float f[8];
+        x.to_float(f);
+        *reinterpret_cast<uint4 *>(dst + 8 * i) = make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7]));
+    }
+}
+hipError_t convert_to_bf16(hipStream_t st, int src_dtype, const void *src, void *dst, int64_t n)
+{
+    const int64_t n8 = n / 8;
+    const unsigned grid = (unsigned)((n8 + 255) / 256 < 16384 ? (n8 + 255) / 256 : 16384);
+    if (src_dtype == kF16) hipLaunchKernelGGL(to_bf16_kernel<f16_t>, dim3(grid), dim3(256), 0, st, (const f16_t *)src, (bf16_t *)dst, n8);
+    else hipLaunchKernelGGL(to_bf16_kernel<float>, dim3(grid), dim3(256), 0, st, (const float *)src, (bf16_t *)dst, n8);
+    return hipGetLastError();
+}
+
+// The saving forward of the training pair for fp16 tensors (y fp32, zero initial state): r, k, w are
+// read as fp16 and unpacked exactly, v_bf16 is the bf16 copy of v the MFMAs take.
+hipError_t chunk_forward_save_f16(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                                  const void *r, const void *k, const void *v, const void *v_bf16, const void *w, const void *u,
+                                  void *y, void *saved_states)
+{
+    FwdArgs a = {};
+    a.T = (int)T; a.H = (int)H; a.nitems = (int)(B * H);
+    a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v_bf16; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
+    a.v_orig = v;
+    a.y = (bf16_t *)y; a.ckpt = (float *)saved_states;
+    a.arrivals = reinterpret_cast<int *>(reinterpret_cast<char *>(saved_states) + chunk_backward_workspace_bytes(B, T, H));
+    bool multi;
+    const unsigned grid = forward_grid(B * H, &multi, &a.split);
+    return (T % CL) != 0 ? launch_fwd<f16_t, float, true, true, false>(st, a, multi, grid)
+                         : launch_fwd<f16_t, float, true, false, false>(st, a, multi, grid);
 }
 
 hipError_t chunk_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
@@ -571,6 +613,7 @@ hipError_t chunk_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64
     a.T = (int)T; a.H = (int)H; a.nitems = (int)(B * H);
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
     a.s0 = s0; a.map = map; a.sT = sT;
+    a.v_orig = v;
     a.gate = (const bf16_t *)gate; a.gn_scale = gn_scale; a.gn_offset = gn_offset; a.gn_eps = gn_eps; a.out = (bf16_t *)out;
     bool multi;
     const unsigned grid = forward_grid(B * H, &multi, &a.split);

@@ -56,6 +56,14 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
                          bool reverse = false,     // the time axis read back to front (T a multiple of 64, no y)
                          bool counters = true);    // saved_states ends with the per-head counters of the fused gu sum (zeroed here)
 
+// fp16 tensors on the chunked kernels (training pair only: y and the gradients are fp32).  r, k, w stay
+// fp16 (the kernels unpack them exactly); v and gy are consumed as bf16 MFMA operands, so the caller
+// keeps bf16 copies of them (convert_to_bf16) next to the saved states.
+hipError_t convert_to_bf16(hipStream_t st, int src_dtype, const void *src, void *dst, int64_t n);
+hipError_t chunk_forward_save_f16(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                                  const void *r, const void *k, const void *v, const void *v_bf16, const void *w, const void *u,
+                                  void *y, void *saved_states);
+
 // Few pairs, long sequence: the forward as P time segments side by side (two passes joined by the
 // affine map of a segment's state).  chunk_forward_segments = P for the shape (1 = does not apply).
 int chunk_forward_segments(int64_t B, int64_t T, int64_t H);
@@ -114,8 +122,11 @@ size_t chunk_saved_bytes(int64_t B, int64_t T, int64_t H);
 hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
                           const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
                           void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, bool states_ready,
-                          void *gu_sum, const float *s0 = nullptr, const float *gsT = nullptr, float *gs0 = nullptr);
+                          void *gu_sum, const float *s0 = nullptr, const float *gsT = nullptr, float *gs0 = nullptr,
+                          int in_dtype = kBF16, const void *v_orig = nullptr, const void *gy_orig = nullptr);
 // s0 / gsT / gs0: gradients through the state, as in scan_backward_state (with states_ready = false)
+// in_dtype kF16 (needs states_ready): r, k, w, u fp16, v and gy their bf16 copies, v_orig / gy_orig the
+// caller's fp16 v and fp32 gy, gradients fp32
 
 // sum over the batch of (B, C) partials -> (C), both in the output type (for the paths without a fused sum)
 hipError_t sum_over_batch(hipStream_t st, int out_dtype, int64_t B, int64_t C, const void *partials, void *sum);

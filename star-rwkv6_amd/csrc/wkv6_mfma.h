@@ -189,6 +189,27 @@ __device__ __forceinline__ void unpack8(const bf16x8 &a, float (&o)[8]) {
 }
 
 
+// The chunked kernels take bf16 tensors (outputs bf16) or fp16 tensors (outputs fp32, the reference's
+// rule for half inputs).  r, k, w go through fp32 code anyway, so their 16-bit tiles are unpacked as
+// what they are; v and gy are consumed as bf16 MFMA operands, so for fp16 tensors the caller passes
+// bf16 copies of them (and the originals for the exact per-timestep pass).
+template <typename Tin> struct OutOf { typedef bf16_t type; };
+template <> struct OutOf<f16_t> { typedef float type; };
+template <typename Tin> __device__ __forceinline__ float in_bits_to_float(uint32_t bits);
+template <> __device__ __forceinline__ float in_bits_to_float<bf16_t>(uint32_t bits) { return __uint_as_float(bits << 16); }
+template <> __device__ __forceinline__ float in_bits_to_float<f16_t>(uint32_t bits) { return (float)__builtin_bit_cast(f16_t, (uint16_t)bits); }
+template <typename Tin> constexpr uint32_t neg_inf_bits() { return 0xff80u; }
+template <> constexpr uint32_t neg_inf_bits<f16_t>() { return 0xfc00u; }
+// four consecutive 16-bit elements of the input type (as read from a tile) -> fp32
+template <typename Tin> __device__ __forceinline__ void unpack4_in(const s16x4 &a, float (&o)[4]);
+template <> __device__ __forceinline__ void unpack4_in<bf16_t>(const s16x4 &a, float (&o)[4]) { unpack4(a, o); }
+template <> __device__ __forceinline__ void unpack4_in<f16_t>(const s16x4 &a, float (&o)[4]) {
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    const h4 x = __builtin_bit_cast(h4, a);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = (float)x[i];
+}
+
 // ------------------------------------------------------------------------------------------
 // LDS tiles: bf16 [token][64 channels], 128-byte rows, no padding; the eight 16-byte pieces of a
 // row are XOR-swizzled with (token & 7).  One layout serves the loads that fill a tile straight

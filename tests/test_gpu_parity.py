@@ -32,7 +32,9 @@ def _run_fwd_bwd(op, dev, algo):
     return y, [x.grad for x in leaves]
 
 
-def _case(op, oracle, B, T, H, seed, dtype, algo, strict=False):
+def _case(op, oracle, B, T, H, seed, dtype, algo, strict=False, tol=None):
+    # tol: the dtype whose tolerance applies (default: the output dtype).  fp16 tensors on the chunked
+    # kernels produce fp32 outputs at bf16 operand precision: they are held to the 1e-2 bound.
     N = 64
     print("case B=%d T=%d H=%d seed=%d dtype=%s algo=%d" % (B, T, H, seed, dtype, algo), flush=True)
     ins = oracle.make_inputs(B, T, H, N, seed)
@@ -45,9 +47,9 @@ def _case(op, oracle, B, T, H, seed, dtype, algo, strict=False):
     g_ref = oracle.backward_c(*ref, gy_ref[0], N)
     if strict:
         assert np.abs(to_np(y) - y_ref).max() <= 1e-4
-    check_close("y", y, y_ref, odt)
+    check_close("y", y, y_ref, tol or odt)
     for name, g, gr in zip("gr gk gv gw gu".split(), grads, g_ref):
-        check_close(name, to_np(g).reshape(gr.shape), gr, odt, is_grad=True)
+        check_close(name, to_np(g).reshape(gr.shape), gr, tol or odt, is_grad=True)
     return y, grads
 
 
@@ -284,6 +286,29 @@ def test_chunk_fwd_bwd_bf16(op, oracle, B, T, H):
     _case(op, oracle, B, T, H, 40 + T, torch.bfloat16, CHUNK)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_mixed_shape_mfma_chains_keep_both_terms(op, oracle, seed):
+    """The chunked kernels chain 16x16x32 and 16x16x16 MFMAs through one accumulator (y = R~ S + A V,
+    and X, W, gv in the backward).  On gfx950 a second MFMA of the other shape issued too close behind the
+    first read a stale accumulator, i.e. dropped the first term; the kernels keep a fixed gap there
+    (chain_gap in wkv6_mfma.h).  With almost no decay (w = -6) the state terms carry most of every
+    output, so a dropped term is an error of order one -- at the smallest shapes, one workgroup, where
+    nothing else perturbs the instruction timing."""
+    N = 64
+    for T in (64, 128, 80):
+        ins = oracle.make_inputs(1, T, 1, N, 900 + seed)
+        ins[3] = torch.full_like(ins[3], -6.0)
+        dev, ref = cast_inputs(ins[:5], torch.bfloat16)
+        gy_dev, gy_ref = cast_inputs(ins[5:6], torch.bfloat16)
+        y, grads = _run_fwd_bwd(op, dev + gy_dev, CHUNK)
+        y_ref, _ = oracle.forward_c(*ref, N)
+        g_ref = oracle.backward_c(*ref, gy_ref[0], N)
+        check_close("y", y, y_ref, torch.bfloat16)
+        for name, g, gr in zip("gr gk gv gw gu".split(), grads, g_ref):
+            check_close(name, to_np(g).reshape(gr.shape), gr, torch.bfloat16, is_grad=True)
+
+
 @pytest.mark.parametrize("B,T,H", [(1, 16, 1), (1, 48, 1), (2, 333, 2), (3, 1024, 4), (1, 80, 5)])
 def test_chunk_more_shapes_bf16(op, oracle, B, T, H):
     # T below the AUTO threshold, T % 64 != 0 with full tiles, ragged T, odd head counts
@@ -337,6 +362,40 @@ def test_chunk_falls_back_on_extreme_decay(op, oracle):
     check_close("y", y, oracle.forward_c(*ref, N)[0], torch.bfloat16)
     for name, g, gr in zip("gr gk gv gw gu".split(), grads, oracle.backward_c(*ref, gy_ref[0], N)):
         check_close(name, to_np(g).reshape(gr.shape), gr, torch.bfloat16, is_grad=True)
+
+
+# fp16 tensors on the chunked kernels (training pair: y and gradients fp32, torch_rwkv_kernel.py:35):
+# r, k, w are unpacked exactly from fp16, v and gy reach the MFMAs through bf16 copies.
+@pytest.mark.parametrize("B,T,H", [(1, 32, 1), (2, 64, 2), (2, 100, 1), (1, 129, 3), (2, 1000, 2), (1, 2048, 1),
+                                   (1, 16, 1), (1, 48, 1), (2, 333, 2), (3, 1024, 4), (1, 80, 5), (75, 64, 4), (300, 32, 1)])
+def test_chunk_fwd_bwd_f16(op, oracle, B, T, H):
+    _case(op, oracle, B, T, H, 140 + T, torch.float16, CHUNK, tol=torch.float16)
+
+
+def test_chunk_f16_falls_back_on_extreme_decay(op, oracle):
+    # as test_chunk_falls_back_on_extreme_decay: the exact second pass reads the fp16 v and the fp32 gy
+    B, T, H, N = 2, 128, 2, 64
+    ins = oracle.make_inputs(B, T, H, N, 54)
+    ins[3][1, 40:60, 70:90] = 6.0
+    ins[3][0, 5, 3] = 20.0
+    ins[3][0, 90:100] = -60000.0      # (fp16 range) decay exactly 1
+    dev, ref = cast_inputs(ins[:5], torch.float16)
+    gy_dev, gy_ref = cast_inputs(ins[5:6], torch.float32)
+    y, grads = _run_fwd_bwd(op, dev + gy_dev, CHUNK)
+    assert y.dtype == torch.float32
+    check_close("y", y, oracle.forward_c(*ref, N)[0], torch.float16)
+    for name, g, gr in zip("gr gk gv gw gu".split(), grads, oracle.backward_c(*ref, gy_ref[0], N)):
+        check_close(name, to_np(g).reshape(gr.shape), gr, torch.float16, is_grad=True)
+
+
+def test_f16_auto_takes_the_chunked_training_pair(op, oracle):
+    # AUTO with fp16 tensors and a gradient wanted: saved states exist, i.e. the chunked pair runs
+    from rwkv_kernel import _native
+    lib = _native.load()
+    assert lib.wkv6_saved_bytes(_native.F16, _native.ALGO_AUTO, 2, 256, 128, 2) > 0
+    assert lib.wkv6_saved_bytes(_native.F16, _native.ALGO_AUTO, 2, 16, 128, 2) == 0      # short: per-timestep kernels
+    assert lib.wkv6_saved_bytes(_native.F16, _native.ALGO_SCAN, 2, 256, 128, 2) == 0
+    _case(op, oracle, 2, 256, 2, 77, torch.float16, 0, tol=torch.float16)
 
 
 # More (batch, head) pairs than the chip has compute units: a forward workgroup then runs several
