@@ -123,6 +123,28 @@ int wkv6_forward_gn_gate_ex(void *stream, int dtype, int state_dtype,
                             const void *s, const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
                             void *out, void *ys, void *workspace, size_t workspace_bytes);
 
+/* The same output stage for TRAINING (no counterpart in the reference, which leaves the group norm and
+ * the gate -- rwkv6_model.py:94-99,158-160 -- and their gradients to framework kernels):
+ *
+ * wkv6_forward_gn_gate_save: zero initial state; writes `out` as above and, for the backward, y
+ * (B,T,C) bf16, the norm's statistics `stats` (B,T,H,2) fp32 = (mean, 1/sqrt(var + gn_eps)) of y over
+ * each head's channels, and the chunk states into `saved` (wkv6_saved_bytes(dtype, WKV6_ALGO_CHUNK, ...)
+ * bytes, as for wkv6_forward_save).  bf16 tensors only; shapes whose training pair runs in time segments
+ * (few pairs, long sequence) return WKV6_ERR_UNSUPPORTED: use the unfused calls there.
+ *
+ * wkv6_gn_gate_backward: given gout = dL/dout, writes gy = dL/dy (feed it to wkv6_backward_saved* with
+ * the same `saved`), ggate = dL/dgate (both (B,T,C) bf16) and gscale, goffset = dL/dgn_scale,
+ * dL/dgn_offset ((H,64) fp32, summed over batch and time; zeroed by the call). */
+int wkv6_forward_gn_gate_save_supported(int dtype, int64_t B, int64_t T, int64_t C, int64_t H);   /* 1: this shape is taken */
+int wkv6_forward_gn_gate_save(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
+                              const void *r, const void *k, const void *v, const void *w, const void *u,
+                              const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
+                              void *out, void *y, float *stats, void *saved, size_t saved_bytes);
+int wkv6_gn_gate_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
+                          const void *gout, const void *y, const float *stats, const void *gate,
+                          const float *gn_scale, const float *gn_offset,
+                          void *gy, void *ggate, float *gscale, float *goffset);
+
 /* Backward of the stateless forward: gr,gk,gv,gw (B,T,C) and gu (B,C), all in the output type.
  * Replaces backward_{bf16,fp16,fp32}(B,T,C,H,r,k,v,w,u,gy,gr,gk,gv,gw,gu),
  * rwkv_kernel/torch_kernel/wkv6_op.cpp:33-41 (kernel_backward_101/102/103/201,

@@ -173,6 +173,41 @@ int wkv6_forward_gn_gate_ex(void *stream, int dtype, int state_dtype,
                                             gate, gn_scale, gn_offset, gn_eps, out, ys));
 }
 
+static int train_segments(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H);
+
+int wkv6_forward_gn_gate_save_supported(int dtype, int64_t B, int64_t T, int64_t C, int64_t H) {
+    return check_shape(dtype, B, T, C, H) == WKV6_OK && dtype == WKV6_BF16 && chunk_possible(dtype, T, C) &&
+           train_segments(dtype, WKV6_ALGO_CHUNK, B, T, C, H) <= 1;
+}
+
+int wkv6_forward_gn_gate_save(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
+                              const void *r, const void *k, const void *v, const void *w, const void *u,
+                              const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
+                              void *out, void *y, float *stats, void *saved, size_t saved_bytes) {
+    int rc = check_shape(dtype, B, T, C, H);
+    if (rc != WKV6_OK) return rc;
+    if (dtype != WKV6_BF16 || !chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;
+    if (train_segments(dtype, WKV6_ALGO_CHUNK, B, T, C, H) > 1) return WKV6_ERR_UNSUPPORTED;   // (time segments: unfused calls)
+    if (!r || !k || !v || !w || !u || !gate || !gn_scale || !gn_offset || !out || !y || !stats) return WKV6_ERR_ARG;
+    if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(gate) || !aligned16(out) || !aligned16(y) ||
+        !aligned16(stats) || !aligned16(gn_scale) || !aligned16(gn_offset)) return WKV6_ERR_ARG;
+    const size_t need = wkv6_saved_bytes(dtype, WKV6_ALGO_CHUNK, B, T, C, H);
+    if (!saved || saved_bytes < need || !aligned16(saved)) return WKV6_ERR_WORKSPACE;
+    return finish(wkv6::chunk_forward_fused_save((hipStream_t)stream, B, T, H, r, k, v, w, u, gate, gn_scale, gn_offset, gn_eps,
+                                                 out, y, stats, saved));
+}
+
+int wkv6_gn_gate_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
+                          const void *gout, const void *y, const float *stats, const void *gate,
+                          const float *gn_scale, const float *gn_offset,
+                          void *gy, void *ggate, float *gscale, float *goffset) {
+    int rc = check_shape(dtype, B, T, C, H);
+    if (rc != WKV6_OK) return rc;
+    if (dtype != WKV6_BF16) return WKV6_ERR_UNSUPPORTED;
+    if (!gout || !y || !stats || !gate || !gn_scale || !gn_offset || !gy || !ggate || !gscale || !goffset) return WKV6_ERR_ARG;
+    return finish(wkv6::gn_gate_backward((hipStream_t)stream, B, T, H, gout, y, stats, gate, gn_scale, gn_offset, gy, ggate, gscale, goffset));
+}
+
 // Size of the part of the saved block that the kernels of one pass use (chunk states, arrival
 // counters; sized so that the guarded per-timestep pass of the backward can use the same buffer).
 static size_t saved_base_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {

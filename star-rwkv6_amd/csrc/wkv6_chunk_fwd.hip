@@ -82,6 +82,8 @@ struct FwdArgs {
     const float *gn_scale, *gn_offset;   // (H, 64)
     float gn_eps;
     bf16_t *out;
+    // training with the fused output stage (then y above is written as well, for the norm's backward):
+    float *stats;    // null, or (B, T, H, 2) fp32: mean and 1/sqrt(var + eps) of y over each head's channels
 };
 
 // ------------------------------------------------------------------------------------------
@@ -230,7 +232,7 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
 // ------------------------------------------------------------------------------------------
 // Loader / producer, lane = channel: wave p <-> tile p of every chunk.
 // ------------------------------------------------------------------------------------------
-template <typename Tin, bool kRagged, bool kMulti, bool kFuse>
+template <typename Tin, bool kSave, bool kRagged, bool kMulti, bool kFuse>
 __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *smem, int *s_wild, int bh0, int part, int pw, int lane)
 {
     constexpr int NT = 16;   // tokens per wave and chunk
@@ -304,10 +306,13 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
     // tile p, lane = channel:  out = ((y - mean) * rstd * gn_scale + gn_offset) * gate, mean and
     // variance over the head's 64 channels of a token (two passes, like a layer norm).
     int fl_c = 0, fl_bh = bh0;
-    bf16_t *ob = nullptr;
+    bf16_t *ob = nullptr, *yb = nullptr;
+    float *sb = nullptr;
+    constexpr bool train = kFuse && kSave;   // training: y and the norm's statistics are written too
     auto point_output = [&]() {
         const int b = fl_bh / H, h = fl_bh - b * H;
         ob = a.out + (int64_t)b * T * C + (int64_t)h * kN;
+        if (train) { yb = a.y + (int64_t)b * T * C + (int64_t)h * kN; sb = a.stats + ((int64_t)b * T * H + h) * 2; }
     };
     if (kFuse) point_output();
     auto output_stage = [&](int it) {   // visit `it` = the output stream's current (pair, chunk)
@@ -317,8 +322,12 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
         const float gsc = tab[ch], gof = tab[kN + ch];
         float yv[16], dv[16];
 #pragma unroll
-        for (int e = 0; e < 16; ++e)
-            yv[e] = bf16_bits_to_float(*reinterpret_cast<const uint16_t *>(ys + ystage_off(16 * p + e, ch)));
+        for (int e = 0; e < 16; ++e) {
+            const uint32_t bits = *reinterpret_cast<const uint16_t *>(ys + ystage_off(16 * p + e, ch));
+            yv[e] = bf16_bits_to_float(bits);
+            const int t = fl_c * CL + 16 * p + e;
+            if (train && (!kRagged || t < T)) *reinterpret_cast<uint16_t *>(reinterpret_cast<char *>(yb) + ((uint32_t)t * rowbytes + 2u * (uint32_t)ch)) = (uint16_t)bits;
+        }
         // lane l of the reduction holds the total of token (l >> 2) & 15
         const float mu_own = transpose_reduce16(yv, lane) * (1.f / kN);
 #pragma unroll
@@ -328,6 +337,10 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
             dv[e] = yv[e] * yv[e];
         }
         const float rstd_own = __builtin_amdgcn_rsqf(transpose_reduce16(dv, lane) * (1.f / kN) + a.gn_eps);
+        if (train && (lane & 3) == 0) {
+            const int t = fl_c * CL + 16 * p + ((lane >> 2) & 15);
+            if (!kRagged || t < T) *reinterpret_cast<float2 *>(sb + (int64_t)t * H * 2) = make_float2(mu_own, rstd_own);
+        }
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
             const float rstd = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(rstd_own), 4 * e));
@@ -411,11 +424,12 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
         // than both.  (With a ragged end the number of store instructions issued is not fixed;
         // they go first then and are waited for with the loads.)
         const bool outputs = kFuse && it > 0;
-        if (outputs && kRagged) output_stage(it - 1);
+        const bool stores_first = kRagged || train;   // (training writes y and the statistics too: not the fixed 16 stores)
+        if (outputs && stores_first) output_stage(it - 1);
         if (it + 2 < nvisit) issue_loads(it + 2);
-        if (outputs && !kRagged) output_stage(it - 1);
+        if (outputs && !stores_first) output_stage(it - 1);
         if (it + 1 < nvisit) {
-            wait_visit_loads(it + 2 < nvisit, outputs && !kRagged);
+            wait_visit_loads(it + 2 < nvisit, outputs && !stores_first);
             prepare(it + 1);
         }
     }
@@ -441,6 +455,7 @@ __device__ __forceinline__ void output_stage_in_place(const FwdArgs &a, int bh) 
     const float gsc = a.gn_scale[h * kN + lane], gof = a.gn_offset[h * kN + lane];
     for (int t = wave; t < a.T; t += nwave) {
         const float y = load1(rowp + (int64_t)t * C);
+        if (a.y) store1(a.y + (int64_t)b * a.T * C + (int64_t)h * kN + lane + (int64_t)t * C, y);
         float sum = y;
 #pragma unroll
         for (int m = 32; m >= 1; m >>= 1) sum += __shfl_xor(sum, m);
@@ -449,6 +464,7 @@ __device__ __forceinline__ void output_stage_in_place(const FwdArgs &a, int bh) 
 #pragma unroll
         for (int m = 32; m >= 1; m >>= 1) sq += __shfl_xor(sq, m);
         const float rstd = __builtin_amdgcn_rsqf(sq * (1.f / kN) + a.gn_eps);
+        if (a.stats && lane == 0) *reinterpret_cast<float2 *>(a.stats + (((int64_t)b * a.T + t) * a.H + h) * 2) = make_float2(sum * (1.f / kN), rstd);
         store1(rowp + (int64_t)t * C, fmaf(d * rstd, gsc, gof) * load1(gp + (int64_t)t * C));
     }
 }
@@ -471,7 +487,7 @@ __global__ __launch_bounds__(kFwdThreads) void chunk_fwd_kernel(FwdArgs a)
     const int bh0 = (int)blockIdx.x / split, part = (int)blockIdx.x - bh0 * split;
     const int nq = 4 / split;   // consumer waves per group
     if (wave < 4) {
-        fwd_producer<Tin, kRagged, kMulti, kFuse>(a, smem, s_wild, bh0, part, wave, lane);
+        fwd_producer<Tin, kSave, kRagged, kMulti, kFuse>(a, smem, s_wild, bh0, part, wave, lane);
     } else {
         const int cw = wave - 4, grp = cw / nq, q = part * nq + (cw - grp * nq);
         if (grp == 0) fwd_consumer<Tin, Ts, kSave, kRagged, kMulti, kFuse, 0>(a, smem, bh0, q, lane);
@@ -621,6 +637,27 @@ hipError_t chunk_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64
     const bool ragged = (T % CL) != 0;
     return state_dtype == kF32 ? launch_fwd_fused<float>(st, a, ragged, multi, grid)
                                : launch_fwd_fused<bf16_t>(st, a, ragged, multi, grid);
+}
+
+// Training with the fused output stage: out = (group_norm_head(y) * gn_scale + gn_offset) * gate, and for
+// the backward y itself (bf16), the norm's statistics and the chunk states.  Zero initial state.
+hipError_t chunk_forward_fused_save(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                                    const void *r, const void *k, const void *v, const void *w, const void *u,
+                                    const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
+                                    void *out, void *y, float *stats, void *saved_states)
+{
+    FwdArgs a = {};
+    a.T = (int)T; a.H = (int)H; a.nitems = (int)(B * H);
+    a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
+    a.v_orig = v;
+    a.gate = (const bf16_t *)gate; a.gn_scale = gn_scale; a.gn_offset = gn_offset; a.gn_eps = gn_eps; a.out = (bf16_t *)out;
+    a.y = (bf16_t *)y; a.stats = stats; a.ckpt = (float *)saved_states;
+    a.arrivals = reinterpret_cast<int *>(reinterpret_cast<char *>(saved_states) + chunk_backward_workspace_bytes(B, T, H));
+    bool multi;
+    const unsigned grid = forward_grid(B * H, &multi, &a.split);
+    a.split = 1;
+    return (T % CL) != 0 ? launch_fwd<bf16_t, float, true, true, true>(st, a, multi, grid)
+                         : launch_fwd<bf16_t, float, true, false, true>(st, a, multi, grid);
 }
 
 // ------------------------------------------------------------------------------------------

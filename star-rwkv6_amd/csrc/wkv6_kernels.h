@@ -113,6 +113,16 @@ hipError_t chunk_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64
                                const void *s0, const int64_t *map, const void *gate, const float *gn_scale,
                                const float *gn_offset, float gn_eps, void *out, void *sT);
 
+// The same for training: also writes y (bf16), the norm's statistics (B,T,H,2: mean, rstd) and the chunk states
+hipError_t chunk_forward_fused_save(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                                    const void *r, const void *k, const void *v, const void *w, const void *u,
+                                    const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
+                                    void *out, void *y, float *stats, void *saved_states);
+// backward of the output stage (wkv6_gn.hip): bf16 tensors, gscale / goffset fp32 (C), zeroed inside
+hipError_t gn_gate_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                            const void *gout, const void *y, const float *stats, const void *gate,
+                            const float *scale, const float *offset, void *gy, void *ggate, float *gscale, float *goffset);
+
 size_t chunk_backward_workspace_bytes(int64_t B, int64_t T, int64_t H);
 // bytes of a forward -> backward hand-over buffer: the workspace plus one arrival counter per head
 // (zeroed by the saving forward, used by the backward's fused batch sum of gu)

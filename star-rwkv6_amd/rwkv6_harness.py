@@ -103,8 +103,9 @@ class TimeMix(nn.Module):
             w = w * m + (1 - m) * -1e9
         u = self.time_faaaa.to(r.dtype)
         fused = getattr(self.rwkv_kernel, "forward_gn_gate", None)
-        if fused is not None and not torch.is_grad_enabled() and r.is_cuda and r.dtype == torch.bfloat16:
-            # inference: group norm and gate come out of the operator's own output stage
+        if fused is not None and r.is_cuda and r.dtype == torch.bfloat16:
+            # group norm and gate come out of the operator's own output stage (inference: y is never
+            # written; training: y and the norm's statistics are kept for one fused backward kernel)
             x, _ = fused(r.contiguous(), k.contiguous(), v.contiguous(), w.contiguous(), u, g.contiguous(),
                          self.group_norm.scale, self.group_norm.offset, self.group_norm.epsilon)
             return self.dense_o(x)

@@ -26,6 +26,9 @@ SIGNATURES = {
     "wkv6_forward_workspace_bytes": (_sz, [_int, _int] + [_i64] * 4),
     "wkv6_forward_gn_gate": (_int, [_p, _int, _int] + [_i64] * 4 + [_int, _p] + [_p] * 9 + [ctypes.c_float, _p, _p]),
     "wkv6_forward_gn_gate_ex": (_int, [_p, _int, _int] + [_i64] * 4 + [_int, _p] + [_p] * 9 + [ctypes.c_float, _p, _p] + [_p, _sz]),
+    "wkv6_forward_gn_gate_save_supported": (_int, [_int] + [_i64] * 4),
+    "wkv6_forward_gn_gate_save": (_int, [_p, _int] + [_i64] * 4 + [_p] * 8 + [ctypes.c_float] + [_p] * 4 + [_sz]),
+    "wkv6_gn_gate_backward": (_int, [_p, _int] + [_i64] * 4 + [_p] * 10),
     "wkv6_backward": (_int, [_p, _int] + [_i64] * 4 + [_p] * 11 + [_p, _sz]),
     "wkv6_backward_workspace_bytes": (_sz, [_int] + [_i64] * 4),
     "wkv6_backward_static": (_int, [_p, _int] + [_i64] * 4 + [_p] * 11),

@@ -119,6 +119,62 @@ class _WKV6(torch.autograd.Function):
             return (None, None, None, None, gr, gk, gv, gw, gu, None)
 
 
+class _WKV6GnGate(torch.autograd.Function):
+    """out = (group_norm_head(wkv6(r, k, v, w, u)) * gn_scale + gn_offset) * gate with gradients, bf16,
+    zero initial state: the operator and what the layer does with its output next
+    (rwkv6_model.py:94-99,158-160) in one forward kernel (wkv6_forward_gn_gate_save: y never makes the
+    trip to the norm's own kernels and back), the norm's and the gate's backward in one elementwise
+    kernel (wkv6_gn_gate_backward), then the operator's backward from the saved chunk states."""
+
+    @staticmethod
+    def forward(ctx, B, T, C, H, r, k, v, w, u, gate, gn_scale, gn_offset, eps):
+        lib = _native.load()
+        with torch.no_grad():
+            code = _DTYPE_CODE[r.dtype]
+            sc = gn_scale.detach().to(dtype=torch.float32).contiguous()
+            of = gn_offset.detach().to(dtype=torch.float32).contiguous()
+            out, y = _staggered(2, (B, T, C), r.dtype, r.device, first=5)
+            stats = torch.empty((B, T, H, 2), device=r.device, dtype=torch.float32)
+            with torch.cuda.device(r.device):
+                nsave = lib.wkv6_saved_bytes(code, _native.ALGO_CHUNK, B, T, C, H)
+                (saved,) = _staggered(1, (nsave,), torch.uint8, r.device, first=7)
+                _native.check(lib.wkv6_forward_gn_gate_save(
+                    _stream(), code, B, T, C, H, _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(gate), _ptr(sc), _ptr(of),
+                    float(eps), _ptr(out), _ptr(y), _ptr(stats), _ptr(saved), nsave))
+            ctx.dims = (B, T, C, H)
+            ctx.saved_states = saved
+            ctx.save_for_backward(r, k, v, w, u, gate, sc, of, y, stats)
+            ctx.param_shapes = (gn_scale.shape, gn_offset.shape, gn_scale.dtype, gn_offset.dtype)
+            return out
+
+    @staticmethod
+    def backward(ctx, gout):
+        lib = _native.load()
+        with torch.no_grad():
+            B, T, C, H = ctx.dims
+            r, k, v, w, u, gate, sc, of, y, stats = ctx.saved_tensors
+            saved, ctx.saved_states = ctx.saved_states, None
+            assert gout.dtype == r.dtype
+            gout = gout.contiguous()
+            code = _DTYPE_CODE[r.dtype]
+            gy, ggate = _staggered(2, (B, T, C), r.dtype, r.device, first=5)
+            gr, gk, gv, gw = _staggered(4, (B, T, C), r.dtype, r.device, first=7)
+            gsc = torch.empty(C, device=r.device, dtype=torch.float32)
+            gof = torch.empty(C, device=r.device, dtype=torch.float32)
+            gu = torch.empty((B, C), device=r.device, dtype=r.dtype)
+            gu_sum = torch.empty(C, device=r.device, dtype=r.dtype)
+            with torch.cuda.device(r.device):
+                _native.check(lib.wkv6_gn_gate_backward(_stream(), code, B, T, C, H, _ptr(gout), _ptr(y), _ptr(stats), _ptr(gate),
+                                                        _ptr(sc), _ptr(of), _ptr(gy), _ptr(ggate), _ptr(gsc), _ptr(gof)))
+                _native.check(lib.wkv6_backward_saved_sum(_stream(), code, _native.ALGO_CHUNK, B, T, C, H,
+                                                          _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(gy),
+                                                          _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu), _ptr(gu_sum),
+                                                          _ptr(saved), saved.numel()))
+            s_shape, o_shape, s_dt, o_dt = ctx.param_shapes
+            return (None, None, None, None, gr, gk, gv, gw, gu_sum.reshape(u.shape), ggate,
+                    gsc.reshape(s_shape).to(s_dt), gof.reshape(o_shape).to(o_dt), None)
+
+
 def _forward_with_state(B, T, C, H, state_map, r, k, v, w, u, init_state, algo=_native.ALGO_AUTO, state_dtype=None):
     """Stateful forward, no gradient (rwkv_kernel/torch_rwkv_kernel.py:76-95)."""
     lib = _native.load()
@@ -283,15 +339,30 @@ class RWKVKernelOperator:
 
     def forward_gn_gate(self, r, k, v, w, u, gate, gn_scale, gn_offset, epsilon=64e-5,
                         return_state=False, init_state=None, state_map=None):
-        """Inference forward with the layer's next two steps fused into the kernel's output stage:
-        returns ``(group_norm(y) * gate, state)`` where group_norm is the per-head layer norm with
-        scale and offset of rwkv6_model.py:94-99 and ``* gate`` is rwkv6_model.py:158-160; y itself is
-        never written.  bf16 tensors; gn_scale / gn_offset hold one value per channel.  No gradient.
-        Not part of the reference's operator."""
+        """Forward with the layer's next two steps fused into the kernel's output stage: returns
+        ``(group_norm(y) * gate, state)`` where group_norm is the per-head layer norm with scale and
+        offset of rwkv6_model.py:94-99 and ``* gate`` is rwkv6_model.py:158-160.  bf16 tensors;
+        gn_scale / gn_offset hold one value per channel.  Without gradients (inference) y itself is
+        never written and the stateful arguments work as in ``__call__``.  With gradients enabled and
+        required (training; no state arguments) the call is differentiable in r, k, v, w, u, gate,
+        gn_scale and gn_offset.  Not part of the reference's operator."""
         B, T, C, H, N, u, init_state, state_map = self._check(r, k, v, w, u, init_state, state_map)
         assert r.dtype == torch.bfloat16, "the fused output stage takes bf16 tensors"
         assert gate.shape == r.shape and gate.dtype == r.dtype and gate.device == r.device
         assert gn_scale.numel() == C and gn_offset.numel() == C
+        if torch.is_grad_enabled() and any(x.requires_grad for x in (r, k, v, w, u, gate, gn_scale, gn_offset)):
+            assert not return_state and init_state is None and state_map is None, \
+                "the differentiable fused call takes no state arguments"
+            for x in (r, k, v, w, u, gate):
+                assert x.is_contiguous()
+            lib = _native.load()
+            if lib.wkv6_forward_gn_gate_save_supported(_DTYPE_CODE[r.dtype], B, T, C, H):
+                return _WKV6GnGate.apply(B, T, C, H, r, k, v, w, u, gate, gn_scale.to(r.device), gn_offset.to(r.device), epsilon), None
+            # (few pairs and a long sequence: the operator runs in time segments; unfused calls)
+            y, _ = self(r, k, v, w, u)
+            z = torch.nn.functional.layer_norm(y.float().view(B, T, H, N), (N,), eps=epsilon).view(B, T, C)
+            out = (z * gn_scale.reshape(1, 1, C).float() + gn_offset.reshape(1, 1, C).float()) * gate.float()
+            return out.to(r.dtype), None
         init_state, state_map = self._resolve_state(B, r, init_state, state_map)
         for x in (r, k, v, w, u, gate):
             assert x.is_contiguous()

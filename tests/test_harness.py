@@ -113,9 +113,9 @@ def test_model_step_hip_operator_matches_python_loop(dtype):
 
 @pytest.mark.gpu
 def test_inference_forward_uses_the_fused_output_stage():
-    """Without gradients and in bf16 the time-mix layer takes group norm and gate from the
-    operator's own output stage; the logits agree with the unfused bf16 path and with the fp32
-    python-loop model on the CPU."""
+    """In bf16 the time-mix layer takes group norm and gate from the operator's own output stage,
+    without gradients (y never written) and with them (the differentiable fused call); the logits
+    agree with the unfused bf16 path and with the fp32 python-loop model on the CPU."""
     from rwkv_kernel import RWKVKernelOperator
     T = 96
     ref = _toy(OPSKernelOperator(64, T), seed=6)
@@ -134,11 +134,16 @@ def test_inference_forward_uses_the_fused_output_stage():
             fused = gpu(ids.to(dev)).float().cpu()
     assert len(calls) == TOY["num_layers"]
     with torch.autocast("cuda", dtype=torch.bfloat16):
-        unfused = gpu(ids.to(dev)).float().cpu()   # gradients enabled: the unfused path
-    assert len(calls) == TOY["num_layers"]
+        trained = gpu(ids.to(dev)).float().cpu()   # gradients enabled: the differentiable fused call
+    assert len(calls) == 2 * TOY["num_layers"] and trained.requires_grad
+    op.forward_gn_gate = None                      # the layer then runs operator, group norm and gate one by one
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        unfused = gpu(ids.to(dev)).float().cpu()
+    assert len(calls) == 2 * TOY["num_layers"]
     scale = float(want.abs().max())
     assert float((fused - want).abs().max()) <= 5e-2 * scale
     assert float((fused - unfused.detach()).abs().max()) <= 3e-2 * scale
+    assert float((trained.detach() - unfused.detach()).abs().max()) <= 3e-2 * scale
 
 
 @pytest.mark.gpu
