@@ -339,7 +339,19 @@ def main():
     ms_per_step = wall / a.steps * 1e3
     tokens = B * T
 
-    # per-call GPU durations with events on the launch stream (torch's current stream)
+    # Per-launch GPU durations with events on the launch stream (torch's current stream), taken inside
+    # the same alternating forward / backward sequence the timed region runs (a kernel launched after
+    # itself instead of after its partner finds other data in the 256 MB Infinity Cache and takes a few
+    # microseconds longer): event, forward, event, backward, event.
+    def gpu_ms_pair(reps):
+        ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(reps)]
+        for e0, e1, e2 in ev:
+            e0.record(); fwd(); e1.record(); bwd_call(); e2.record()
+        torch.cuda.synchronize()
+        tf = sorted(e0.elapsed_time(e1) for e0, e1, _ in ev)
+        tb = sorted(e1.elapsed_time(e2) for _, e1, e2 in ev)
+        return sum(tf) / len(tf), tf[len(tf) // 2], sum(tb) / len(tb), tb[len(tb) // 2]
+
     def gpu_ms(fn, reps):
         ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(reps)]
         for s, e in ev:
@@ -349,8 +361,7 @@ def main():
         return sum(ts) / len(ts), ts[len(ts) // 2]
 
     reps = max(10, min(a.steps, 50))
-    f_avg, f_med = gpu_ms(fwd, reps)
-    b_avg, b_med = gpu_ms(bwd_call, reps)   # the kernel alone (one launch per call)
+    f_avg, f_med, b_avg, b_med = gpu_ms_pair(reps)   # (the backward: the kernel alone, one launch per call)
 
     # stream-copy bandwidth actually reachable on this box (read + write of a 1 GiB buffer)
     src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
