@@ -145,6 +145,44 @@ int wkv6_gn_gate_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t
                           const float *gn_scale, const float *gn_offset,
                           void *gy, void *ggate, float *gscale, float *goffset);
 
+/* The INPUT side of the layer around the operator (no counterpart in the reference, which leaves it
+ * to framework kernels): the token shift and the five low-rank mixers of rwkv6_model.py:134-146 that
+ * turn the layer input x into the inputs xr, xk, xv, xw, xg of the projections producing r, k, v, w
+ * and the gate.  With xx = (previous token, zero before the first) - x  (TimeShift, :40-43):
+ *
+ *   wkv6_shift_mix_x:     x_mix = x + xx * mix_x                                  (:136)
+ *   (caller)              h[:, :, s, :] = tanh(x_mix A_s^T), s = r,k,v,w,g        (DecomposerDense.dense_a, :20)
+ *   wkv6_shift_mix_five:  x_s = x + xx * (h_s W_s^T + bias_s)                     (dense_b :21, :141-145)
+ *
+ * The rank-R product h_s W_s^T runs on the matrix cores inside the kernel that writes the five
+ * outputs, so the five (B,T,C) coefficient tensors are never stored.  bf16 tensors; C a multiple
+ * of 64; R (decomposer_size) 32 or 64 -- wkv6_shift_mix_supported says whether a shape is taken,
+ * WKV6_ERR_UNSUPPORTED otherwise.  x, x_mix, x_s and their gradients (B,T,C); h (B,T,5,R);
+ * w2t (5,C,R): each mixer's dense_b weight as (out, in); bias (5,C) and mix_x (C) fp32.
+ *
+ * Backward, in the order the chain rule needs it:
+ *   wkv6_shift_mix_five_backward: from the gradients gx_s of the five outputs writes
+ *       gcoef (5,B,T,C) = gx_s * xx  -- the caller's GEMMs turn it into the gradients of h
+ *       (gcoef_s W_s), of W_s (gcoef_s^T h_s) and of bias_s (sum over tokens) --,
+ *       gxx = sum_s gx_s * coef_s and gp = sum_s gx_s - gxx  (both (B,T,C)).
+ *   (caller) gh -> through tanh and A -> gxm = dL/dx_mix (B,T,C)
+ *   wkv6_shift_mix_x_backward: gx = gp + gxm (1 - mix_x) + z[t+1] with z = gxx + gxm mix_x
+ *       (nothing from beyond a sequence's last token), gmix_x (C) fp32 = sum over tokens of gxm * xx
+ *       (zeroed by the call). */
+int wkv6_shift_mix_supported(int dtype, int64_t C, int64_t R);
+int wkv6_shift_mix_x(void *stream, int dtype, int64_t B, int64_t T, int64_t C,
+                     const void *x, const float *mix_x, void *x_mix);
+int wkv6_shift_mix_five(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t R,
+                        const void *x, const void *h, const void *w2t, const float *bias,
+                        void *xr, void *xk, void *xv, void *xw, void *xg);
+int wkv6_shift_mix_five_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t R,
+                                 const void *x, const void *h, const void *w2t, const float *bias,
+                                 const void *gxr, const void *gxk, const void *gxv, const void *gxw, const void *gxg,
+                                 void *gcoef, void *gp, void *gxx);
+int wkv6_shift_mix_x_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C,
+                              const void *x, const float *mix_x, const void *gp, const void *gxx, const void *gxm,
+                              void *gx, float *gmix_x);
+
 /* Backward of the stateless forward: gr,gk,gv,gw (B,T,C) and gu (B,C), all in the output type.
  * Replaces backward_{bf16,fp16,fp32}(B,T,C,H,r,k,v,w,u,gy,gr,gk,gv,gw,gu),
  * rwkv_kernel/torch_kernel/wkv6_op.cpp:33-41 (kernel_backward_101/102/103/201,

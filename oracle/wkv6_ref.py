@@ -230,6 +230,30 @@ def group_norm_gate_np(y, gate, scale, offset, head_size, epsilon=64e-5):
     return x.reshape(B, T, C) * np.asarray(gate, dtype=np.float64)
 
 
+def shift_mix_np(x, mix_x, a, w2t, bias):
+    """What the reference model does with the layer input before the projections that feed the
+    operator, in float64 (rwkv6_model.py:134-146):
+        xx = TimeShift(x) = (x padded with one zero token in front, last dropped) - x       :40-43
+        x_mix = x + xx * mix_x                                                              :136
+        coef_s = DecomposerDense_s(x_mix) = tanh(x_mix a_s^T) w2t_s^T + bias_s              :11-25, :139
+        x_s = x + xx * coef_s  for s = r, k, v, w, g                                        :141-145
+    a (5R, C): dense_a kernels stacked, as (out, in); w2t (5, C, R): dense_b kernels as (out, in);
+    bias (5, C).  Returns (x_mix, h (B,T,5,R), [xr, xk, xv, xw, xg])."""
+    x = np.asarray(x, dtype=np.float64)
+    B, T, C = x.shape
+    w2t = np.asarray(w2t, dtype=np.float64)
+    R = w2t.shape[2]
+    prev = np.concatenate([np.zeros((B, 1, C)), x[:, :-1]], axis=1)
+    xx = prev - x
+    x_mix = x + xx * np.asarray(mix_x, dtype=np.float64).reshape(1, 1, C)
+    h = np.tanh(x_mix @ np.asarray(a, dtype=np.float64).T).reshape(B, T, 5, R)
+    outs = []
+    for s in range(5):
+        coef = h[:, :, s, :] @ w2t[s].T + np.asarray(bias, dtype=np.float64)[s].reshape(1, 1, C)
+        outs.append(x + xx * coef)
+    return x_mix, h, outs
+
+
 def make_inputs(B, T, H, N, seed, with_gy=True, with_state=False):
     """The benchmark's seeded distributions, drawn on the CPU in float32:
     r,k,v ~ N(0,1); w = x ~ U(-6,1) passed raw; u ~ N(0,0.5^2) (H,N); gy ~ N(0,1);

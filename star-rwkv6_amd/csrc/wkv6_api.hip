@@ -208,6 +208,55 @@ int wkv6_gn_gate_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t
     return finish(wkv6::gn_gate_backward((hipStream_t)stream, B, T, H, gout, y, stats, gate, gn_scale, gn_offset, gy, ggate, gscale, goffset));
 }
 
+static int check_mix(int dtype, int64_t B, int64_t T, int64_t C, int64_t R) {
+    if (B <= 0 || T <= 0 || C <= 0 || R <= 0) return WKV6_ERR_ARG;
+    if (dtype != WKV6_BF16 || !wkv6::shift_mix_supported(C, R)) return WKV6_ERR_UNSUPPORTED;
+    if (B * T > ((int64_t)1 << 31) / 256 * 64) return WKV6_ERR_UNSUPPORTED;   // the launch grids are 32-bit
+    return WKV6_OK;
+}
+
+int wkv6_shift_mix_supported(int dtype, int64_t C, int64_t R) {
+    return dtype == WKV6_BF16 && wkv6::shift_mix_supported(C, R);
+}
+
+int wkv6_shift_mix_x(void *stream, int dtype, int64_t B, int64_t T, int64_t C,
+                     const void *x, const float *mix_x, void *x_mix) {
+    const int rc = check_mix(dtype, B, T, C, 32);
+    if (rc != WKV6_OK) return rc;
+    if (!x || !mix_x || !x_mix) return WKV6_ERR_ARG;
+    return finish(wkv6::shift_mix_x((hipStream_t)stream, B, T, C, x, mix_x, x_mix));
+}
+
+int wkv6_shift_mix_five(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t R,
+                        const void *x, const void *h, const void *w2t, const float *bias,
+                        void *xr, void *xk, void *xv, void *xw, void *xg) {
+    const int rc = check_mix(dtype, B, T, C, R);
+    if (rc != WKV6_OK) return rc;
+    if (!x || !h || !w2t || !bias || !xr || !xk || !xv || !xw || !xg) return WKV6_ERR_ARG;
+    void *const out[5] = {xr, xk, xv, xw, xg};
+    return finish(wkv6::shift_mix_five((hipStream_t)stream, B, T, C, R, x, h, w2t, bias, out));
+}
+
+int wkv6_shift_mix_five_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t R,
+                                 const void *x, const void *h, const void *w2t, const float *bias,
+                                 const void *gxr, const void *gxk, const void *gxv, const void *gxw, const void *gxg,
+                                 void *gcoef, void *gp, void *gxx) {
+    const int rc = check_mix(dtype, B, T, C, R);
+    if (rc != WKV6_OK) return rc;
+    if (!x || !h || !w2t || !bias || !gxr || !gxk || !gxv || !gxw || !gxg || !gcoef || !gp || !gxx) return WKV6_ERR_ARG;
+    const void *const gout[5] = {gxr, gxk, gxv, gxw, gxg};
+    return finish(wkv6::shift_mix_five_backward((hipStream_t)stream, B, T, C, R, x, h, w2t, bias, gout, gcoef, gp, gxx));
+}
+
+int wkv6_shift_mix_x_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C,
+                              const void *x, const float *mix_x, const void *gp, const void *gxx, const void *gxm,
+                              void *gx, float *gmix_x) {
+    const int rc = check_mix(dtype, B, T, C, 32);
+    if (rc != WKV6_OK) return rc;
+    if (!x || !mix_x || !gp || !gxx || !gxm || !gx || !gmix_x) return WKV6_ERR_ARG;
+    return finish(wkv6::shift_mix_x_backward((hipStream_t)stream, B, T, C, x, mix_x, gp, gxx, gxm, gx, gmix_x));
+}
+
 // Size of the part of the saved block that the kernels of one pass use (chunk states, arrival
 // counters; sized so that the guarded per-timestep pass of the backward can use the same buffer).
 static size_t saved_base_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {

@@ -123,6 +123,19 @@ hipError_t gn_gate_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
                             const void *gout, const void *y, const float *stats, const void *gate,
                             const float *scale, const float *offset, void *gy, void *ggate, float *gscale, float *goffset);
 
+// input side of the time-mix layer (wkv6_mix.hip): token shift and the five low-rank mixers, bf16 tensors,
+// rank R in {32, 64}.  h (B,T,5,R), w2t (5,C,R), bias (5,C) and mix_x (C) fp32.
+bool shift_mix_supported(int64_t C, int64_t R);
+hipError_t shift_mix_x(hipStream_t st, int64_t B, int64_t T, int64_t C, const void *x, const float *mix_x, void *x_mix);
+hipError_t shift_mix_five(hipStream_t st, int64_t B, int64_t T, int64_t C, int64_t R, const void *x, const void *h,
+                          const void *w2t, const float *bias, void *const out[5]);
+// gcoef (5,B,T,C), gp and gxx (B,T,C)
+hipError_t shift_mix_five_backward(hipStream_t st, int64_t B, int64_t T, int64_t C, int64_t R, const void *x, const void *h,
+                                   const void *w2t, const float *bias, const void *const gout[5], void *gcoef, void *gp, void *gxx);
+// gx (B,T,C), gmix_x (C) fp32, zeroed inside
+hipError_t shift_mix_x_backward(hipStream_t st, int64_t B, int64_t T, int64_t C, const void *x, const float *mix_x,
+                                const void *gp, const void *gxx, const void *gxm, void *gx, float *gmix_x);
+
 size_t chunk_backward_workspace_bytes(int64_t B, int64_t T, int64_t H);
 // bytes of a forward -> backward hand-over buffer: the workspace plus one arrival counter per head
 // (zeroed by the saving forward, used by the backward's fused batch sum of gu)

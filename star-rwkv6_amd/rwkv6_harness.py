@@ -83,14 +83,24 @@ class TimeMix(nn.Module):
         with torch.no_grad():
             self.dense_w.dense_b.bias.uniform_(-6.0, 1.0)
 
-    def forward(self, x, mask=None):
+    def _mixed_inputs(self, x):
+        """xr, xk, xv, xw, xg of rwkv6_model.py:134-145."""
+        mixers = (self.dense_xr, self.dense_xk, self.dense_xv, self.dense_xw, self.dense_xg)
+        fused = getattr(self.rwkv_kernel, "shift_mix", None)
+        if fused is not None and x.is_cuda and torch.is_autocast_enabled() and torch.get_autocast_gpu_dtype() == torch.bfloat16:
+            xb = x.to(torch.bfloat16).contiguous()
+            if self.rwkv_kernel.shift_mix_supported(xb, mixers[0].dense_a.out_features):
+                # token shift, x_mix and the five rank-R expansions in the operator library's kernels
+                return fused(xb, self.time_mix_x,
+                             torch.cat([m.dense_a.weight for m in mixers]),
+                             torch.stack([m.dense_b.weight for m in mixers]),
+                             torch.stack([m.dense_b.bias for m in mixers]))
         x_shift = time_shift(x)
         x_mix = x + x_shift * self.time_mix_x.to(x.dtype)
-        xr = x + x_shift * self.dense_xr(x_mix)
-        xk = x + x_shift * self.dense_xk(x_mix)
-        xv = x + x_shift * self.dense_xv(x_mix)
-        xw = x + x_shift * self.dense_xw(x_mix)
-        xg = x + x_shift * self.dense_xg(x_mix)
+        return tuple(x + x_shift * m(x_mix) for m in mixers)
+
+    def forward(self, x, mask=None):
+        xr, xk, xv, xw, xg = self._mixed_inputs(x)
         r, k, v, w, g = self.dense_r(xr), self.dense_k(xk), self.dense_v(xv), self.dense_w(xw), F.silu(self.dense_g(xg))
         if mask is not None:
             # Padded tokens neither write to the state nor decay it.  rwkv6_model.py:149-152 sets

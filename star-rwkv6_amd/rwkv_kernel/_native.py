@@ -29,6 +29,11 @@ SIGNATURES = {
     "wkv6_forward_gn_gate_save_supported": (_int, [_int] + [_i64] * 4),
     "wkv6_forward_gn_gate_save": (_int, [_p, _int] + [_i64] * 4 + [_p] * 8 + [ctypes.c_float] + [_p] * 4 + [_sz]),
     "wkv6_gn_gate_backward": (_int, [_p, _int] + [_i64] * 4 + [_p] * 10),
+    "wkv6_shift_mix_supported": (_int, [_int, _i64, _i64]),
+    "wkv6_shift_mix_x": (_int, [_p, _int] + [_i64] * 3 + [_p] * 3),
+    "wkv6_shift_mix_five": (_int, [_p, _int] + [_i64] * 4 + [_p] * 9),
+    "wkv6_shift_mix_five_backward": (_int, [_p, _int] + [_i64] * 4 + [_p] * 12),
+    "wkv6_shift_mix_x_backward": (_int, [_p, _int] + [_i64] * 3 + [_p] * 7),
     "wkv6_backward": (_int, [_p, _int] + [_i64] * 4 + [_p] * 11 + [_p, _sz]),
     "wkv6_backward_workspace_bytes": (_sz, [_int] + [_i64] * 4),
     "wkv6_backward_static": (_int, [_p, _int] + [_i64] * 4 + [_p] * 11),

@@ -175,6 +175,68 @@ class _WKV6GnGate(torch.autograd.Function):
                     gsc.reshape(s_shape).to(s_dt), gof.reshape(o_shape).to(o_dt), None)
 
 
+class _ShiftMix(torch.autograd.Function):
+    """The layer's input side (rwkv6_model.py:134-146) with gradients, bf16: x -> (xr, xk, xv, xw, xg).
+    Token shift and x_mix in one kernel (wkv6_shift_mix_x), the GEMM against the stacked first mixer
+    weights and its tanh in torch, then one kernel that expands the rank-R coefficients on the matrix
+    cores and writes the five outputs (wkv6_shift_mix_five).  Backward: wkv6_shift_mix_five_backward,
+    the reductions over channels and over tokens as batched GEMMs, wkv6_shift_mix_x_backward."""
+
+    @staticmethod
+    def forward(ctx, x, mix_x, a, w2t, bias):
+        lib = _native.load()
+        with torch.no_grad():
+            B, T, C = x.shape
+            R = w2t.shape[2]
+            code = _DTYPE_CODE[x.dtype]
+            mx = mix_x.detach().to(torch.float32).contiguous()
+            a16 = a.detach().to(x.dtype).contiguous()
+            w16 = w2t.detach().to(x.dtype).contiguous()
+            b32 = bias.detach().to(torch.float32).contiguous()
+            x_mix = torch.empty_like(x)
+            outs = _staggered(5, (B, T, C), x.dtype, x.device, first=1)
+            with torch.cuda.device(x.device):
+                _native.check(lib.wkv6_shift_mix_x(_stream(), code, B, T, C, _ptr(x), _ptr(mx), _ptr(x_mix)))
+                h = torch.tanh(x_mix.view(B * T, C) @ a16.t())            # (B*T, 5R)
+                _native.check(lib.wkv6_shift_mix_five(_stream(), code, B, T, C, R, _ptr(x), _ptr(h), _ptr(w16), _ptr(b32),
+                                                      *[_ptr(o) for o in outs]))
+            ctx.save_for_backward(x, x_mix, h, mx, a16, w16, b32)
+            ctx.param_dtypes = (mix_x.dtype, a.dtype, w2t.dtype, bias.dtype)
+            return tuple(outs)
+
+    @staticmethod
+    def backward(ctx, *gouts):
+        lib = _native.load()
+        with torch.no_grad():
+            x, x_mix, h, mx, a16, w16, b32 = ctx.saved_tensors
+            B, T, C = x.shape
+            n, R = B * T, w16.shape[2]
+            code = _DTYPE_CODE[x.dtype]
+            gouts = [torch.zeros_like(x) if g is None else g.to(x.dtype).contiguous() for g in gouts]
+            gcoef = torch.empty((5, n, C), device=x.device, dtype=x.dtype)
+            gp, gxx, gx = _staggered(3, (B, T, C), x.dtype, x.device, first=1)
+            gmx = torch.empty(C, device=x.device, dtype=torch.float32)
+            with torch.cuda.device(x.device):
+                _native.check(lib.wkv6_shift_mix_five_backward(
+                    _stream(), code, B, T, C, R, _ptr(x), _ptr(h), _ptr(w16), _ptr(b32), *[_ptr(g) for g in gouts],
+                    _ptr(gcoef), _ptr(gp), _ptr(gxx)))
+                gh = torch.bmm(gcoef, w16)                                   # (5, n, R): summed over channels
+                # sums over tokens: gcoef^T h for the weights and, through eight more columns of which
+                # the first holds ones, gcoef^T 1 for the biases -- one pass over gcoef for both
+                h3 = torch.zeros((5, n, R + 8), device=x.device, dtype=x.dtype)
+                h3[:, :, :R] = h.view(n, 5, R).permute(1, 0, 2)
+                h3[:, :, R] = 1
+                gwb = torch.bmm(gcoef.transpose(1, 2), h3)                   # (5, C, R + 8)
+                gw2t, gbias = gwb[:, :, :R], gwb[:, :, R]
+                gpre = (gh.permute(1, 0, 2).reshape(n, 5 * R).float() * (1.0 - h.float() ** 2)).to(x.dtype)
+                ga = gpre.t() @ x_mix.view(n, C)                             # (5R, C)
+                gxm = (gpre @ a16).view(B, T, C)
+                _native.check(lib.wkv6_shift_mix_x_backward(_stream(), code, B, T, C, _ptr(x), _ptr(mx), _ptr(gp), _ptr(gxx),
+                                                            _ptr(gxm), _ptr(gx), _ptr(gmx)))
+            dm, da, dw, db = ctx.param_dtypes
+            return gx, gmx.to(dm), ga.to(da), gw2t.to(dw), gbias.to(db)
+
+
 def _forward_with_state(B, T, C, H, state_map, r, k, v, w, u, init_state, algo=_native.ALGO_AUTO, state_dtype=None):
     """Stateful forward, no gradient (rwkv_kernel/torch_rwkv_kernel.py:76-95)."""
     lib = _native.load()
@@ -336,6 +398,26 @@ class RWKVKernelOperator:
             return _forward_with_state(B, T, C, H, state_map, r, k, v, w, u, init_state, self.algo)
         o = _WKV6.apply(B, T, C, H, r, k, v, w, u, self.algo)
         return o, None
+
+    def shift_mix_supported(self, x, decomposer_size):
+        """Whether ``shift_mix`` takes this tensor (bf16 on the GPU, rank 32 or 64)."""
+        if not (x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 3):
+            return False
+        return bool(_native.load().wkv6_shift_mix_supported(_DTYPE_CODE[x.dtype], x.shape[2], decomposer_size))
+
+    def shift_mix(self, x, mix_x, a, w2t, bias):
+        """The layer's input side, rwkv6_model.py:134-146: from the layer input ``x`` (B,T,C) to the
+        inputs ``(xr, xk, xv, xw, xg)`` of the projections that produce r, k, v, w and the gate:
+        ``x_s = x + xx * (tanh((x + xx * mix_x) a_s^T) w2t_s^T + bias_s)`` with ``xx`` the previous token
+        minus the token.  ``a`` (5R, C): the five mixers' first weights stacked in the order r, k, v, w, g;
+        ``w2t`` (5, C, R) and ``bias`` (5, C): their second weights and biases.  Differentiable in all
+        five arguments.  Not part of the reference's operator."""
+        B, T, C = x.shape
+        assert x.is_contiguous() and mix_x.numel() == C
+        R = w2t.shape[2]
+        assert a.shape == (5 * R, C) and w2t.shape == (5, C, R) and bias.shape == (5, C)
+        assert self.shift_mix_supported(x, R), "shift_mix takes bf16 tensors on the GPU with rank 32 or 64"
+        return _ShiftMix.apply(x, mix_x.reshape(C), a, w2t, bias)
 
     def forward_gn_gate(self, r, k, v, w, u, gate, gn_scale, gn_offset, epsilon=64e-5,
                         return_state=False, init_state=None, state_map=None):

@@ -147,6 +147,52 @@ def test_inference_forward_uses_the_fused_output_stage():
 
 
 @pytest.mark.gpu
+def test_training_step_uses_the_fused_input_side():
+    """With mixers of rank 32 (the rank of configuration 4) the time-mix layer under bf16 autocast takes
+    its five mixed inputs from the library's shift-mix kernels: loss and gradients of one step against
+    the fp32 python-loop model on the CPU, and against the same GPU model with that path switched off."""
+    from rwkv_kernel import RWKVKernelOperator
+    T = 128
+    cfg = dict(TOY, decomposer_size=32)
+    torch.manual_seed(8)
+    ref = hz.RWKV6(OPSKernelOperator(64, T), **cfg)
+    dev = torch.device("cuda:0")
+    gpu = hz.RWKV6(RWKVKernelOperator(64, T), **cfg).to(dev)
+    gpu.load_state_dict(ref.state_dict())
+    torch.manual_seed(9)
+    ids = torch.randint(0, TOY["vocabulary_size"], (2, T + 1))
+    calls = []
+    op = gpu.blocks[0].time_mix.rwkv_kernel
+    inner = op.shift_mix
+    op.shift_mix = lambda *a, **kw: (calls.append(1), inner(*a, **kw))[1]
+
+    def loss_and_grads(model, ids, autocast):
+        model.zero_grad(set_to_none=True)
+        with torch.autocast(ids.device.type, dtype=autocast, enabled=autocast is not None):
+            logits = model(ids[:, :-1])
+        loss = F.cross_entropy(logits.float().reshape(-1, logits.shape[-1]), ids[:, 1:].reshape(-1))
+        loss.backward()
+        return float(loss.detach()), {n: p.grad.detach().float().cpu() for n, p in model.named_parameters()}
+
+    l_ref, g_ref = loss_and_grads(ref, ids, None)
+    l_gpu, g_gpu = loss_and_grads(gpu, ids.to(dev), torch.bfloat16)
+    assert len(calls) == TOY["num_layers"]
+    op.shift_mix = None
+    l_off, g_off = loss_and_grads(gpu, ids.to(dev), torch.bfloat16)
+    assert len(calls) == TOY["num_layers"]
+    assert abs(l_gpu - l_ref) <= 3e-2 * max(1.0, abs(l_ref)), (l_gpu, l_ref)
+
+    def worst(ga, gb):
+        return max(float((ga[n] - gb[n]).abs().max()) / (float(gb[n].abs().max()) + 1e-12) for n in gb)
+
+    w_fused, w_off = worst(g_gpu, g_ref), worst(g_off, g_ref)
+    print("worst relative gradient error vs fp32: fused input side %.3e, torch ops %.3e" % (w_fused, w_off))
+    assert w_fused <= 8e-2, w_fused
+    mix_names = [n for n in g_ref if "dense_x" in n or "time_mix_x" in n]
+    assert mix_names and all(torch.isfinite(g_gpu[n]).all() and float(g_gpu[n].abs().max()) > 0 for n in mix_names)
+
+
+@pytest.mark.gpu
 def test_config4_full_size_train_step(oracle):
     """Configuration 4 at its real size through the torch binding: 24 layers, d_model 2048, 32 heads
     of 64, FFN 7168, vocabulary 65536 (rwkv6_model.py:261-276), 8 x 1024 uniform random token ids,

@@ -216,6 +216,46 @@ def test_group_norm_gate_is_a_per_head_layer_norm(oracle):
     assert np.abs(out - 0.25).max() < 1e-12
 
 
+def test_shift_mix_special_cases_and_layer_modules(oracle):
+    # the restated input side of the layer: cases whose answer is known without the formula, then the
+    # same computation assembled from torch's own Linear / pad modules with separately held weights
+    import torch
+    import torch.nn.functional as F
+
+    g = torch.Generator().manual_seed(11)
+    B, T, C, R = 2, 6, 64, 4
+    x = torch.randn(B, T, C, generator=g, dtype=torch.float64)
+    mix_x = torch.rand(C, generator=g, dtype=torch.float64)
+    a = torch.randn(5 * R, C, generator=g, dtype=torch.float64) * 0.2
+    w2t = torch.randn(5, C, R, generator=g, dtype=torch.float64)
+    bias = torch.randn(5, C, generator=g, dtype=torch.float64)
+    zero_w, zero_b, ones_b = torch.zeros_like(w2t), torch.zeros_like(bias), torch.ones_like(bias)
+    # coefficient 0: every output is x itself; coefficient 1: every output is the PREVIOUS token
+    # (zero for the first) -- a shift in the wrong direction or a sign error in xx fails here
+    _, _, outs = oracle.shift_mix_np(x.numpy(), mix_x.numpy(), a.numpy(), zero_w.numpy(), zero_b.numpy())
+    assert all(np.array_equal(o, x.numpy()) for o in outs)
+    _, _, outs = oracle.shift_mix_np(x.numpy(), mix_x.numpy(), a.numpy(), zero_w.numpy(), ones_b.numpy())
+    prev = torch.cat([torch.zeros(B, 1, C, dtype=torch.float64), x[:, :-1]], 1).numpy()
+    assert all(np.abs(o - prev).max() < 1e-14 for o in outs)
+    # mix_x = 1: x_mix is the previous token as well
+    xm, _, _ = oracle.shift_mix_np(x.numpy(), np.ones(C), a.numpy(), w2t.numpy(), bias.numpy())
+    assert np.abs(xm - prev).max() < 1e-14
+    # each mixer as two Linear modules on a padded-and-sliced shift; mixer s only sees its own weights
+    xm, h, outs = oracle.shift_mix_np(x.numpy(), mix_x.numpy(), a.numpy(), w2t.numpy(), bias.numpy())
+    xs = F.pad(x, (0, 0, 1, 0))[:, :-1] - x
+    x_mix = x + xs * mix_x
+    assert np.abs(xm - x_mix.numpy()).max() < 1e-13
+    for s in range(5):
+        first = torch.nn.Linear(C, R, bias=False, dtype=torch.float64)
+        second = torch.nn.Linear(R, C, bias=True, dtype=torch.float64)
+        with torch.no_grad():
+            first.weight.copy_(a[s * R:(s + 1) * R]); second.weight.copy_(w2t[s]); second.bias.copy_(bias[s])
+            hs = torch.tanh(first(x_mix))
+            want = x + xs * second(hs)
+        assert np.abs(h[:, :, s] - hs.numpy()).max() < 1e-13
+        assert np.abs(outs[s] - want.numpy()).max() < 1e-12
+
+
 def test_state_gradients_vs_autograd(oracle):
     # gradient into the initial state and from the final state: the adjoint-form C oracle against
     # torch.autograd through the python loop (float64), for  L = sum(y*gy) + sum(S_T*gS)
