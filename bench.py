@@ -49,7 +49,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--preheat-ms", type=float, default=600.0,
                     help="untimed run of the same step before --warmup, so that the clocks are up whatever --warmup is")
-    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c4", "c5"])
+    ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c4", "c5", "mix"])
     ap.add_argument("--algo", default="auto", choices=["auto", "scan", "chunk"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--plain-pair", action="store_true", help="time forward()+backward() without saved states")
@@ -233,6 +233,64 @@ def bench_model_step(a):
         "loss_first_last": [losses[0], losses[-1]], "dtype": "bf16", "data": "synthetic"}))
 
 
+def bench_shift_mix(a):
+    """The input side of the time-mix layer at the layer shape of configuration 2 (B=8, T=1024, C=2048,
+    mixers of rank 32): the four kernels through the C ABI with pre-allocated buffers, each timed on
+    its own with events on torch's current stream.  Prints its own JSON line: microseconds per kernel
+    and the rate at which each moves its algorithmic bytes (the (B,T,C) tensors it must read and write)."""
+    import torch
+    from rwkv_kernel import _native
+
+    lib = _native.load()
+    B, T, C, R = 8, 1024, 2048, 32
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(a.seed)
+    unit = B * T * C * 2                                   # bytes of one (B,T,C) bf16 tensor
+    # all (B,T,C) tensors out of one pool, each base --stagger bytes further on than the one before
+    pitch = unit + a.stagger
+    pool = torch.empty(22 * pitch, dtype=torch.uint8, device=dev)
+    slot = lambda i: pool[i * pitch: i * pitch + unit].view(torch.bfloat16).view(B, T, C)
+    fill = lambda i: slot(i).copy_(torch.randn(B, T, C, generator=g).to(torch.bfloat16))
+    x, gxm = fill(0), fill(1)
+    h = torch.tanh(torch.randn(B, T, 5, R, generator=g)).to(torch.bfloat16).to(dev)
+    w2t = (torch.randn(5, C, R, generator=g) / R ** 0.5).to(torch.bfloat16).to(dev)
+    bias, mix = torch.rand(5, C, generator=g).to(dev), torch.rand(C, generator=g).to(dev)
+    outs, gouts = [slot(2 + i) for i in range(5)], [fill(7 + i) for i in range(5)]
+    x_mix, gp, gxx, gx = (slot(12 + i) for i in range(4))
+    gcoef, plane = slot(16), pitch // 2                    # five slots in a row
+    gmix = torch.empty(C, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    P = lambda t: t.data_ptr()
+    calls = {   # name: (call, (B,T,C) tensors read + written)
+        "shift_mix_x": (lambda: lib.wkv6_shift_mix_x(st, _native.BF16, B, T, C, P(x), P(mix), P(x_mix)), 2),
+        "shift_mix_five": (lambda: lib.wkv6_shift_mix_five(st, _native.BF16, B, T, C, R, P(x), P(h), P(w2t), P(bias),
+                                                           *[P(o) for o in outs]), 6),
+        "shift_mix_five_backward": (lambda: lib.wkv6_shift_mix_five_backward(
+            st, _native.BF16, B, T, C, R, P(x), P(h), P(w2t), P(bias), *[P(o) for o in gouts], P(gcoef), plane, P(gp), P(gxx)), 13),
+        "shift_mix_x_backward": (lambda: lib.wkv6_shift_mix_x_backward(st, _native.BF16, B, T, C, P(x), P(mix), P(gp), P(gxx),
+                                                                       P(gxm), P(gx), P(gmix)), 5),
+    }
+    res = {}
+    for name, (call, units) in calls.items():
+        for _ in range(a.warmup):
+            _native.check(call())
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(a.steps):
+            call()
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / a.steps * 1e3
+        res[name] = {"us": us, "algorithmic_bytes": units * unit, "GB/s": units * unit / us * 1e-3,
+                     "frac_of_hbm_peak": units * unit / us * 1e-3 / HBM_PEAK_GBS}
+    total = sum(v["us"] for v in res.values())
+    print(json.dumps({
+        "metric": "time-mix input side (token shift + five low-rank mixers), forward + backward kernels, Mtokens/s",
+        "n_gpus": 1, "value": B * T / total, "unit": "Mtokens/s", "us_all_four_kernels": total, "steps": a.steps, "warmup": a.warmup,
+        "config": {"workload": "mix: B=8 T=1024 C=2048 rank 32, bf16", "allocation": "one pool, tensor bases %d B apart mod 2 MiB" % a.stagger}, "kernels": res, "dtype": "bf16", "data": "synthetic"}))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -249,6 +307,9 @@ def main():
     if a.workload == "c4":
         torch.cuda.set_device(0)
         return bench_model_step(a)
+    if a.workload == "mix":
+        torch.cuda.set_device(0)
+        return bench_shift_mix(a)
     lib = _native.load()
     B, T, H, dt_name = WORKLOADS[a.workload]
     N = 64

@@ -162,7 +162,8 @@ int wkv6_gn_gate_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t
  *
  * Backward, in the order the chain rule needs it:
  *   wkv6_shift_mix_five_backward: from the gradients gx_s of the five outputs writes
- *       gcoef (5,B,T,C) = gx_s * xx  -- the caller's GEMMs turn it into the gradients of h
+ *       gcoef = gx_s * xx, five (B,T,C) planes gcoef_stride elements apart (at least B*T*C, a
+ *       multiple of 8)  -- the caller's GEMMs turn it into the gradients of h
  *       (gcoef_s W_s), of W_s (gcoef_s^T h_s) and of bias_s (sum over tokens) --,
  *       gxx = sum_s gx_s * coef_s and gp = sum_s gx_s - gxx  (both (B,T,C)).
  *   (caller) gh -> through tanh and A -> gxm = dL/dx_mix (B,T,C)
@@ -178,7 +179,7 @@ int wkv6_shift_mix_five(void *stream, int dtype, int64_t B, int64_t T, int64_t C
 int wkv6_shift_mix_five_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t R,
                                  const void *x, const void *h, const void *w2t, const float *bias,
                                  const void *gxr, const void *gxk, const void *gxv, const void *gxw, const void *gxg,
-                                 void *gcoef, void *gp, void *gxx);
+                                 void *gcoef, int64_t gcoef_stride, void *gp, void *gxx);
 int wkv6_shift_mix_x_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C,
                               const void *x, const float *mix_x, const void *gp, const void *gxx, const void *gxm,
                               void *gx, float *gmix_x);

@@ -240,12 +240,13 @@ int wkv6_shift_mix_five(void *stream, int dtype, int64_t B, int64_t T, int64_t C
 int wkv6_shift_mix_five_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t R,
                                  const void *x, const void *h, const void *w2t, const float *bias,
                                  const void *gxr, const void *gxk, const void *gxv, const void *gxw, const void *gxg,
-                                 void *gcoef, void *gp, void *gxx) {
+                                 void *gcoef, int64_t gcoef_stride, void *gp, void *gxx) {
     const int rc = check_mix(dtype, B, T, C, R);
     if (rc != WKV6_OK) return rc;
     if (!x || !h || !w2t || !bias || !gxr || !gxk || !gxv || !gxw || !gxg || !gcoef || !gp || !gxx) return WKV6_ERR_ARG;
+    if (gcoef_stride < B * T * C || gcoef_stride % 8 != 0) return WKV6_ERR_ARG;
     const void *const gout[5] = {gxr, gxk, gxv, gxw, gxg};
-    return finish(wkv6::shift_mix_five_backward((hipStream_t)stream, B, T, C, R, x, h, w2t, bias, gout, gcoef, gp, gxx));
+    return finish(wkv6::shift_mix_five_backward((hipStream_t)stream, B, T, C, R, x, h, w2t, bias, gout, gcoef, gcoef_stride, gp, gxx));
 }
 
 int wkv6_shift_mix_x_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C,

@@ -129,9 +129,10 @@ bool shift_mix_supported(int64_t C, int64_t R);
 hipError_t shift_mix_x(hipStream_t st, int64_t B, int64_t T, int64_t C, const void *x, const float *mix_x, void *x_mix);
 hipError_t shift_mix_five(hipStream_t st, int64_t B, int64_t T, int64_t C, int64_t R, const void *x, const void *h,
                           const void *w2t, const float *bias, void *const out[5]);
-// gcoef (5,B,T,C), gp and gxx (B,T,C)
+// gcoef: five (B,T,C) planes gcoef_stride elements apart; gp and gxx (B,T,C)
 hipError_t shift_mix_five_backward(hipStream_t st, int64_t B, int64_t T, int64_t C, int64_t R, const void *x, const void *h,
-                                   const void *w2t, const float *bias, const void *const gout[5], void *gcoef, void *gp, void *gxx);
+                                   const void *w2t, const float *bias, const void *const gout[5], void *gcoef, int64_t gcoef_stride,
+                                   void *gp, void *gxx);
 // gx (B,T,C), gmix_x (C) fp32, zeroed inside
 hipError_t shift_mix_x_backward(hipStream_t st, int64_t B, int64_t T, int64_t C, const void *x, const float *mix_x,
                                 const void *gp, const void *gxx, const void *gxm, void *gx, float *gmix_x);

@@ -32,7 +32,7 @@ SIGNATURES = {
     "wkv6_shift_mix_supported": (_int, [_int, _i64, _i64]),
     "wkv6_shift_mix_x": (_int, [_p, _int] + [_i64] * 3 + [_p] * 3),
     "wkv6_shift_mix_five": (_int, [_p, _int] + [_i64] * 4 + [_p] * 9),
-    "wkv6_shift_mix_five_backward": (_int, [_p, _int] + [_i64] * 4 + [_p] * 12),
+    "wkv6_shift_mix_five_backward": (_int, [_p, _int] + [_i64] * 4 + [_p] * 10 + [_i64, _p, _p]),
     "wkv6_shift_mix_x_backward": (_int, [_p, _int] + [_i64] * 3 + [_p] * 7),
     "wkv6_backward": (_int, [_p, _int] + [_i64] * 4 + [_p] * 11 + [_p, _sz]),
     "wkv6_backward_workspace_bytes": (_sz, [_int] + [_i64] * 4),

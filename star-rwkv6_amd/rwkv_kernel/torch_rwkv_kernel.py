@@ -213,13 +213,15 @@ class _ShiftMix(torch.autograd.Function):
             n, R = B * T, w16.shape[2]
             code = _DTYPE_CODE[x.dtype]
             gouts = [torch.zeros_like(x) if g is None else g.to(x.dtype).contiguous() for g in gouts]
-            gcoef = torch.empty((5, n, C), device=x.device, dtype=x.dtype)
+            # the five planes of gcoef 256 bytes further apart than they are long (see _staggered)
+            plane = n * C + _STAGGER // 2
+            gcoef = torch.empty(5 * plane, device=x.device, dtype=x.dtype).as_strided((5, n, C), (plane, C, 1))
             gp, gxx, gx = _staggered(3, (B, T, C), x.dtype, x.device, first=1)
             gmx = torch.empty(C, device=x.device, dtype=torch.float32)
             with torch.cuda.device(x.device):
                 _native.check(lib.wkv6_shift_mix_five_backward(
                     _stream(), code, B, T, C, R, _ptr(x), _ptr(h), _ptr(w16), _ptr(b32), *[_ptr(g) for g in gouts],
-                    _ptr(gcoef), _ptr(gp), _ptr(gxx)))
+                    _ptr(gcoef), plane, _ptr(gp), _ptr(gxx)))
                 gh = torch.bmm(gcoef, w16)                                   # (5, n, R): summed over channels
                 # sums over tokens: gcoef^T h for the weights and, through eight more columns of which
                 # the first holds ones, gcoef^T 1 for the biases -- one pass over gcoef for both

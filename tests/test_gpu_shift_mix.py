@@ -93,13 +93,14 @@ def test_backward_kernels(lib, B, T, C, R):
     want_gxx = xx_leaf.grad.numpy()
     want_gcoef = np.stack([c.grad.numpy() for c in coef_leaf])
     want_gp = sum(to_np(go) for go in gouts) - want_gxx
-    gcoef = torch.full((5, B * T, C), float("nan"), dtype=BF16, device="cuda")
+    plane = B * T * C + 128 * (T % 2)        # planes back to back, or 256 bytes apart
+    gcoef = torch.full((5 * plane,), float("nan"), dtype=BF16, device="cuda").as_strided((5, B * T, C), (plane, C, 1))
     gp, gxx = torch.empty_like(dev["x"]), torch.empty_like(dev["x"])
     _native.check(lib.wkv6_shift_mix_five_backward(
         _stream(), _native.BF16, B, T, C, R, dev["x"].data_ptr(), h.data_ptr(), dev["w2t"].data_ptr(), dev["bias"].data_ptr(),
-        *[go.data_ptr() for go in gouts], gcoef.data_ptr(), gp.data_ptr(), gxx.data_ptr()))
+        *[go.data_ptr() for go in gouts], gcoef.data_ptr(), plane, gp.data_ptr(), gxx.data_ptr()))
     torch.cuda.synchronize()
-    check_close("gcoef", gcoef.view(5, B, T, C), want_gcoef, BF16, is_grad=True)
+    check_close("gcoef", gcoef.reshape(5, B, T, C), want_gcoef, BF16, is_grad=True)
     check_close("gxx", gxx, want_gxx, BF16, is_grad=True)
     check_close("gp", gp, want_gp, BF16, is_grad=True)
     # second kernel: all of x's gradient, with gp and gxx as the first kernel wrote them (bf16)
