@@ -87,7 +87,7 @@ class TimeMix(nn.Module):
         """xr, xk, xv, xw, xg of rwkv6_model.py:134-145."""
         mixers = (self.dense_xr, self.dense_xk, self.dense_xv, self.dense_xw, self.dense_xg)
         fused = getattr(self.rwkv_kernel, "shift_mix", None)
-        if fused is not None and x.is_cuda and torch.is_autocast_enabled() and torch.get_autocast_gpu_dtype() == torch.bfloat16:
+        if fused is not None and x.is_cuda and torch.is_autocast_enabled('cuda') and torch.get_autocast_dtype('cuda') == torch.bfloat16:
             xb = x.to(torch.bfloat16).contiguous()
             if self.rwkv_kernel.shift_mix_supported(xb, mixers[0].dense_a.out_features):
                 # token shift, x_mix and the five rank-R expansions in the operator library's kernels
