@@ -22,21 +22,23 @@ __device__ __forceinline__ void lds_store8(float *p, const float (&f)[8]) {
 }
 
 // ------------------------------------------------------------------------------------------
-// Forward.  wave q owns key rows j in [16q,16q+16); lane i owns value column i.
+// Forward.  wave q of NW owns key rows j in [64/NW q, 64/NW (q+1)); lane i owns value column i.
 //   y_t[i]  = v_t[i] * sum_j r_t[j] u[j] k_t[j]  +  sum_j r_t[j] S[j][i]
 //   S[j][i] = S[j][i] * d_t[j] + k_t[j] v_t[i]
 // ------------------------------------------------------------------------------------------
-struct alignas(16) ScanFwdLds {
+template <int NW> struct alignas(16) ScanFwdLdsT {
     float s_r[TC][kN], s_k[TC][kN], s_d[TC][kN], s_v[TC][kN];
-    float s_part[4][TC][kN];
+    float s_part[NW][TC][kN];
     float s_ruk[TC];
     float s_u[kN];
 };
+typedef ScanFwdLdsT<4> ScanFwdLds;
 
-// Work of one (b, h) pair by threads 0..255 of the workgroup; further threads only keep the
-// barriers company (the chunked kernels call this with 512 threads).
-template <typename Tin, typename Tout, typename Ts>
-__device__ __forceinline__ void scan_fwd_body(ScanFwdLds &L, int b, int h, int T, int H,
+// Work of one (b, h) pair by the first NW waves of the workgroup (wave q owns key rows
+// [64/NW * q, 64/NW * (q+1)); the first 256 threads also stage the tiles and fold the partials);
+// further threads only keep the barriers company (the chunked kernels call this with NW = 4 and 768 threads).
+template <typename Tin, typename Tout, typename Ts, int NW = 4>
+__device__ __forceinline__ void scan_fwd_body(ScanFwdLdsT<NW> &L, int b, int h, int T, int H,
         const Tin *__restrict__ r, const Tin *__restrict__ k, const Tin *__restrict__ v,
         const Tin *__restrict__ w, const Tin *__restrict__ u,
         const Ts *__restrict__ s0, const int64_t *__restrict__ map,
@@ -45,7 +47,8 @@ __device__ __forceinline__ void scan_fwd_body(ScanFwdLds &L, int b, int h, int T
     auto &s_r = L.s_r; auto &s_k = L.s_k; auto &s_d = L.s_d; auto &s_v = L.s_v;
     auto &s_part = L.s_part; auto &s_ruk = L.s_ruk; auto &s_u = L.s_u;
     const int tid = threadIdx.x, lane = tid & 63, q = tid >> 6;
-    if (tid >= 256) {   // same barrier sequence as below, no work
+    constexpr int RW = kN / NW;   // key rows per wave
+    if (tid >= 64 * NW) {   // same barrier sequence as below, no work
         __syncthreads();
         for (int t0 = 0; t0 < T; t0 += TC) { __syncthreads(); __syncthreads(); }
         return;
@@ -59,20 +62,21 @@ __device__ __forceinline__ void scan_fwd_body(ScanFwdLds &L, int b, int h, int T
     const Tin *pb = (half == 0 ? k : w) + base + sc;
     Raw8<Tin> ra, rb;
 
-    float s[16];
+    float s[RW];
     if (s0 != nullptr) {
         const int64_t row = map ? map[b] : (int64_t)b;
-        const Ts *p = s0 + ((row * H + h) * kN + 16 * q) * kN + lane;
+        const Ts *p = s0 + ((row * H + h) * kN + RW * q) * kN + lane;
 #pragma unroll
-        for (int jj = 0; jj < 16; ++jj) s[jj] = load1(p + jj * kN);
+        for (int jj = 0; jj < RW; ++jj) s[jj] = load1(p + jj * kN);
     } else {
 #pragma unroll
-        for (int jj = 0; jj < 16; ++jj) s[jj] = 0.f;
+        for (int jj = 0; jj < RW; ++jj) s[jj] = 0.f;
     }
     if (tid < kN) s_u[tid] = load1(u + h * kN + tid);
 
     auto prefetch = [&](int t0) {
         const int t = t0 + st;
+        if (tid >= 256) return;
         if (t < T) { const int64_t row = reverse ? T - 1 - t : t; ra.load(pa + row * C); rb.load(pb + row * C); }
         else { ra.zero(); rb.zero(); }
     };
@@ -80,7 +84,7 @@ __device__ __forceinline__ void scan_fwd_body(ScanFwdLds &L, int b, int h, int T
     __syncthreads();
 
     for (int t0 = 0; t0 < T; t0 += TC) {
-        {   // registers -> LDS tile
+        if (tid < 256) {   // registers -> LDS tile
             float fa[8], fb[8];
             ra.to_float(fa); rb.to_float(fb);
             if (half == 0) {
@@ -102,12 +106,12 @@ __device__ __forceinline__ void scan_fwd_body(ScanFwdLds &L, int b, int h, int T
         prefetch(t0 + TC);
         const int nt = min(TC, T - t0);
         for (int t = 0; t < nt; ++t) {
-            float rr[16], kk[16], dd[16];
+            float rr[RW], kk[RW], dd[RW];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const float4 a = *reinterpret_cast<const float4 *>(&s_r[t][16 * q + 4 * g]);
-                const float4 c = *reinterpret_cast<const float4 *>(&s_k[t][16 * q + 4 * g]);
-                const float4 e = *reinterpret_cast<const float4 *>(&s_d[t][16 * q + 4 * g]);
+            for (int g = 0; g < RW / 4; ++g) {
+                const float4 a = *reinterpret_cast<const float4 *>(&s_r[t][RW * q + 4 * g]);
+                const float4 c = *reinterpret_cast<const float4 *>(&s_k[t][RW * q + 4 * g]);
+                const float4 e = *reinterpret_cast<const float4 *>(&s_d[t][RW * q + 4 * g]);
                 rr[4 * g] = a.x; rr[4 * g + 1] = a.y; rr[4 * g + 2] = a.z; rr[4 * g + 3] = a.w;
                 kk[4 * g] = c.x; kk[4 * g + 1] = c.y; kk[4 * g + 2] = c.z; kk[4 * g + 3] = c.w;
                 dd[4 * g] = e.x; dd[4 * g + 1] = e.y; dd[4 * g + 2] = e.z; dd[4 * g + 3] = e.w;
@@ -115,7 +119,7 @@ __device__ __forceinline__ void scan_fwd_body(ScanFwdLds &L, int b, int h, int T
             const float vi = s_v[t][lane];
             float acc0 = (q == 0) ? vi * s_ruk[t] : 0.f, acc1 = 0.f;
 #pragma unroll
-            for (int jj = 0; jj < 16; jj += 2) {
+            for (int jj = 0; jj < RW; jj += 2) {
                 const float x0 = kk[jj] * vi, x1 = kk[jj + 1] * vi;
                 acc0 = fmaf(rr[jj], s[jj], acc0);
                 acc1 = fmaf(rr[jj + 1], s[jj + 1], acc1);
@@ -127,10 +131,10 @@ __device__ __forceinline__ void scan_fwd_body(ScanFwdLds &L, int b, int h, int T
         __syncthreads();
         {   // sum the four wave partials, one rounding, coalesced store
             const int t = tid >> 4, c4 = (tid & 15) * 4;
-            if (t < nt) {
+            if (t < nt && tid < 256) {
                 float4 a = *reinterpret_cast<const float4 *>(&s_part[0][t][c4]);
 #pragma unroll
-                for (int qq = 1; qq < 4; ++qq) {
+                for (int qq = 1; qq < NW; ++qq) {
                     const float4 c = *reinterpret_cast<const float4 *>(&s_part[qq][t][c4]);
                     a.x += c.x; a.y += c.y; a.z += c.z; a.w += c.w;
                 }
@@ -141,9 +145,9 @@ __device__ __forceinline__ void scan_fwd_body(ScanFwdLds &L, int b, int h, int T
         // past the barrier above; s_part is rewritten only after the barrier that follows them.
     }
     if (sT != nullptr) {
-        Ts *p = sT + (((int64_t)b * H + h) * kN + 16 * q) * kN + lane;
+        Ts *p = sT + (((int64_t)b * H + h) * kN + RW * q) * kN + lane;
 #pragma unroll
-        for (int jj = 0; jj < 16; ++jj) store1(p + jj * kN, s[jj]);
+        for (int jj = 0; jj < RW; ++jj) store1(p + jj * kN, s[jj]);
     }
 }
 
