@@ -156,18 +156,20 @@ __device__ __forceinline__ void scan_fwd_body(ScanFwdLdsT<NW> &L, int b, int h, 
 // workspace), where gr'_t[j] = sum_i gy_t[i] S_t[j][i] is gr without the u term.
 // lane j owns key row j; wave q owns value columns [16q,16q+16).
 // ------------------------------------------------------------------------------------------
-struct alignas(16) ScanBwdALds {
+template <int NW> struct alignas(16) ScanBwdALdsT {
     float s_r[TC][kN], s_k[TC][kN], s_d[TC][kN], s_v[TC][kN], s_g[TC][kN];
-    float s_part[4][TC][kN];
+    float s_part[NW][TC][kN];
     float s_vgy[TC];
     float s_u[kN];
 };
+typedef ScanBwdALdsT<4> ScanBwdALds;
 
 // P is addressed as wsP[t * pstride + channel-in-head]: the caller points wsP at this head's
 // first element ((B,T,C) layout: pstride = C; a private [T][64] block: pstride = 64).
-// Threads 0..255 work; further threads only keep the barriers company.
-template <typename Tin, typename Tout>
-__device__ __forceinline__ void scan_bwd_a_body(ScanBwdALds &L, int b, int h, int T, int H,
+// The first NW waves work (wave q owns value columns [64/NW q, 64/NW (q+1)); NW <= 16; the first
+// 256 threads also stage the tiles and finish the rows); further threads only keep the barriers company.
+template <typename Tin, typename Tout, int NW = 4>
+__device__ __forceinline__ void scan_bwd_a_body(ScanBwdALdsT<NW> &L, int b, int h, int T, int H,
         const Tin *__restrict__ r, const Tin *__restrict__ k, const Tin *__restrict__ v,
         const Tin *__restrict__ w, const Tin *__restrict__ u, const Tout *__restrict__ gy,
         Tout *__restrict__ gr, Tout *__restrict__ gu, float *__restrict__ wsP, int64_t pstride,
@@ -179,7 +181,9 @@ __device__ __forceinline__ void scan_bwd_a_body(ScanBwdALds &L, int b, int h, in
     auto &s_r = L.s_r; auto &s_k = L.s_k; auto &s_d = L.s_d; auto &s_v = L.s_v; auto &s_g = L.s_g;
     auto &s_part = L.s_part; auto &s_vgy = L.s_vgy; auto &s_u = L.s_u;
     const int tid = threadIdx.x, lane = tid & 63, q = tid >> 6;
-    if (tid >= 256) {   // same barrier sequence as below, no work
+    constexpr int RW = kN / NW;   // value columns per wave
+    const bool first256 = tid < 256;
+    if (tid >= 64 * NW) {   // same barrier sequence as below, no work
         __syncthreads();
         for (int t0 = 0; t0 < T; t0 += TC) { __syncthreads(); __syncthreads(); __syncthreads(); }
         __syncthreads();
@@ -193,15 +197,16 @@ __device__ __forceinline__ void scan_bwd_a_body(ScanBwdALds &L, int b, int h, in
     Raw8<Tin> ra, rb, rc;
     Raw8<Tout> rg;
 
-    float s[16];
+    float s[RW];
 #pragma unroll
-    for (int ii = 0; ii < 16; ++ii) s[ii] = s0 ? s0[lane * kN + 16 * q + ii] : 0.f;
+    for (int ii = 0; ii < RW; ++ii) s[ii] = s0 ? s0[lane * kN + RW * q + ii] : 0.f;
     if (tid < kN) s_u[tid] = load1(u + h * kN + tid);
     float gu_acc[4] = {0.f, 0.f, 0.f, 0.f};
 
     auto prefetch = [&](int t0) {
         const int t = t0 + st;
         const int64_t o = base + (int64_t)t * C + sc;
+        if (!first256) return;
         if (t < T) {
             if (half == 0) { ra.load(v + o); rg.load(gy + o); }
             else { ra.load(k + o); rb.load(w + o); rc.load(r + o); }
@@ -211,7 +216,7 @@ __device__ __forceinline__ void scan_bwd_a_body(ScanBwdALds &L, int b, int h, in
     __syncthreads();
 
     for (int t0 = 0; t0 < T; t0 += TC) {
-        {
+        if (first256) {
             float fa[8], fb[8];
             ra.to_float(fa);
             if (half == 0) {
@@ -237,18 +242,18 @@ __device__ __forceinline__ void scan_bwd_a_body(ScanBwdALds &L, int b, int h, in
         prefetch(t0 + TC);
         const int nt = min(TC, T - t0);
         for (int t = 0; t < nt; ++t) {
-            float vv[16], gg[16];
+            float vv[RW], gg[RW];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const float4 a = *reinterpret_cast<const float4 *>(&s_v[t][16 * q + 4 * g]);
-                const float4 c = *reinterpret_cast<const float4 *>(&s_g[t][16 * q + 4 * g]);
+            for (int g = 0; g < RW / 4; ++g) {
+                const float4 a = *reinterpret_cast<const float4 *>(&s_v[t][RW * q + 4 * g]);
+                const float4 c = *reinterpret_cast<const float4 *>(&s_g[t][RW * q + 4 * g]);
                 vv[4 * g] = a.x; vv[4 * g + 1] = a.y; vv[4 * g + 2] = a.z; vv[4 * g + 3] = a.w;
                 gg[4 * g] = c.x; gg[4 * g + 1] = c.y; gg[4 * g + 2] = c.z; gg[4 * g + 3] = c.w;
             }
             const float kj = s_k[t][lane], dj = s_d[t][lane];
             float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll
-            for (int ii = 0; ii < 16; ii += 2) {
+            for (int ii = 0; ii < RW; ii += 2) {
                 const float x0 = kj * vv[ii], x1 = kj * vv[ii + 1];
                 acc0 = fmaf(gg[ii], s[ii], acc0);
                 acc1 = fmaf(gg[ii + 1], s[ii + 1], acc1);
@@ -260,10 +265,10 @@ __device__ __forceinline__ void scan_bwd_a_body(ScanBwdALds &L, int b, int h, in
         __syncthreads();
         {
             const int t = tid >> 4, c4 = (tid & 15) * 4;
-            if (t < nt) {
+            if (t < nt && first256) {
                 float4 a = *reinterpret_cast<const float4 *>(&s_part[0][t][c4]);
 #pragma unroll
-                for (int qq = 1; qq < 4; ++qq) {
+                for (int qq = 1; qq < NW; ++qq) {
                     const float4 c = *reinterpret_cast<const float4 *>(&s_part[qq][t][c4]);
                     a.x += c.x; a.y += c.y; a.z += c.z; a.w += c.w;
                 }
@@ -292,21 +297,26 @@ __device__ __forceinline__ void scan_bwd_a_body(ScanBwdALds &L, int b, int h, in
         gu_acc[i] += __shfl_xor(gu_acc[i], 16);
         gu_acc[i] += __shfl_xor(gu_acc[i], 32);
     }
-    if (lane < 16) {
+    if (lane < 16 && first256) {   // (the finishing threads: waves 0..3)
 #pragma unroll
         for (int i = 0; i < 4; ++i) s_part[0][q][lane * 4 + i] = gu_acc[i];
     }
     if (fT) {   // s now holds S_T
         float f = 0.f;
 #pragma unroll
-        for (int ii = 0; ii < 16; ++ii) f = fmaf(s[ii], gsT ? gsT[lane * kN + 16 * q + ii] : 0.f, f);
+        for (int ii = 0; ii < RW; ++ii) f = fmaf(s[ii], gsT ? gsT[lane * kN + RW * q + ii] : 0.f, f);
         s_part[1][q][lane] = f;
     }
     __syncthreads();
     if (tid < kN) {
         const float g = s_part[0][0][tid] + s_part[0][1][tid] + s_part[0][2][tid] + s_part[0][3][tid];
         store1(gu + (int64_t)b * C + h * kN + tid, g);
-        if (fT) fT[tid] = s_part[1][0][tid] + s_part[1][1][tid] + s_part[1][2][tid] + s_part[1][3][tid];
+        if (fT) {
+            float f = 0.f;
+#pragma unroll
+            for (int qq = 0; qq < NW; ++qq) f += s_part[1][qq][tid];
+            fT[tid] = f;
+        }
     }
 }
 
@@ -320,17 +330,20 @@ __device__ __forceinline__ void scan_bwd_a_body(ScanBwdALds &L, int b, int h, in
 // rwkv_kernels.cu:358-405):   gw_t[j] = -exp(w_t[j]) * ( sum_{m>t} P_m[j] - sum_{m>=t} Q_m[j] ),
 // Q_m[j] = k_m[j] gk'_m[j], P from sweep A; accumulated as one running difference per channel.
 // ------------------------------------------------------------------------------------------
-struct alignas(16) ScanBwdBLds {
+template <int NWR> struct alignas(16) ScanBwdBLdsT {
     float s_r[TC][kN], s_k[TC][kN], s_d[TC][kN], s_v[TC][kN], s_g[TC][kN];
-    float s_pk[4][TC][kN], s_pv[4][TC][kN];
+    float s_pk[NWR][TC][kN], s_pv[NWR][TC][kN];
     float s_e[TC][kN];
     float s_vgy[TC], s_ruk[TC];
     float s_u[kN];
 };
+typedef ScanBwdBLdsT<4> ScanBwdBLds;
 
-// Threads 0..511 of the workgroup work.  P addressed as in sweep A.
-template <typename Tin, typename Tout>
-__device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLds &L, int b, int h, int T, int H,
+// The first 2 NWR waves of the workgroup work: NWR in the K role, then NWR in the V role, each
+// owning 64/NWR value columns / key rows; the first 512 threads also stage the tiles and finish the
+// rows.  P addressed as in sweep A.
+template <typename Tin, typename Tout, int NWR = 4>
+__device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLdsT<NWR> &L, int b, int h, int T, int H,
         const Tin *__restrict__ r, const Tin *__restrict__ k, const Tin *__restrict__ v,
         const Tin *__restrict__ w, const Tin *__restrict__ u, const Tout *__restrict__ gy,
         const float *__restrict__ wsP, int64_t pstride,
@@ -345,13 +358,14 @@ __device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLds &L, int b, int h, in
     auto &s_pk = L.s_pk; auto &s_pv = L.s_pv; auto &s_e = L.s_e;
     auto &s_vgy = L.s_vgy; auto &s_ruk = L.s_ruk; auto &s_u = L.s_u;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    if (tid >= 512) {   // a larger workgroup: same barrier sequence as below, no work
+    constexpr int RW = kN / NWR;
+    if (tid >= 128 * NWR) {   // a larger workgroup: same barrier sequence as below, no work
         __syncthreads();
         for (int t0 = ((T - 1) / TC) * TC; t0 >= 0; t0 -= TC) { __syncthreads(); __syncthreads(); __syncthreads(); }
         return;
     }
-    const int q = wave & 3;
-    const bool role_k = wave < 4;
+    const int q = wave % NWR;
+    const bool role_k = wave < NWR;
     const int64_t C = (int64_t)H * kN;
     const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
 
@@ -364,10 +378,10 @@ __device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLds &L, int b, int h, in
     float4 preP = make_float4(0, 0, 0, 0), curP;
     float preW[4] = {0, 0, 0, 0}, curW[4];
 
-    float g[16];
+    float g[RW];
 #pragma unroll
-    for (int i = 0; i < 16; ++i)
-        g[i] = !gsT ? 0.f : role_k ? gsT[lane * kN + 16 * q + i] : gsT[(16 * q + i) * kN + lane];
+    for (int i = 0; i < RW; ++i)
+        g[i] = !gsT ? 0.f : role_k ? gsT[lane * kN + RW * q + i] : gsT[(RW * q + i) * kN + lane];
     if (tid < kN) s_u[tid] = load1(u + h * kN + tid);
     float carry[4] = {0.f, 0.f, 0.f, 0.f};  // sum over later tiles of (P - Q), finaliser channels
     if (fT && tid < 256) {
@@ -434,18 +448,18 @@ __device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLds &L, int b, int h, in
         const int nt = min(TC, T - t0);
         if (role_k) {
             for (int t = nt - 1; t >= 0; --t) {
-                float vv[16], gg[16];
+                float vv[RW], gg[RW];
 #pragma unroll
-                for (int a4 = 0; a4 < 4; ++a4) {
-                    const float4 a = *reinterpret_cast<const float4 *>(&s_v[t][16 * q + 4 * a4]);
-                    const float4 c = *reinterpret_cast<const float4 *>(&s_g[t][16 * q + 4 * a4]);
+                for (int a4 = 0; a4 < RW / 4; ++a4) {
+                    const float4 a = *reinterpret_cast<const float4 *>(&s_v[t][RW * q + 4 * a4]);
+                    const float4 c = *reinterpret_cast<const float4 *>(&s_g[t][RW * q + 4 * a4]);
                     vv[4 * a4] = a.x; vv[4 * a4 + 1] = a.y; vv[4 * a4 + 2] = a.z; vv[4 * a4 + 3] = a.w;
                     gg[4 * a4] = c.x; gg[4 * a4 + 1] = c.y; gg[4 * a4 + 2] = c.z; gg[4 * a4 + 3] = c.w;
                 }
                 const float rj = s_r[t][lane], dj = s_d[t][lane];
                 float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll
-                for (int ii = 0; ii < 16; ii += 2) {
+                for (int ii = 0; ii < RW; ii += 2) {
                     acc0 = fmaf(vv[ii], g[ii], acc0);
                     acc1 = fmaf(vv[ii + 1], g[ii + 1], acc1);
                     g[ii] = fmaf(g[ii], dj, rj * gg[ii]);
@@ -455,12 +469,12 @@ __device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLds &L, int b, int h, in
             }
         } else {
             for (int t = nt - 1; t >= 0; --t) {
-                float rr[16], kk[16], dd[16];
+                float rr[RW], kk[RW], dd[RW];
 #pragma unroll
-                for (int a4 = 0; a4 < 4; ++a4) {
-                    const float4 a = *reinterpret_cast<const float4 *>(&s_r[t][16 * q + 4 * a4]);
-                    const float4 c = *reinterpret_cast<const float4 *>(&s_k[t][16 * q + 4 * a4]);
-                    const float4 e = *reinterpret_cast<const float4 *>(&s_d[t][16 * q + 4 * a4]);
+                for (int a4 = 0; a4 < RW / 4; ++a4) {
+                    const float4 a = *reinterpret_cast<const float4 *>(&s_r[t][RW * q + 4 * a4]);
+                    const float4 c = *reinterpret_cast<const float4 *>(&s_k[t][RW * q + 4 * a4]);
+                    const float4 e = *reinterpret_cast<const float4 *>(&s_d[t][RW * q + 4 * a4]);
                     rr[4 * a4] = a.x; rr[4 * a4 + 1] = a.y; rr[4 * a4 + 2] = a.z; rr[4 * a4 + 3] = a.w;
                     kk[4 * a4] = c.x; kk[4 * a4 + 1] = c.y; kk[4 * a4 + 2] = c.z; kk[4 * a4 + 3] = c.w;
                     dd[4 * a4] = e.x; dd[4 * a4 + 1] = e.y; dd[4 * a4 + 2] = e.z; dd[4 * a4 + 3] = e.w;
@@ -468,7 +482,7 @@ __device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLds &L, int b, int h, in
                 const float gi = s_g[t][lane];
                 float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll
-                for (int jj = 0; jj < 16; jj += 2) {
+                for (int jj = 0; jj < RW; jj += 2) {
                     acc0 = fmaf(kk[jj], g[jj], acc0);
                     acc1 = fmaf(kk[jj + 1], g[jj + 1], acc1);
                     g[jj] = fmaf(g[jj], dd[jj], rr[jj] * gi);
@@ -485,7 +499,7 @@ __device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLds &L, int b, int h, in
             if (ft < nt) {
                 float4 a = *reinterpret_cast<const float4 *>(&s_pk[0][ft][fc]);
 #pragma unroll
-                for (int qq = 1; qq < 4; ++qq) {
+                for (int qq = 1; qq < NWR; ++qq) {
                     const float4 c = *reinterpret_cast<const float4 *>(&s_pk[qq][ft][fc]);
                     a.x += c.x; a.y += c.y; a.z += c.z; a.w += c.w;
                 }
@@ -499,11 +513,11 @@ __device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLds &L, int b, int h, in
                 e[0] = curP.x - Qv[0]; e[1] = curP.y - Qv[1]; e[2] = curP.z - Qv[2]; e[3] = curP.w - Qv[3];
             }
             *reinterpret_cast<float4 *>(&s_e[ft][fc]) = make_float4(e[0], e[1], e[2], e[3]);
-        } else {                    // gv
+        } else if (tid < 512) {     // gv
             if (ft < nt) {
                 float4 a = *reinterpret_cast<const float4 *>(&s_pv[0][ft][fc]);
 #pragma unroll
-                for (int qq = 1; qq < 4; ++qq) {
+                for (int qq = 1; qq < NWR; ++qq) {
                     const float4 c = *reinterpret_cast<const float4 *>(&s_pv[qq][ft][fc]);
                     a.x += c.x; a.y += c.y; a.z += c.z; a.w += c.w;
                 }
@@ -546,7 +560,7 @@ __device__ __forceinline__ void scan_bwd_b_body(ScanBwdBLds &L, int b, int h, in
     }
     if (gs0 && role_k) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) gs0[lane * kN + 16 * q + i] = g[i];
+        for (int i = 0; i < RW; ++i) gs0[lane * kN + RW * q + i] = g[i];
     }
 }
 
