@@ -39,10 +39,7 @@ namespace wkv6 {
 constexpr int kMixers = 5;
 constexpr int kMixTiles = 2;       // 16-channel MFMA tiles per wave: 32 channels, 64 contiguous bytes per token
 constexpr int kMixWaveCh = 16 * kMixTiles, kMixGroupCh = 4 * kMixWaveCh;   // channels per wave, per workgroup
-#ifndef WKV6_MIX_TB
-#define WKV6_MIX_TB 8
-#endif
-constexpr int kMixTokBlocks = WKV6_MIX_TB;   // 16-token blocks one workgroup walks through (the W fragments stay in registers)
+constexpr int kMixTokBlocks = 8;   // 16-token blocks one workgroup walks through (the W fragments stay in registers)
 
 // what one wave keeps for its channels: the W fragments and the biases of the five mixers
 template <int R> struct MixWeights {

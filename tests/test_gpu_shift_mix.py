@@ -163,3 +163,108 @@ def test_unsupported_shapes_are_refused(lib):
     assert rc == 2          # WKV6_ERR_UNSUPPORTED
     rc = lib.wkv6_shift_mix_x(_stream(), _native.BF16, 1, 4, 128, None, m.data_ptr(), x.data_ptr())
     assert rc == 1          # WKV6_ERR_ARG
+
+
+def test_full_size_known_answers(lib):
+    """At the benchmark's layer shape (B=8, T=1024, C=2048, rank 32), where a float64 reference of
+    everything is too slow: cases whose exact answer needs no arithmetic.  Coefficient 0 (W = 0,
+    bias = 0) must return x bit for bit in all five outputs; coefficient 1 must return the previous
+    token (x + (prev - x) in fp32: to one bf16 rounding plus 2^-23 of |x|; exactly zero at the start
+    of every sequence); and with coefficient 1 the backward
+    kernel's gp = sum_s g_s - gxx must be exactly zero wherever gxx, five bf16 values summed in
+    fp32, is itself a bf16 number -- checked through gp + gxx = sum_s g_s to one rounding."""
+    from rwkv_kernel import _native
+    B, T, C, R = 8, 1024, 2048, 32
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(B, T, C, generator=g).to(BF16).cuda()
+    h = torch.tanh(torch.randn(B, T, 5, R, generator=g)).to(BF16).cuda()
+    zero_w = torch.zeros(5, C, R, dtype=BF16, device="cuda")
+    outs = [torch.full((B, T, C), float("nan"), dtype=BF16, device="cuda") for _ in range(5)]
+
+    def five(bias):
+        _native.check(lib.wkv6_shift_mix_five(_stream(), _native.BF16, B, T, C, R, x.data_ptr(), h.data_ptr(), zero_w.data_ptr(),
+                                              bias.data_ptr(), *[o.data_ptr() for o in outs]))
+        torch.cuda.synchronize()
+
+    five(torch.zeros(5, C, device="cuda"))
+    assert all(torch.equal(o, x) for o in outs)
+    five(torch.ones(5, C, device="cuda"))
+    prev = torch.cat([torch.zeros(B, 1, C, dtype=BF16, device="cuda"), x[:, :-1]], 1)
+    slack = 2.0 ** -23 * float(x.float().abs().max())
+    for o in outs:
+        assert torch.allclose(o.float(), prev.float(), rtol=2.0 ** -8, atol=slack)
+        assert float(o[:, 0].float().abs().max()) == 0.0
+    # x_mix with mix_x = 1 is the previous token as well, with mix_x = 0 it is x
+    x_mix = torch.empty_like(x)
+    for val, want in ((1.0, prev), (0.0, x)):
+        m = torch.full((C,), val, device="cuda")
+        _native.check(lib.wkv6_shift_mix_x(_stream(), _native.BF16, B, T, C, x.data_ptr(), m.data_ptr(), x_mix.data_ptr()))
+        torch.cuda.synchronize()
+        assert torch.allclose(x_mix.float(), want.float(), rtol=2.0 ** -8, atol=slack)
+    assert torch.equal(x_mix, x)                       # (mix_x = 0: bit for bit)
+    # backward with coefficient 1: gcoef_s = g_s * xx, gxx = sum_s g_s, gp = 0 up to gxx's own rounding
+    gouts = [torch.randn(B, T, C, generator=g).to(BF16).cuda() for _ in range(5)]
+    plane = B * T * C
+    gcoef = torch.empty(5, B * T, C, dtype=BF16, device="cuda")
+    gp, gxx = torch.empty_like(x), torch.empty_like(x)
+    _native.check(lib.wkv6_shift_mix_five_backward(
+        _stream(), _native.BF16, B, T, C, R, x.data_ptr(), h.data_ptr(), zero_w.data_ptr(), torch.ones(5, C, device="cuda").data_ptr(),
+        *[go.data_ptr() for go in gouts], gcoef.data_ptr(), plane, gp.data_ptr(), gxx.data_ptr()))
+    torch.cuda.synchronize()
+    total = sum(go.float() for go in gouts)
+    assert torch.equal(gxx, total.to(BF16))
+    assert float(gp.float().abs().max()) == 0.0       # sum - gxx in fp32, before gxx is rounded: exactly zero
+    xx = prev.float() - x.float()
+    for s in range(5):
+        assert torch.equal(gcoef[s].view(B, T, C), (gouts[s].float() * xx).to(BF16))
+
+
+def test_calls_replay_in_a_hip_graph(lib):
+    """The four calls captured once into a graph (they allocate nothing, enqueue on the given stream
+    only and clear gmix_x with a kernel of their own) and replayed with eager work in between: every
+    replay reproduces the eager results (bit for bit, except gmix_x whose atomic sums may come in
+    another order)."""
+    from rwkv_kernel import _native
+    B, T, C, R = 3, 200, 320, 32
+    dev, _ = _inputs(B, T, C, R, 5)
+    g = torch.Generator().manual_seed(6)
+    h = torch.tanh(torch.randn(B, T, 5, R, generator=g)).to(BF16).cuda()
+    gouts = [torch.randn(B, T, C, generator=g).to(BF16).cuda() for _ in range(5)]
+    gxm = torch.randn(B, T, C, generator=g).to(BF16).cuda()
+    res = {n: torch.empty_like(dev["x"]) for n in ("x_mix", "o0", "o1", "o2", "o3", "o4", "gp", "gxx", "gx")}
+    res["gcoef"] = torch.empty(5, B * T, C, dtype=BF16, device="cuda")
+    res["gmix"] = torch.empty(C, device="cuda")
+    P = lambda t: t.data_ptr()
+
+    def step():
+        st = torch.cuda.current_stream().cuda_stream
+        _native.check(lib.wkv6_shift_mix_x(st, _native.BF16, B, T, C, P(dev["x"]), P(dev["mix_x"]), P(res["x_mix"])))
+        _native.check(lib.wkv6_shift_mix_five(st, _native.BF16, B, T, C, R, P(dev["x"]), P(h), P(dev["w2t"]), P(dev["bias"]),
+                                              *[P(res["o%d" % s]) for s in range(5)]))
+        _native.check(lib.wkv6_shift_mix_five_backward(st, _native.BF16, B, T, C, R, P(dev["x"]), P(h), P(dev["w2t"]), P(dev["bias"]),
+                                                       *[P(go) for go in gouts], P(res["gcoef"]), B * T * C, P(res["gp"]), P(res["gxx"])))
+        _native.check(lib.wkv6_shift_mix_x_backward(st, _native.BF16, B, T, C, P(dev["x"]), P(dev["mix_x"]), P(res["gp"]), P(res["gxx"]),
+                                                    P(gxm), P(res["gx"]), P(res["gmix"])))
+
+    step()
+    torch.cuda.synchronize()
+    eager = {n: t.clone() for n, t in res.items()}
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                      # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    for rep in range(3):
+        for t in res.values():
+            t.fill_(float("nan"))   # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for n, t in res.items():
+            if n == "gmix":
+                assert torch.allclose(t, eager[n], rtol=1e-5, atol=1e-5), (rep, n)
+            else:
+                assert torch.equal(t, eager[n]), (rep, n)
