@@ -516,7 +516,7 @@ __global__ __launch_bounds__(kFwdThreads) void chunk_fwd_kernel(FwdArgs a)
 }
 
 // compute units of the current device (an immutable device property, looked up once per device)
-static int compute_units() {
+int compute_units() {
     static int cached[64] = {0};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;

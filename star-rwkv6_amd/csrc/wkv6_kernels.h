@@ -25,6 +25,9 @@ inline hipError_t allow_dynamic_lds(int bytes) {
 
 enum { kBF16 = 0, kF16 = 1, kF32 = 2 };  // same numbering as the public header
 
+// compute units of the current device (an immutable device property, looked up once per device)
+int compute_units();
+
 // --- per-timestep recurrence (wkv6_scan.hip) ---
 hipError_t scan_forward(hipStream_t st, int dtype, int state_dtype, int64_t B, int64_t T, int64_t H,
                         const void *r, const void *k, const void *v, const void *w, const void *u,

@@ -756,14 +756,43 @@ def test_chunk_matches_scan_on_padding_mask(op, oracle):
     check_close("y", y, oracle.forward_c(*ref, N)[0], torch.bfloat16)
 
 
-def test_plain_backward_equals_saved_backward(op, oracle):
+@pytest.mark.parametrize("B,T,H", [(40, 128, 8), (5, 100, 64), (100, 64, 3), (300, 37, 1), (33, 200, 10), (130, 512, 2)])
+def test_chunk_backward_with_more_pairs_than_compute_units(op, oracle, B, T, H):
+    """More (batch, head) pairs than the GPU has compute units and a short sequence: the backward runs one
+    workgroup per compute unit, each taking several pairs back to back (different batch rows of one
+    head); every pair's gradients, and gu summed over the batch, against the oracle.  Head counts
+    that divide the number of compute units and ones that do not, one chunk per pair and several, a
+    ragged last chunk."""
+    _case(op, oracle, B, T, H, 500 + T, torch.bfloat16, CHUNK)
+
+
+def test_chunk_many_pairs_fall_back_on_extreme_decay(op, oracle):
+    # as test_chunk_falls_back_on_extreme_decay with 280 pairs: pairs that are a workgroup's first and
+    # ones that are its second leave the chunked form's range and are redone exactly after the
+    # workgroup's last pair, their neighbours in the same workgroup keep their MFMA results
+    B, T, H, N = 70, 128, 4, 64
+    ins = oracle.make_inputs(B, T, H, N, 57)
+    ins[3][0, 40:60, 70:90] = 6.0          # pair (0, 1)
+    ins[3][69, 10:30, 200:230] = 6.0       # pair (69, 3): index 279, the second pair of its workgroup
+    ins[3][66, 100:110, 0:64] = 7.0        # pair (66, 0): index 264
+    ins[3][3, 90:100] = -1e9               # decay exactly 1
+    dev, ref = cast_inputs(ins[:5], torch.bfloat16)
+    gy_dev, gy_ref = cast_inputs(ins[5:6], torch.bfloat16)
+    y, grads = _run_fwd_bwd(op, dev + gy_dev, CHUNK)
+    check_close("y", y, oracle.forward_c(*ref, N)[0], torch.bfloat16)
+    for name, g, gr in zip("gr gk gv gw gu".split(), grads, oracle.backward_c(*ref, gy_ref[0], N)):
+        check_close(name, to_np(g).reshape(gr.shape), gr, torch.bfloat16, is_grad=True)
+
+
+@pytest.mark.parametrize("B,T,H", [(2, 320, 2), (150, 192, 2)])
+def test_plain_backward_equals_saved_backward(op, oracle, B, T, H):
     # wkv6_backward (recomputes the chunk states) and wkv6_backward_saved (takes them from the
     # forward) agree to rounding (the two sweeps scale k differently before the bf16 rounding),
-    # and both meet the tolerance against the oracle
+    # and both meet the tolerance against the oracle; with few pairs and with more pairs than compute units
     from rwkv_kernel import _native
 
     lib = _native.load()
-    B, T, H, N = 2, 320, 2, 64
+    N = 64
     C = H * N
     ins = oracle.make_inputs(B, T, H, N, 77)
     dev, _ = cast_inputs(ins[:6], torch.bfloat16)
