@@ -60,7 +60,8 @@ struct BwdLds {
     static constexpr int kState = kOp + 2 * kOpBytes;                  // [item & 1] saved forward state of the chunk, bf16 [i][j] (transposed) as a tile
     static constexpr int kVgy = kState + 2 * kTileBytes;                    // [8 consumer waves][16] fp32: <v_t, gy_t>
     static constexpr int kGu = kVgy + 8 * 16 * 4;                      // [pair parity][64] fp32: gu partial of consumer group 1
-    static constexpr int kBytes = kGu + 2 * kN * 4;
+    static constexpr int kGuSum = kGu + 2 * kN * 4;                    // [64] fp32: gu summed over the workgroup's pairs (several-pairs variant)
+    static constexpr int kBytes = kGuSum + kN * 4;
 };
 static_assert(BwdLds::kBytes <= 160 * 1024, "LDS block of the backward kernel");
 
@@ -116,11 +117,17 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     // kMulti, group 0: gu of the pair just finished, waiting for group 1's half (it is in LDS once the
     // next barrier has been passed)
     float gu_prev = 0.f;
+    float gu_wg = 0.f;   // kMulti, group 0: gu summed over the workgroup's pairs, as stored (for the fused batch sum)
     int prev_slot = -1, prev_b = 0;
     float *gu_lds = reinterpret_cast<float *>(smem + BwdLds::kGu);
+    auto store_gu = [&](int b_, float total) {
+        Tout *dst = reinterpret_cast<Tout *>(a.gu) + (int64_t)b_ * C + h * kN + col;
+        store1(dst, total);
+        if (kMulti) gu_wg += sizeof(Tout) == 2 ? bf16_bits_to_float(pack_bf16x2(total, 0.f) & 0xffffu) : total;   // (as store1 rounds it)
+    };
     auto deliver_gu = [&]() {
         if (g == 0 && !s_wild[prev_slot])   // (the exact second pass writes gu itself)
-            store1(reinterpret_cast<Tout *>(a.gu) + (int64_t)prev_b * C + h * kN + col, gu_prev + gu_lds[(prev_slot & 1) * kN + col]);
+            store_gu(prev_b, gu_prev + gu_lds[(prev_slot & 1) * kN + col]);
         prev_slot = -1;
     };
     // Saved forward state of a chunk as packed bf16: Sraw[m] = S^T[i = 16m + 4g .. +3][j = col].  It
@@ -366,10 +373,9 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     __threadfence_block();
     __syncthreads();
     if (kMulti && GRP == 0 && prev_slot >= 0) deliver_gu();   // (a last pair of no chunks cannot happen: T >= 1)
-    if (GRP == 0 && g == 0 && !s_wild[last_slot]) {   // (the exact second pass writes gu itself)
-        gu_acc += gu_lds[(last_slot & 1) * kN + col];
-        store1(reinterpret_cast<Tout *>(a.gu) + (int64_t)b * C + h * kN + col, gu_acc);
-    }
+    if (GRP == 0 && g == 0 && !s_wild[last_slot])     // (the exact second pass writes gu itself)
+        store_gu(b, gu_acc + gu_lds[(last_slot & 1) * kN + col]);
+    if (kMulti && GRP == 0 && g == 0) reinterpret_cast<float *>(smem + BwdLds::kGuSum)[col] = gu_wg;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -700,9 +706,12 @@ __global__ __launch_bounds__(kBwdWaves * 64) void chunk_bwd_kernel(BwdArgs a)
         __syncthreads();
         const int tid = threadIdx.x;
         if (tid < kN) {          // wave 0
-            float part = 0.f;
+            // kMulti: the pairs done by the chunked code were summed by consumer group 0 as it stored them
+            // (LDS); only what an exact second pass wrote is read back
+            float part = kMulti ? reinterpret_cast<const float *>(smem + BwdLds::kGuSum)[tid] : 0.f;
             for (int slot = 0; slot < npw; ++slot)
-                part += load1(reinterpret_cast<const Tout *>(a.gu) + (int64_t)((pair0 + slot * (int)gridDim.x) / a.H) * C + h * kN + tid);
+                if (!kMulti || s_wild[slot])
+                    part += load1(reinterpret_cast<const Tout *>(a.gu) + (int64_t)((pair0 + slot * (int)gridDim.x) / a.H) * C + h * kN + tid);
             __hip_atomic_store(a.ckpt + (int64_t)pair0 * slice + slice / 2 + tid, part, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             if (tid == 0)
@@ -770,8 +779,9 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
     bool multi = false;
     {
         const int64_t cus = compute_units(), pairs = B * H;
-        // (from 1024 tokens on a pair's start-up no longer shows and one workgroup per pair is 1-2 % faster)
-        if (!s0 && !gsT && !gs0 && pairs > cus && H <= cus && T < 16 * CL) {
+        // (beyond 1024 tokens a pair's start-up no longer shows: B16 T2048 runs in the same time either way,
+        // B12 T4096 is 1 % faster with one workgroup per pair)
+        if (!s0 && !gsT && !gs0 && pairs > cus && H <= cus && T <= 16 * CL) {
             const int64_t g = cus / H * H;
             if ((pairs + g - 1) / g <= kBwdMaxPairs) { multi = true; grid = (unsigned)g; }
         }

@@ -868,7 +868,7 @@ def test_fused_gu_batch_sum(op, oracle, B, T, H, dt):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("B,T,H", [(2, 256, 4), (1, 2048, 3)])   # the second: seven launches (time segments)
+@pytest.mark.parametrize("B,T,H", [(2, 256, 4), (1, 2048, 3), (70, 128, 4)])   # the second: seven launches (time segments); the third: several pairs per workgroup
 def test_training_pair_replays_in_a_hip_graph(op, oracle, B, T, H):
     """forward_save + backward_saved_sum captured once into a graph (the library allocates nothing
     and only enqueues on the given stream), replayed several times with eager work and
