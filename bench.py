@@ -29,6 +29,7 @@ WORKLOADS = {
     "c1": (2, 128, 4, "f32"),
     "c2_f16": (8, 1024, 32, "f16"),   # the c2 shape with fp16 tensors: y, gy and the gradients are fp32
     "long1": (1, 8192, 32, "bf16"),   # one long sequence per GPU (fine-tuning): 32 pairs, runs as time segments
+    "short": (128, 256, 32, "bf16"),  # many short sequences: 4096 pairs, every workgroup takes 16 of them back to back
 }
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (separate runs), scaled
