@@ -782,8 +782,10 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
         // (beyond 1024 tokens a pair's start-up no longer shows: B16 T2048 runs in the same time either way,
         // B12 T4096 is 1 % faster with one workgroup per pair)
         if (!s0 && !gsT && !gs0 && pairs > cus && H <= cus && T <= 16 * CL) {
-            const int64_t g = cus / H * H;
-            if ((pairs + g - 1) / g <= kBwdMaxPairs) { multi = true; grid = (unsigned)g; }
+            // (more workgroups than that only where one would get more pairs than it keeps flags for)
+            const int64_t g = cus / H * H, per = (pairs + g - 1) / g;
+            multi = true;
+            grid = (unsigned)(g * ((per + kBwdMaxPairs - 1) / kBwdMaxPairs));
         }
     }
     auto launch_as = [&](auto in_tag, auto ragged_tag, auto multi_tag) -> hipError_t {

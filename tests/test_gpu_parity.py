@@ -766,6 +766,30 @@ def test_chunk_backward_with_more_pairs_than_compute_units(op, oracle, B, T, H):
     _case(op, oracle, B, T, H, 500 + T, torch.bfloat16, CHUNK)
 
 
+def test_chunk_backward_with_more_pairs_than_a_workgroup_keeps_flags_for(op, oracle):
+    """16 500 single-head sequences of 32 tokens: more than 64 pairs per compute unit, so the grid of the
+    several-pairs backward is a multiple of its usual size.  The rows are independent: a few of them
+    (first, last, around the places where a workgroup's pair list wraps) against the oracle, and gu
+    summed over all rows against its closed form  sum_{b,t} r k <v, gy>  in float64."""
+    B, T, H, N = 16500, 32, 1, 64
+    g = torch.Generator().manual_seed(91)
+    mk = lambda: torch.randn(B, T, N, generator=g).to(torch.bfloat16)
+    r, k, v, gy = mk(), mk(), mk(), mk()
+    w = (torch.rand(B, T, N, generator=g) * 7 - 6).to(torch.bfloat16)
+    u = (torch.randn(H, N, generator=g) * 0.5).to(torch.bfloat16)
+    dev = [x.cuda() for x in (r, k, v, w, u, gy)]
+    y, grads = _run_fwd_bwd(op, dev, CHUNK)
+    rows = [0, 1, 255, 256, 257, 511, 512, 8191, 8192, 16383, 16384, 16385, B - 2, B - 1]
+    sub = [to_np(x[rows]) for x in (r, k, v, w)] + [to_np(u)]
+    check_close("y", y[rows], oracle.forward_c(*sub, N)[0], torch.bfloat16)
+    g_ref = oracle.backward_c(*sub, to_np(gy[rows]), N)
+    for name, got, want in zip("gr gk gv gw".split(), grads[:4], g_ref[:4]):
+        check_close(name, got[rows], want, torch.bfloat16, is_grad=True)
+    rd, kd, vd, gd = (x.cuda().double() for x in (r, k, v, gy))
+    gu_ref = (rd * kd * (vd * gd).sum(-1, keepdim=True)).sum((0, 1)).cpu().numpy().reshape(H, N)
+    check_close("gu", to_np(grads[4]).reshape(H, N), gu_ref, torch.bfloat16, is_grad=True)
+
+
 def test_chunk_many_pairs_fall_back_on_extreme_decay(op, oracle):
     # as test_chunk_falls_back_on_extreme_decay with 280 pairs: pairs that are a workgroup's first and
     # ones that are its second leave the chunked form's range and are redone exactly after the
