@@ -43,9 +43,12 @@ struct FwdLds {
     static constexpr int kOp = kRawV + 3 * kTileBytes;                  // [2] operand blocks
     static constexpr int kOpRt = 0, kOpKt = kTileBytes, kOpG = 2 * kTileBytes, kOpRuk = kOpG + 4 * kN * 4;
     static constexpr int kOpBytes = kOpRuk + CL * 4;
-    static constexpr int kBytes = kOp + 2 * kOpBytes;
+    static constexpr int kBytes0 = kOp + 2 * kOpBytes;
+    // only WITHOUT the fused output stage: [2] K^ = K~ g, k decayed to the END of its tile (exponents <= 0)
+    static constexpr int kKg = kBytes0;
+    static constexpr int kBytes = kKg + 2 * kTileBytes;
     // only with the fused output stage (group norm and gate):
-    static constexpr int kYStage = kBytes;                              // [2 visit parities] y of one chunk, bf16
+    static constexpr int kYStage = kBytes0;                             // [2 visit parities] y of one chunk, bf16
     static constexpr int kRawG = kYStage + 2 * kTileBytes;              // [4] raw gate tiles (visit & 3)
     static constexpr int kGnTab = kRawG + 4 * kTileBytes;               // [4][scale, offset][64] floats of the visit's head
     static constexpr int kBytesFused = kGnTab + 4 * 2 * kN * 4;
@@ -151,18 +154,32 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
                 // (fresh_s: form the tile addresses per tile instead of holding them all across the chunk)
-                op_off = fresh_s(op_off); v_off = fresh_s(v_off);
                 const unsigned char *rt = smem + op_off + FwdLds::kOpRt, *kt = smem + op_off + FwdLds::kOpKt;
                 const float *gv_ = reinterpret_cast<const float *>(smem + op_off + FwdLds::kOpG);
                 const float *ruk = reinterpret_cast<const float *>(smem + op_off + FwdLds::kOpRuk);
                 const unsigned char *vt = smem + v_off;
                 const s16x4 vf = tile_frag_tok(vt, 16 * q, 16 * p, l16, g);
-                // U = K~^T V in accumulators of its own: these MFMAs do not wait for the state, which keeps
-                // the chain from one tile's state to the next down to the VALU update at the end
+                const bool minep = (p & 1) == GRP && (kFuse || a.y != nullptr);   // (no y wanted: a pass that only builds the state)
                 f32x4 U[4];
+                bf16x8 sop0, sop1;
+                if (minep) { sop0 = acc_as_operand(S[0], S[1]); sop1 = acc_as_operand(S[2], S[3]); }
+                if (kFuse) {
+                    // U = K~^T V in accumulators of its own, added to the state by VALU code at the end of the tile
 #pragma unroll
-                for (int m = 0; m < 4; ++m) U[m] = mfma16(tile_frag_tok(kt, 16 * m, 16 * p, l16, g), vf, (f32x4){0.f, 0.f, 0.f, 0.f});
-                if ((p & 1) == GRP && (kFuse || a.y != nullptr)) {   // (no y wanted: a pass that only builds the state)
+                    for (int m = 0; m < 4; ++m) U[m] = mfma16(tile_frag_tok(kt, 16 * m, 16 * p, l16, g), vf, (f32x4){0.f, 0.f, 0.f, 0.f});
+                } else {
+                    // S <- diag(g) S + K^^T V: the new contributions' decay is folded into the operand, so the
+                    // update is one scaling and an MFMA accumulation onto the state itself
+                    const unsigned char *kgt = smem + FwdLds::kKg + (it & 1) * kTileBytes;
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) {
+                        const float4 gg = *reinterpret_cast<const float4 *>(&gv_[p * kN + 16 * m + 4 * g]);
+                        S[m][0] *= gg.x; S[m][1] *= gg.y; S[m][2] *= gg.z; S[m][3] *= gg.w;
+                    }
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) S[m] = mfma16(tile_frag_tok(kgt, 16 * m, 16 * p, l16, g), vf, S[m]);
+                }
+                if (minep) {
                     const int row = 16 * p + l16;
                     const bf16x8 rf0 = tile_frag_ch(rt, row, 0, g), rf1 = tile_frag_ch(rt, row, 1, g);
                     const bf16x8 kf0 = tile_frag_ch(kt, row, 0, g), kf1 = tile_frag_ch(kt, row, 1, g);
@@ -177,11 +194,11 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
                     // neighbouring channels of one token and writes them with one 8-byte store.
                     f32x4 Y = {0.f, 0.f, 0.f, 0.f};
                     if (kFuse) {
-                        Y = mfma32(rf0, acc_as_operand(S[0], S[1]), Y);
-                        Y = mfma32(rf1, acc_as_operand(S[2], S[3]), Y);
+                        Y = mfma32(rf0, sop0, Y);
+                        Y = mfma32(rf1, sop1, Y);
                     } else {
-                        Y = mfma32(acc_as_operand(S[0], S[1]), rf0, Y);
-                        Y = mfma32(acc_as_operand(S[2], S[3]), rf1, Y);
+                        Y = mfma32(sop0, rf0, Y);
+                        Y = mfma32(sop1, rf1, Y);
                     }
                     settle(AT);
 #pragma unroll
@@ -207,13 +224,17 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
                         if (!kRagged || t < T) store4(y_h + ((uint32_t)t * (uint32_t)C + (uint32_t)(16 * q + 4 * g)), Y[0], Y[1], Y[2], Y[3]);
                     }
                 }
-                // S <- diag(g) (S + U)
-                settle(U[0], U[1], U[2], U[3]);
+                if (kFuse) {
+                    // S <- diag(g) (S + U)
+                    settle(U[0], U[1], U[2], U[3]);
 #pragma unroll
-                for (int m = 0; m < 4; ++m) {
-                    const float4 gg = *reinterpret_cast<const float4 *>(&gv_[p * kN + 16 * m + 4 * g]);
-                    S[m][0] = (S[m][0] + U[m][0]) * gg.x; S[m][1] = (S[m][1] + U[m][1]) * gg.y;
-                    S[m][2] = (S[m][2] + U[m][2]) * gg.z; S[m][3] = (S[m][3] + U[m][3]) * gg.w;
+                    for (int m = 0; m < 4; ++m) {
+                        const float4 gg = *reinterpret_cast<const float4 *>(&gv_[p * kN + 16 * m + 4 * g]);
+                        S[m][0] = (S[m][0] + U[m][0]) * gg.x; S[m][1] = (S[m][1] + U[m][1]) * gg.y;
+                        S[m][2] = (S[m][2] + U[m][2]) * gg.z; S[m][3] = (S[m][3] + U[m][3]) * gg.w;
+                    }
+                } else {
+                    settle(S[0], S[1], S[2], S[3]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -389,6 +410,17 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
             *reinterpret_cast<uint16_t *>(op + FwdLds::kOpRt + o1) = (uint16_t)(pr2 >> 16);
             *reinterpret_cast<uint16_t *>(op + FwdLds::kOpKt + o0) = (uint16_t)pk2;
             *reinterpret_cast<uint16_t *>(op + FwdLds::kOpKt + o1) = (uint16_t)(pk2 >> 16);
+        }
+        if (!kFuse) {
+            // K^ = K~ g = k exp(-(c_16 - c_{t+1})): the state update's operand
+            unsigned char *kg = smem + FwdLds::kKg + (it & 1) * kTileBytes;
+#pragma unroll
+            for (int e = 0; e < NT; e += 2) {
+                const uint32_t pg2 = pack_bf16x2(xk[e] * pa, xk[e + 1] * pa);
+                const uint32_t o0 = choff[e & 7] + e * kTileRow, o1 = choff[(e + 1) & 7] + (e + 1) * kTileRow;
+                *reinterpret_cast<uint16_t *>(kg + o0) = (uint16_t)pg2;
+                *reinterpret_cast<uint16_t *>(kg + o1) = (uint16_t)(pg2 >> 16);
+            }
         }
         // the whole tile's decay: g, and the range check of exp(+c)
         if (__builtin_amdgcn_ballot_w64(!(cs2 <= kWildLimit * kLog2e)) != 0ull) {

@@ -127,10 +127,11 @@ def test_config5_prefill_with_fused_output_stage(op):
     y, sT = op(r, k, v, w, u, return_state=True, init_state=s0)
     out, sT2 = op.forward_gn_gate(r, k, v, w, u, gate, scale, offset, 64e-5, return_state=True, init_state=s0)
     torch.cuda.synchronize()
-    # (same arithmetic in both kernels; the compiler is free to contract products and sums
-    # differently in the two instantiations, so not bit for bit)
+    # (the two kernels round k at different scalings before it enters the state update's MFMA -- decayed
+    # to the end of its tile in the unfused kernel, to its own token in the fused one --, so the carried
+    # states agree to the rounding of a bf16 operand, not bit for bit)
     ds = float((sT - sT2).abs().max()) / float(sT.abs().max())
-    assert ds <= 1e-5, ds
+    assert ds <= 1e-2, ds
     x = F.layer_norm(y.float().reshape(B, T, H, N), (N,), None, None, 64e-5)
     want = ((x * scale + offset).reshape(B, T, H * N) * gate.float())
     err = float((out.float() - want).abs().max()) / float(want.abs().max())
