@@ -169,7 +169,8 @@ int wkv6_gn_gate_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t
  *   (caller) gh -> through tanh and A -> gxm = dL/dx_mix (B,T,C)
  *   wkv6_shift_mix_x_backward: gx = gp + gxm (1 - mix_x) + z[t+1] with z = gxx + gxm mix_x
  *       (nothing from beyond a sequence's last token), gmix_x (C) fp32 = sum over tokens of gxm * xx
- *       (zeroed by the call). */
+ *       (zeroed by the call).  gp and gxx may both be NULL (zero): the backward of x_mix alone, e.g. for
+ *       the channel-mix layer's two fixed token-shift mixes (rwkv6_model.py:57-60). */
 int wkv6_shift_mix_supported(int dtype, int64_t C, int64_t R);
 int wkv6_shift_mix_x(void *stream, int dtype, int64_t B, int64_t T, int64_t C,
                      const void *x, const float *mix_x, void *x_mix);

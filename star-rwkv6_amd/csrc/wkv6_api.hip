@@ -254,7 +254,7 @@ int wkv6_shift_mix_x_backward(void *stream, int dtype, int64_t B, int64_t T, int
                               void *gx, float *gmix_x) {
     const int rc = check_mix(dtype, B, T, C, 32);
     if (rc != WKV6_OK) return rc;
-    if (!x || !mix_x || !gp || !gxx || !gxm || !gx || !gmix_x) return WKV6_ERR_ARG;
+    if (!x || !mix_x || !gxm || !gx || !gmix_x || (gp == nullptr) != (gxx == nullptr)) return WKV6_ERR_ARG;
     return finish(wkv6::shift_mix_x_backward((hipStream_t)stream, B, T, C, x, mix_x, gp, gxx, gxm, gx, gmix_x));
 }
 

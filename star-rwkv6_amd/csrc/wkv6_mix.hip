@@ -246,6 +246,7 @@ constexpr int kMixRows = 8;        // token rows a workgroup of the kernel below
 constexpr int kMixRun = 64;        // tokens per workgroup
 
 // gx = gp + gxm (1 - mix_x) + z[t+1],  z = gxx + gxm mix_x;  gmix_x += gxm * xx.
+// gp and gxx may be null (both zero): the backward of x_mix = x + xx * mix_x on its own.
 // Thread (row, column group): 8 channels of every 8th token of the workgroup's 64 tokens; the
 // per-channel sums go through LDS to one atomic per channel and workgroup.
 __global__ __launch_bounds__(256) void shift_mix_x_bwd_kernel(int64_t n_tok, int T, int C,
@@ -270,9 +271,10 @@ __global__ __launch_bounds__(256) void shift_mix_x_bwd_kernel(int64_t n_tok, int
             const size_t e = (size_t)tok * C + c;
             const int t = (int)(tok % T);
             Raw8<bf16_t> rx, rp, rg, rm, rzn, rmn;
-            rx.load(x + e); rg.load(gp + e); rm.load(gxm + e);
+            rx.load(x + e); rm.load(gxm + e);
+            if (gp) rg.load(gp + e); else rg.zero();
             if (t != 0) rp.load(x + e - C); else rp.zero();
-            if (t != T - 1) { rzn.load(gxx + e + C); rmn.load(gxm + e + C); } else { rzn.zero(); rmn.zero(); }
+            if (t != T - 1) { rmn.load(gxm + e + C); if (gxx) rzn.load(gxx + e + C); else rzn.zero(); } else { rzn.zero(); rmn.zero(); }
             float xa[8], xp[8], p[8], m[8], zn[8], mn[8], o[8];
             rx.to_float(xa); rp.to_float(xp); rg.to_float(p); rm.to_float(m); rzn.to_float(zn); rmn.to_float(mn);
 #pragma unroll

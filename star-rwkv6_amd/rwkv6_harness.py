@@ -124,8 +124,9 @@ class TimeMix(nn.Module):
 
 
 class ChannelMix(nn.Module):
-    def __init__(self, hidden_size, expand_size):
+    def __init__(self, hidden_size, expand_size, rwkv_kernel=None):
         super().__init__()
+        self.rwkv_kernel = rwkv_kernel   # optional: its shift_mix_x kernel does the two token-shift mixes in bf16
         self.time_mix_k = nn.Parameter(torch.rand(hidden_size))
         self.time_mix_r = nn.Parameter(torch.rand(hidden_size))
         self.dense_key = nn.Linear(hidden_size, expand_size, bias=False)
@@ -133,9 +134,15 @@ class ChannelMix(nn.Module):
         self.dense_receptance = nn.Linear(hidden_size, hidden_size, bias=False)
 
     def forward(self, x):
-        xx = time_shift(x)
-        xk = x + xx * self.time_mix_k.to(x.dtype)
-        xr = x + xx * self.time_mix_r.to(x.dtype)
+        fused = getattr(self.rwkv_kernel, "shift_mix_x", None)
+        if fused is not None and x.is_cuda and torch.is_autocast_enabled('cuda') and torch.get_autocast_dtype('cuda') == torch.bfloat16 \
+                and x.shape[-1] % 64 == 0:
+            xb = x.to(torch.bfloat16).contiguous()
+            xk, xr = fused(xb, self.time_mix_k), fused(xb, self.time_mix_r)
+        else:
+            xx = time_shift(x)
+            xk = x + xx * self.time_mix_k.to(x.dtype)
+            xr = x + xx * self.time_mix_r.to(x.dtype)
         k = torch.square(torch.relu(self.dense_key(xk)))
         return torch.sigmoid(self.dense_receptance(xr)) * self.dense_value(k)
 
@@ -146,7 +153,7 @@ class Block(nn.Module):
         self.layer_norm_att = nn.LayerNorm(hidden_size, eps=1e-5)
         self.layer_norm_ffn = nn.LayerNorm(hidden_size, eps=1e-5)
         self.time_mix = TimeMix(rwkv_kernel, hidden_size, decomposer_size, head_size)
-        self.channel_mix = ChannelMix(hidden_size, expand_size)
+        self.channel_mix = ChannelMix(hidden_size, expand_size, rwkv_kernel)
 
     def forward(self, x, mask=None):
         x = x + self.time_mix(self.layer_norm_att(x), mask)

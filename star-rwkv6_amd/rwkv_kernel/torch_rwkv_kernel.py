@@ -239,6 +239,38 @@ class _ShiftMix(torch.autograd.Function):
             return gx, gmx.to(dm), ga.to(da), gw2t.to(dw), gbias.to(db)
 
 
+class _ShiftMixX(torch.autograd.Function):
+    """x + (previous token - x) * mix with gradients, bf16 (wkv6_shift_mix_x and its backward): the fixed
+    token-shift mix of rwkv6_model.py:136 (time mix) and :57-60 (channel mix)."""
+
+    @staticmethod
+    def forward(ctx, x, mix):
+        lib = _native.load()
+        with torch.no_grad():
+            B, T, C = x.shape
+            mx = mix.detach().to(torch.float32).contiguous()
+            out = torch.empty_like(x)
+            with torch.cuda.device(x.device):
+                _native.check(lib.wkv6_shift_mix_x(_stream(), _DTYPE_CODE[x.dtype], B, T, C, _ptr(x), _ptr(mx), _ptr(out)))
+            ctx.save_for_backward(x, mx)
+            ctx.mix_dtype = mix.dtype
+            return out
+
+    @staticmethod
+    def backward(ctx, gout):
+        lib = _native.load()
+        with torch.no_grad():
+            x, mx = ctx.saved_tensors
+            B, T, C = x.shape
+            gout = gout.to(x.dtype).contiguous()
+            gx = torch.empty_like(x)
+            gmx = torch.empty(C, device=x.device, dtype=torch.float32)
+            with torch.cuda.device(x.device):
+                _native.check(lib.wkv6_shift_mix_x_backward(_stream(), _DTYPE_CODE[x.dtype], B, T, C, _ptr(x), _ptr(mx), None, None,
+                                                            _ptr(gout), _ptr(gx), _ptr(gmx)))
+            return gx, gmx.to(ctx.mix_dtype)
+
+
 def _forward_with_state(B, T, C, H, state_map, r, k, v, w, u, init_state, algo=_native.ALGO_AUTO, state_dtype=None):
     """Stateful forward, no gradient (rwkv_kernel/torch_rwkv_kernel.py:76-95)."""
     lib = _native.load()
@@ -406,6 +438,14 @@ class RWKVKernelOperator:
         if not (x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 3):
             return False
         return bool(_native.load().wkv6_shift_mix_supported(_DTYPE_CODE[x.dtype], x.shape[2], decomposer_size))
+
+    def shift_mix_x(self, x, mix):
+        """``x + (previous token - x) * mix`` (zero before a sequence's first token), differentiable in both
+        arguments: the fixed token-shift mix of rwkv6_model.py:136 and of the channel-mix layer
+        (:57-60).  bf16 tensors on the GPU, ``mix`` one value per channel.  Not part of the reference's operator."""
+        assert x.is_contiguous() and x.dim() == 3 and mix.numel() == x.shape[2]
+        assert self.shift_mix_supported(x, 32), "shift_mix_x takes bf16 tensors on the GPU, channels a multiple of 64"
+        return _ShiftMixX.apply(x, mix.reshape(x.shape[2]))
 
     def shift_mix(self, x, mix_x, a, w2t, bias):
         """The layer's input side, rwkv6_model.py:134-146: from the layer input ``x`` (B,T,C) to the

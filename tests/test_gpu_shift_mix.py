@@ -268,3 +268,26 @@ def test_calls_replay_in_a_hip_graph(lib):
                 assert torch.allclose(t, eager[n], rtol=1e-5, atol=1e-5), (rep, n)
             else:
                 assert torch.equal(t, eager[n]), (rep, n)
+
+
+@pytest.mark.parametrize("B,T,C", [(2, 64, 128), (3, 37, 64), (5, 1, 192), (1, 300, 320)])
+def test_fixed_mix_on_its_own(B, T, C):
+    """op.shift_mix_x: x + xx * mix and its gradients (the backward kernel with no gp / gxx) against
+    float64 autograd."""
+    import rwkv_kernel
+    op = rwkv_kernel.RWKVKernelOperator(64, 4096)
+    g = torch.Generator().manual_seed(40 + T)
+    x = torch.randn(B, T, C, generator=g).to(BF16).cuda().requires_grad_(True)
+    mix = torch.rand(C, generator=g).cuda().requires_grad_(True)
+    gout = torch.randn(B, T, C, generator=g).to(BF16).cuda()
+    out = op.shift_mix_x(x, mix)
+    out.backward(gout)
+    torch.cuda.synchronize()
+    xr = x.detach().double().cpu().requires_grad_(True)
+    mr = mix.detach().double().cpu().requires_grad_(True)
+    xx = torch.cat([torch.zeros(B, 1, C, dtype=torch.float64), xr[:, :-1]], 1) - xr
+    want = xr + xx * mr
+    want.backward(gout.double().cpu())
+    check_close("x_mix", out, want.detach().numpy(), BF16)
+    check_close("gx", x.grad, xr.grad.numpy(), BF16, is_grad=True)
+    check_close("gmix", mix.grad.double().cpu().numpy(), mr.grad.numpy(), torch.float32, is_grad=True)
