@@ -39,7 +39,8 @@ bool chunk_eligible(int dtype, int64_t T, int64_t C) { return chunk_possible(dty
 // kernels: r, k, w are unpacked exactly, v and gy go through bf16 copies kept behind the saved states.
 bool train_chunk(int dtype, int algo, int64_t T, int64_t C) {
     if (dtype != WKV6_BF16 && dtype != WKV6_F16) return false;
-    if (T * C >= (1LL << 31)) return false;
+    // (the kernels address a (b, h) pair's rows with 32-bit byte offsets; fp16 tensors have 4-byte outputs)
+    if (T * C >= (dtype == WKV6_F16 ? 1LL << 30 : 1LL << 31)) return false;
     return algo == WKV6_ALGO_CHUNK || (algo == WKV6_ALGO_AUTO && T >= 32);
 }
 
