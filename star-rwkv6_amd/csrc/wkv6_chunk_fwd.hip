@@ -253,7 +253,8 @@ __device__ __forceinline__ void fwd_consumer(const FwdArgs &a, const unsigned ch
 // ------------------------------------------------------------------------------------------
 // Loader / producer, lane = channel: wave p <-> tile p of every chunk.
 // ------------------------------------------------------------------------------------------
-template <typename Tin, bool kSave, bool kRagged, bool kMulti, bool kFuse>
+// kNoR: a pass that only builds states (no y wanted): r is neither loaded nor prepared
+template <typename Tin, bool kSave, bool kRagged, bool kMulti, bool kFuse, bool kNoR>
 __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *smem, int *s_wild, int bh0, int part, int pw, int lane)
 {
     constexpr int NT = 16;   // tokens per wave and chunk
@@ -286,7 +287,7 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
     // preparation turns them into r = k = 0, w = -inf (decay 1), and the v rows only ever meet zero
     // operands.  Each wave loads what it reads itself, so its own vmcnt covers its inputs; v is
     // picked up by the consumers a barrier later.
-    constexpr int kLoads = 8 + (kFuse ? 2 : 0);   // per chunk and wave
+    constexpr int kLoads = 8 + (kFuse ? 2 : 0) - (kNoR ? 2 : 0);   // per chunk and wave
     constexpr int kLoads0 = kLoads + (kFuse ? 2 : 0);                  // wave 0 also brings the norm's scale and offset
     auto issue_loads = [&](int it) {   // visit `it` = the load stream's current (pair, chunk)
         const int tb = ld_c * CL + 16 * p;
@@ -297,7 +298,7 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
             const int t = tb + 8 * blk + lrow;
             const uint32_t o = (uint32_t)(kRagged ? min(t, T - 1) : a.reverse ? T - 1 - t : t) * rowbytes + lpiece;
             load_rows8_to_lds(wb, o, rkw + 2 * kTileBytes + 8 * blk * kTileRow);
-            load_rows8_to_lds(rb, o, rkw + 8 * blk * kTileRow);
+            if (!kNoR) load_rows8_to_lds(rb, o, rkw + 8 * blk * kTileRow);
             load_rows8_to_lds(kb_, o, rkw + kTileBytes + 8 * blk * kTileRow);
             load_rows8_to_lds(vb, o, vv + 8 * blk * kTileRow);
             if (kFuse) load_rows8_to_lds(gb, o, lds0 + FwdLds::kRawG + (it & 3) * kTileBytes + (16 * p + 8 * blk) * kTileRow);
@@ -386,7 +387,7 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
 #pragma unroll
         for (int e = 0; e < NT; ++e) {
             const uint32_t o = choff[e & 7] + e * kTileRow;
-            uint32_t ra = *reinterpret_cast<const uint16_t *>(raw + o);
+            uint32_t ra = kNoR ? 0u : *reinterpret_cast<const uint16_t *>(raw + o);
             uint32_t rk = *reinterpret_cast<const uint16_t *>(raw + kTileBytes + o);
             uint32_t rw = *reinterpret_cast<const uint16_t *>(raw + 2 * kTileBytes + o);
             if (kRagged && tb + e >= T) { ra = 0u; rk = 0u; rw = neg_inf_bits<Tin>(); }
@@ -406,8 +407,10 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
         for (int e = 0; e < NT; e += 2) {
             const uint32_t pr2 = pack_bf16x2(xr[e], xr[e + 1]), pk2 = pack_bf16x2(xk[e], xk[e + 1]);
             const uint32_t o0 = choff[e & 7] + e * kTileRow, o1 = choff[(e + 1) & 7] + (e + 1) * kTileRow;
-            *reinterpret_cast<uint16_t *>(op + FwdLds::kOpRt + o0) = (uint16_t)pr2;
-            *reinterpret_cast<uint16_t *>(op + FwdLds::kOpRt + o1) = (uint16_t)(pr2 >> 16);
+            if (!kNoR) {
+                *reinterpret_cast<uint16_t *>(op + FwdLds::kOpRt + o0) = (uint16_t)pr2;
+                *reinterpret_cast<uint16_t *>(op + FwdLds::kOpRt + o1) = (uint16_t)(pr2 >> 16);
+            }
             *reinterpret_cast<uint16_t *>(op + FwdLds::kOpKt + o0) = (uint16_t)pk2;
             *reinterpret_cast<uint16_t *>(op + FwdLds::kOpKt + o1) = (uint16_t)(pk2 >> 16);
         }
@@ -428,8 +431,10 @@ __device__ __forceinline__ void fwd_producer(const FwdArgs &a, unsigned char *sm
         }
         dacc += cs2;
         reinterpret_cast<float *>(op + FwdLds::kOpG)[p * kN + ch] = pa;
-        const float tot = transpose_reduce16(pr, lane);
-        if ((lane & 3) == 0) reinterpret_cast<float *>(op + FwdLds::kOpRuk)[16 * p + ((lane >> 2) & 15)] = tot;
+        if (!kNoR) {
+            const float tot = transpose_reduce16(pr, lane);
+            if ((lane & 3) == 0) reinterpret_cast<float *>(op + FwdLds::kOpRuk)[16 * p + ((lane >> 2) & 15)] = tot;
+        }
         if (pp_c + 1 == nchunk && a.dsum != nullptr && part == 0) {   // the pair's total decay, this wave's tiles
             a.dsum[((int64_t)p * a.nitems + (bh0 + pp_n * stride)) * kN + ch] = dacc;
             dacc = 0.f;
@@ -501,7 +506,7 @@ __device__ __forceinline__ void output_stage_in_place(const FwdArgs &a, int bh) 
     }
 }
 
-template <typename Tin, typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse>
+template <typename Tin, typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse, bool kNoR = false>
 __global__ __launch_bounds__(kFwdThreads) void chunk_fwd_kernel(FwdArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -519,7 +524,7 @@ __global__ __launch_bounds__(kFwdThreads) void chunk_fwd_kernel(FwdArgs a)
     const int bh0 = (int)blockIdx.x / split, part = (int)blockIdx.x - bh0 * split;
     const int nq = 4 / split;   // consumer waves per group
     if (wave < 4) {
-        fwd_producer<Tin, kSave, kRagged, kMulti, kFuse>(a, smem, s_wild, bh0, part, wave, lane);
+        fwd_producer<Tin, kSave, kRagged, kMulti, kFuse, kNoR>(a, smem, s_wild, bh0, part, wave, lane);
     } else {
         const int cw = wave - 4, grp = cw / nq, q = part * nq + (cw - grp * nq);
         if (grp == 0) fwd_consumer<Tin, Ts, kSave, kRagged, kMulti, kFuse, 0>(a, smem, bh0, q, lane);
@@ -560,9 +565,9 @@ int compute_units() {
     return cached[dev];
 }
 
-template <typename Tin, typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse>
+template <typename Tin, typename Ts, bool kSave, bool kRagged, bool kMulti, bool kFuse, bool kNoR = false>
 static hipError_t launch_fwd(hipStream_t st, const FwdArgs &a, unsigned grid) {
-    constexpr auto kern = chunk_fwd_kernel<Tin, Ts, kSave, kRagged, kMulti, kFuse>;
+    constexpr auto kern = chunk_fwd_kernel<Tin, Ts, kSave, kRagged, kMulti, kFuse, kNoR>;
     const size_t lds = kFuse ? FwdLds::kBytesFused : FwdLds::kBytes;
     hipError_t e = allow_dynamic_lds<kern>((int)lds);
     if (e != hipSuccess) return e;
@@ -572,6 +577,13 @@ static hipError_t launch_fwd(hipStream_t st, const FwdArgs &a, unsigned grid) {
 }
 template <typename Tin, typename Ts, bool kSave, bool kRagged, bool kFuse>
 static hipError_t launch_fwd(hipStream_t st, const FwdArgs &a, bool multi, unsigned grid) {
+    // no y wanted and fp32 states (the state-only passes of the backward and of the time segments):
+    // the variant that leaves r alone
+    if constexpr (!kFuse && std::is_same<Ts, float>::value && std::is_same<Tin, bf16_t>::value) {
+        if (a.y == nullptr)
+            return multi ? launch_fwd<Tin, Ts, kSave, kRagged, true, kFuse, true>(st, a, grid)
+                         : launch_fwd<Tin, Ts, kSave, kRagged, false, kFuse, true>(st, a, grid);
+    }
     return multi ? launch_fwd<Tin, Ts, kSave, kRagged, true, kFuse>(st, a, grid) : launch_fwd<Tin, Ts, kSave, kRagged, false, kFuse>(st, a, grid);
 }
 template <typename Ts>
