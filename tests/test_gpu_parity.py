@@ -766,6 +766,14 @@ def test_chunk_backward_with_more_pairs_than_compute_units(op, oracle, B, T, H):
     _case(op, oracle, B, T, H, 500 + T, torch.bfloat16, CHUNK)
 
 
+@pytest.mark.parametrize("B,T,H", [(208, 51, 7), (323, 134, 3), (60, 33, 12), (146, 69, 12), (140, 290, 3), (49, 273, 6),
+                                   (29, 475, 9), (49, 173, 7), (109, 53, 3), (99, 167, 5)])
+def test_chunk_many_pairs_drawn_shapes(op, oracle, B, T, H):
+    # shapes drawn once at random among those with more pairs than compute units: ragged lengths, head
+    # counts that do not divide the number of compute units, workgroups with unequal numbers of pairs
+    _case(op, oracle, B, T, H, 700 + B, torch.bfloat16, CHUNK)
+
+
 def test_chunk_backward_with_more_pairs_than_a_workgroup_keeps_flags_for(op, oracle):
     """16 500 single-head sequences of 32 tokens: more than 64 pairs per compute unit, so the grid of the
     several-pairs backward is a multiple of its usual size.  The rows are independent: a few of them
