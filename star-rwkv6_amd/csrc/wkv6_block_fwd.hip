@@ -1,0 +1,316 @@
+// WKV6 forward in block form for gfx950 (bf16 MFMA for the dense products, fp32 state), for bf16
+// tensors, sequence lengths that are a multiple of 64 and between half a pair and one (batch, head)
+// pair per compute unit.  The tile form in wkv6_chunk_fwd.hip (state advanced every 16 tokens)
+// serves every other case.  Notation and the operand scaling are in wkv6_block.h.
+//
+// Per block of 32 tokens (S = state entering it, rows j):
+//   A[t][s] = R~_t . K~_s (s < t),   A[t][t] = sum_j r_t[j] u[j] k_t[j]
+//   Y  = R~ (g1 o S) + A V
+//   S <- g2 o (g1 o S + K~^T V)
+// The state is touched twice per block (two scalings and one MFMA accumulation over its 32 tokens)
+// instead of once per 16-token tile; A is three 16x16 blocks; nothing but the scalings and the masks
+// of the diagonal blocks is VALU work in the consumer waves.
+//
+// Workgroup: 12 waves.  Four producer waves (wave p <-> tokens 16p..16p+15 of every chunk) bring the
+// raw rows from global memory straight into LDS three chunk visits ahead, turn r, k, w of the next
+// chunk into R~, K~, g1, g2 and the diagonal, and write out what the consumers staged during the
+// previous visit.  Eight consumer waves (q, half): value columns 16q..16q+15; both halves carry the
+// state through both blocks of a visit, half h produces y of block h.  y and the saved chunk states
+// never leave a consumer wave as partial rows: they are staged in LDS as [token][channel] tiles and
+// stored one visit later by the producer waves as whole 128-byte rows.
+#include "wkv6_mfma.h"
+#include "wkv6_kernels.h"
+#include "wkv6_scan_body.h"
+#include "wkv6_block.h"
+
+#include <type_traits>
+
+namespace wkv6 {
+
+struct BlockFwdLds {
+    static constexpr int kRaw = 0;                                       // [2 visit parities][r, k, w] raw tiles
+    static constexpr int kRawV = kRaw + 2 * 3 * kTileBytes;              // [visit & 3] raw v tiles
+    static constexpr int kOp = kRawV + 4 * kTileBytes;                   // [2][R~, K~]
+    static constexpr int kVec = kOp + 2 * 2 * kTileBytes;                // [2] per-visit vectors
+    static constexpr int kYStage = kVec + 2 * kBlockVecBytes;            // [2] y of one chunk, bf16 tile
+    static constexpr int kSStage = kYStage + 2 * kTileBytes;             // [2] state at a chunk start, bf16 [i][j] tile
+    static constexpr int kBytes = kSStage + 2 * kTileBytes;
+};
+static_assert(BlockFwdLds::kBytes <= 160 * 1024, "LDS block of the block-form forward kernel");
+
+struct BlockFwdArgs {
+    int T, H;
+    const bf16_t *r, *k, *v, *w, *u;
+    const void *s0;          // initial state (B or n_state, H, 64, 64) [key][value] in Ts, or null
+    const int64_t *map;      // batch row -> state row, or null
+    bf16_t *y;
+    void *sT;                // final state in Ts, or null
+    float *ckpt;             // saved chunk states (bf16 [chunk][value][key] in the first half of each pair's slice), or null
+    int *arrivals;           // with ckpt: per-head counters of the backward's fused gu sum, zeroed here
+};
+
+// ------------------------------------------------------------------------------------------
+// Consumer wave (q, HALF): value columns i = 16q + l16; y of block HALF (tokens 32 HALF .. +31).
+// State S[m]: rows j = block_row_channel(m, g) + rr, column i.
+// ------------------------------------------------------------------------------------------
+template <typename Ts, bool kSave, int HALF>
+__device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsigned char *smem, int bh, int q, int lane)
+{
+    const int T = a.T, H = a.H;
+    const int g = lane >> 4, l16 = lane & 15;
+    const int nchunk = T / kBlockTokens;
+    const int b = bh / H, h = bh - b * H;
+    f32x4 S[4];
+    if (a.s0 != nullptr) {
+        const int64_t row = a.map ? a.map[b] : (int64_t)b;
+        const Ts *p = reinterpret_cast<const Ts *>(a.s0) + (row * H + h) * kN * kN + 16 * q + l16;
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) S[m][rr] = load1(p + (block_row_channel(m, g) + rr) * kN);
+    } else {
+#pragma unroll
+        for (int m = 0; m < 4; ++m) S[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
+    if (kSave && HALF == 0 && b == 0 && q == 0 && lane == 0 && a.arrivals) a.arrivals[h] = 0;
+    for (int it = 0; it < nchunk; ++it) {
+        __syncthreads();
+        const unsigned char *rt = smem + BlockFwdLds::kOp + (it & 1) * 2 * kTileBytes, *kt = rt + kTileBytes;
+        const float *vec = reinterpret_cast<const float *>(smem + BlockFwdLds::kVec + (it & 1) * kBlockVecBytes);
+        const float *ruk = vec + 4 * kN;
+        const unsigned char *vt = smem + BlockFwdLds::kRawV + (it & 3) * kTileBytes;
+        if (kSave && HALF == 0) {
+            // the state at the chunk start, as the backward wants it: bf16, transposed ([i][j] rows of 128 bytes)
+            unsigned char *ss = smem + BlockFwdLds::kSStage + (it & 1) * kTileBytes;
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+                *reinterpret_cast<uint2 *>(ss + tile_off(16 * q + l16, block_row_channel(m, g))) =
+                    make_uint2(pack_bf16x2(S[m][0], S[m][1]), pack_bf16x2(S[m][2], S[m][3]));
+        }
+        unsigned char *ys = smem + BlockFwdLds::kYStage + (it & 1) * kTileBytes;
+        auto scale = [&](const float *gv) {
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                const float4 gg = *reinterpret_cast<const float4 *>(&gv[block_row_channel(m, g)]);
+                S[m][0] *= gg.x; S[m][1] *= gg.y; S[m][2] *= gg.z; S[m][3] *= gg.w;
+            }
+        };
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+            scale(vec + 2 * blk * kN);   // g1 of the block
+            if (blk == HALF) {
+                // y of this block's two 16-token row groups; products transposed (accumulator rows i = 4g + rr,
+                // column t = l16: a lane holds four neighbouring channels of one token).  Every fragment is
+                // fetched first, then the MFMAs run as independent chains.
+                const bf16x8 sop0 = acc_as_operand(S[0], S[1]), sop1 = acc_as_operand(S[2], S[3]);
+                const int r0 = 32 * blk + l16, r1 = r0 + 16;
+                const bf16x8 rf0a = block_frag_ch(rt, r0, 0, g), rf0b = block_frag_ch(rt, r0, 1, g);
+                const bf16x8 rf1a = block_frag_ch(rt, r1, 0, g), rf1b = block_frag_ch(rt, r1, 1, g);
+                const bf16x8 kf0a = block_frag_ch(kt, r0, 0, g), kf0b = block_frag_ch(kt, r0, 1, g);
+                const bf16x8 kf1a = block_frag_ch(kt, r1, 0, g), kf1b = block_frag_ch(kt, r1, 1, g);
+                const s16x4 vf0 = tile_frag_tok(vt, 16 * q, 32 * blk, l16, g), vf1 = tile_frag_tok(vt, 16 * q, 32 * blk + 16, l16, g);
+                const float ruk0 = ruk[r0], ruk1 = ruk[r1];
+                const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+                // A^T[s][t] = K~_s . R~_t (rows s = 4g + rr, column t = l16): blocks (0,0), (0,1), (1,1)
+                f32x4 A00 = mfma32(kf0a, rf0a, zero), A01 = mfma32(kf0a, rf1a, zero), A11 = mfma32(kf1a, rf1a, zero);
+                f32x4 Y0 = mfma32(sop0, rf0a, zero), Y1 = mfma32(sop0, rf1a, zero);
+                A00 = mfma32(kf0b, rf0b, A00); A01 = mfma32(kf0b, rf1b, A01); A11 = mfma32(kf1b, rf1b, A11);
+                Y0 = mfma32(sop1, rf0b, Y0); Y1 = mfma32(sop1, rf1b, Y1);
+                settle(A00, A01, A11, Y0, Y1);
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr) {
+                    const int s_ = 4 * g + rr;
+                    A00[rr] = (l16 > s_) ? A00[rr] : ((l16 == s_) ? ruk0 : 0.f);
+                    A11[rr] = (l16 > s_) ? A11[rr] : ((l16 == s_) ? ruk1 : 0.f);
+                }
+                Y0 = mfma16(vf0, pack4(A00), Y0);
+                Y1 = mfma16(vf0, pack4(A01), Y1);
+                Y1 = mfma16(vf1, pack4(A11), Y1);
+                settle(Y0, Y1);
+                *reinterpret_cast<uint2 *>(ys + tile_off(r0, 16 * q + 4 * g)) = make_uint2(pack_bf16x2(Y0[0], Y0[1]), pack_bf16x2(Y0[2], Y0[3]));
+                *reinterpret_cast<uint2 *>(ys + tile_off(r1, 16 * q + 4 * g)) = make_uint2(pack_bf16x2(Y1[0], Y1[1]), pack_bf16x2(Y1[2], Y1[3]));
+            }
+            // S <- g2 o (g1 o S + K~^T V) over the block's 32 tokens
+            {
+                s16x4 vf[2], kq[2][4];
+#pragma unroll
+                for (int pp = 0; pp < 2; ++pp) {
+                    vf[pp] = tile_frag_tok(vt, 16 * q, 32 * blk + 16 * pp, l16, g);
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) kq[pp][m] = block_frag_tok_rows(kt, m, 32 * blk + 16 * pp, l16, g);
+                }
+#pragma unroll
+                for (int pp = 0; pp < 2; ++pp)
+#pragma unroll
+                    for (int m = 0; m < 4; ++m) S[m] = mfma16(kq[pp][m], vf[pp], S[m]);
+            }
+            settle(S[0], S[1], S[2], S[3]);
+            scale(vec + (2 * blk + 1) * kN);   // g2 of the block
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (a.sT != nullptr && HALF == 0) {
+        Ts *p = reinterpret_cast<Ts *>(a.sT) + (int64_t)bh * kN * kN + 16 * q + l16;
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) store1(p + (block_row_channel(m, g) + rr) * kN, S[m][rr]);
+    }
+    __syncthreads();   // the producers write out the last chunk's staged rows behind this one
+}
+
+// ------------------------------------------------------------------------------------------
+// Producer wave p: tokens 16p..16p+15 of every chunk.
+// ------------------------------------------------------------------------------------------
+template <bool kSave>
+__device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsigned char *smem, int *s_wild, int bh, int p, int lane)
+{
+    const int T = a.T, H = a.H;
+    const int g = lane >> 4, l16 = lane & 15;
+    const int64_t C = (int64_t)H * kN;
+    const int nchunk = T / kBlockTokens;
+    const int b = bh / H, h = bh - b * H;
+    const uint32_t rowbytes = (uint32_t)C * 2u;
+    const uint32_t lds0 = lds_address(smem);
+    const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
+    const bf16_t *rb = a.r + base, *kb_ = a.k + base, *vb = a.v + base, *wb = a.w + base;
+    bf16_t *yb = a.y + base;
+    char *ckb = kSave ? reinterpret_cast<char *>(a.ckpt + (int64_t)bh * nchunk * (kN * kN)) : nullptr;
+    // this lane's part of an 8-row block: row (lane >> 3), 16-byte piece swizzled with the row
+    const int lrow = lane >> 3;
+    const uint32_t lpiece = (uint32_t)(((lane & 7) ^ lrow) << 4);
+    // Vector-memory operations this wave has issued so far, and the count right after the r, k, w loads
+    // of visit j went out: a wave's operations complete in program order, so "the loads of visit j have
+    // landed" is "at most (issued - mark of j) operations are still in flight".
+    int issued = 0, mark_even = 0, mark_odd = 0;
+    auto issue_v = [&](int it) {
+        const uint32_t vv = lds0 + BlockFwdLds::kRawV + (it & 3) * kTileBytes + 16 * p * kTileRow;
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+            load_rows8_to_lds(vb, (uint32_t)(it * kBlockTokens + 16 * p + 8 * blk + lrow) * rowbytes + lpiece, vv + 8 * blk * kTileRow);
+        issued += 2;
+    };
+    auto issue_rkw = [&](int it) {
+        const uint32_t raw = lds0 + BlockFwdLds::kRaw + (it & 1) * 3 * kTileBytes + 16 * p * kTileRow;
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+            const uint32_t o = (uint32_t)(it * kBlockTokens + 16 * p + 8 * blk + lrow) * rowbytes + lpiece;
+            load_rows8_to_lds(wb, o, raw + 2 * kTileBytes + 8 * blk * kTileRow);
+            load_rows8_to_lds(rb, o, raw + 8 * blk * kTileRow);
+            load_rows8_to_lds(kb_, o, raw + kTileBytes + 8 * blk * kTileRow);
+        }
+        issued += 6;
+        if (it & 1) mark_odd = issued; else mark_even = issued;
+    };
+    // what the consumers staged during visit `it`, as whole rows: y rows of this wave's tokens and rows
+    // 16p..16p+15 of the chunk's state
+    auto store_staged = [&](int it) {
+        const unsigned char *ys = smem + BlockFwdLds::kYStage + (it & 1) * kTileBytes;
+        const unsigned char *ss = smem + BlockFwdLds::kSStage + (it & 1) * kTileBytes;
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+            const int row = 16 * p + 8 * blk + lrow;
+            const uint4 x = *reinterpret_cast<const uint4 *>(ys + row * kTileRow + (lane & 7) * 16);
+            *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(yb) + ((uint32_t)(it * kBlockTokens + row) * rowbytes + lpiece)) = x;
+            if (kSave) {
+                const uint4 s = *reinterpret_cast<const uint4 *>(ss + row * kTileRow + (lane & 7) * 16);
+                *reinterpret_cast<uint4 *>(ckb + ((uint32_t)it * (uint32_t)(kN * kN * 2) + (uint32_t)(row * kTileRow) + lpiece)) = s;
+            }
+        }
+        issued += kSave ? 4 : 2;
+    };
+    float u4[4];
+    load4(a.u + h * kN + 4 * l16, u4);
+    // visit `it` (its r, k, w loads have been issued); `next` >= 0: the visit whose r, k, w loads go out
+    // as soon as this one's raw rows are in registers (into the same LDS block)
+    auto prepare = [&](int it, int next) {
+        const unsigned char *raw = smem + BlockFwdLds::kRaw + (it & 1) * 3 * kTileBytes;
+        unsigned char *op = smem + BlockFwdLds::kOp + (it & 1) * 2 * kTileBytes;
+        float *vec = reinterpret_cast<float *>(smem + BlockFwdLds::kVec + (it & 1) * kBlockVecBytes);
+        wait_in_flight(issued - ((it & 1) ? mark_odd : mark_even));
+        const bool ok = block_prepare(raw, raw + kTileBytes, raw + 2 * kTileBytes, vec, u4, p, l16, g,
+            [&]() {
+                if (next >= 0) {
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    issue_rkw(next);
+                }
+            },
+            [&](uint32_t o, const float (&xr)[4], const float (&xk)[4], const float (&)[4], const float (&)[4]) {
+                *reinterpret_cast<uint2 *>(op + o) = make_uint2(pack_bf16x2(xr[0], xr[1]), pack_bf16x2(xr[2], xr[3]));
+                *reinterpret_cast<uint2 *>(op + kTileBytes + o) = make_uint2(pack_bf16x2(xk[0], xk[1]), pack_bf16x2(xk[2], xk[3]));
+            });
+        if (!ok && lane == 0) *s_wild = 1;
+    };
+    // r, k, w of visit j are requested three visits ahead (two in the prologue), v three visits ahead
+    issue_v(0);
+    issue_rkw(0);
+    if (nchunk > 1) { issue_v(1); issue_rkw(1); }
+    if (nchunk > 2) issue_v(2);
+    prepare(0, nchunk > 2 ? 2 : -1);
+    for (int it = 0; it < nchunk; ++it) {
+        __syncthreads();
+        // free again: the raw v block of visit it-1; the staging tiles of visit it-1 are complete
+        if (it + 3 < nchunk) issue_v(it + 3);
+        if (it > 0) store_staged(it - 1);
+        if (it + 1 < nchunk) prepare(it + 1, it + 3 < nchunk ? it + 3 : -1);
+    }
+    __syncthreads();
+    store_staged(nchunk - 1);
+    wait_loads<0>();
+}
+
+constexpr int kBlockFwdThreads = 12 * 64;
+
+template <typename Ts, bool kSave>
+__global__ __launch_bounds__(kBlockFwdThreads) void block_fwd_kernel(BlockFwdArgs a)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    __shared__ int s_wild;
+    static_assert(sizeof(ScanFwdLds) <= BlockFwdLds::kBytes, "the exact second pass reuses the LDS block");
+    if (threadIdx.x == 0) s_wild = 0;
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int bh = (int)blockIdx.x;
+    if (wave < 4) block_fwd_producer<kSave>(a, smem, &s_wild, bh, wave, lane);
+    else if (wave < 8) block_fwd_consumer<Ts, kSave, 0>(a, smem, bh, wave - 4, lane);
+    else block_fwd_consumer<Ts, kSave, 1>(a, smem, bh, wave - 8, lane);
+    // exact second pass if 16 tokens of this pair left the range the scaled operands can hold
+    __threadfence_block();
+    __syncthreads();
+    if (s_wild) {
+        __syncthreads();
+        scan_fwd_body<bf16_t, bf16_t, Ts>(*reinterpret_cast<ScanFwdLds *>(smem), bh / a.H, bh % a.H, a.T, a.H, a.r, a.k, a.v, a.w, a.u,
+                                          reinterpret_cast<const Ts *>(a.s0), a.map, a.y, reinterpret_cast<Ts *>(a.sT), false);
+    }
+}
+
+bool block_forward_applies(int64_t B, int64_t T, int64_t H) {
+    const int64_t pairs = B * H, cus = compute_units();
+    // (with fewer pairs than half the compute units the tile form shares a pair out over several workgroups)
+    return T >= kBlockTokens && (T % kBlockTokens) == 0 && pairs <= cus && 2 * pairs > cus;
+}
+
+hipError_t block_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
+                         const void *r, const void *k, const void *v, const void *w, const void *u,
+                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states, bool counters)
+{
+    BlockFwdArgs a = {};
+    a.T = (int)T; a.H = (int)H;
+    a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
+    a.s0 = s0; a.map = map; a.y = (bf16_t *)y; a.sT = sT; a.ckpt = (float *)saved_states;
+    a.arrivals = saved_states && counters ? reinterpret_cast<int *>(reinterpret_cast<char *>(saved_states) + chunk_backward_workspace_bytes(B, T, H)) : nullptr;
+    auto launch = [&](auto ts_tag, auto save_tag) -> hipError_t {
+        constexpr auto kern = block_fwd_kernel<decltype(ts_tag), decltype(save_tag)::value>;
+        hipError_t e = allow_dynamic_lds<kern>(BlockFwdLds::kBytes);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(kBlockFwdThreads), BlockFwdLds::kBytes, st, a);
+        return hipGetLastError();
+    };
+    const bool save = saved_states != nullptr;
+    if (state_dtype == kF32) return save ? launch(float{}, std::true_type{}) : launch(float{}, std::false_type{});
+    return save ? launch(bf16_t{}, std::true_type{}) : launch(bf16_t{}, std::false_type{});
+}
+
+}  // namespace wkv6

@@ -610,6 +610,8 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
                          const void *s0, const int64_t *map, void *y, void *sT, void *saved_states, float *dsum, bool reverse,
                          bool counters)
 {
+    if (y != nullptr && dsum == nullptr && !reverse && block_forward_applies(B, T, H))
+        return block_forward(st, state_dtype, B, T, H, r, k, v, w, u, s0, map, y, sT, saved_states, counters);
     FwdArgs a = {};
     a.dsum = dsum;
     a.reverse = reverse && (T % CL) == 0;

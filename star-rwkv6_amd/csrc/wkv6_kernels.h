@@ -59,6 +59,20 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
                          bool reverse = false,     // the time axis read back to front (T a multiple of 64, no y)
                          bool counters = true);    // saved_states ends with the per-head counters of the fused gu sum (zeroed here)
 
+// --- block form (wkv6_block_fwd.hip, wkv6_block_bwd.hip): a 64-token chunk as one block of the
+// recurrence; bf16 tensors, T a multiple of 64, between half a pair and one pair per compute unit.
+// Same arguments and the same saved-state layout as the tile form above, which takes every other case.
+bool block_forward_applies(int64_t B, int64_t T, int64_t H);
+hipError_t block_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
+                         const void *r, const void *k, const void *v, const void *w, const void *u,
+                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states, bool counters);
+
+bool block_backward_applies(int64_t B, int64_t T, int64_t H);
+// workspace: the chunk-start states as a forward pass leaves them, followed by the per-head counters; gu_sum may be null
+hipError_t block_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                          const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, void *gu_sum);
+
 // fp16 tensors on the chunked kernels (training pair only: y and the gradients are fp32).  r, k, w stay
 // fp16 (the kernels unpack them exactly); v and gy are consumed as bf16 MFMA operands, so the caller
 // keeps bf16 copies of them (convert_to_bf16) next to the saved states.
