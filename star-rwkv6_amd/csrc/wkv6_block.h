@@ -185,17 +185,20 @@ __device__ __forceinline__ bool block_prepare(const unsigned char *raw_r, const 
         for (int e = 0; e < 4; ++e) d[e] = sum_row16(d[e]);
         if (l16 == 0) *reinterpret_cast<float4 *>(&vec[4 * kN + 16 * p + 4 * g]) = make_float4(d[0], d[1], d[2], d[3]);
     }
+    float al[4];   // alpha_t of the lane's current token (the previous token's alpha_{t+1})
+#pragma unroll
+    for (int c = 0; c < 4; ++c) al[c] = exp2_fast(-ex[c]);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        float xr[4], xk[4], xa[4];
+        float xr[4], xk[4];
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            xr[c] = fr[e][c] * exp2_fast(-ex[c]);
+            xr[c] = fr[e][c] * al[c];
             ex[c] += ew2[e][c];
-            xa[c] = exp2_fast(-ex[c]);   // alpha_{t+1}
+            al[c] = exp2_fast(-ex[c]);   // alpha_{t+1}
             xk[c] = fk[e][c] * exp2_fast(ex[c]);
         }
-        emit(tile_off(16 * p + 4 * g + e, 4 * l16), xr, xk, xa, ew2[e]);
+        emit(tile_off(16 * p + 4 * g + e, 4 * l16), xr, xk, al, ew2[e]);
     }
     return __builtin_amdgcn_ballot_w64(!ok) == 0ull;
 }

@@ -74,6 +74,17 @@ __device__ __forceinline__ float prev_in_row16(float x, float first) {
     return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(first), __float_as_int(x), 0x111, 0xF, 0xF, false));
 }
 
+// Two 16-token row groups, each lane holding four channels (8 bytes: `a` of the first group's token l16,
+// `b` of the second group's) -> one 16-byte piece per lane: lanes of even g receive the channels
+// 4g .. 4g+7 of the first group's token, lanes of odd g the channels 4(g-1) .. 4g+3 of the second
+// group's (rows of 16 lanes are swapped between the two registers).
+__device__ __forceinline__ u32x4 pair_rows_8ch(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1)
+{
+    const auto x = __builtin_amdgcn_permlane16_swap(a0, b0, false, false);
+    const auto y = __builtin_amdgcn_permlane16_swap(a1, b1, false, false);
+    return (u32x4){x[0], y[0], x[1], y[1]};
+}
+
 // ------------------------------------------------------------------------------------------
 // Wave (q, HALF): key channels j = 16q .. 16q+15, block HALF of the visit (tokens 32 HALF .. +31):
 // gr, gk, gw, gu.  Gj[m]: reverse state, rows i = block_row_channel(m, g) + rr, column j = 16q + l16.
@@ -253,9 +264,9 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
         settle(X1[0], X1[1], W1[0], W1[1]);
         // elementwise pass: lane (l16, g) <-> token of row group n, channels 16q + 4g + rr
         const float g1s[4] = {g1r.x, g1r.y, g1r.z, g1r.w};
+        uint32_t packed[3][2][2];   // [gr, gk, gw][row group][channel pair]
 #pragma unroll
         for (int n = 0; n < 2; ++n) {
-            const int trow = (n == 0 ? R0 : R1) + l16;
             const uint32_t o = la_cols + (uint32_t)((n == 0 ? R0 : R1) * kTileRow);
             float rt_[4], kt_[4], an[4], ew[4];
             {
@@ -269,10 +280,11 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
             for (int rr = 0; rr < 4; ++rr) {
                 // alpha_t is the previous token's alpha_{t+1} (the lane before); the block's first token has
                 // 1 / g1, its middle token (the second group's first) exactly 1
-                const float a_t = prev_in_row16(an[rr], n == 0 ? __builtin_amdgcn_rcpf(g1s[rr]) : 1.f), a_n = an[rr];
+                const float a_n = an[rr], ia_n = __builtin_amdgcn_rcpf(a_n);
+                const float a_t = prev_in_row16(a_n, n == 0 ? __builtin_amdgcn_rcpf(g1s[rr]) : 1.f);
+                const float ia_t = prev_in_row16(ia_n, n == 0 ? g1s[rr] : 1.f);
                 const float X = fmaf(g1s[rr], X0[n][rr], X1[n][rr]);
                 const float W = W0[n][rr] + W1[n][rr];
-                const float ia_t = __builtin_amdgcn_rcpf(a_t), ia_n = __builtin_amdgcn_rcpf(a_n);
                 const float rraw = rt_[rr] * ia_t, kraw = kt_[rr] * a_n;
                 const float uvg = u4[rr] * vg[n];
                 Pv[rr] = rt_[rr] * X;
@@ -292,10 +304,16 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
             if ((HALF == 0 && n == 0 && c == 0 && l16 == 0) || (HALF == 1 && n == 1 && c == nchunk - 1 && l16 == 15)) {
                 gwo[0] = gwo[1] = gwo[2] = gwo[3] = 0.f;
             }
-            const uint32_t go = (uint32_t)(c * kBlockTokens + trow) * rowbytes + 2u * (uint32_t)(16 * q + 4 * g);
-            *reinterpret_cast<uint2 *>(gr_h + go) = make_uint2(pack_bf16x2(gro[0], gro[1]), pack_bf16x2(gro[2], gro[3]));
-            *reinterpret_cast<uint2 *>(gk_h + go) = make_uint2(pack_bf16x2(gko[0], gko[1]), pack_bf16x2(gko[2], gko[3]));
-            *reinterpret_cast<uint2 *>(gw_h + go) = make_uint2(pack_bf16x2(gwo[0], gwo[1]), pack_bf16x2(gwo[2], gwo[3]));
+            packed[0][n][0] = pack_bf16x2(gro[0], gro[1]); packed[0][n][1] = pack_bf16x2(gro[2], gro[3]);
+            packed[1][n][0] = pack_bf16x2(gko[0], gko[1]); packed[1][n][1] = pack_bf16x2(gko[2], gko[3]);
+            packed[2][n][0] = pack_bf16x2(gwo[0], gwo[1]); packed[2][n][1] = pack_bf16x2(gwo[2], gwo[3]);
+        }
+        {
+            // 16 bytes per lane: token (g odd ? R1 : R0) + l16, channels 16q + 8 (g >> 1) .. +7
+            const uint32_t go = (uint32_t)(c * kBlockTokens + R0 + 16 * (g & 1) + l16) * rowbytes + 2u * (uint32_t)(16 * q + 8 * (g >> 1));
+            *reinterpret_cast<u32x4 *>(gr_h + go) = pair_rows_8ch(packed[0][0][0], packed[0][0][1], packed[0][1][0], packed[0][1][1]);
+            *reinterpret_cast<u32x4 *>(gk_h + go) = pair_rows_8ch(packed[1][0][0], packed[1][0][1], packed[1][1][0], packed[1][1][1]);
+            *reinterpret_cast<u32x4 *>(gw_h + go) = pair_rows_8ch(packed[2][0][0], packed[2][0][1], packed[2][1][0], packed[2][1][1]);
         }
         __builtin_amdgcn_sched_barrier(0);
     }
@@ -379,10 +397,10 @@ __device__ __forceinline__ void block_bwd_gv(BlockGvState &st, const unsigned ch
             for (int m = 0; m < 4; ++m) { Gi[m] = mfma16(rq[0][m], gyq0, Gi[m]); Gi[m] = mfma16(rq[1][m], gyq1, Gi[m]); }
         }
         settle(GV0, GV1, V0, V1);
-        store4(gv_h + ((uint32_t)(c * kBlockTokens + r0) * rowelems + (uint32_t)(16 * q + 4 * g)),
-               GV0[0] + V0[0], GV0[1] + V0[1], GV0[2] + V0[2], GV0[3] + V0[3]);
-        store4(gv_h + ((uint32_t)(c * kBlockTokens + r1) * rowelems + (uint32_t)(16 * q + 4 * g)),
-               GV1[0] + V1[0], GV1[1] + V1[1], GV1[2] + V1[2], GV1[3] + V1[3]);
+        // 16 bytes per lane: token (g odd ? R1 : R0) + l16, channels 16q + 8 (g >> 1) .. +7
+        *reinterpret_cast<u32x4 *>(gv_h + ((uint32_t)(c * kBlockTokens + R0 + 16 * (g & 1) + l16) * rowelems + (uint32_t)(16 * q + 8 * (g >> 1)))) =
+            pair_rows_8ch(pack_bf16x2(GV0[0] + V0[0], GV0[1] + V0[1]), pack_bf16x2(GV0[2] + V0[2], GV0[3] + V0[3]),
+                          pack_bf16x2(GV1[0] + V1[0], GV1[1] + V1[1]), pack_bf16x2(GV1[2] + V1[2], GV1[3] + V1[3]));
         settle(Gi[0], Gi[1], Gi[2], Gi[3]);
         scale(vec + 2 * blk * kN);   // g1 of the block
     }
@@ -454,7 +472,7 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
 #pragma unroll
     for (int m = 0; m < 4; ++m) gvst.Gi[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
     // item `it` is loaded during visit it-2 (or the prologue), its state during visit it-1, and it is prepared during visit it-1
-    constexpr int kTileLoads = 10, kStateLoads = 2, kGvStores = 4;
+    constexpr int kTileLoads = 10, kStateLoads = 2, kGvStores = 2;
     issue_state(0);
     issue_loads(0);
     if (nchunk > 1) issue_loads(1);
