@@ -130,6 +130,17 @@ __device__ __forceinline__ void wait_in_flight(int n) {
     else wait_loads<0>();
 }
 
+// Two 16-token row groups, each lane holding four channels (8 bytes: `a` of the first group's token l16,
+// `b` of the second group's) -> one 16-byte piece per lane: lanes of even g receive the channels
+// 4g .. 4g+7 of the first group's token, lanes of odd g the channels 4(g-1) .. 4g+3 of the second
+// group's (rows of 16 lanes are swapped between the two registers).
+__device__ __forceinline__ u32x4 pair_rows_8ch(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1)
+{
+    const auto x = __builtin_amdgcn_permlane16_swap(a0, b0, false, false);
+    const auto y = __builtin_amdgcn_permlane16_swap(a1, b1, false, false);
+    return (u32x4){x[0], y[0], x[1], y[1]};
+}
+
 // Operand preparation of one producer wave (tokens 16p .. 16p+15 of a chunk; lane (l16, g) holds
 // channels 4 l16 .. +3 of tokens 4g .. 4g+3, all LDS accesses 8 bytes wide).  Reads the raw r, k, w
 // rows, leaves the per-visit vectors of this wave (its g1 or g2 row, its 16 diagonal sums) and hands

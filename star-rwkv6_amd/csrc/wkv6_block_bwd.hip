@@ -38,13 +38,15 @@ namespace wkv6 {
 struct BlockBwdLds {
     static constexpr int kRawRK = 0;                                   // [item % 3][r, k] raw tiles, turned into R~, K~ in place
     static constexpr int kRawW = kRawRK + 3 * 2 * kTileBytes;          // [item % 3] raw w tiles, turned into exp(w) in place
-    static constexpr int kRawVG = kRawW + 3 * kTileBytes;              // [item % 3][v, gy] raw tiles
-    static constexpr int kAlpha = kRawVG + 3 * 2 * kTileBytes;         // [item & 1] row t: alpha_{t+1}
+    static constexpr int kRawVG = kRawW + 3 * kTileBytes;              // [item & 1][v, gy] raw tiles
+    static constexpr int kAlpha = kRawVG + 2 * 2 * kTileBytes;         // [item & 1] row t: alpha_{t+1}
     static constexpr int kVec = kAlpha + 2 * kTileBytes;               // [item & 1] per-visit vectors
     static constexpr int kState = kVec + 2 * kBlockVecBytes;           // [item & 1] saved forward state of the chunk, bf16 [i][j] as a tile
     static constexpr int kScratch = kState + 2 * kTileBytes;           // [8 waves][16] floats
     static constexpr int kGu = kScratch + 8 * 16 * 4;                  // [64] floats: gu partial of half 1
-    static constexpr int kBytes = kGu + kN * 4;
+    static constexpr int kGFlags = kGu + kN * 4;                       // [2 blocks][4 q] visit number + 1 once the wave has written its columns of kGt
+    static constexpr int kGt = kGFlags + 64;                           // [2 blocks] g2 o G at the block's end, bf16 [j][i] tiles (what gv and W take)
+    static constexpr int kBytes = kGt + 2 * kTileBytes;
 };
 static_assert(BlockBwdLds::kBytes <= 160 * 1024, "LDS block of the block-form backward kernel");
 
@@ -74,16 +76,7 @@ __device__ __forceinline__ float prev_in_row16(float x, float first) {
     return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(first), __float_as_int(x), 0x111, 0xF, 0xF, false));
 }
 
-// Two 16-token row groups, each lane holding four channels (8 bytes: `a` of the first group's token l16,
-// `b` of the second group's) -> one 16-byte piece per lane: lanes of even g receive the channels
-// 4g .. 4g+7 of the first group's token, lanes of odd g the channels 4(g-1) .. 4g+3 of the second
-// group's (rows of 16 lanes are swapped between the two registers).
-__device__ __forceinline__ u32x4 pair_rows_8ch(uint32_t a0, uint32_t a1, uint32_t b0, uint32_t b1)
-{
-    const auto x = __builtin_amdgcn_permlane16_swap(a0, b0, false, false);
-    const auto y = __builtin_amdgcn_permlane16_swap(a1, b1, false, false);
-    return (u32x4){x[0], y[0], x[1], y[1]};
-}
+typedef volatile int __attribute__((address_space(3))) *LdsFlag;
 
 // ------------------------------------------------------------------------------------------
 // Wave (q, HALF): key channels j = 16q .. 16q+15, block HALF of the visit (tokens 32 HALF .. +31):
@@ -107,16 +100,19 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
     float u4[4];
     load4(a.u + h * kN + 16 * q + 4 * g, u4);   // u of this lane's four channels 16q + 4g + rr
     float gu_acc[4] = {0.f, 0.f, 0.f, 0.f};
+    float pend = 1.f;   // per-column factor the reverse state Gj has still to be multiplied with
     float *scratch = reinterpret_cast<float *>(smem + BlockBwdLds::kScratch) + (4 * HALF + q) * 16;
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
     const BlockLane la(l16, g);
     const uint32_t la_state = block_lane_state(q, l16, g), la_cols = block_lane_cols4(q, l16, g);
+    const uint32_t gt_lo = tile_off(col, 8 * g), gt_hi = tile_off(col, 32 + 8 * g);
+    LdsFlag g_flags = (LdsFlag)(smem + BlockBwdLds::kGFlags);
     for (int it = 0; it < nchunk; ++it) {
         const int c = nchunk - 1 - it;
         __syncthreads();
         const unsigned char *rt = smem + BlockBwdLds::kRawRK + (it % 3) * 2 * kTileBytes, *kt = rt + kTileBytes;
         const unsigned char *wt = smem + BlockBwdLds::kRawW + (it % 3) * kTileBytes;
-        const unsigned char *vt = smem + BlockBwdLds::kRawVG + (it % 3) * 2 * kTileBytes, *gyt = vt + kTileBytes;
+        const unsigned char *vt = smem + BlockBwdLds::kRawVG + (it & 1) * 2 * kTileBytes, *gyt = vt + kTileBytes;
         const unsigned char *at = smem + BlockBwdLds::kAlpha + (it & 1) * kTileBytes;
         const float *vec = reinterpret_cast<const float *>(smem + BlockBwdLds::kVec + (it & 1) * kBlockVecBytes);
         const unsigned char *stt = smem + BlockBwdLds::kState + (it & 1) * kTileBytes;
@@ -130,9 +126,18 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
         // One step of the reverse state over block `blk`; leaves g2 o G (what W of that block takes) as operands.
         bf16x8 GmL, GmH;
         auto step_G = [&](int blk, float g1c, float g2c, bool keep_operand) {
+            const float f = pend * g2c;   // (the g1 of the step before is still owed)
 #pragma unroll
-            for (int m = 0; m < 4; ++m) { Gj[m][0] *= g2c; Gj[m][1] *= g2c; Gj[m][2] *= g2c; Gj[m][3] *= g2c; }
-            if (keep_operand) { GmL = acc_as_operand(Gj[0], Gj[1]); GmH = acc_as_operand(Gj[2], Gj[3]); }
+            for (int m = 0; m < 4; ++m) { Gj[m][0] *= f; Gj[m][1] *= f; Gj[m][2] *= f; Gj[m][3] *= f; }
+            if (keep_operand) {
+                GmL = acc_as_operand(Gj[0], Gj[1]); GmH = acc_as_operand(Gj[2], Gj[3]);
+                // also for the gv role of the producer waves: row j = col, value channels 8g .. 8g+7 and 32 + 8g .. +7
+                unsigned char *gt = smem + BlockBwdLds::kGt + blk * kTileBytes;
+                *reinterpret_cast<bf16x8 *>(gt + gt_lo) = GmL;
+                *reinterpret_cast<bf16x8 *>(gt + gt_hi) = GmH;
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                if (lane == 0) g_flags[4 * blk + q] = it + 1;
+            }
             s16x4 gq[2][4], rtq[2];
 #pragma unroll
             for (int pp = 0; pp < 2; ++pp) {
@@ -145,8 +150,7 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
 #pragma unroll
                 for (int m = 0; m < 4; ++m) Gj[m] = mfma16(gq[pp][m], rtq[pp], Gj[m]);
             settle(Gj[0], Gj[1], Gj[2], Gj[3]);
-#pragma unroll
-            for (int m = 0; m < 4; ++m) { Gj[m][0] *= g1c; Gj[m][1] *= g1c; Gj[m][2] *= g1c; Gj[m][3] *= g1c; }
+            pend = g1c;
         };
         // E[j = col] = sum_i S[j][i] G[j][i] with S as fp32 values in the layout of Gj; then to the lanes that hold channel col as a row
         float pre[4];
@@ -157,7 +161,7 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
                 e0 = fmaf(Sv[m][0], Gj[m][0], e0); e1 = fmaf(Sv[m][1], Gj[m][1], e1);
                 e0 = fmaf(Sv[m][2], Gj[m][2], e0); e1 = fmaf(Sv[m][3], Gj[m][3], e1);
             }
-            const float E = sum_rows(e0 + e1);
+            const float E = sum_rows((e0 + e1) * pend);
             if (g == 0) scratch[l16] = E;
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // (one wave: its LDS accesses are executed in order)
             const float4 E4 = *reinterpret_cast<const float4 *>(&scratch[4 * g]);
@@ -331,32 +335,33 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
 }
 
 // ------------------------------------------------------------------------------------------
-// gv role of a producer wave: wave q owns value columns i = 16q..16q+15 of the reverse state,
-// Gi[m]: rows j = block_row_channel(m, g) + rr, column i = 16q + l16.
+// gv role of a producer wave: wave q owns value columns i = 16q..16q+15.  The reverse state comes from
+// the waves that step it (g2 o G at the end of each block, as they publish it in kGt).
 // ------------------------------------------------------------------------------------------
-struct BlockGvState { f32x4 Gi[4]; };
-
-__device__ __forceinline__ void block_bwd_gv(BlockGvState &st, const unsigned char *smem, bf16_t *gv_h, uint32_t rowelems,
-                                             int c, int it, int q, int lane)
+__device__ __forceinline__ void block_bwd_gv(const unsigned char *smem, bf16_t *gv_h, uint32_t rowelems, int c, int it, int q, int lane)
 {
     const int g = lane >> 4, l16 = lane & 15;
-    f32x4 (&Gi)[4] = st.Gi;
     const unsigned char *rt = smem + BlockBwdLds::kRawRK + (it % 3) * 2 * kTileBytes, *kt = rt + kTileBytes;
-    const unsigned char *gyt = smem + BlockBwdLds::kRawVG + (it % 3) * 2 * kTileBytes + kTileBytes;
+    const unsigned char *gyt = smem + BlockBwdLds::kRawVG + (it & 1) * 2 * kTileBytes + kTileBytes;
     const float *vec = reinterpret_cast<const float *>(smem + BlockBwdLds::kVec + (it & 1) * kBlockVecBytes), *ruk = vec + 4 * kN;
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
     const BlockLane la(l16, g);
-    auto scale = [&](const float *gv) {
-#pragma unroll
-        for (int m = 0; m < 4; ++m) {
-            const float4 gg = *reinterpret_cast<const float4 *>(&gv[block_row_channel(m, g)]);
-            Gi[m][0] *= gg.x; Gi[m][1] *= gg.y; Gi[m][2] *= gg.z; Gi[m][3] *= gg.w;
-        }
-    };
+    // operand fragment G[j = 32h + 8g + e][i = 16q + l16], e < 8, out of the [j][i] tile: two transposing reads of
+    // four rows each (rows 8g + (l16 >> 2) and four further on, the lane's 8-byte piece of channels 16q + 4 (l16 & 3) ..)
+    const uint32_t gt_a = ((uint32_t)(8 * g + (l16 >> 2)) << 7) + ((((uint32_t)(2 * q) | (((uint32_t)l16 >> 1) & 1u)) ^ ((uint32_t)l16 >> 2)) << 4) + (((uint32_t)l16 & 1u) << 3);
+    const uint32_t gt_b = (gt_a ^ 64u) + 4 * kTileRow;
+    LdsFlag g_flags = (LdsFlag)(smem + BlockBwdLds::kGFlags);
 #pragma unroll
     for (int blk = 1; blk >= 0; --blk) {
-        scale(vec + (2 * blk + 1) * kN);   // g2 of the block: G decayed from the block's end to its middle
-        const bf16x8 GmL = acc_as_operand(Gi[0], Gi[1]), GmH = acc_as_operand(Gi[2], Gi[3]);
+        while (g_flags[4 * blk] < it + 1 || g_flags[4 * blk + 1] < it + 1 || g_flags[4 * blk + 2] < it + 1 || g_flags[4 * blk + 3] < it + 1)
+            __builtin_amdgcn_s_sleep(1);
+        const unsigned char *gt = smem + BlockBwdLds::kGt + blk * kTileBytes;
+        auto g_frag = [&](int h) {
+            const u32x2 lo = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(gt + gt_a + h * 32 * kTileRow)));
+            const u32x2 hi = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(gt + gt_b + h * 32 * kTileRow)));
+            return make_bf16x8(lo[0], lo[1], hi[0], hi[1]);
+        };
+        const bf16x8 GmL = g_frag(0), GmH = g_frag(1);
         const int R0 = 32 * blk, R1 = R0 + 16, r0 = R0 + l16, r1 = R1 + l16;
         const s16x4 gyq0 = la.frag_tok(gyt, q, R0), gyq1 = la.frag_tok(gyt, q, R1);
         const float ruk0 = ruk[r0], ruk1 = ruk[r1];
@@ -386,23 +391,11 @@ __device__ __forceinline__ void block_bwd_gv(BlockGvState &st, const unsigned ch
         }
         f32x4 V0 = mfma16(gyq0, pack4(A00), zero), V1 = mfma16(gyq1, pack4(A11), zero);
         V0 = mfma16(gyq1, pack4(A10), V0);
-        // G <- g1 o (g2 o G + R~^T gY) over the block
-        {
-            s16x4 rq[2][4];
-#pragma unroll
-            for (int pp = 0; pp < 2; ++pp)
-#pragma unroll
-                for (int m = 0; m < 4; ++m) rq[pp][m] = la.frag_tok_rows(rt, m, 32 * blk + 16 * pp);
-#pragma unroll
-            for (int m = 0; m < 4; ++m) { Gi[m] = mfma16(rq[0][m], gyq0, Gi[m]); Gi[m] = mfma16(rq[1][m], gyq1, Gi[m]); }
-        }
         settle(GV0, GV1, V0, V1);
         // 16 bytes per lane: token (g odd ? R1 : R0) + l16, channels 16q + 8 (g >> 1) .. +7
         *reinterpret_cast<u32x4 *>(gv_h + ((uint32_t)(c * kBlockTokens + R0 + 16 * (g & 1) + l16) * rowelems + (uint32_t)(16 * q + 8 * (g >> 1)))) =
             pair_rows_8ch(pack_bf16x2(GV0[0] + V0[0], GV0[1] + V0[1]), pack_bf16x2(GV0[2] + V0[2], GV0[3] + V0[3]),
                           pack_bf16x2(GV1[0] + V1[0], GV1[1] + V1[1]), pack_bf16x2(GV1[2] + V1[2], GV1[3] + V1[3]));
-        settle(Gi[0], Gi[1], Gi[2], Gi[3]);
-        scale(vec + 2 * blk * kN);   // g1 of the block
     }
 }
 
@@ -424,28 +417,32 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
     bf16_t *gvb = a.gv + base;
     const int lrow = lane >> 3;
     const uint32_t lpiece = (uint32_t)(((lane & 7) ^ lrow) << 4);
-    // item `it` = chunk nchunk-1-it
-    auto issue_loads = [&](int it) {
+    // item `it` = chunk nchunk-1-it.  r, k, w go out two visits ahead (they are prepared one visit ahead),
+    // v, gy and the chunk's saved state one visit ahead.
+    auto issue_rkw = [&](int it) {
         const int tb = (nchunk - 1 - it) * kBlockTokens + 16 * p;
         const uint32_t rk = lds0 + BlockBwdLds::kRawRK + (it % 3) * 2 * kTileBytes + 16 * p * kTileRow;
         const uint32_t ww = lds0 + BlockBwdLds::kRawW + (it % 3) * kTileBytes + 16 * p * kTileRow;
-        const uint32_t vg = lds0 + BlockBwdLds::kRawVG + (it % 3) * 2 * kTileBytes + 16 * p * kTileRow;
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
             const uint32_t o = (uint32_t)(tb + 8 * hf + lrow) * rowbytes + lpiece;
             load_rows8_to_lds(kb_, o, rk + kTileBytes + 8 * hf * kTileRow);
             load_rows8_to_lds(wb, o, ww + 8 * hf * kTileRow);
-            load_rows8_to_lds(vb, o, vg + 8 * hf * kTileRow);
             load_rows8_to_lds(rb, o, rk + 8 * hf * kTileRow);
-            load_rows8_to_lds(gb, o, vg + kTileBytes + 8 * hf * kTileRow);
         }
     };
-    auto issue_state = [&](int it) {
+    auto issue_vg_state = [&](int it) {
+        const int tb = (nchunk - 1 - it) * kBlockTokens + 16 * p;
+        const uint32_t vg = lds0 + BlockBwdLds::kRawVG + (it & 1) * 2 * kTileBytes + 16 * p * kTileRow;
         const bf16_t *src = ckb + (int64_t)(nchunk - 1 - it) * (kN * kN);
         const uint32_t dst = lds0 + BlockBwdLds::kState + (it & 1) * kTileBytes + 16 * p * kTileRow;
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf)
+        for (int hf = 0; hf < 2; ++hf) {
+            const uint32_t o = (uint32_t)(tb + 8 * hf + lrow) * rowbytes + lpiece;
             load_rows8_to_lds(src, (uint32_t)((16 * p + 8 * hf + lrow) * kTileRow) + lpiece, dst + 8 * hf * kTileRow);
+            load_rows8_to_lds(vb, o, vg + 8 * hf * kTileRow);
+            load_rows8_to_lds(gb, o, vg + kTileBytes + 8 * hf * kTileRow);
+        }
     };
     float u4[4];
     load4(a.u + h * kN + 4 * l16, u4);
@@ -468,26 +465,22 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
             });
         if (!ok && lane == 0) *s_wild = 1;
     };
-    BlockGvState gvst;
-#pragma unroll
-    for (int m = 0; m < 4; ++m) gvst.Gi[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    // item `it` is loaded during visit it-2 (or the prologue), its state during visit it-1, and it is prepared during visit it-1
-    constexpr int kTileLoads = 10, kStateLoads = 2, kGvStores = 2;
-    issue_state(0);
-    issue_loads(0);
-    if (nchunk > 1) issue_loads(1);
-    prepare(0, nchunk > 1 ? kTileLoads : 0);
+    constexpr int kRkwLoads = 6, kVgStateLoads = 6, kGvStores = 2;
+    issue_vg_state(0);
+    issue_rkw(0);
+    if (nchunk > 1) issue_rkw(1);
+    prepare(0, nchunk > 1 ? kRkwLoads : 0);
     for (int it = 0; it < nchunk; ++it) {
         __syncthreads();
-        // free again: the r, k, w, v, gy blocks and the state tile of item it-1
-        const int state_loads = it + 1 < nchunk ? kStateLoads : 0, tile_loads = it + 2 < nchunk ? kTileLoads : 0;
-        if (it + 1 < nchunk) issue_state(it + 1);
-        if (it + 2 < nchunk) issue_loads(it + 2);
-        // behind the tile loads of item it+1 (issued one visit ago): that visit's gv stores, and this visit's loads
-        if (it + 1 < nchunk) prepare(it + 1, (it > 0 ? kGvStores : 0) + state_loads + tile_loads);
-        block_bwd_gv(gvst, smem, gvb, (uint32_t)C, nchunk - 1 - it, it, p, lane);
-        // the next item's state has to be in LDS when the other waves pass the barrier
-        if (it + 1 < nchunk) wait_in_flight(tile_loads + kGvStores);
+        // free again: every tile of item it-1
+        const int vgs = it + 1 < nchunk ? kVgStateLoads : 0, rkw = it + 2 < nchunk ? kRkwLoads : 0;
+        if (it + 1 < nchunk) issue_vg_state(it + 1);
+        if (it + 2 < nchunk) issue_rkw(it + 2);
+        // behind the r, k, w loads of item it+1 (issued one visit ago): that visit's gv stores, and this visit's loads
+        if (it + 1 < nchunk) prepare(it + 1, (it > 0 ? kGvStores : 0) + vgs + rkw);
+        block_bwd_gv(smem, gvb, (uint32_t)C, nchunk - 1 - it, it, p, lane);
+        // v, gy and the state of the next item have to be in LDS when the other waves pass the barrier
+        if (it + 1 < nchunk) wait_in_flight(rkw + kGvStores);
     }
     wait_loads<0>();
     __threadfence_block();
@@ -503,6 +496,7 @@ __global__ __launch_bounds__(kBlockBwdThreads) void block_bwd_kernel(BlockBwdArg
     static_assert(sizeof(ScanBwdALds) <= BlockBwdLds::kBytes && sizeof(ScanBwdBLds) <= BlockBwdLds::kBytes,
                   "the exact second pass reuses the LDS block");
     if (threadIdx.x == 0) s_wild = 0;
+    if (threadIdx.x < 8) reinterpret_cast<int *>(smem + BlockBwdLds::kGFlags)[threadIdx.x] = 0;
     __syncthreads();
 
     const int bh = (int)blockIdx.x;
