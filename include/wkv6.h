@@ -44,17 +44,22 @@ enum {
 
 /* Algorithm selector for the *_ex entry points. */
 enum {
-    WKV6_ALGO_AUTO = 0,  /* library picks: chunked MFMA path for bf16 tensors with T >= 32 (and for
-                            fp16 tensors in the training pair wkv6_forward_save / wkv6_backward_saved*),
-                            else scan                                                          */
+    WKV6_ALGO_AUTO = 0,  /* library picks: chunked MFMA path for bf16 tensors with T >= 32, else scan.
+                            fp16 and fp32 tensors always take the scan: their results are fp32-exact
+                            (1e-4 class), the same with and without a gradient                   */
     WKV6_ALGO_SCAN = 1,  /* per-timestep fp32 recurrence, state in VGPRs                       */
     WKV6_ALGO_CHUNK = 2  /* chunk-parallel form, bf16 MFMA for the dense intra-chunk products: bf16
                             tensors in every call; fp16 tensors (fp32 outputs) in the training pair
-                            only, where r, k, w are unpacked exactly and v, gy reach the MFMAs as
-                            bf16 copies kept in the saved block.  A workgroup whose (batch, head)
-                            pair has a 16-token tile with decay beyond what the operand scaling can
-                            hold redoes that pair with the exact per-timestep code inside the same
-                            launch                                                             */
+                            wkv6_forward_save / wkv6_backward_saved* only, where r, k, w are
+                            unpacked exactly and v, gy reach the MFMAs as bf16 copies kept in the
+                            saved block.  ACCURACY: for fp16 tensors this is an explicit trade --
+                            the fp32-typed y and gradients then carry bf16 operand precision
+                            (relative error up to 1e-2, against 1e-4 of the scan), and differ by
+                            that much from what wkv6_forward returns for the same inputs (calls
+                            without a gradient always take the scan for fp16).  A workgroup whose
+                            (batch, head) pair has a 16-token tile with decay beyond what the
+                            operand scaling can hold redoes that pair with the exact per-timestep
+                            code inside the same launch                                        */
 };
 
 const char *wkv6_status_string(int status);

@@ -35,13 +35,16 @@ void *static_scratch(hipError_t *err) {
 bool chunk_possible(int dtype, int64_t T, int64_t C) { return dtype == WKV6_BF16 && T * C < (1LL << 31); }
 bool chunk_eligible(int dtype, int64_t T, int64_t C) { return chunk_possible(dtype, T, C) && T >= 32; }
 
-// The training pair (wkv6_forward_save / wkv6_backward_saved*) also runs fp16 tensors on the chunked
+// The training pair (wkv6_forward_save / wkv6_backward_saved*) can also run fp16 tensors on the chunked
 // kernels: r, k, w are unpacked exactly, v and gy go through bf16 copies kept behind the saved states.
+// That gives fp32-typed outputs of bf16 operand precision (1e-2 class), which differ from what the
+// exact per-timestep kernels return for the same fp16 inputs (every call without a gradient takes
+// those): only on request (WKV6_ALGO_CHUNK), never under WKV6_ALGO_AUTO.
 bool train_chunk(int dtype, int algo, int64_t T, int64_t C) {
     if (dtype != WKV6_BF16 && dtype != WKV6_F16) return false;
     // (the kernels address a (b, h) pair's rows with 32-bit byte offsets; fp16 tensors have 4-byte outputs)
     if (T * C >= (dtype == WKV6_F16 ? 1LL << 30 : 1LL << 31)) return false;
-    return algo == WKV6_ALGO_CHUNK || (algo == WKV6_ALGO_AUTO && T >= 32);
+    return algo == WKV6_ALGO_CHUNK || (algo == WKV6_ALGO_AUTO && dtype == WKV6_BF16 && T >= 32);
 }
 
 thread_local int g_last_status = WKV6_OK;
@@ -192,6 +195,7 @@ int wkv6_forward_gn_gate_save(void *stream, int dtype, int64_t B, int64_t T, int
     if (!r || !k || !v || !w || !u || !gate || !gn_scale || !gn_offset || !out || !y || !stats) return WKV6_ERR_ARG;
     if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(gate) || !aligned16(out) || !aligned16(y) ||
         !aligned16(stats) || !aligned16(gn_scale) || !aligned16(gn_offset)) return WKV6_ERR_ARG;
+    if (!(gn_eps >= 0.f)) return WKV6_ERR_ARG;
     const size_t need = wkv6_saved_bytes(dtype, WKV6_ALGO_CHUNK, B, T, C, H);
     if (!saved || saved_bytes < need || !aligned16(saved)) return WKV6_ERR_WORKSPACE;
     return finish(wkv6::chunk_forward_fused_save((hipStream_t)stream, B, T, H, r, k, v, w, u, gate, gn_scale, gn_offset, gn_eps,
@@ -206,6 +210,8 @@ int wkv6_gn_gate_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t
     if (rc != WKV6_OK) return rc;
     if (dtype != WKV6_BF16) return WKV6_ERR_UNSUPPORTED;
     if (!gout || !y || !stats || !gate || !gn_scale || !gn_offset || !gy || !ggate || !gscale || !goffset) return WKV6_ERR_ARG;
+    if (!aligned16(gout) || !aligned16(y) || !aligned16(stats) || !aligned16(gate) || !aligned16(gn_scale) || !aligned16(gn_offset) ||
+        !aligned16(gy) || !aligned16(ggate) || !aligned16(gscale) || !aligned16(goffset)) return WKV6_ERR_ARG;
     return finish(wkv6::gn_gate_backward((hipStream_t)stream, B, T, H, gout, y, stats, gate, gn_scale, gn_offset, gy, ggate, gscale, goffset));
 }
 
@@ -225,6 +231,7 @@ int wkv6_shift_mix_x(void *stream, int dtype, int64_t B, int64_t T, int64_t C,
     const int rc = check_mix(dtype, B, T, C, 32);
     if (rc != WKV6_OK) return rc;
     if (!x || !mix_x || !x_mix) return WKV6_ERR_ARG;
+    if (!aligned16(x) || !aligned16(mix_x) || !aligned16(x_mix)) return WKV6_ERR_ARG;
     return finish(wkv6::shift_mix_x((hipStream_t)stream, B, T, C, x, mix_x, x_mix));
 }
 
@@ -234,6 +241,8 @@ int wkv6_shift_mix_five(void *stream, int dtype, int64_t B, int64_t T, int64_t C
     const int rc = check_mix(dtype, B, T, C, R);
     if (rc != WKV6_OK) return rc;
     if (!x || !h || !w2t || !bias || !xr || !xk || !xv || !xw || !xg) return WKV6_ERR_ARG;
+    if (!aligned16(x) || !aligned16(h) || !aligned16(w2t) || !aligned16(bias) || !aligned16(xr) || !aligned16(xk) || !aligned16(xv) ||
+        !aligned16(xw) || !aligned16(xg)) return WKV6_ERR_ARG;
     void *const out[5] = {xr, xk, xv, xw, xg};
     return finish(wkv6::shift_mix_five((hipStream_t)stream, B, T, C, R, x, h, w2t, bias, out));
 }
@@ -246,6 +255,8 @@ int wkv6_shift_mix_five_backward(void *stream, int dtype, int64_t B, int64_t T, 
     if (rc != WKV6_OK) return rc;
     if (!x || !h || !w2t || !bias || !gxr || !gxk || !gxv || !gxw || !gxg || !gcoef || !gp || !gxx) return WKV6_ERR_ARG;
     if (gcoef_stride < B * T * C || gcoef_stride % 8 != 0) return WKV6_ERR_ARG;
+    if (!aligned16(x) || !aligned16(h) || !aligned16(w2t) || !aligned16(bias) || !aligned16(gxr) || !aligned16(gxk) || !aligned16(gxv) ||
+        !aligned16(gxw) || !aligned16(gxg) || !aligned16(gcoef) || !aligned16(gp) || !aligned16(gxx)) return WKV6_ERR_ARG;
     const void *const gout[5] = {gxr, gxk, gxv, gxw, gxg};
     return finish(wkv6::shift_mix_five_backward((hipStream_t)stream, B, T, C, R, x, h, w2t, bias, gout, gcoef, gcoef_stride, gp, gxx));
 }
@@ -256,6 +267,8 @@ int wkv6_shift_mix_x_backward(void *stream, int dtype, int64_t B, int64_t T, int
     const int rc = check_mix(dtype, B, T, C, 32);
     if (rc != WKV6_OK) return rc;
     if (!x || !mix_x || !gxm || !gx || !gmix_x || (gp == nullptr) != (gxx == nullptr)) return WKV6_ERR_ARG;
+    if (!aligned16(x) || !aligned16(mix_x) || !aligned16(gp) || !aligned16(gxx) || !aligned16(gxm) || !aligned16(gx) || !aligned16(gmix_x))
+        return WKV6_ERR_ARG;
     return finish(wkv6::shift_mix_x_backward((hipStream_t)stream, B, T, C, x, mix_x, gp, gxx, gxm, gx, gmix_x));
 }
 

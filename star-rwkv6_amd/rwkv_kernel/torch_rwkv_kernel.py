@@ -166,10 +166,20 @@ class _WKV6GnGate(torch.autograd.Function):
             with torch.cuda.device(r.device):
                 _native.check(lib.wkv6_gn_gate_backward(_stream(), code, B, T, C, H, _ptr(gout), _ptr(y), _ptr(stats), _ptr(gate),
                                                         _ptr(sc), _ptr(of), _ptr(gy), _ptr(ggate), _ptr(gsc), _ptr(gof)))
-                _native.check(lib.wkv6_backward_saved_sum(_stream(), code, _native.ALGO_CHUNK, B, T, C, H,
-                                                          _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(gy),
-                                                          _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu), _ptr(gu_sum),
-                                                          _ptr(saved), saved.numel()))
+                if saved is not None:
+                    _native.check(lib.wkv6_backward_saved_sum(_stream(), code, _native.ALGO_CHUNK, B, T, C, H,
+                                                              _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(gy),
+                                                              _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu), _ptr(gu_sum),
+                                                              _ptr(saved), saved.numel()))
+                else:
+                    # a second backward over the same graph (retain_graph): the saved block went with the
+                    # first one (its counters are used up); the plain backward rebuilds the states itself
+                    ws_bytes = lib.wkv6_backward_workspace_bytes_ex(code, _native.ALGO_CHUNK, B, T, C, H)
+                    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=r.device) if ws_bytes else None
+                    _native.check(lib.wkv6_backward_ex(_stream(), code, _native.ALGO_CHUNK, B, T, C, H,
+                                                       _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(gy),
+                                                       _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu), _ptr(ws), ws_bytes))
+                    gu_sum = torch.sum(gu, 0)
             s_shape, o_shape, s_dt, o_dt = ctx.param_shapes
             return (None, None, None, None, gr, gk, gv, gw, gu_sum.reshape(u.shape), ggate,
                     gsc.reshape(s_shape).to(s_dt), gof.reshape(o_shape).to(o_dt), None)

@@ -80,6 +80,33 @@ def test_argument_validation_returns_status_codes(native):
     assert lib.wkv6_forward_with_state(None, native.BF16, 2, 16, 128, 2, 1, None, *args[:5], None, fake, fake) == 1
 
 
+def test_misaligned_pointers_are_refused_by_the_fused_entry_points(native):
+    """The token-shift, low-rank-mixer and group-norm entry points use 16-byte vector accesses on every
+    tensor argument: a pointer off a 16-byte boundary is WKV6_ERR_ARG before anything is launched, as in
+    the operator's own entry points; so is a negative or NaN epsilon."""
+    lib = native.load()
+    ok, off = 0x10000, 0x10008
+    B, T, C, R, H = 2, 64, 128, 32, 2
+
+    def variants(n):
+        for i in range(n):
+            yield [off if j == i else ok for j in range(n)]
+
+    for a in variants(3):
+        assert lib.wkv6_shift_mix_x(None, native.BF16, B, T, C, *a) == 1, a
+    for a in variants(9):
+        assert lib.wkv6_shift_mix_five(None, native.BF16, B, T, C, R, *a) == 1, a
+    for a in variants(12):
+        assert lib.wkv6_shift_mix_five_backward(None, native.BF16, B, T, C, R, *a[:10], B * T * C, *a[10:]) == 1, a
+    for a in variants(7):
+        assert lib.wkv6_shift_mix_x_backward(None, native.BF16, B, T, C, *a) == 1, a
+    for a in variants(10):
+        assert lib.wkv6_gn_gate_backward(None, native.BF16, B, T, C, H, *a) == 1, a
+    saved = lib.wkv6_saved_bytes(native.BF16, native.ALGO_CHUNK, B, T, C, H)
+    for eps in (-1.0, float("nan")):
+        assert lib.wkv6_forward_gn_gate_save(None, native.BF16, B, T, C, H, *([ok] * 8), eps, ok, ok, ok, ok, saved) == 1, eps
+
+
 def test_custom_call_rejects_bad_opaque_without_throwing(native):
     lib = native.load()
     arr = (ctypes.c_void_p * 12)(*([0x1000] * 12))

@@ -116,6 +116,53 @@ def test_backward_kernels(lib, B, T, C, R):
     check_close("gmix_x", gmix.cpu().double().numpy(), mix.grad.numpy(), torch.float32, is_grad=True)
 
 
+def test_backward_kernels_full_size(lib):
+    """The two backward kernels at the training benchmark's layer shape (B=8, T=1024, C=2048, rank 32)
+    with random coefficients: every output of one batch row (a row's tokens only see that row) against
+    the formulas' autograd in float64, and gmix_x -- a sum over all rows and tokens -- against its
+    float64 value over everything."""
+    from rwkv_kernel import _native
+    B, T, C, R, row = 8, 1024, 2048, 32, 5
+    print("shift_mix backward kernels, full size", flush=True)
+    dev, ref = _inputs(B, T, C, R, 4242)
+    g = torch.Generator().manual_seed(4243)
+    h = torch.tanh(torch.randn(B, T, 5, R, generator=g)).to(BF16).cuda()
+    gouts = [torch.randn(B, T, C, generator=g).to(BF16).cuda() for _ in range(5)]
+    gxm = torch.randn(B, T, C, generator=g).to(BF16).cuda()
+    plane = B * T * C
+    gcoef = torch.full((5, B * T, C), float("nan"), dtype=BF16, device="cuda")
+    gp, gxx, gx = (torch.full_like(dev["x"], float("nan")) for _ in range(3))
+    gmix = torch.full((C,), 7.0, device="cuda")
+    _native.check(lib.wkv6_shift_mix_five_backward(
+        _stream(), _native.BF16, B, T, C, R, dev["x"].data_ptr(), h.data_ptr(), dev["w2t"].data_ptr(), dev["bias"].data_ptr(),
+        *[go.data_ptr() for go in gouts], gcoef.data_ptr(), plane, gp.data_ptr(), gxx.data_ptr()))
+    _native.check(lib.wkv6_shift_mix_x_backward(_stream(), _native.BF16, B, T, C, dev["x"].data_ptr(), dev["mix_x"].data_ptr(),
+                                                gp.data_ptr(), gxx.data_ptr(), gxm.data_ptr(), gx.data_ptr(), gmix.data_ptr()))
+    torch.cuda.synchronize()
+    # one row in float64
+    x = torch.tensor(ref["x"][row:row + 1], requires_grad=True)
+    mix = torch.tensor(ref["mix_x"], requires_grad=True)
+    hh = torch.tensor(to_np(h[row:row + 1]))
+    go = [torch.tensor(to_np(t[row:row + 1])) for t in gouts]
+    coef_leaf = [(hh[:, :, s] @ torch.tensor(ref["w2t"][s]).T + torch.tensor(ref["bias"][s])).requires_grad_(True) for s in range(5)]
+    xx = torch.cat([torch.zeros(1, 1, C, dtype=torch.float64), x[:, :-1]], 1) - x
+    xx_leaf = xx.detach().requires_grad_(True)
+    sum(((x.detach() + xx_leaf * coef_leaf[s]) * go[s]).sum() for s in range(5)).backward()
+    want_gxx = xx_leaf.grad.numpy()
+    check_close("gcoef", gcoef.view(5, B, T, C)[:, row:row + 1], np.stack([c.grad.numpy() for c in coef_leaf]), BF16, is_grad=True)
+    check_close("gxx", gxx[row:row + 1], want_gxx, BF16, is_grad=True)
+    check_close("gp", gp[row:row + 1], sum(t.numpy() for t in go) - want_gxx, BF16, is_grad=True)
+    coefs = [c.detach() for c in coef_leaf]
+    (sum(((x + xx * coefs[s]) * go[s]).sum() for s in range(5)) + ((x + xx * mix) * torch.tensor(to_np(gxm[row:row + 1]))).sum()).backward()
+    check_close("gx", gx[row:row + 1], x.grad.numpy(), BF16, is_grad=True)
+    # gmix_x over everything: sum_{b,t} gxm * xx
+    xa = ref["x"]
+    xxa = np.concatenate([np.zeros((B, 1, C)), xa[:, :-1]], 1) - xa
+    check_close("gmix_x", gmix.cpu().double().numpy(), (to_np(gxm) * xxa).sum((0, 1)), torch.float32, is_grad=True)
+    for t in (gcoef, gp, gxx, gx):
+        assert bool(torch.isfinite(t.float()).all())
+
+
 @pytest.mark.parametrize("B,T,C,R", [(2, 64, 128, 32), (3, 37, 64, 32), (1, 300, 320, 64), (4, 128, 512, 32)])
 def test_autograd_through_the_operator_object(oracle, B, T, C, R):
     """op.shift_mix end to end, gradients of all five arguments, against float64 autograd through the

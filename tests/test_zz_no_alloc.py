@@ -28,11 +28,19 @@ def _pair(lib, native, B, T, H, dtype, seed):
     want = outs()
     native.check(lib.wkv6_backward(st, code, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy), *[P(x) for x in want], P(ws), n))
     got = outs()
-    torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
-    native.check(lib.wkv6_backward_static(st, code, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy), *[P(x) for x in got]))
-    torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+
+    def call():
+        native.check(lib.wkv6_backward_static(st, code, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy), *[P(x) for x in got]))
+        torch.cuda.synchronize()
+
+    call()   # (the first call on a device looks the array's address up and sets the kernels' attributes)
+    # the device's own count of free memory, which sees every allocation of the process, not only torch's
+    free_before = torch.cuda.mem_get_info()[0]
+    torch_before = torch.cuda.memory_allocated()
+    for x in got:
+        x.fill_(float("nan"))
+    call()
+    assert torch.cuda.mem_get_info()[0] == free_before and torch.cuda.memory_allocated() == torch_before
     return got, want
 
 
@@ -63,3 +71,51 @@ def test_static_scratch_backward_refuses_what_does_not_fit():
     p = x.data_ptr()
     rc = lib.wkv6_backward_static(None, _native.BF16, B, T, C, H, *([p] * 11))
     assert rc == 3 and b"workspace" in lib.wkv6_status_string(rc)
+
+
+def test_static_scratch_backward_replays_in_a_hip_graph():
+    """The call captured once into a graph (it allocates nothing and enqueues on the given stream only) and
+    replayed on changed inputs, with eager work in between: every replay equals wkv6_backward on the same
+    inputs."""
+    from rwkv_kernel import _native
+
+    lib = _native.load()
+    torch.cuda.set_device(0)
+    B, T, H, N = 4, 256, 8, 64
+    C = H * N
+    g = torch.Generator().manual_seed(31)
+    src = [torch.randn(B, T, C, generator=g) for _ in range(4)] + [torch.rand(B, T, C, generator=g) * 7.0 - 6.0]
+    r, k, v, gy, w = (x.to(torch.bfloat16).cuda() for x in src)
+    u = (torch.randn(H, N, generator=g) * 0.5).to(torch.bfloat16).cuda()
+    got = [torch.empty(B, T, C, dtype=torch.bfloat16, device="cuda") for _ in range(4)] + [torch.empty(B, C, dtype=torch.bfloat16, device="cuda")]
+    P = lambda t: t.data_ptr()
+
+    def step():
+        st = torch.cuda.current_stream().cuda_stream
+        _native.check(lib.wkv6_backward_static(st, _native.BF16, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy), *[P(x) for x in got]))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()                      # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    n = lib.wkv6_backward_workspace_bytes(_native.BF16, B, T, C, H)
+    ws = torch.empty(n, dtype=torch.uint8, device="cuda")
+    for rep in range(3):
+        # changed inputs (in place: the graph holds the addresses), eager work between the replays
+        v.copy_((torch.randn(B, T, C, generator=g)).to(torch.bfloat16))
+        gy.copy_((torch.randn(B, T, C, generator=g)).to(torch.bfloat16))
+        for x in got:
+            x.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        want = [torch.empty_like(x) for x in got]
+        st = torch.cuda.current_stream().cuda_stream
+        _native.check(lib.wkv6_backward(st, _native.BF16, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy), *[P(x) for x in want], P(ws), n))
+        torch.cuda.synchronize()
+        for name, a, b in zip("gr gk gv gw gu".split(), got, want):
+            assert torch.equal(a, b), (rep, name)
