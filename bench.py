@@ -329,66 +329,71 @@ def main():
     # step, and tensors whose bases agree modulo 4 KiB send all those streams to the same memory
     # channel at the same time (which costs about 5 % at this size; torch's own allocator returns
     # 2 MiB-aligned blocks).  The torch flavour carves the tensors it allocates itself the same way.
-    nbytes = B * T * C * max(es, eo)
-    slot = (nbytes + (2 << 20) - 1) // (2 << 20) * (2 << 20) + (2 << 20)
     nsave = 0 if a.plain_pair else lib.wkv6_saved_bytes(code, algo, B, T, C, H)
-    pool = torch.empty(11 * slot + nsave + (2 << 20), dtype=torch.uint8, device=dev)
-    first = -pool.data_ptr() % (2 << 20)
-
-    def carve(i, nb=nbytes):
-        o = first + i * slot + i * a.stagger
-        return pool[o:o + nb]
-
-    def big(i, src=None, dt=None):
-        dt = dt or dtype
-        t = carve(i, B * T * C * torch.empty((), dtype=dt).element_size()).view(dt).view(B, T, C)
-        if src is not None:
-            t.copy_(src.to(dt))
-        return t
-
     ins = synthetic_inputs(B, T, H, N, a.seed)
-    r, k, v, w = (big(i, ins[i]) for i in range(4))
-    gy = big(4, ins[5], odtype)
     u = ins[4].to(dtype).to(dev).contiguous()
-    y, gr, gk, gv, gw = (big(5 + i, None, odtype) for i in range(5))
-    gu_part = torch.empty(B, C, dtype=odtype, device=dev)
-    fws_bytes = lib.wkv6_forward_workspace_bytes(code, algo, B, T, C, H)
-    bws_bytes = lib.wkv6_backward_workspace_bytes_ex(code, algo, B, T, C, H)
-    fws = torch.empty(max(fws_bytes, 16), dtype=torch.uint8, device=dev)
-    bws = torch.empty(max(bws_bytes, 16), dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
     P = lambda t: t.data_ptr()
 
-    # the pair a training step uses (the torch autograd.Function does the same): the forward saves the
-    # per-chunk states the backward would otherwise recompute; --plain-pair times the two calls the
-    # reference's binding corresponds to (forward(r..y), backward(r..gu)) instead
-    saved = carve(10, max(nsave, 16))
+    def make_calls(stagger):
+        nbytes = B * T * C * max(es, eo)
+        slot = (nbytes + (2 << 20) - 1) // (2 << 20) * (2 << 20) + (2 << 20)
+        pool = torch.empty(11 * slot + nsave + (2 << 20), dtype=torch.uint8, device=dev)
+        first = -pool.data_ptr() % (2 << 20)
 
-    def fwd():
-        if nsave:
-            _native.check(lib.wkv6_forward_save(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(y),
-                                                P(saved), nsave))
-        else:
-            _native.check(lib.wkv6_forward_ex(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(y),
-                                              P(fws), fws_bytes))
+        def carve(i, nb=nbytes):
+            o = first + i * slot + i * stagger
+            return pool[o:o + nb]
 
-    gu_sum = torch.empty(C, dtype=odtype, device=dev)
+        def big(i, src=None, dt=None):
+            dt = dt or dtype
+            t = carve(i, B * T * C * torch.empty((), dtype=dt).element_size()).view(dt).view(B, T, C)
+            if src is not None:
+                t.copy_(src.to(dt))
+            return t
 
-    def bwd_call():
-        if nsave:   # the batch sum of gu comes out of the same launch
-            _native.check(lib.wkv6_backward_saved_sum(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy),
-                                                      P(gr), P(gk), P(gv), P(gw), P(gu_part), P(gu_sum), P(saved), nsave))
-        else:
-            _native.check(lib.wkv6_backward_ex(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy),
-                                               P(gr), P(gk), P(gv), P(gw), P(gu_part), P(bws), bws_bytes))
+        r, k, v, w = (big(i, ins[i]) for i in range(4))
+        gy = big(4, ins[5], odtype)
+        y, gr, gk, gv, gw = (big(5 + i, None, odtype) for i in range(5))
+        gu_part = torch.empty(B, C, dtype=odtype, device=dev)
+        fws_bytes = lib.wkv6_forward_workspace_bytes(code, algo, B, T, C, H)
+        bws_bytes = lib.wkv6_backward_workspace_bytes_ex(code, algo, B, T, C, H)
+        fws = torch.empty(max(fws_bytes, 16), dtype=torch.uint8, device=dev)
+        bws = torch.empty(max(bws_bytes, 16), dtype=torch.uint8, device=dev)
 
-    def bwd():   # what a training step does: the library call plus the batch sum of gu, as the reference's binding
-        bwd_call()
-        return gu_sum if nsave else torch.sum(gu_part, 0)
+        # the pair a training step uses (the torch autograd.Function does the same): the forward saves the
+        # per-chunk states the backward would otherwise recompute; --plain-pair times the two calls the
+        # reference's binding corresponds to (forward(r..y), backward(r..gu)) instead
+        saved = carve(10, max(nsave, 16))
 
-    def step():
-        fwd(); bwd()
+        def fwd():
+            if nsave:
+                _native.check(lib.wkv6_forward_save(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(y),
+                                                    P(saved), nsave))
+            else:
+                _native.check(lib.wkv6_forward_ex(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(y),
+                                                  P(fws), fws_bytes))
 
+        gu_sum = torch.empty(C, dtype=odtype, device=dev)
+
+        def bwd_call():
+            if nsave:   # the batch sum of gu comes out of the same launch
+                _native.check(lib.wkv6_backward_saved_sum(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy),
+                                                          P(gr), P(gk), P(gv), P(gw), P(gu_part), P(gu_sum), P(saved), nsave))
+            else:
+                _native.check(lib.wkv6_backward_ex(stream, code, algo, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy),
+                                                   P(gr), P(gk), P(gv), P(gw), P(gu_part), P(bws), bws_bytes))
+
+        def bwd():   # what a training step does: the library call plus the batch sum of gu, as the reference's binding
+            bwd_call()
+            return gu_sum if nsave else torch.sum(gu_part, 0)
+
+        def step():
+            fwd(); bwd()
+
+        return fwd, bwd_call, bwd, step
+
+    fwd, bwd_call, bwd, step = make_calls(a.stagger)
     preheat_ms = preheat(step, a.preheat_ms) if a.preheat_ms > 0 else 0.0
     for _ in range(a.warmup):
         step()
@@ -465,6 +470,56 @@ def main():
             "fwd_GBps": bytes_fwd / (f_avg * 1e-3) / 1e9, "bwd_GBps": bytes_bwd / (b_avg * 1e-3) / 1e9,
         },
     }
+    def timed_ms(fn, steps):
+        """GPU time per call of fn over `steps` back-to-back calls (events on the launch stream)."""
+        for _ in range(max(5, a.warmup // 5)):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+    if a.stagger and not a.plain_pair:
+        # the same calls on tensors whose bases all sit on 2 MiB boundaries (what a framework's allocator returns)
+        out["unstaggered_ms_per_step"] = timed_ms(make_calls(0)[3], a.steps)
+    if dt_name == "bf16" and not a.plain_pair and a.algo == "auto":
+        # what a caller of the torch binding gets: op(r, k, v, w, u) and y.backward(gy) on tensors from separate
+        # torch.empty calls (the binding staggers only what it allocates itself: y, the saved block, the gradients).
+        # The binding's host side (autograd bookkeeping, seven allocations per step) is inside this figure.
+        from rwkv_kernel import RWKVKernelOperator
+        op = RWKVKernelOperator(N, T)
+        leaves = []
+        for i in range(4):
+            t = torch.empty(B, T, C, dtype=dtype, device=dev)
+            t.copy_(ins[i].to(dtype))
+            leaves.append(t.requires_grad_(True))
+        ub = u.clone().requires_grad_(True)
+        gyb = torch.empty(B, T, C, dtype=odtype, device=dev)
+        gyb.copy_(ins[5].to(odtype))
+
+        def binding_step():
+            for t in leaves:
+                t.grad = None
+            ub.grad = None
+            yb, _ = op(*leaves, ub)
+            yb.backward(gyb)
+
+        out["binding_ms_per_step"] = timed_ms(binding_step, a.steps)
+        # the same step captured once and replayed: the binding's kernels on the binding's own allocation, without its
+        # host side (the situation inside a model step, where the host runs ahead of the GPU)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            binding_step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            binding_step()
+        out["binding_replayed_ms_per_step"] = timed_ms(graph.replay, a.steps)
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(B, T, H, N, a.seed, a.cpu_tokens)
     print(json.dumps(out))
