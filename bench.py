@@ -36,9 +36,9 @@ WORKLOADS = {
 # by the same counters' reading for a device-to-device copy of known size; see profiles/.
 # Keyed by (workload, algo, "fwd"|"bwd").  None = not measured.
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/c2_fwd_bwd_hbm_traffic_pmc.md: backward_saved_sum 201.8 MB read + 134.4 MB written,
+    # profiles/c2_fwd_bwd_hbm_traffic_pmc.md: backward_saved_sum 201.8 MB read + 135.8 MB written,
     # forward_save 134.5 MB read + 67.1 MB written
-    ("c2", "auto", "bwd"): 336.2e6, ("c2", "chunk", "bwd"): 336.2e6,
+    ("c2", "auto", "bwd"): 337.5e6, ("c2", "chunk", "bwd"): 337.5e6,
     ("c2", "auto", "fwd"): 201.6e6, ("c2", "chunk", "fwd"): 201.6e6,
 }
 
@@ -53,6 +53,8 @@ def parse():
     ap.add_argument("--workload", default="c2", choices=sorted(WORKLOADS) + ["c4", "c5", "mix"])
     ap.add_argument("--algo", default="auto", choices=["auto", "scan", "chunk"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra-timings", action="store_true",
+                    help="skip the unstaggered and the through-the-binding steps (profiles of the headline step alone)")
     ap.add_argument("--plain-pair", action="store_true", help="time forward()+backward() without saved states")
     ap.add_argument("--cpu-tokens", type=int, default=0, help="tokens in the CPU baseline sample (0 = default)")
     ap.add_argument("--seed", type=int, default=0)
@@ -483,10 +485,10 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / steps
 
-    if a.stagger and not a.plain_pair:
+    if a.stagger and not a.plain_pair and not a.no_extra_timings:
         # the same calls on tensors whose bases all sit on 2 MiB boundaries (what a framework's allocator returns)
         out["unstaggered_ms_per_step"] = timed_ms(make_calls(0)[3], a.steps)
-    if dt_name == "bf16" and not a.plain_pair and a.algo == "auto":
+    if dt_name == "bf16" and not a.plain_pair and a.algo == "auto" and not a.no_extra_timings:
         # what a caller of the torch binding gets: op(r, k, v, w, u) and y.backward(gy) on tensors from separate
         # torch.empty calls (the binding staggers only what it allocates itself: y, the saved block, the gradients).
         # The binding's host side (autograd bookkeeping, seven allocations per step) is inside this figure.
