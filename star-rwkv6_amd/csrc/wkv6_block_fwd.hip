@@ -1,7 +1,12 @@
 // WKV6 forward in block form for gfx950 (bf16 MFMA for the dense products, fp32 state), for bf16
-// tensors, sequence lengths that are a multiple of 64 and between half a pair and one (batch, head)
-// pair per compute unit.  The tile form in wkv6_chunk_fwd.hip (state advanced every 16 tokens)
-// serves every other case.  Notation and the operand scaling are in wkv6_block.h.
+// tensors, sequence lengths that are a multiple of 64 and more than half a (batch, head) pair per
+// compute unit.  The tile form in wkv6_chunk_fwd.hip (state advanced every 16 tokens) serves every
+// other case.  Notation and the operand scaling are in wkv6_block.h.
+//
+// One workgroup per pair; with more pairs than compute units one workgroup per compute unit, which runs
+// its pairs (same head, `bstep` batch rows apart) back to back through ONE pipeline: the loads, the
+// operand preparation and the stores each walk the flat sequence of (pair, chunk) visits with a cursor
+// of their own, so a pair's first chunks are loaded and prepared while the pair before it finishes.
 //
 // Per block of 32 tokens (S = state entering it, rows j):
 //   A[t][s] = R~_t . K~_s (s < t),   A[t][t] = sum_j r_t[j] u[j] k_t[j]
@@ -38,8 +43,11 @@ struct BlockFwdLds {
 };
 static_assert(BlockFwdLds::kBytes <= 160 * 1024, "LDS block of the block-form forward kernel");
 
+constexpr int kBlockMaxSlots = 64;   // pairs one workgroup takes at most
+
 struct BlockFwdArgs {
-    int T, H;
+    int T, H, B;
+    int bstep;               // batch rows between two pairs of a workgroup (B: one pair per workgroup)
     const bf16_t *r, *k, *v, *w, *u;
     const void *s0;          // initial state (B or n_state, H, 64, 64) [key][value] in Ts, or null
     const int64_t *map;      // batch row -> state row, or null
@@ -54,27 +62,35 @@ struct BlockFwdArgs {
 // State S[m]: rows j = block_row_channel(m, g) + rr, column i.
 // ------------------------------------------------------------------------------------------
 template <typename Ts, bool kSave, int HALF>
-__device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsigned char *smem, int bh, int q, int lane)
+__device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsigned char *smem, int pair0, int q, int lane)
 {
     const int T = a.T, H = a.H;
     const int g = lane >> 4, l16 = lane & 15;
     const int nchunk = T / kBlockTokens;
-    const int b = bh / H, h = bh - b * H;
-    f32x4 S[4];
-    if (a.s0 != nullptr) {
+    const int b0 = pair0 / H, h = pair0 - b0 * H;
+    const int npw = (a.B - b0 + a.bstep - 1) / a.bstep;   // pairs of this workgroup: batch rows b0, b0 + bstep, ...
+    const int nvisit = npw * nchunk;
+    f32x4 S[4], Snext[4];
+    // initial state of the workgroup's pair number `slot`, requested one visit before the pair begins
+    auto request_state = [&](int slot) {
+        const int b = b0 + slot * a.bstep;
         const int64_t row = a.map ? a.map[b] : (int64_t)b;
         const Ts *p = reinterpret_cast<const Ts *>(a.s0) + (row * H + h) * kN * kN + 16 * q + l16;
 #pragma unroll
         for (int m = 0; m < 4; ++m)
 #pragma unroll
-            for (int rr = 0; rr < 4; ++rr) S[m][rr] = load1(p + (block_row_channel(m, g) + rr) * kN);
-    } else {
-#pragma unroll
-        for (int m = 0; m < 4; ++m) S[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    }
-    if (kSave && HALF == 0 && b == 0 && q == 0 && lane == 0 && a.arrivals) a.arrivals[h] = 0;
-    for (int it = 0; it < nchunk; ++it) {
+            for (int rr = 0; rr < 4; ++rr) Snext[m][rr] = load1(p + (block_row_channel(m, g) + rr) * kN);
+    };
+    if (a.s0 != nullptr) request_state(0);
+    if (kSave && HALF == 0 && b0 == 0 && q == 0 && lane == 0 && a.arrivals) a.arrivals[h] = 0;
+    int c = 0, slot = 0;   // visit `it` is chunk c of pair number `slot`
+    for (int it = 0; it < nvisit; ++it) {
         __syncthreads();
+        if (c == 0) {
+#pragma unroll
+            for (int m = 0; m < 4; ++m) S[m] = a.s0 != nullptr ? Snext[m] : (f32x4){0.f, 0.f, 0.f, 0.f};
+        }
+        if (a.s0 != nullptr && c == nchunk - 1 && slot + 1 < npw) request_state(slot + 1);
         const unsigned char *rt = smem + BlockFwdLds::kOp + (it & 1) * 2 * kTileBytes, *kt = rt + kTileBytes;
         const float *vec = reinterpret_cast<const float *>(smem + BlockFwdLds::kVec + (it & 1) * kBlockVecBytes);
         const float *ruk = vec + 4 * kN;
@@ -148,13 +164,17 @@ __device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsign
             scale(vec + (2 * blk + 1) * kN);   // g2 of the block
         }
         __builtin_amdgcn_sched_barrier(0);
-    }
-    if (a.sT != nullptr && HALF == 0) {
-        Ts *p = reinterpret_cast<Ts *>(a.sT) + (int64_t)bh * kN * kN + 16 * q + l16;
+        if (++c == nchunk) {
+            if (a.sT != nullptr && HALF == 0) {   // the pair's final state
+                Ts *p = reinterpret_cast<Ts *>(a.sT) + ((int64_t)(b0 + slot * a.bstep) * H + h) * (kN * kN) + 16 * q + l16;
 #pragma unroll
-        for (int m = 0; m < 4; ++m)
+                for (int m = 0; m < 4; ++m)
 #pragma unroll
-            for (int rr = 0; rr < 4; ++rr) store1(p + (block_row_channel(m, g) + rr) * kN, S[m][rr]);
+                    for (int rr = 0; rr < 4; ++rr) store1(p + (block_row_channel(m, g) + rr) * kN, S[m][rr]);
+            }
+            c = 0;
+            ++slot;
+        }
     }
     __syncthreads();   // the producers write out the last chunk's staged rows behind this one
 }
@@ -163,99 +183,125 @@ __device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsign
 // Producer wave p: tokens 16p..16p+15 of every chunk.
 // ------------------------------------------------------------------------------------------
 template <bool kSave>
-__device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsigned char *smem, int *s_wild, int bh, int p, int lane)
+__device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsigned char *smem, int *s_wild, int pair0, int p, int lane)
 {
     const int T = a.T, H = a.H;
     const int g = lane >> 4, l16 = lane & 15;
     const int64_t C = (int64_t)H * kN;
     const int nchunk = T / kBlockTokens;
-    const int b = bh / H, h = bh - b * H;
+    const int b0 = pair0 / H, h = pair0 - b0 * H;
+    const int npw = (a.B - b0 + a.bstep - 1) / a.bstep;
+    const int nvisit = npw * nchunk;
     const uint32_t rowbytes = (uint32_t)C * 2u;
     const uint32_t lds0 = lds_address(smem);
-    const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
-    const bf16_t *rb = a.r + base, *kb_ = a.k + base, *vb = a.v + base, *wb = a.w + base;
-    bf16_t *yb = a.y + base;
-    char *ckb = kSave ? reinterpret_cast<char *>(a.ckpt + (int64_t)bh * nchunk * (kN * kN)) : nullptr;
+    // first element of the workgroup's pair number `slot` in a (B,T,C) tensor
+    auto pair_base = [&](int slot) { return (int64_t)(b0 + slot * a.bstep) * T * C + (int64_t)h * kN; };
     // this lane's part of an 8-row block: row (lane >> 3), 16-byte piece swizzled with the row
     const int lrow = lane >> 3;
     const uint32_t lpiece = (uint32_t)(((lane & 7) ^ lrow) << 4);
+    // Every stream walks the flat sequence of visits (pair 0 chunk 0, 1, .., pair 1 chunk 0, ..) with a cursor
+    // of its own: visit number `it`, its chunk `c`, and the pointers of its pair.
+    struct Cursor {
+        int it = 0, c = 0, slot = 0;
+    };
+    Cursor cv, cr, co, cp;   // v loads, r/k/w loads, stores of staged rows, operand preparation
+    const bf16_t *vb = a.v + pair_base(0), *rb = a.r + pair_base(0), *kb_ = a.k + pair_base(0), *wb = a.w + pair_base(0);
+    bf16_t *yb = a.y + pair_base(0);
+    char *ckb = kSave ? reinterpret_cast<char *>(a.ckpt + (int64_t)(b0 * H + h) * nchunk * (kN * kN)) : nullptr;
     // Vector-memory operations this wave has issued so far, and the count right after the r, k, w loads
     // of visit j went out: a wave's operations complete in program order, so "the loads of visit j have
     // landed" is "at most (issued - mark of j) operations are still in flight".
     int issued = 0, mark_even = 0, mark_odd = 0;
-    auto issue_v = [&](int it) {
-        const uint32_t vv = lds0 + BlockFwdLds::kRawV + (it & 3) * kTileBytes + 16 * p * kTileRow;
+    auto issue_v = [&]() {   // the next visit's v
+        const uint32_t vv = lds0 + BlockFwdLds::kRawV + (cv.it & 3) * kTileBytes + 16 * p * kTileRow;
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk)
-            load_rows8_to_lds(vb, (uint32_t)(it * kBlockTokens + 16 * p + 8 * blk + lrow) * rowbytes + lpiece, vv + 8 * blk * kTileRow);
+            load_rows8_to_lds(vb, (uint32_t)(cv.c * kBlockTokens + 16 * p + 8 * blk + lrow) * rowbytes + lpiece, vv + 8 * blk * kTileRow);
         issued += 2;
+        ++cv.it;
+        if (++cv.c == nchunk) { cv.c = 0; ++cv.slot; vb = a.v + pair_base(cv.slot); }
     };
-    auto issue_rkw = [&](int it) {
-        const uint32_t raw = lds0 + BlockFwdLds::kRaw + (it & 1) * 3 * kTileBytes + 16 * p * kTileRow;
+    auto issue_rkw = [&]() {   // the next visit's r, k, w
+        const uint32_t raw = lds0 + BlockFwdLds::kRaw + (cr.it & 1) * 3 * kTileBytes + 16 * p * kTileRow;
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
-            const uint32_t o = (uint32_t)(it * kBlockTokens + 16 * p + 8 * blk + lrow) * rowbytes + lpiece;
+            const uint32_t o = (uint32_t)(cr.c * kBlockTokens + 16 * p + 8 * blk + lrow) * rowbytes + lpiece;
             load_rows8_to_lds(wb, o, raw + 2 * kTileBytes + 8 * blk * kTileRow);
             load_rows8_to_lds(rb, o, raw + 8 * blk * kTileRow);
             load_rows8_to_lds(kb_, o, raw + kTileBytes + 8 * blk * kTileRow);
         }
         issued += 6;
-        if (it & 1) mark_odd = issued; else mark_even = issued;
+        if (cr.it & 1) mark_odd = issued; else mark_even = issued;
+        ++cr.it;
+        if (++cr.c == nchunk) {
+            cr.c = 0; ++cr.slot;
+            const int64_t nb = pair_base(cr.slot);
+            rb = a.r + nb; kb_ = a.k + nb; wb = a.w + nb;
+        }
     };
-    // what the consumers staged during visit `it`, as whole rows: y rows of this wave's tokens and rows
-    // 16p..16p+15 of the chunk's state
-    auto store_staged = [&](int it) {
-        const unsigned char *ys = smem + BlockFwdLds::kYStage + (it & 1) * kTileBytes;
-        const unsigned char *ss = smem + BlockFwdLds::kSStage + (it & 1) * kTileBytes;
+    // what the consumers staged during the next visit in line, as whole rows: y rows of this wave's tokens
+    // and rows 16p..16p+15 of the chunk's state
+    auto store_staged = [&]() {
+        const unsigned char *ys = smem + BlockFwdLds::kYStage + (co.it & 1) * kTileBytes;
+        const unsigned char *ss = smem + BlockFwdLds::kSStage + (co.it & 1) * kTileBytes;
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
             const int row = 16 * p + 8 * blk + lrow;
             const uint4 x = *reinterpret_cast<const uint4 *>(ys + row * kTileRow + (lane & 7) * 16);
-            *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(yb) + ((uint32_t)(it * kBlockTokens + row) * rowbytes + lpiece)) = x;
+            *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(yb) + ((uint32_t)(co.c * kBlockTokens + row) * rowbytes + lpiece)) = x;
             if (kSave) {
                 const uint4 s = *reinterpret_cast<const uint4 *>(ss + row * kTileRow + (lane & 7) * 16);
-                *reinterpret_cast<uint4 *>(ckb + ((uint32_t)it * (uint32_t)(kN * kN * 2) + (uint32_t)(row * kTileRow) + lpiece)) = s;
+                *reinterpret_cast<uint4 *>(ckb + ((uint32_t)co.c * (uint32_t)(kN * kN * 2) + (uint32_t)(row * kTileRow) + lpiece)) = s;
             }
         }
         issued += kSave ? 4 : 2;
+        ++co.it;
+        if (++co.c == nchunk) {
+            co.c = 0; ++co.slot;
+            yb = a.y + pair_base(co.slot);
+            if (kSave) ckb = reinterpret_cast<char *>(a.ckpt + (int64_t)((b0 + co.slot * a.bstep) * H + h) * nchunk * (kN * kN));
+        }
     };
     float u4[4];
-    load4(a.u + h * kN + 4 * l16, u4);
-    // visit `it` (its r, k, w loads have been issued); `next` >= 0: the visit whose r, k, w loads go out
-    // as soon as this one's raw rows are in registers (into the same LDS block)
-    auto prepare = [&](int it, int next) {
+    load4(a.u + h * kN + 4 * l16, u4);   // (all pairs of a workgroup belong to one head)
+    // the next visit in line (its r, k, w loads have been issued); `more`: the r, k, w loads of the next visit
+    // not yet requested go out as soon as this one's raw rows are in registers (into the same LDS block)
+    auto prepare = [&](bool more) {
+        const int it = cp.it;
         const unsigned char *raw = smem + BlockFwdLds::kRaw + (it & 1) * 3 * kTileBytes;
         unsigned char *op = smem + BlockFwdLds::kOp + (it & 1) * 2 * kTileBytes;
         float *vec = reinterpret_cast<float *>(smem + BlockFwdLds::kVec + (it & 1) * kBlockVecBytes);
         wait_in_flight(issued - ((it & 1) ? mark_odd : mark_even));
         const bool ok = block_prepare(raw, raw + kTileBytes, raw + 2 * kTileBytes, vec, u4, p, l16, g,
             [&]() {
-                if (next >= 0) {
+                if (more) {
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-                    issue_rkw(next);
+                    issue_rkw();
                 }
             },
             [&](uint32_t o, const float (&xr)[4], const float (&xk)[4], const float (&)[4], const float (&)[4]) {
                 *reinterpret_cast<uint2 *>(op + o) = make_uint2(pack_bf16x2(xr[0], xr[1]), pack_bf16x2(xr[2], xr[3]));
                 *reinterpret_cast<uint2 *>(op + kTileBytes + o) = make_uint2(pack_bf16x2(xk[0], xk[1]), pack_bf16x2(xk[2], xk[3]));
             });
-        if (!ok && lane == 0) *s_wild = 1;
+        if (!ok && lane == 0) s_wild[cp.slot] = 1;
+        ++cp.it;
+        if (++cp.c == nchunk) { cp.c = 0; ++cp.slot; }
     };
     // r, k, w of visit j are requested three visits ahead (two in the prologue), v three visits ahead
-    issue_v(0);
-    issue_rkw(0);
-    if (nchunk > 1) { issue_v(1); issue_rkw(1); }
-    if (nchunk > 2) issue_v(2);
-    prepare(0, nchunk > 2 ? 2 : -1);
-    for (int it = 0; it < nchunk; ++it) {
+    issue_v();
+    issue_rkw();
+    if (nvisit > 1) { issue_v(); issue_rkw(); }
+    if (nvisit > 2) issue_v();
+    prepare(nvisit > 2);
+    for (int it = 0; it < nvisit; ++it) {
         __syncthreads();
         // free again: the raw v block of visit it-1; the staging tiles of visit it-1 are complete
-        if (it + 3 < nchunk) issue_v(it + 3);
-        if (it > 0) store_staged(it - 1);
-        if (it + 1 < nchunk) prepare(it + 1, it + 3 < nchunk ? it + 3 : -1);
+        if (it + 3 < nvisit) issue_v();
+        if (it > 0) store_staged();
+        if (it + 1 < nvisit) prepare(it + 3 < nvisit);
     }
     __syncthreads();
-    store_staged(nchunk - 1);
+    store_staged();
     wait_loads<0>();
 }
 
@@ -265,31 +311,46 @@ template <typename Ts, bool kSave>
 __global__ __launch_bounds__(kBlockFwdThreads) void block_fwd_kernel(BlockFwdArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ int s_wild;
+    __shared__ int s_wild[kBlockMaxSlots];   // per pair of the workgroup: 16 tokens left the scaled operands' range
     static_assert(sizeof(ScanFwdLds) <= BlockFwdLds::kBytes, "the exact second pass reuses the LDS block");
-    if (threadIdx.x == 0) s_wild = 0;
+    if (threadIdx.x < kBlockMaxSlots) s_wild[threadIdx.x] = 0;
     __syncthreads();
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int bh = (int)blockIdx.x;
-    if (wave < 4) block_fwd_producer<kSave>(a, smem, &s_wild, bh, wave, lane);
-    else if (wave < 8) block_fwd_consumer<Ts, kSave, 0>(a, smem, bh, wave - 4, lane);
-    else block_fwd_consumer<Ts, kSave, 1>(a, smem, bh, wave - 8, lane);
-    // exact second pass if 16 tokens of this pair left the range the scaled operands can hold
+    const int pair0 = (int)blockIdx.x;
+    if (wave < 4) block_fwd_producer<kSave>(a, smem, s_wild, pair0, wave, lane);
+    else if (wave < 8) block_fwd_consumer<Ts, kSave, 0>(a, smem, pair0, wave - 4, lane);
+    else block_fwd_consumer<Ts, kSave, 1>(a, smem, pair0, wave - 8, lane);
+    // exact second pass for the pairs of which 16 tokens left the range the scaled operands can hold
     __threadfence_block();
     __syncthreads();
-    if (s_wild) {
+    const int b0 = pair0 / a.H, h = pair0 - b0 * a.H;
+    const int npw = (a.B - b0 + a.bstep - 1) / a.bstep;
+    for (int slot = 0; slot < npw; ++slot) {
+        if (!s_wild[slot]) continue;   // (uniform over the workgroup)
         __syncthreads();
-        scan_fwd_body<bf16_t, bf16_t, Ts>(*reinterpret_cast<ScanFwdLds *>(smem), bh / a.H, bh % a.H, a.T, a.H, a.r, a.k, a.v, a.w, a.u,
+        scan_fwd_body<bf16_t, bf16_t, Ts>(*reinterpret_cast<ScanFwdLds *>(smem), b0 + slot * a.bstep, h, a.T, a.H, a.r, a.k, a.v, a.w, a.u,
                                           reinterpret_cast<const Ts *>(a.s0), a.map, a.y, reinterpret_cast<Ts *>(a.sT), false);
     }
+}
+
+// Workgroups of a launch: one per pair, or -- more pairs than compute units -- as many as there are compute
+// units, rounded down to a multiple of H (so that a workgroup's pairs belong to one head); 0: the block form
+// does not take the shape.
+static int64_t block_grid(int64_t B, int64_t H) {
+    const int64_t pairs = B * H, cus = compute_units();
+    if (pairs <= cus) return pairs;
+    const int64_t grid = cus / H * H;
+    // (heads that leave a tenth of the compute units idle, or more pairs per workgroup than its flags hold: tile form)
+    if (grid * 10 < cus * 9 || (pairs + grid - 1) / grid > kBlockMaxSlots) return 0;
+    return grid;
 }
 
 bool block_forward_applies(int64_t B, int64_t T, int64_t H) {
     const int64_t pairs = B * H, cus = compute_units();
     // (with fewer pairs than half the compute units the tile form shares a pair out over several workgroups)
-    return T >= kBlockTokens && (T % kBlockTokens) == 0 && pairs <= cus && 2 * pairs > cus;
+    return T >= kBlockTokens && (T % kBlockTokens) == 0 && 2 * pairs > cus && block_grid(B, H) > 0;
 }
 
 hipError_t block_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
@@ -297,7 +358,9 @@ hipError_t block_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
                          const void *s0, const int64_t *map, void *y, void *sT, void *saved_states, bool counters)
 {
     BlockFwdArgs a = {};
-    a.T = (int)T; a.H = (int)H;
+    a.T = (int)T; a.H = (int)H; a.B = (int)B;
+    const int64_t grid = block_grid(B, H);
+    a.bstep = B * H <= grid ? (int)B : (int)(grid / H);
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
     a.s0 = s0; a.map = map; a.y = (bf16_t *)y; a.sT = sT; a.ckpt = (float *)saved_states;
     a.arrivals = saved_states && counters ? reinterpret_cast<int *>(reinterpret_cast<char *>(saved_states) + chunk_backward_workspace_bytes(B, T, H)) : nullptr;
@@ -305,7 +368,7 @@ hipError_t block_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
         constexpr auto kern = block_fwd_kernel<decltype(ts_tag), decltype(save_tag)::value>;
         hipError_t e = allow_dynamic_lds<kern>(BlockFwdLds::kBytes);
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3((unsigned)(B * H)), dim3(kBlockFwdThreads), BlockFwdLds::kBytes, st, a);
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kBlockFwdThreads), BlockFwdLds::kBytes, st, a);
         return hipGetLastError();
     };
     const bool save = saved_states != nullptr;

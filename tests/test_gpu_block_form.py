@@ -1,8 +1,8 @@
 """The block-form MFMA kernels (32-token blocks scaled from the block middle; taken for bf16 tensors with
-T a multiple of 64 and between half as many and as many (batch, head) pairs as the chip has compute
-units) through the C ABI and the torch binding against the float64 oracle: shapes at the edges of their
-range, states in and out of the forward, decay beyond the scaled operands' range, and the mixing of
-either form's forward with either form's backward."""
+T a multiple of 64 and more than half as many (batch, head) pairs as the chip has compute units; the
+forward also takes several pairs per workgroup) through the C ABI and the torch binding against the float64
+oracle: shapes at the edges of their range, states in and out of the forward, decay beyond the scaled
+operands' range, and the mixing of either form's forward with either form's backward."""
 import numpy as np
 import pytest
 import torch
@@ -26,6 +26,14 @@ def op():
 def _pairs_in_range(B, H):
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     return cus // 2 < B * H <= cus
+
+
+def _several_pairs_per_workgroup(B, H):
+    # more pairs than compute units: one workgroup per compute unit (rounded down to a multiple of H) runs
+    # its pairs back to back through one pipeline
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    grid = cus // H * H
+    return B * H > cus and grid * 10 >= cus * 9 and -(-B * H // grid) <= 64
 
 
 def _fwd_bwd(op, ins, algo=CHUNK):
@@ -56,6 +64,39 @@ def test_block_form_fwd_bwd(op, oracle, B, T, H):
     print("block form B=%d T=%d H=%d" % (B, T, H), flush=True)
     y, grads, ref, gy_ref = _fwd_bwd(op, oracle.make_inputs(B, T, H, N, 500 + T + H))
     _check(oracle, y, grads, ref, gy_ref)
+
+
+# More pairs than compute units.  (B, T, H): one chunk per pair (the pipeline's start spans three pairs), pairs
+# that do not fill the last round of workgroups, a head count that does not divide the compute units (grid 240),
+# many pairs per workgroup
+@pytest.mark.parametrize("B,T,H", [(40, 64, 32), (75, 128, 4), (13, 192, 40), (300, 64, 8), (33, 256, 32)])
+def test_block_form_several_pairs_per_workgroup(op, oracle, B, T, H):
+    assert _several_pairs_per_workgroup(B, H) and T % 64 == 0
+    print("block form, several pairs per workgroup B=%d T=%d H=%d" % (B, T, H), flush=True)
+    y, grads, ref, gy_ref = _fwd_bwd(op, oracle.make_inputs(B, T, H, N, 700 + T + H))
+    _check(oracle, y, grads, ref, gy_ref)
+
+
+def test_block_form_several_pairs_state_in_out_and_fallback(op, oracle):
+    """Several pairs per workgroup with an initial state through a state map and the final state out; pairs in the
+    first, a middle and the last position of their workgroup leave the scaled operands' range and are redone
+    exactly after the workgroup's last pair."""
+    B, T, H, nstate = 40, 128, 32, 9
+    assert _several_pairs_per_workgroup(B, H)
+    ins = oracle.make_inputs(B, T, H, N, 91, with_state=True)
+    ins[3][0, 10:30, 64:128] = 6.0        # batch row 0, head 1: first pair of its workgroup
+    ins[3][17, 70:90, 0:64] = 6.0         # a middle one
+    ins[3][39, 100:120, 31 * 64:] = 6.0   # the last
+    dev, ref = cast_inputs(ins[:5], BF16)
+    op.algo = CHUNK
+    for sdt in (BF16, torch.float32):
+        s_dev, s_ref = cast_inputs([ins[6][:nstate]], sdt)
+        smap = [(5 * i + 2) % nstate for i in range(B)]
+        y, sT = op(*dev, return_state=True, init_state=s_dev[0], state_map=smap)
+        torch.cuda.synchronize()
+        y_ref, sT_ref = oracle.forward_c(*ref, N, s_ref[0], smap)
+        check_close("y", y, y_ref, BF16)
+        check_close("sT", sT, sT_ref, BF16)
 
 
 def test_block_form_extreme_decay(op, oracle):

@@ -109,16 +109,15 @@ def test_config5_prefill_then_decode(op, oracle):
     assert rel_inf(to_np(s), to_np(s_one)) <= 1e-2
 
 
-def test_config5_prefill_with_fused_output_stage(op):
-    # B=64 T=512 C=2048: the fused group norm + gate against the same two steps applied on the GPU to
-    # the unfused kernel's own y (both normalise the bf16-rounded y, so they agree to output rounding),
-    # and the carried state is the unfused one
-    import torch.nn.functional as F
-    from oracle import wkv6_ref
+def test_config5_prefill_with_fused_output_stage(op, oracle):
+    # B=64 T=512 C=2048: the fused group norm + gate against the oracle's y (float64, four batch rows) pushed
+    # through the float64 restatement of the norm and the gate; the carried state against the oracle's and
+    # against the unfused kernel's
     B, T, H, N = 64, 512, 32, 64
     print("config 5 prefill, fused output stage", flush=True)
-    ins = wkv6_ref.make_inputs(B, T, H, N, 3, with_state=True)
-    r, k, v, w, u = (x.to(torch.bfloat16).cuda().contiguous() for x in ins[:5])
+    ins = oracle.make_inputs(B, T, H, N, 3, with_state=True)
+    dev, ref = cast_inputs(ins[:5], torch.bfloat16)
+    r, k, v, w, u = dev
     s0 = ins[6].float().cuda()
     g = torch.Generator().manual_seed(9)
     gate = torch.randn(B, T, H * N, generator=g).to(torch.bfloat16).cuda()
@@ -127,65 +126,16 @@ def test_config5_prefill_with_fused_output_stage(op):
     y, sT = op(r, k, v, w, u, return_state=True, init_state=s0)
     out, sT2 = op.forward_gn_gate(r, k, v, w, u, gate, scale, offset, 64e-5, return_state=True, init_state=s0)
     torch.cuda.synchronize()
-    # (the two kernels round k at different scalings before it enters the state update's MFMA -- decayed
-    # to the end of its tile in the unfused kernel, to its own token in the fused one --, so the carried
-    # states agree to the rounding of a bf16 operand, not bit for bit)
+    # (the two kernels scale k differently before it enters the state update's MFMA, so the carried states
+    # agree to the rounding of a bf16 operand, not bit for bit)
     ds = float((sT - sT2).abs().max()) / float(sT.abs().max())
     assert ds <= 1e-2, ds
-    x = F.layer_norm(y.float().reshape(B, T, H, N), (N,), None, None, 64e-5)
-    want = ((x * scale + offset).reshape(B, T, H * N) * gate.float())
-    err = float((out.float() - want).abs().max()) / float(want.abs().max())
-    assert err <= 1e-2, err
+    rows = [0, 17, 42, 63]
+    sub = [x[rows] for x in ref[:4]] + [ref[4]]
+    y_ref, s_ref = oracle.forward_c(*sub, N, to_np(s0)[rows])
+    want = oracle.group_norm_gate_np(y_ref, to_np(gate)[rows], to_np(scale), to_np(offset), N, 64e-5)
+    check_close("out", out[rows], want, torch.bfloat16)
+    check_close("y (unfused)", y[rows], y_ref, torch.bfloat16)
+    check_close("state (fused)", sT2[rows], s_ref, torch.bfloat16)
+    check_close("state (unfused)", sT[rows], s_ref, torch.bfloat16)
     assert bool(torch.isfinite(out.float()).all())
-
-
-def test_config2_state_gradients_across_a_cut(op):
-    # B=8 C=2048 at T=1024 cut into 512 + 512: with the state and its gradient handed across the cut
-    # the chunked bf16 kernels give the gradients of the uncut call (to bf16 rounding of y and the
-    # state's bf16 operands)
-    from oracle import wkv6_ref
-    B, T, H, N, cut = 8, 1024, 32, 64, 512
-    print("config 2 size, state gradients across a cut", flush=True)
-    ins = wkv6_ref.make_inputs(B, T, H, N, 4)
-    r, k, v, w, u, gy = (x.to(torch.bfloat16).cuda().contiguous() for x in ins[:6])
-    op.algo = AUTO
-    whole = [x.clone().requires_grad_(True) for x in (r, k, v, w, u)]
-    y, _ = op(*whole)
-    g_whole = torch.autograd.grad((y.float() * gy.float()).sum(), whole)
-    parts = [x.clone().requires_grad_(True) for x in (r, k, v, w, u)]
-    a = [x[:, :cut].contiguous() for x in parts[:4]] + [parts[4]]
-    b = [x[:, cut:].contiguous() for x in parts[:4]] + [parts[4]]
-    ya, sa = op(*a, return_state=True)
-    yb, _ = op(*b, return_state=True, init_state=sa)
-    g_parts = torch.autograd.grad((torch.cat([ya, yb], 1).float() * gy.float()).sum(), parts)
-    torch.cuda.synchronize()
-    for name, x, z in zip("gr gk gv gw gu".split(), g_parts, g_whole):
-        assert bool(torch.isfinite(x.float()).all())
-        err = float((x.float() - z.float()).abs().max()) / float(z.float().abs().max())
-        assert err <= 1e-2, (name, err)
-
-
-def test_long_single_sequence_in_time_segments_vs_oracle(op, oracle):
-    # bench.py's long1 shape (B=1 T=8192 C=2048 H=32 bf16): the training pair runs as 8 time segments
-    # side by side; forward and gradients against the float64 oracle over the whole sequence, and
-    # against the exact per-timestep kernels, which walk the sequence in one piece
-    from rwkv_kernel import _native
-    B, T, H, N = 1, 8192, 32, 64
-    C = H * N
-    print("long1 full size", flush=True)
-    lib = _native.load()
-    one_piece = B * H * (T // 64) * N * N * 4          # chunk states of the sequence in one piece
-    assert lib.wkv6_saved_bytes(_native.BF16, AUTO, B, T, C, H) >= one_piece + 2 * 8 * B * H * N * N * 4   # + 8 segments' states
-    ins = oracle.make_inputs(B, T, H, N, 3)
-    dev, ref = cast_inputs(ins[:5], torch.bfloat16)
-    gyd, gyr = cast_inputs(ins[5:6], torch.bfloat16)
-    y, grads = _fwd_bwd(op, dev, gyd[0], AUTO)
-    y_ref, _ = oracle.forward_c(*ref, N)
-    check_close("y", y, y_ref, torch.bfloat16)
-    g_ref = oracle.backward_c(*ref, gyr[0], N)
-    for name, g, gr in zip("gr gk gv gw gu".split(), grads, g_ref):
-        check_close(name, to_np(g).reshape(gr.shape), gr, torch.bfloat16, is_grad=True)
-    y1, grads1 = _fwd_bwd(op, dev, gyd[0], SCAN)
-    assert rel_inf(to_np(y), to_np(y1).astype(np.float64)) <= 1e-2
-    for name, g, g1 in zip("gr gk gv gw gu".split(), grads, grads1):
-        assert rel_inf(to_np(g), to_np(g1).astype(np.float64)) <= 1e-2, name
