@@ -14,6 +14,7 @@
 namespace wkv6 {
 
 constexpr int kBlockTokens = 64;                      // tokens per chunk visit (two blocks of 32)
+constexpr int kBlockMaxSlots = 64;   // (batch, head) pairs one workgroup takes at most
 constexpr float kLog2Log2e = 0.5287663729448977f;     // log2(log2(e)): exp(w) log2(e) = 2^(w log2(e) + this)
 
 // Per-visit vectors the producer waves leave for the others: [g1 of block 0, g2 of block 0, g1 of

@@ -43,8 +43,8 @@ struct BlockBwdLds {
     static constexpr int kVec = kAlpha + 2 * kTileBytes;               // [item & 1] per-visit vectors
     static constexpr int kState = kVec + 2 * kBlockVecBytes;           // [item & 1] saved forward state of the chunk, bf16 [i][j] as a tile
     static constexpr int kScratch = kState + 2 * kTileBytes;           // [8 waves][16] floats
-    static constexpr int kGu = kScratch + 8 * 16 * 4;                  // [64] floats: gu partial of half 1
-    static constexpr int kGFlags = kGu + kN * 4;                       // [2 blocks][4 q] visit number + 1 once the wave has written its columns of kGt
+    static constexpr int kGu = kScratch + 8 * 16 * 4;                  // [2 pair parities][2 halves][64] floats: gu partials of a pair; [64]: gu summed over the workgroup's pairs
+    static constexpr int kGFlags = kGu + 5 * kN * 4;                       // [2 blocks][4 q] visit number + 1 once the wave has written its columns of kGt
     static constexpr int kGt = kGFlags + 64;                           // [2 blocks] g2 o G at the block's end, bf16 [j][i] tiles (what gv and W take)
     static constexpr int kBytes = kGt + 2 * kTileBytes;
 };
@@ -52,6 +52,7 @@ static_assert(BlockBwdLds::kBytes <= 160 * 1024, "LDS block of the block-form ba
 
 struct BlockBwdArgs {
     int T, H, B;
+    int bstep;        // batch rows between two pairs of a workgroup (B: one pair per workgroup)
     const bf16_t *r, *k, *v, *w, *u, *gy;
     bf16_t *gr, *gk, *gv, *gw, *gu;
     bf16_t *gu_sum;   // null, or C elements: receives the sum of gu over the batch
@@ -82,18 +83,20 @@ typedef volatile int __attribute__((address_space(3))) *LdsFlag;
 // Wave (q, HALF): key channels j = 16q .. 16q+15, block HALF of the visit (tokens 32 HALF .. +31):
 // gr, gk, gw, gu.  Gj[m]: reverse state, rows i = block_row_channel(m, g) + rr, column j = 16q + l16.
 // ------------------------------------------------------------------------------------------
-template <int HALF>
-__device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned char *smem, const int *s_wild, int bh, int q, int lane)
+template <int HALF, bool kMulti>
+__device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned char *smem, const int *s_wild, int pair0, int q, int lane)
 {
     const int T = a.T, H = a.H;
     const int g = lane >> 4, l16 = lane & 15;
     const int col = 16 * q + l16;
     const int64_t C = (int64_t)H * kN;
     const int nchunk = T / kBlockTokens;
-    const int b = bh / H, h = bh - b * H;
-    const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
+    const int b0 = pair0 / H, h = pair0 - b0 * H;
+    const int npw = kMulti ? (a.B - b0 + a.bstep - 1) / a.bstep : 1;   // pairs of this workgroup: batch rows b0, b0 + bstep, ... (one head)
+    const int nvisit = npw * nchunk;
     const uint32_t rowbytes = (uint32_t)C * 2u;
-    char *gr_h = reinterpret_cast<char *>(a.gr + base), *gk_h = reinterpret_cast<char *>(a.gk + base), *gw_h = reinterpret_cast<char *>(a.gw + base);
+    const int64_t base0 = (int64_t)b0 * T * C + (int64_t)h * kN;
+    char *gr_h = reinterpret_cast<char *>(a.gr + base0), *gk_h = reinterpret_cast<char *>(a.gk + base0), *gw_h = reinterpret_cast<char *>(a.gw + base0);
     f32x4 Gj[4];
 #pragma unroll
     for (int m = 0; m < 4; ++m) Gj[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -101,15 +104,44 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
     load4(a.u + h * kN + 16 * q + 4 * g, u4);   // u of this lane's four channels 16q + 4g + rr
     float gu_acc[4] = {0.f, 0.f, 0.f, 0.f};
     float pend = 1.f;   // per-column factor the reverse state Gj has still to be multiplied with
+    // gu of a pair: both halves leave their part in LDS (rows of the pair's parity); after the next barrier
+    // half 0 adds them, stores the pair's row and adds it, as stored, to the sum over the workgroup's pairs
+    // (for the fused batch sum; a lane owns its four channels of that row)
+    float *gu_lds = reinterpret_cast<float *>(smem + BlockBwdLds::kGu);
+    auto deliver_gu = [&](int done) {   // done: number of the pair
+        if (l16 == 0 && !s_wild[done]) {   // (the exact second pass writes a pair's gu itself)
+            const float *rows = gu_lds + (done & 1) * 2 * kN + 16 * q + 4 * g;
+            const float4 x = *reinterpret_cast<const float4 *>(rows), y = *reinterpret_cast<const float4 *>(rows + kN);
+            const float t0 = x.x + y.x, t1 = x.y + y.y, t2 = x.z + y.z, t3 = x.w + y.w;
+            store4(a.gu + (int64_t)(b0 + done * a.bstep) * C + h * kN + 16 * q + 4 * g, t0, t1, t2, t3);
+            const uint32_t p01 = pack_bf16x2(t0, t1), p23 = pack_bf16x2(t2, t3);
+            float4 *sum = reinterpret_cast<float4 *>(gu_lds + 4 * kN + 16 * q + 4 * g);
+            float4 acc = *sum;
+            acc.x += __uint_as_float(p01 << 16); acc.y += __uint_as_float(p01 & 0xffff0000u);
+            acc.z += __uint_as_float(p23 << 16); acc.w += __uint_as_float(p23 & 0xffff0000u);
+            *sum = acc;
+        }
+    };
+    if (HALF == 0 && l16 == 0) *reinterpret_cast<float4 *>(gu_lds + 4 * kN + 16 * q + 4 * g) = make_float4(0.f, 0.f, 0.f, 0.f);
     float *scratch = reinterpret_cast<float *>(smem + BlockBwdLds::kScratch) + (4 * HALF + q) * 16;
     const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
     const BlockLane la(l16, g);
     const uint32_t la_state = block_lane_state(q, l16, g), la_cols = block_lane_cols4(q, l16, g);
     const uint32_t gt_lo = tile_off(col, 8 * g), gt_hi = tile_off(col, 32 + 8 * g);
     LdsFlag g_flags = (LdsFlag)(smem + BlockBwdLds::kGFlags);
-    for (int it = 0; it < nchunk; ++it) {
-        const int c = nchunk - 1 - it;
+    int cv = 0, slot = 0;   // visit `it` is the cv-th visit of pair number `slot`: chunk nchunk-1-cv
+    for (int it = 0; it < nvisit; ++it) {
+        const int c = nchunk - 1 - cv;
         __syncthreads();
+        if (kMulti && HALF == 0 && cv == 0 && slot > 0) deliver_gu(slot - 1);
+        if (kMulti && cv == 0 && slot > 0) {   // a new pair: its rows, the reverse state from zero
+            const int64_t base = (int64_t)(b0 + slot * a.bstep) * T * C + (int64_t)h * kN;
+            gr_h = reinterpret_cast<char *>(a.gr + base); gk_h = reinterpret_cast<char *>(a.gk + base); gw_h = reinterpret_cast<char *>(a.gw + base);
+#pragma unroll
+            for (int m = 0; m < 4; ++m) Gj[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            pend = 1.f;
+            gu_acc[0] = gu_acc[1] = gu_acc[2] = gu_acc[3] = 0.f;
+        }
         const unsigned char *rt = smem + BlockBwdLds::kRawRK + (it % 3) * 2 * kTileBytes, *kt = rt + kTileBytes;
         const unsigned char *wt = smem + BlockBwdLds::kRawW + (it % 3) * kTileBytes;
         const unsigned char *vt = smem + BlockBwdLds::kRawVG + (it & 1) * 2 * kTileBytes, *gyt = vt + kTileBytes;
@@ -320,18 +352,18 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
             *reinterpret_cast<u32x4 *>(gw_h + go) = pair_rows_8ch(packed[2][0][0], packed[2][0][1], packed[2][1][0], packed[2][1][1]);
         }
         __builtin_amdgcn_sched_barrier(0);
-    }
-    // gu: fold the 16 tokens of a row, then the two halves; lanes l16 = 0 hold channels 16q + 4g + rr
+        if (++cv == nchunk) {
+            // the pair is done.  gu: fold the 16 tokens of a row; lanes l16 = 0 hold channels 16q + 4g + rr
 #pragma unroll
-    for (int rr = 0; rr < 4; ++rr) gu_acc[rr] = sum_row16(gu_acc[rr]);
-    float *gu_lds = reinterpret_cast<float *>(smem + BlockBwdLds::kGu);
-    if (HALF == 1 && l16 == 0) *reinterpret_cast<float4 *>(&gu_lds[16 * q + 4 * g]) = make_float4(gu_acc[0], gu_acc[1], gu_acc[2], gu_acc[3]);
+            for (int rr = 0; rr < 4; ++rr) gu_acc[rr] = sum_row16(gu_acc[rr]);
+            if (l16 == 0) *reinterpret_cast<float4 *>(&gu_lds[((slot & 1) * 2 + HALF) * kN + 16 * q + 4 * g]) = make_float4(gu_acc[0], gu_acc[1], gu_acc[2], gu_acc[3]);
+            cv = 0;
+            ++slot;
+        }
+    }
     __threadfence_block();
     __syncthreads();
-    if (HALF == 0 && l16 == 0 && !*s_wild) {   // (the exact second pass writes gu itself)
-        const float4 o = *reinterpret_cast<const float4 *>(&gu_lds[16 * q + 4 * g]);
-        store4(a.gu + (int64_t)b * C + h * kN + 16 * q + 4 * g, gu_acc[0] + o.x, gu_acc[1] + o.y, gu_acc[2] + o.z, gu_acc[3] + o.w);
-    }
+    if (HALF == 0) deliver_gu(npw - 1);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -402,27 +434,40 @@ __device__ __forceinline__ void block_bwd_gv(const unsigned char *smem, bf16_t *
 // ------------------------------------------------------------------------------------------
 // Producer wave p: loads, operand preparation of tokens 16p..16p+15, then the gv role.
 // ------------------------------------------------------------------------------------------
-__device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsigned char *smem, int *s_wild, int bh, int p, int lane)
+template <bool kMulti>
+__device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsigned char *smem, int *s_wild, int pair0, int p, int lane)
 {
     const int T = a.T, H = a.H;
     const int g = lane >> 4, l16 = lane & 15;
     const int64_t C = (int64_t)H * kN;
     const int nchunk = T / kBlockTokens;
-    const int b = bh / H, h = bh - b * H;
+    const int b0 = pair0 / H, h = pair0 - b0 * H;
+    const int npw = kMulti ? (a.B - b0 + a.bstep - 1) / a.bstep : 1;
+    const int nvisit = npw * nchunk;
     const uint32_t rowbytes = (uint32_t)C * 2u;
     const uint32_t lds0 = lds_address(smem);
-    const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
-    const bf16_t *rb = a.r + base, *kb_ = a.k + base, *vb = a.v + base, *wb = a.w + base, *gb = a.gy + base;
-    const bf16_t *ckb = reinterpret_cast<const bf16_t *>(a.ckpt + (int64_t)bh * nchunk * (kN * kN));
-    bf16_t *gvb = a.gv + base;
+    // first element of the workgroup's pair number `slot` in a (B,T,C) tensor; its saved states
+    auto pair_base = [&](int slot) { return (int64_t)(b0 + slot * a.bstep) * T * C + (int64_t)h * kN; };
+    auto pair_states = [&](int slot) {
+        return reinterpret_cast<const bf16_t *>(a.ckpt + (int64_t)((b0 + slot * a.bstep) * H + h) * nchunk * (kN * kN));
+    };
     const int lrow = lane >> 3;
     const uint32_t lpiece = (uint32_t)(((lane & 7) ^ lrow) << 4);
-    // item `it` = chunk nchunk-1-it.  r, k, w go out two visits ahead (they are prepared one visit ahead),
-    // v, gy and the chunk's saved state one visit ahead.
-    auto issue_rkw = [&](int it) {
-        const int tb = (nchunk - 1 - it) * kBlockTokens + 16 * p;
-        const uint32_t rk = lds0 + BlockBwdLds::kRawRK + (it % 3) * 2 * kTileBytes + 16 * p * kTileRow;
-        const uint32_t ww = lds0 + BlockBwdLds::kRawW + (it % 3) * kTileBytes + 16 * p * kTileRow;
+    // Every stream walks the flat sequence of visits (pair 0 chunk nchunk-1, .., 0, pair 1 chunk nchunk-1, ..) with
+    // a cursor of its own: visit number `it`, its position `c` in its pair (chunk nchunk-1-c), the pair's number.
+    struct Cursor {
+        int it = 0, c = 0, slot = 0;
+    };
+    Cursor cr, cg, cp, co;   // r/k/w loads, v/gy/state loads, operand preparation, gv role
+    const bf16_t *rb = a.r + pair_base(0), *kb_ = a.k + pair_base(0), *wb = a.w + pair_base(0);
+    const bf16_t *vb = a.v + pair_base(0), *gb = a.gy + pair_base(0), *ckb = pair_states(0);
+    bf16_t *gvb = a.gv + pair_base(0);
+    // r, k, w go out two visits ahead (they are prepared one visit ahead), v, gy and the chunk's saved state one
+    // visit ahead.
+    auto issue_rkw = [&]() {
+        const int tb = (nchunk - 1 - cr.c) * kBlockTokens + 16 * p;
+        const uint32_t rk = lds0 + BlockBwdLds::kRawRK + (cr.it % 3) * 2 * kTileBytes + 16 * p * kTileRow;
+        const uint32_t ww = lds0 + BlockBwdLds::kRawW + (cr.it % 3) * kTileBytes + 16 * p * kTileRow;
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
             const uint32_t o = (uint32_t)(tb + 8 * hf + lrow) * rowbytes + lpiece;
@@ -430,12 +475,18 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
             load_rows8_to_lds(wb, o, ww + 8 * hf * kTileRow);
             load_rows8_to_lds(rb, o, rk + 8 * hf * kTileRow);
         }
+        ++cr.it;
+        if (kMulti && ++cr.c == nchunk) {
+            cr.c = 0; ++cr.slot;
+            const int64_t nb = pair_base(cr.slot);
+            rb = a.r + nb; kb_ = a.k + nb; wb = a.w + nb;
+        } else if (!kMulti) ++cr.c;
     };
-    auto issue_vg_state = [&](int it) {
-        const int tb = (nchunk - 1 - it) * kBlockTokens + 16 * p;
-        const uint32_t vg = lds0 + BlockBwdLds::kRawVG + (it & 1) * 2 * kTileBytes + 16 * p * kTileRow;
-        const bf16_t *src = ckb + (int64_t)(nchunk - 1 - it) * (kN * kN);
-        const uint32_t dst = lds0 + BlockBwdLds::kState + (it & 1) * kTileBytes + 16 * p * kTileRow;
+    auto issue_vg_state = [&]() {
+        const int tb = (nchunk - 1 - cg.c) * kBlockTokens + 16 * p;
+        const uint32_t vg = lds0 + BlockBwdLds::kRawVG + (cg.it & 1) * 2 * kTileBytes + 16 * p * kTileRow;
+        const bf16_t *src = ckb + (int64_t)(nchunk - 1 - cg.c) * (kN * kN);
+        const uint32_t dst = lds0 + BlockBwdLds::kState + (cg.it & 1) * kTileBytes + 16 * p * kTileRow;
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
             const uint32_t o = (uint32_t)(tb + 8 * hf + lrow) * rowbytes + lpiece;
@@ -443,12 +494,19 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
             load_rows8_to_lds(vb, o, vg + 8 * hf * kTileRow);
             load_rows8_to_lds(gb, o, vg + kTileBytes + 8 * hf * kTileRow);
         }
+        ++cg.it;
+        if (kMulti && ++cg.c == nchunk) {
+            cg.c = 0; ++cg.slot;
+            const int64_t nb = pair_base(cg.slot);
+            vb = a.v + nb; gb = a.gy + nb; ckb = pair_states(cg.slot);
+        } else if (!kMulti) ++cg.c;
     };
     float u4[4];
-    load4(a.u + h * kN + 4 * l16, u4);
-    // `younger`: vector-memory operations this wave has issued behind the tile loads of item `it` (a
-    // wave's operations complete in program order, so those may stay in flight)
-    auto prepare = [&](int it, int younger) {
+    load4(a.u + h * kN + 4 * l16, u4);   // (all pairs of a workgroup belong to one head)
+    // the next visit in line; `younger`: vector-memory operations this wave has issued behind that visit's tile
+    // loads (a wave's operations complete in program order, so those may stay in flight)
+    auto prepare = [&](int younger) {
+        const int it = cp.it;
         unsigned char *rk = smem + BlockBwdLds::kRawRK + (it % 3) * 2 * kTileBytes;
         unsigned char *ww = smem + BlockBwdLds::kRawW + (it % 3) * kTileBytes;
         unsigned char *al = smem + BlockBwdLds::kAlpha + (it & 1) * kTileBytes;
@@ -463,24 +521,28 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
                 *reinterpret_cast<uint2 *>(al + o) = make_uint2(pack_bf16x2(xa[0], xa[1]), pack_bf16x2(xa[2], xa[3]));
                 *reinterpret_cast<uint2 *>(ww + o) = make_uint2(pack_bf16x2(ew2[0] * kLn2, ew2[1] * kLn2), pack_bf16x2(ew2[2] * kLn2, ew2[3] * kLn2));
             });
-        if (!ok && lane == 0) *s_wild = 1;
+        if (!ok && lane == 0) s_wild[cp.slot] = 1;
+        ++cp.it;
+        if (kMulti && ++cp.c == nchunk) { cp.c = 0; ++cp.slot; }
     };
     constexpr int kRkwLoads = 6, kVgStateLoads = 6, kGvStores = 2;
-    issue_vg_state(0);
-    issue_rkw(0);
-    if (nchunk > 1) issue_rkw(1);
-    prepare(0, nchunk > 1 ? kRkwLoads : 0);
-    for (int it = 0; it < nchunk; ++it) {
+    issue_vg_state();
+    issue_rkw();
+    if (nvisit > 1) issue_rkw();
+    prepare(nvisit > 1 ? kRkwLoads : 0);
+    for (int it = 0; it < nvisit; ++it) {
         __syncthreads();
-        // free again: every tile of item it-1
-        const int vgs = it + 1 < nchunk ? kVgStateLoads : 0, rkw = it + 2 < nchunk ? kRkwLoads : 0;
-        if (it + 1 < nchunk) issue_vg_state(it + 1);
-        if (it + 2 < nchunk) issue_rkw(it + 2);
-        // behind the r, k, w loads of item it+1 (issued one visit ago): that visit's gv stores, and this visit's loads
-        if (it + 1 < nchunk) prepare(it + 1, (it > 0 ? kGvStores : 0) + vgs + rkw);
-        block_bwd_gv(smem, gvb, (uint32_t)C, nchunk - 1 - it, it, p, lane);
-        // v, gy and the state of the next item have to be in LDS when the other waves pass the barrier
-        if (it + 1 < nchunk) wait_in_flight(rkw + kGvStores);
+        // free again: every tile of visit it-1
+        const int vgs = it + 1 < nvisit ? kVgStateLoads : 0, rkw = it + 2 < nvisit ? kRkwLoads : 0;
+        if (it + 1 < nvisit) issue_vg_state();
+        if (it + 2 < nvisit) issue_rkw();
+        // behind the r, k, w loads of visit it+1 (issued one visit ago): that visit's gv stores, and this visit's loads
+        if (it + 1 < nvisit) prepare((it > 0 ? kGvStores : 0) + vgs + rkw);
+        block_bwd_gv(smem, gvb, (uint32_t)C, nchunk - 1 - co.c, it, p, lane);
+        ++co.c;
+        if (kMulti && co.c == nchunk) { co.c = 0; ++co.slot; gvb = a.gv + pair_base(co.slot); }
+        // v, gy and the state of the next visit have to be in LDS when the other waves pass the barrier
+        if (it + 1 < nvisit) wait_in_flight(rkw + kGvStores);
     }
     wait_loads<0>();
     __threadfence_block();
@@ -489,60 +551,82 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
 
 constexpr int kBlockBwdThreads = 12 * 64;
 
+template <bool kMulti>   // kMulti: a workgroup takes several pairs, one after the other
 __global__ __launch_bounds__(kBlockBwdThreads) void block_bwd_kernel(BlockBwdArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    __shared__ int s_wild;
+    __shared__ int s_wild[kBlockMaxSlots];   // per pair of the workgroup: 16 tokens left the scaled operands' range
     static_assert(sizeof(ScanBwdALds) <= BlockBwdLds::kBytes && sizeof(ScanBwdBLds) <= BlockBwdLds::kBytes,
                   "the exact second pass reuses the LDS block");
-    if (threadIdx.x == 0) s_wild = 0;
+    if (threadIdx.x < kBlockMaxSlots) s_wild[threadIdx.x] = 0;
     if (threadIdx.x < 8) reinterpret_cast<int *>(smem + BlockBwdLds::kGFlags)[threadIdx.x] = 0;
     __syncthreads();
 
-    const int bh = (int)blockIdx.x;
+    const int pair0 = (int)blockIdx.x;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if (wave < 4) block_bwd_producer(a, smem, &s_wild, bh, wave, lane);
-    else if (wave < 8) block_bwd_xw<0>(a, smem, &s_wild, bh, wave - 4, lane);
-    else block_bwd_xw<1>(a, smem, &s_wild, bh, wave - 8, lane);
-    const int b = bh / a.H, h = bh % a.H;
+    if (wave < 4) block_bwd_producer<kMulti>(a, smem, s_wild, pair0, wave, lane);
+    else if (wave < 8) block_bwd_xw<0, kMulti>(a, smem, s_wild, pair0, wave - 4, lane);
+    else block_bwd_xw<1, kMulti>(a, smem, s_wild, pair0, wave - 8, lane);
+    const int b0 = pair0 / a.H, h = pair0 - b0 * a.H;
+    const int npw = kMulti ? (a.B - b0 + a.bstep - 1) / a.bstep : 1;
     const int nchunk = a.T / kBlockTokens;
-    // exact second pass if 16 tokens of this pair left the range the scaled operands can hold; the
+    const int64_t slice = (int64_t)nchunk * (kN * kN), C = (int64_t)a.H * kN;
+    const int tid = threadIdx.x;
+    __threadfence_block();
+    __syncthreads();
+    // gu summed over the workgroup's pairs that the chunked code did (half 0 added them up as it stored them): out
+    // of the way of the second pass, which uses the whole LDS block
+    __shared__ float s_gu_wg[kN];
+    if (tid < kN) s_gu_wg[tid] = reinterpret_cast<const float *>(smem + BlockBwdLds::kGu)[4 * kN + tid];
+    // exact second pass for the pairs of which 16 tokens left the range the scaled operands can hold; the
     // pair's own slice of the state workspace (nchunk x 64 x 64 floats = T x 64) holds P
-    if (s_wild) {
-        float *ck = a.ckpt + (int64_t)bh * nchunk * (kN * kN);
+    for (int slot = 0; slot < npw; ++slot) {
+        if (!s_wild[slot]) continue;   // (uniform over the workgroup)
+        const int b = b0 + slot * a.bstep;
+        // (the pointers pass through a value the compiler cannot see through, so that nothing derived from them is
+        // computed ahead of the loop and kept in registers across the chunked code)
+        const int z = fresh_s(0);
+        float *ck = a.ckpt + (int64_t)(b * a.H + h) * slice + z;
         __syncthreads();
-        scan_bwd_a_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdALds *>(smem), b, h, a.T, a.H, a.r, a.k, a.v, a.w, a.u, a.gy,
-                                        a.gr, a.gu, ck, kN, nullptr, nullptr, nullptr);
+        scan_bwd_a_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdALds *>(smem), b, h, a.T, a.H, a.r + z, a.k + z, a.v + z, a.w + z, a.u + z, a.gy + z,
+                                        a.gr + z, a.gu + z, ck, kN, nullptr, nullptr, nullptr);
         __threadfence_block();
         __syncthreads();
-        scan_bwd_b_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdBLds *>(smem), b, h, a.T, a.H, a.r, a.k, a.v, a.w, a.u, a.gy, ck, kN,
-                                        a.gk, a.gv, a.gw, nullptr, nullptr, nullptr, true);
+        const int z2 = fresh_s(0);
+        scan_bwd_b_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdBLds *>(smem), b, h, a.T, a.H, a.r + z2, a.k + z2, a.v + z2, a.w + z2, a.u + z2, a.gy + z2,
+                                        ck + z2, kN, a.gk + z2, a.gv + z2, a.gw + z2, nullptr, nullptr, nullptr, true);
+        __threadfence_block();
         __syncthreads();
     }
-    // Fused batch sum of gu: the workgroup that is the last of its head to deliver adds up the B partials.
-    // The partials travel as written-through (agent scope) stores into the unused second half of each
-    // workgroup's workspace slice, completed before the arrival counter is bumped; no fence, which would
-    // write back the whole L2.
+    // (addresses formed from here on are not to be computed ahead of the second pass and kept across it)
+    int lane_id = tid;
+    asm volatile("" : "+v"(lane_id));
+    float part = 0.f;
+    if (a.gu_sum != nullptr && lane_id < kN) {
+        part = s_gu_wg[lane_id];
+        for (int slot = 0; slot < npw; ++slot)   // the redone pairs' rows, as the second pass stored them
+            if (s_wild[slot]) part += load1(a.gu + (int64_t)(b0 + slot * a.bstep) * C + h * kN + lane_id);
+    }
+    // Fused batch sum of gu: the workgroup that is the last of its head to deliver adds up the partials, one per
+    // workgroup of the head.  They travel as written-through (agent scope) stores into the unused second half of
+    // the workspace slice of each workgroup's first pair, completed before the arrival counter is bumped; no
+    // fence, which would write back the whole L2.
     if (a.gu_sum != nullptr) {
         __shared__ int s_last;
-        const int64_t slice = (int64_t)nchunk * (kN * kN), C = (int64_t)a.H * kN;
-        __threadfence_block();   // this workgroup's gu row (half 0 or the second pass) is written
-        __syncthreads();
-        const int tid = threadIdx.x;
+        const int nparts = a.bstep;   // workgroups of this head (first pairs h, h + H, ..)
         if (tid < kN) {          // wave 0
-            const float part = load1(a.gu + (int64_t)b * C + h * kN + tid);
-            __hip_atomic_store(a.ckpt + (int64_t)bh * slice + slice / 2 + tid, part, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(a.ckpt + (int64_t)pair0 * slice + slice / 2 + lane_id, part, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             if (tid == 0)
-                s_last = __hip_atomic_fetch_add(a.arrivals + h, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.B - 1;
+                s_last = __hip_atomic_fetch_add(a.arrivals + h, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nparts - 1;
         }
         __syncthreads();
         if (s_last && tid < kN) {
             float acc = 0.f;
-            for (int j = 0; j < a.B; ++j)
-                acc += __hip_atomic_load(a.ckpt + (int64_t)(h + j * a.H) * slice + slice / 2 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            store1(a.gu_sum + h * kN + tid, acc);
+            for (int j = 0; j < nparts; ++j)
+                acc += __hip_atomic_load(a.ckpt + (int64_t)(h + j * a.H) * slice + slice / 2 + lane_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            store1(a.gu_sum + h * kN + lane_id, acc);
             if (tid == 0) __hip_atomic_store(a.arrivals + h, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // armed again
         }
     }
@@ -556,15 +640,19 @@ hipError_t block_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
 {
     BlockBwdArgs a = {};
     a.T = (int)T; a.H = (int)H; a.B = (int)B;
+    const int64_t grid = block_grid(B, H);
+    a.bstep = B * H <= grid ? (int)B : (int)(grid / H);
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w;
     a.u = (const bf16_t *)u; a.gy = (const bf16_t *)gy;
     a.gr = (bf16_t *)gr; a.gk = (bf16_t *)gk; a.gv = (bf16_t *)gv; a.gw = (bf16_t *)gw; a.gu = (bf16_t *)gu;
     a.gu_sum = (bf16_t *)gu_sum;
     a.ckpt = (float *)workspace;
     a.arrivals = reinterpret_cast<int *>(reinterpret_cast<char *>(workspace) + chunk_backward_workspace_bytes(B, T, H));
-    hipError_t e = allow_dynamic_lds<block_bwd_kernel>(BlockBwdLds::kBytes);
+    const bool multi = B * H > grid;
+    hipError_t e = multi ? allow_dynamic_lds<block_bwd_kernel<true>>(BlockBwdLds::kBytes) : allow_dynamic_lds<block_bwd_kernel<false>>(BlockBwdLds::kBytes);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(block_bwd_kernel, dim3((unsigned)(B * H)), dim3(kBlockBwdThreads), BlockBwdLds::kBytes, st, a);
+    if (multi) hipLaunchKernelGGL(block_bwd_kernel<true>, dim3((unsigned)grid), dim3(kBlockBwdThreads), BlockBwdLds::kBytes, st, a);
+    else hipLaunchKernelGGL(block_bwd_kernel<false>, dim3((unsigned)grid), dim3(kBlockBwdThreads), BlockBwdLds::kBytes, st, a);
     return hipGetLastError();
 }
 

@@ -43,8 +43,6 @@ struct BlockFwdLds {
 };
 static_assert(BlockFwdLds::kBytes <= 160 * 1024, "LDS block of the block-form forward kernel");
 
-constexpr int kBlockMaxSlots = 64;   // pairs one workgroup takes at most
-
 struct BlockFwdArgs {
     int T, H, B;
     int bstep;               // batch rows between two pairs of a workgroup (B: one pair per workgroup)
@@ -338,7 +336,7 @@ __global__ __launch_bounds__(kBlockFwdThreads) void block_fwd_kernel(BlockFwdArg
 // Workgroups of a launch: one per pair, or -- more pairs than compute units -- as many as there are compute
 // units, rounded down to a multiple of H (so that a workgroup's pairs belong to one head); 0: the block form
 // does not take the shape.
-static int64_t block_grid(int64_t B, int64_t H) {
+int64_t block_grid(int64_t B, int64_t H) {
     const int64_t pairs = B * H, cus = compute_units();
     if (pairs <= cus) return pairs;
     const int64_t grid = cus / H * H;

@@ -62,6 +62,8 @@ hipError_t chunk_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
 // --- block form (wkv6_block_fwd.hip, wkv6_block_bwd.hip): a 64-token chunk as one block of the
 // recurrence; bf16 tensors, T a multiple of 64, between half a pair and one pair per compute unit.
 // Same arguments and the same saved-state layout as the tile form above, which takes every other case.
+// workgroups of a block-form launch (0: the shape is not taken)
+int64_t block_grid(int64_t B, int64_t H);
 bool block_forward_applies(int64_t B, int64_t T, int64_t H);
 hipError_t block_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
                          const void *r, const void *k, const void *v, const void *w, const void *u,

@@ -99,6 +99,21 @@ def test_block_form_several_pairs_state_in_out_and_fallback(op, oracle):
         check_close("sT", sT, sT_ref, BF16)
 
 
+def test_block_form_several_pairs_fallback_in_the_backward(op, oracle):
+    """Forward and backward with several pairs per workgroup, of which the first, a middle and the last one of
+    a workgroup are redone exactly: every gradient, and gu summed over the batch (the chunked pairs' rows
+    added up inside the kernel as they are stored, the redone pairs' rows read back)."""
+    B, T, H = 40, 128, 32
+    assert _several_pairs_per_workgroup(B, H)
+    ins = oracle.make_inputs(B, T, H, N, 93)
+    ins[3][0, 10:30, 64:128] = 6.0
+    ins[3][17, 70:90, 0:64] = 6.0
+    ins[3][39, 100:120, 31 * 64:] = 6.0
+    ins[3][39, 5:25, 0:64] = 6.0
+    y, grads, ref, gy_ref = _fwd_bwd(op, ins)
+    _check(oracle, y, grads, ref, gy_ref)
+
+
 def test_block_form_extreme_decay(op, oracle):
     """Pairs whose decay leaves the scaled operands' range are redone with the exact per-timestep code inside
     the same launch (forward and backward decide alike); decay exactly 0 and exactly 1; a 16-token stretch
