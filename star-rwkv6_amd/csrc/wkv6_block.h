@@ -150,9 +150,12 @@ __device__ __forceinline__ u32x4 pair_rows_8ch(uint32_t a0, uint32_t a1, uint32_
 // ew2 = exp(w) log2(e).  Returns false if the wave's 16 tokens leave the range the scaled operands
 // can hold (any channel).
 // `after_read()` runs once the raw rows are in registers (their LDS block may be refilled from then on).
-template <typename AfterRead, typename Emit>
+// kRagged: only the first `valid` tokens of the chunk exist; the others are prepared as r = k = 0 with
+// decay 1 (exp(w) = 0), so that they leave both states alone and contribute nothing (their rows hold
+// copies of the last token that exists).
+template <bool kRagged, typename AfterRead, typename Emit>
 __device__ __forceinline__ bool block_prepare(const unsigned char *raw_r, const unsigned char *raw_k, const unsigned char *raw_w,
-                                              float *vec, const float (&u4)[4], int p, int l16, int g, AfterRead after_read, Emit emit)
+                                              float *vec, const float (&u4)[4], int p, int l16, int g, int valid, AfterRead after_read, Emit emit)
 {
     uint2 qr[4], qk[4], qw[4];
 #pragma unroll
@@ -172,6 +175,10 @@ __device__ __forceinline__ bool block_prepare(const unsigned char *raw_r, const 
         unpack4(make_s16x4(qw[e].x, qw[e].y), fw);
 #pragma unroll
         for (int c = 0; c < 4; ++c) ew2[e][c] = exp2_fast(fmaf(fw[c], kLog2e, kLog2Log2e));   // exp(w) log2(e): exponents in base 2
+        if (kRagged && 16 * p + 4 * g + e >= valid) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) { fr[e][c] = 0.f; fk[e][c] = 0.f; ew2[e][c] = 0.f; }
+        }
     }
     // running sums: inside the lane (4 tokens), across the four lane groups; relative to the block's
     // middle, which is the END of an even wave's tokens and the START of an odd wave's

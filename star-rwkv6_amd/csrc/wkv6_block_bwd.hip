@@ -83,14 +83,14 @@ typedef volatile int __attribute__((address_space(3))) *LdsFlag;
 // Wave (q, HALF): key channels j = 16q .. 16q+15, block HALF of the visit (tokens 32 HALF .. +31):
 // gr, gk, gw, gu.  Gj[m]: reverse state, rows i = block_row_channel(m, g) + rr, column j = 16q + l16.
 // ------------------------------------------------------------------------------------------
-template <int HALF, bool kMulti>
+template <int HALF, bool kMulti, bool kRagged>
 __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned char *smem, const int *s_wild, int pair0, int q, int lane)
 {
     const int T = a.T, H = a.H;
     const int g = lane >> 4, l16 = lane & 15;
     const int col = 16 * q + l16;
     const int64_t C = (int64_t)H * kN;
-    const int nchunk = T / kBlockTokens;
+    const int nchunk = (T + kBlockTokens - 1) / kBlockTokens;
     const int b0 = pair0 / H, h = pair0 - b0 * H;
     const int npw = kMulti ? (a.B - b0 + a.bstep - 1) / a.bstep : 1;   // pairs of this workgroup: batch rows b0, b0 + bstep, ... (one head)
     const int nvisit = npw * nchunk;
@@ -337,7 +337,8 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
             }
             // the gradient of the first and the last decay of the sequence is zero by definition (the flow
             // balance leaves rounding residue there)
-            if ((HALF == 0 && n == 0 && c == 0 && l16 == 0) || (HALF == 1 && n == 1 && c == nchunk - 1 && l16 == 15)) {
+            if ((HALF == 0 && n == 0 && c == 0 && l16 == 0) ||
+                (kRagged ? c * kBlockTokens + (n == 0 ? R0 : R1) + l16 == T - 1 : (HALF == 1 && n == 1 && c == nchunk - 1 && l16 == 15))) {
                 gwo[0] = gwo[1] = gwo[2] = gwo[3] = 0.f;
             }
             packed[0][n][0] = pack_bf16x2(gro[0], gro[1]); packed[0][n][1] = pack_bf16x2(gro[2], gro[3]);
@@ -346,10 +347,16 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
         }
         {
             // 16 bytes per lane: token (g odd ? R1 : R0) + l16, channels 16q + 8 (g >> 1) .. +7
-            const uint32_t go = (uint32_t)(c * kBlockTokens + R0 + 16 * (g & 1) + l16) * rowbytes + 2u * (uint32_t)(16 * q + 8 * (g >> 1));
-            *reinterpret_cast<u32x4 *>(gr_h + go) = pair_rows_8ch(packed[0][0][0], packed[0][0][1], packed[0][1][0], packed[0][1][1]);
-            *reinterpret_cast<u32x4 *>(gk_h + go) = pair_rows_8ch(packed[1][0][0], packed[1][0][1], packed[1][1][0], packed[1][1][1]);
-            *reinterpret_cast<u32x4 *>(gw_h + go) = pair_rows_8ch(packed[2][0][0], packed[2][0][1], packed[2][1][0], packed[2][1][1]);
+            const int tok = c * kBlockTokens + R0 + 16 * (g & 1) + l16;
+            const uint32_t go = (uint32_t)tok * rowbytes + 2u * (uint32_t)(16 * q + 8 * (g >> 1));
+            const u32x4 o_r = pair_rows_8ch(packed[0][0][0], packed[0][0][1], packed[0][1][0], packed[0][1][1]);
+            const u32x4 o_k = pair_rows_8ch(packed[1][0][0], packed[1][0][1], packed[1][1][0], packed[1][1][1]);
+            const u32x4 o_w = pair_rows_8ch(packed[2][0][0], packed[2][0][1], packed[2][1][0], packed[2][1][1]);
+            if (!kRagged || tok < T) {   // (rows past the end of the sequence are not written)
+                *reinterpret_cast<u32x4 *>(gr_h + go) = o_r;
+                *reinterpret_cast<u32x4 *>(gk_h + go) = o_k;
+                *reinterpret_cast<u32x4 *>(gw_h + go) = o_w;
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
         if (++cv == nchunk) {
@@ -370,7 +377,8 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
 // gv role of a producer wave: wave q owns value columns i = 16q..16q+15.  The reverse state comes from
 // the waves that step it (g2 o G at the end of each block, as they publish it in kGt).
 // ------------------------------------------------------------------------------------------
-__device__ __forceinline__ void block_bwd_gv(const unsigned char *smem, bf16_t *gv_h, uint32_t rowelems, int c, int it, int q, int lane)
+template <bool kRagged>
+__device__ __forceinline__ void block_bwd_gv(const unsigned char *smem, bf16_t *gv_h, uint32_t rowelems, int T, int c, int it, int q, int lane)
 {
     const int g = lane >> 4, l16 = lane & 15;
     const unsigned char *rt = smem + BlockBwdLds::kRawRK + (it % 3) * 2 * kTileBytes, *kt = rt + kTileBytes;
@@ -425,22 +433,23 @@ __device__ __forceinline__ void block_bwd_gv(const unsigned char *smem, bf16_t *
         V0 = mfma16(gyq1, pack4(A10), V0);
         settle(GV0, GV1, V0, V1);
         // 16 bytes per lane: token (g odd ? R1 : R0) + l16, channels 16q + 8 (g >> 1) .. +7
-        *reinterpret_cast<u32x4 *>(gv_h + ((uint32_t)(c * kBlockTokens + R0 + 16 * (g & 1) + l16) * rowelems + (uint32_t)(16 * q + 8 * (g >> 1)))) =
-            pair_rows_8ch(pack_bf16x2(GV0[0] + V0[0], GV0[1] + V0[1]), pack_bf16x2(GV0[2] + V0[2], GV0[3] + V0[3]),
-                          pack_bf16x2(GV1[0] + V1[0], GV1[1] + V1[1]), pack_bf16x2(GV1[2] + V1[2], GV1[3] + V1[3]));
+        const int tok = c * kBlockTokens + R0 + 16 * (g & 1) + l16;
+        const u32x4 o_v = pair_rows_8ch(pack_bf16x2(GV0[0] + V0[0], GV0[1] + V0[1]), pack_bf16x2(GV0[2] + V0[2], GV0[3] + V0[3]),
+                                        pack_bf16x2(GV1[0] + V1[0], GV1[1] + V1[1]), pack_bf16x2(GV1[2] + V1[2], GV1[3] + V1[3]));
+        if (!kRagged || tok < T) *reinterpret_cast<u32x4 *>(gv_h + ((uint32_t)tok * rowelems + (uint32_t)(16 * q + 8 * (g >> 1)))) = o_v;
     }
 }
 
 // ------------------------------------------------------------------------------------------
 // Producer wave p: loads, operand preparation of tokens 16p..16p+15, then the gv role.
 // ------------------------------------------------------------------------------------------
-template <bool kMulti>
+template <bool kMulti, bool kRagged>
 __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsigned char *smem, int *s_wild, int pair0, int p, int lane)
 {
     const int T = a.T, H = a.H;
     const int g = lane >> 4, l16 = lane & 15;
     const int64_t C = (int64_t)H * kN;
-    const int nchunk = T / kBlockTokens;
+    const int nchunk = (T + kBlockTokens - 1) / kBlockTokens;
     const int b0 = pair0 / H, h = pair0 - b0 * H;
     const int npw = kMulti ? (a.B - b0 + a.bstep - 1) / a.bstep : 1;
     const int nvisit = npw * nchunk;
@@ -453,6 +462,8 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
     };
     const int lrow = lane >> 3;
     const uint32_t lpiece = (uint32_t)(((lane & 7) ^ lrow) << 4);
+    // byte offset of this lane's piece of token row t of a pair (kRagged: rows past the end read the last row)
+    auto row_offset = [&](int t) { return (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes + lpiece; };
     // Every stream walks the flat sequence of visits (pair 0 chunk nchunk-1, .., 0, pair 1 chunk nchunk-1, ..) with
     // a cursor of its own: visit number `it`, its position `c` in its pair (chunk nchunk-1-c), the pair's number.
     struct Cursor {
@@ -470,7 +481,7 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
         const uint32_t ww = lds0 + BlockBwdLds::kRawW + (cr.it % 3) * kTileBytes + 16 * p * kTileRow;
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
-            const uint32_t o = (uint32_t)(tb + 8 * hf + lrow) * rowbytes + lpiece;
+            const uint32_t o = row_offset(tb + 8 * hf + lrow);
             load_rows8_to_lds(kb_, o, rk + kTileBytes + 8 * hf * kTileRow);
             load_rows8_to_lds(wb, o, ww + 8 * hf * kTileRow);
             load_rows8_to_lds(rb, o, rk + 8 * hf * kTileRow);
@@ -489,7 +500,7 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
         const uint32_t dst = lds0 + BlockBwdLds::kState + (cg.it & 1) * kTileBytes + 16 * p * kTileRow;
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
-            const uint32_t o = (uint32_t)(tb + 8 * hf + lrow) * rowbytes + lpiece;
+            const uint32_t o = row_offset(tb + 8 * hf + lrow);
             load_rows8_to_lds(src, (uint32_t)((16 * p + 8 * hf + lrow) * kTileRow) + lpiece, dst + 8 * hf * kTileRow);
             load_rows8_to_lds(vb, o, vg + 8 * hf * kTileRow);
             load_rows8_to_lds(gb, o, vg + kTileBytes + 8 * hf * kTileRow);
@@ -513,7 +524,7 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
         float *vec = reinterpret_cast<float *>(smem + BlockBwdLds::kVec + (it & 1) * kBlockVecBytes);
         wait_in_flight(younger);
         const float kLn2 = 0.6931471805599453f;
-        const bool ok = block_prepare(rk, rk + kTileBytes, ww, vec, u4, p, l16, g, []() {},
+        const bool ok = block_prepare<kRagged>(rk, rk + kTileBytes, ww, vec, u4, p, l16, g, T - (nchunk - 1 - cp.c) * kBlockTokens, []() {},
             [&](uint32_t o, const float (&xr)[4], const float (&xk)[4], const float (&xa)[4], const float (&ew2)[4]) {
                 // R~ and K~ take the place of the raw r and k, exp(w) that of the raw w
                 *reinterpret_cast<uint2 *>(rk + o) = make_uint2(pack_bf16x2(xr[0], xr[1]), pack_bf16x2(xr[2], xr[3]));
@@ -523,7 +534,8 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
             });
         if (!ok && lane == 0) s_wild[cp.slot] = 1;
         ++cp.it;
-        if (kMulti && ++cp.c == nchunk) { cp.c = 0; ++cp.slot; }
+        ++cp.c;
+        if (kMulti && cp.c == nchunk) { cp.c = 0; ++cp.slot; }
     };
     constexpr int kRkwLoads = 6, kVgStateLoads = 6, kGvStores = 2;
     issue_vg_state();
@@ -538,7 +550,7 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
         if (it + 2 < nvisit) issue_rkw();
         // behind the r, k, w loads of visit it+1 (issued one visit ago): that visit's gv stores, and this visit's loads
         if (it + 1 < nvisit) prepare((it > 0 ? kGvStores : 0) + vgs + rkw);
-        block_bwd_gv(smem, gvb, (uint32_t)C, nchunk - 1 - co.c, it, p, lane);
+        block_bwd_gv<kRagged>(smem, gvb, (uint32_t)C, T, nchunk - 1 - co.c, it, p, lane);
         ++co.c;
         if (kMulti && co.c == nchunk) { co.c = 0; ++co.slot; gvb = a.gv + pair_base(co.slot); }
         // v, gy and the state of the next visit have to be in LDS when the other waves pass the barrier
@@ -551,7 +563,7 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
 
 constexpr int kBlockBwdThreads = 12 * 64;
 
-template <bool kMulti>   // kMulti: a workgroup takes several pairs, one after the other
+template <bool kMulti, bool kRagged>   // kMulti: a workgroup takes several pairs, one after the other; kRagged: T is no multiple of 64
 __global__ __launch_bounds__(kBlockBwdThreads) void block_bwd_kernel(BlockBwdArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -565,12 +577,12 @@ __global__ __launch_bounds__(kBlockBwdThreads) void block_bwd_kernel(BlockBwdArg
     const int pair0 = (int)blockIdx.x;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if (wave < 4) block_bwd_producer<kMulti>(a, smem, s_wild, pair0, wave, lane);
-    else if (wave < 8) block_bwd_xw<0, kMulti>(a, smem, s_wild, pair0, wave - 4, lane);
-    else block_bwd_xw<1, kMulti>(a, smem, s_wild, pair0, wave - 8, lane);
+    if (wave < 4) block_bwd_producer<kMulti, kRagged>(a, smem, s_wild, pair0, wave, lane);
+    else if (wave < 8) block_bwd_xw<0, kMulti, kRagged>(a, smem, s_wild, pair0, wave - 4, lane);
+    else block_bwd_xw<1, kMulti, kRagged>(a, smem, s_wild, pair0, wave - 8, lane);
     const int b0 = pair0 / a.H, h = pair0 - b0 * a.H;
     const int npw = kMulti ? (a.B - b0 + a.bstep - 1) / a.bstep : 1;
-    const int nchunk = a.T / kBlockTokens;
+    const int nchunk = (a.T + kBlockTokens - 1) / kBlockTokens;
     const int64_t slice = (int64_t)nchunk * (kN * kN), C = (int64_t)a.H * kN;
     const int tid = threadIdx.x;
     __threadfence_block();
@@ -648,12 +660,16 @@ hipError_t block_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
     a.gu_sum = (bf16_t *)gu_sum;
     a.ckpt = (float *)workspace;
     a.arrivals = reinterpret_cast<int *>(reinterpret_cast<char *>(workspace) + chunk_backward_workspace_bytes(B, T, H));
-    const bool multi = B * H > grid;
-    hipError_t e = multi ? allow_dynamic_lds<block_bwd_kernel<true>>(BlockBwdLds::kBytes) : allow_dynamic_lds<block_bwd_kernel<false>>(BlockBwdLds::kBytes);
-    if (e != hipSuccess) return e;
-    if (multi) hipLaunchKernelGGL(block_bwd_kernel<true>, dim3((unsigned)grid), dim3(kBlockBwdThreads), BlockBwdLds::kBytes, st, a);
-    else hipLaunchKernelGGL(block_bwd_kernel<false>, dim3((unsigned)grid), dim3(kBlockBwdThreads), BlockBwdLds::kBytes, st, a);
-    return hipGetLastError();
+    const bool multi = B * H > grid, ragged = (T % kBlockTokens) != 0;
+    auto launch = [&](auto multi_tag, auto ragged_tag) -> hipError_t {
+        constexpr auto kern = block_bwd_kernel<decltype(multi_tag)::value, decltype(ragged_tag)::value>;
+        hipError_t e = allow_dynamic_lds<kern>(BlockBwdLds::kBytes);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kBlockBwdThreads), BlockBwdLds::kBytes, st, a);
+        return hipGetLastError();
+    };
+    if (multi) return ragged ? launch(std::true_type{}, std::true_type{}) : launch(std::true_type{}, std::false_type{});
+    return ragged ? launch(std::false_type{}, std::true_type{}) : launch(std::false_type{}, std::false_type{});
 }
 
 }  // namespace wkv6

@@ -1,6 +1,6 @@
 // WKV6 forward in block form for gfx950 (bf16 MFMA for the dense products, fp32 state), for bf16
-// tensors, sequence lengths that are a multiple of 64 and more than half a (batch, head) pair per
-// compute unit.  The tile form in wkv6_chunk_fwd.hip (state advanced every 16 tokens) serves every
+// tensors and more than half a (batch, head) pair per compute unit (a sequence length that is no
+// multiple of 64 leaves the last chunk with tokens past the end: kRagged).  The tile form in wkv6_chunk_fwd.hip (state advanced every 16 tokens) serves every
 // other case.  Notation and the operand scaling are in wkv6_block.h.
 //
 // One workgroup per pair; with more pairs than compute units one workgroup per compute unit, which runs
@@ -64,7 +64,7 @@ __device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsign
 {
     const int T = a.T, H = a.H;
     const int g = lane >> 4, l16 = lane & 15;
-    const int nchunk = T / kBlockTokens;
+    const int nchunk = (T + kBlockTokens - 1) / kBlockTokens;
     const int b0 = pair0 / H, h = pair0 - b0 * H;
     const int npw = (a.B - b0 + a.bstep - 1) / a.bstep;   // pairs of this workgroup: batch rows b0, b0 + bstep, ...
     const int nvisit = npw * nchunk;
@@ -180,13 +180,13 @@ __device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsign
 // ------------------------------------------------------------------------------------------
 // Producer wave p: tokens 16p..16p+15 of every chunk.
 // ------------------------------------------------------------------------------------------
-template <bool kSave>
+template <bool kSave, bool kRagged>
 __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsigned char *smem, int *s_wild, int pair0, int p, int lane)
 {
     const int T = a.T, H = a.H;
     const int g = lane >> 4, l16 = lane & 15;
     const int64_t C = (int64_t)H * kN;
-    const int nchunk = T / kBlockTokens;
+    const int nchunk = (T + kBlockTokens - 1) / kBlockTokens;
     const int b0 = pair0 / H, h = pair0 - b0 * H;
     const int npw = (a.B - b0 + a.bstep - 1) / a.bstep;
     const int nvisit = npw * nchunk;
@@ -197,6 +197,8 @@ __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsign
     // this lane's part of an 8-row block: row (lane >> 3), 16-byte piece swizzled with the row
     const int lrow = lane >> 3;
     const uint32_t lpiece = (uint32_t)(((lane & 7) ^ lrow) << 4);
+    // byte offset of this lane's piece of token row t of a pair (kRagged: rows past the end read the last row)
+    auto row_offset = [&](int t) { return (uint32_t)(kRagged ? min(t, T - 1) : t) * rowbytes + lpiece; };
     // Every stream walks the flat sequence of visits (pair 0 chunk 0, 1, .., pair 1 chunk 0, ..) with a cursor
     // of its own: visit number `it`, its chunk `c`, and the pointers of its pair.
     struct Cursor {
@@ -214,7 +216,7 @@ __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsign
         const uint32_t vv = lds0 + BlockFwdLds::kRawV + (cv.it & 3) * kTileBytes + 16 * p * kTileRow;
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk)
-            load_rows8_to_lds(vb, (uint32_t)(cv.c * kBlockTokens + 16 * p + 8 * blk + lrow) * rowbytes + lpiece, vv + 8 * blk * kTileRow);
+            load_rows8_to_lds(vb, row_offset(cv.c * kBlockTokens + 16 * p + 8 * blk + lrow), vv + 8 * blk * kTileRow);
         issued += 2;
         ++cv.it;
         if (++cv.c == nchunk) { cv.c = 0; ++cv.slot; vb = a.v + pair_base(cv.slot); }
@@ -223,7 +225,7 @@ __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsign
         const uint32_t raw = lds0 + BlockFwdLds::kRaw + (cr.it & 1) * 3 * kTileBytes + 16 * p * kTileRow;
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
-            const uint32_t o = (uint32_t)(cr.c * kBlockTokens + 16 * p + 8 * blk + lrow) * rowbytes + lpiece;
+            const uint32_t o = row_offset(cr.c * kBlockTokens + 16 * p + 8 * blk + lrow);
             load_rows8_to_lds(wb, o, raw + 2 * kTileBytes + 8 * blk * kTileRow);
             load_rows8_to_lds(rb, o, raw + 8 * blk * kTileRow);
             load_rows8_to_lds(kb_, o, raw + kTileBytes + 8 * blk * kTileRow);
@@ -246,7 +248,8 @@ __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsign
         for (int blk = 0; blk < 2; ++blk) {
             const int row = 16 * p + 8 * blk + lrow;
             const uint4 x = *reinterpret_cast<const uint4 *>(ys + row * kTileRow + (lane & 7) * 16);
-            *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(yb) + ((uint32_t)(co.c * kBlockTokens + row) * rowbytes + lpiece)) = x;
+            if (!kRagged || co.c * kBlockTokens + row < T)
+                *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(yb) + ((uint32_t)(co.c * kBlockTokens + row) * rowbytes + lpiece)) = x;
             if (kSave) {
                 const uint4 s = *reinterpret_cast<const uint4 *>(ss + row * kTileRow + (lane & 7) * 16);
                 *reinterpret_cast<uint4 *>(ckb + ((uint32_t)co.c * (uint32_t)(kN * kN * 2) + (uint32_t)(row * kTileRow) + lpiece)) = s;
@@ -270,7 +273,7 @@ __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsign
         unsigned char *op = smem + BlockFwdLds::kOp + (it & 1) * 2 * kTileBytes;
         float *vec = reinterpret_cast<float *>(smem + BlockFwdLds::kVec + (it & 1) * kBlockVecBytes);
         wait_in_flight(issued - ((it & 1) ? mark_odd : mark_even));
-        const bool ok = block_prepare(raw, raw + kTileBytes, raw + 2 * kTileBytes, vec, u4, p, l16, g,
+        const bool ok = block_prepare<kRagged>(raw, raw + kTileBytes, raw + 2 * kTileBytes, vec, u4, p, l16, g, T - cp.c * kBlockTokens,
             [&]() {
                 if (more) {
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -305,7 +308,7 @@ __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsign
 
 constexpr int kBlockFwdThreads = 12 * 64;
 
-template <typename Ts, bool kSave>
+template <typename Ts, bool kSave, bool kRagged>
 __global__ __launch_bounds__(kBlockFwdThreads) void block_fwd_kernel(BlockFwdArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
@@ -317,7 +320,7 @@ __global__ __launch_bounds__(kBlockFwdThreads) void block_fwd_kernel(BlockFwdArg
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int pair0 = (int)blockIdx.x;
-    if (wave < 4) block_fwd_producer<kSave>(a, smem, s_wild, pair0, wave, lane);
+    if (wave < 4) block_fwd_producer<kSave, kRagged>(a, smem, s_wild, pair0, wave, lane);
     else if (wave < 8) block_fwd_consumer<Ts, kSave, 0>(a, smem, pair0, wave - 4, lane);
     else block_fwd_consumer<Ts, kSave, 1>(a, smem, pair0, wave - 8, lane);
     // exact second pass for the pairs of which 16 tokens left the range the scaled operands can hold
@@ -348,7 +351,7 @@ int64_t block_grid(int64_t B, int64_t H) {
 bool block_forward_applies(int64_t B, int64_t T, int64_t H) {
     const int64_t pairs = B * H, cus = compute_units();
     // (with fewer pairs than half the compute units the tile form shares a pair out over several workgroups)
-    return T >= kBlockTokens && (T % kBlockTokens) == 0 && 2 * pairs > cus && block_grid(B, H) > 0;
+    return 2 * pairs > cus && block_grid(B, H) > 0 && T * H * kN < (1LL << 31);
 }
 
 hipError_t block_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
@@ -362,16 +365,19 @@ hipError_t block_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
     a.s0 = s0; a.map = map; a.y = (bf16_t *)y; a.sT = sT; a.ckpt = (float *)saved_states;
     a.arrivals = saved_states && counters ? reinterpret_cast<int *>(reinterpret_cast<char *>(saved_states) + chunk_backward_workspace_bytes(B, T, H)) : nullptr;
-    auto launch = [&](auto ts_tag, auto save_tag) -> hipError_t {
-        constexpr auto kern = block_fwd_kernel<decltype(ts_tag), decltype(save_tag)::value>;
+    auto launch = [&](auto ts_tag, auto save_tag, auto ragged_tag) -> hipError_t {
+        constexpr auto kern = block_fwd_kernel<decltype(ts_tag), decltype(save_tag)::value, decltype(ragged_tag)::value>;
         hipError_t e = allow_dynamic_lds<kern>(BlockFwdLds::kBytes);
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kBlockFwdThreads), BlockFwdLds::kBytes, st, a);
         return hipGetLastError();
     };
+    auto launch_ts = [&](auto ts_tag, auto save_tag) -> hipError_t {
+        return (T % kBlockTokens) != 0 ? launch(ts_tag, save_tag, std::true_type{}) : launch(ts_tag, save_tag, std::false_type{});
+    };
     const bool save = saved_states != nullptr;
-    if (state_dtype == kF32) return save ? launch(float{}, std::true_type{}) : launch(float{}, std::false_type{});
-    return save ? launch(bf16_t{}, std::true_type{}) : launch(bf16_t{}, std::false_type{});
+    if (state_dtype == kF32) return save ? launch_ts(float{}, std::true_type{}) : launch_ts(float{}, std::false_type{});
+    return save ? launch_ts(bf16_t{}, std::true_type{}) : launch_ts(bf16_t{}, std::false_type{});
 }
 
 }  // namespace wkv6

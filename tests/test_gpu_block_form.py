@@ -220,24 +220,35 @@ def test_either_forward_feeds_either_backward(oracle):
         assert float((a.float() - b.float()).abs().max()) <= 2e-2 * float(a.float().abs().max())
 
 
-def test_block_form_is_taken(oracle):
-    """The saving pair at the benchmark's shape agrees with the tile-form kernels to rounding but not bit for
-    bit (a different operand scaling): the block form is what runs there.  (T = 1000 is outside its range and
-    runs the tile form in both calls of the comparison, bit for bit.)"""
+def test_sequence_end_does_not_reach_back(oracle):
+    """The first T tokens of a sequence that is 8 tokens longer (its last chunk then has tokens past the end,
+    which are prepared as r = k = 0 with decay 1) give the y of the T-token sequence: bit for bit where the extra
+    tokens have a chunk of their own, to rounding where they share the last chunk."""
     import rwkv_kernel
 
     op = rwkv_kernel.RWKVKernelOperator(N, 4096)
     B, H = 8, 32
-    for T, same in ((1024, False), (1000, True)):
+    for T in (1024, 1000, 64):
         ins = oracle.make_inputs(B, T, H, N, 5)
         dev, _ = cast_inputs(ins[:5], BF16)
         op.algo = CHUNK
         with torch.no_grad():
-            y1, _ = op(*dev)
-            # the same tokens as the first part of a sequence that is 8 tokens longer: the tile form takes it
+            y1, s1 = op(*dev, return_state=True)
             longer = [torch.cat([x, x[:, :8]], 1).contiguous() for x in dev[:4]] + [dev[4]]
             y2, _ = op(*longer)
         torch.cuda.synchronize()
-        y2 = y2[:, :T]
-        assert float((y1.float() - y2.float()).abs().max()) <= 2e-2 * float(y1.float().abs().max())
-        assert torch.equal(y1, y2) == same, T
+        if T % 64 == 0:
+            assert torch.equal(y1, y2[:, :T]), T
+        else:   # (the extra tokens share the last chunk: its blocks are scaled from other reference values)
+            assert float((y1.float() - y2[:, :T].float()).abs().max()) <= 2e-2 * float(y1.float().abs().max()), T
+
+
+# (B, T, H): sequence lengths that are no multiple of 64 -- one token more than a chunk, one less, T < 64, an odd
+# number of chunks, several pairs per workgroup
+@pytest.mark.parametrize("B,T,H", [(5, 250, 32), (3, 65, 64), (5, 63, 32), (129, 1, 1), (8, 1000, 32), (40, 100, 32), (75, 150, 4),
+                                   (300, 33, 1)])
+def test_block_form_ragged_sequence_end(op, oracle, B, T, H):
+    assert _pairs_in_range(B, H) or _several_pairs_per_workgroup(B, H)
+    print("block form, ragged B=%d T=%d H=%d" % (B, T, H), flush=True)
+    y, grads, ref, gy_ref = _fwd_bwd(op, oracle.make_inputs(B, T, H, N, 800 + T + H))
+    _check(oracle, y, grads, ref, gy_ref)
