@@ -20,11 +20,9 @@
 //   gw_t[j]  = -exp(w_t[j]) ( E[j] + sum_{m<t} (Q_m - P_m) - P_t ),  E[j] = sum_i S0[j][i] G_new[j][i]
 // (the last line is the flow balance across decay step t, anchored at the exact tile-boundary term E).
 //
-// Workgroup: one per (batch, head) -- or, with more pairs than compute units (kMulti), one per
-// compute unit that takes every gridDim.x-th pair, back to back through the same pipeline: the next
-// pair's first chunks are loaded and prepared while the last chunks of the current one are worked on
-// (a workgroup fills the LDS of its compute unit, so nothing else would hide that).  The grid is then a
-// multiple of H, so that all pairs of a workgroup belong to the same head.
+// Workgroup: one per (batch, head).  (With more pairs than half the compute units the block-form
+// kernel in wkv6_block_bwd.hip runs instead, unless gradients flow through the state or the tensors
+// are fp16.)
 // 12 waves in four-wave roles (one wave of each role per SIMD):
 //   loader/producer (wave p <-> tile p, lane = channel): brings the raw r, k, w, v, gy rows of a
 //       chunk from global memory straight into LDS tiles two items ahead (and the chunk's saved
@@ -59,9 +57,8 @@ struct BwdLds {
     static constexpr int kOpBytes = kOpRuk + CL * 4;
     static constexpr int kState = kOp + 2 * kOpBytes;                  // [item & 1] saved forward state of the chunk, bf16 [i][j] (transposed) as a tile
     static constexpr int kVgy = kState + 2 * kTileBytes;                    // [8 consumer waves][16] fp32: <v_t, gy_t>
-    static constexpr int kGu = kVgy + 8 * 16 * 4;                      // [pair parity][64] fp32: gu partial of consumer group 1
-    static constexpr int kGuSum = kGu + 2 * kN * 4;                    // [64] fp32: gu summed over the workgroup's pairs (several-pairs variant)
-    static constexpr int kBytes = kGuSum + kN * 4;
+    static constexpr int kGu = kVgy + 8 * 16 * 4;                      // [64] fp32: gu partial of consumer group 1
+    static constexpr int kBytes = kGu + kN * 4;
 };
 static_assert(BwdLds::kBytes <= 160 * 1024, "LDS block of the backward kernel");
 
@@ -73,7 +70,6 @@ struct BwdArgs {
     bf16_t *gu_sum;   // null, or C elements: receives the sum of gu over the batch
     int *arrivals;    // per head: workgroups that have delivered their gu partial (zero on entry)
     int B;
-    int npairs;       // B * H (a workgroup of the several-pairs variant takes every gridDim.x-th pair)
     float *ckpt;
     // gradients through the state (all null for the stateless operator): fp32 (B,H,64,64) [key][value]
     const float *s0, *gsT;   // initial state; gradient arriving at the final state
@@ -83,22 +79,15 @@ struct BwdArgs {
 // ------------------------------------------------------------------------------------------
 // Consumer group GRP of two: gr, gk, gw, gu.
 // ------------------------------------------------------------------------------------------
-// pairs a workgroup of the several-pairs variant takes at most (one flag each for the exact second pass)
-constexpr int kBwdMaxPairs = 64;
-
-template <typename Tin, bool kRagged, bool kMulti, int GRP>
+template <typename Tin, bool kRagged, int GRP>
 __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *smem, const int *s_wild, int pair0, int q, int lane)
 {
     const int T = a.T, H = a.H;
     const int g = lane >> 4, l16 = lane & 15;
     const int col = 16 * q + l16;   // the key channel j this lane's accumulator column holds
     const int64_t C = (int64_t)H * kN;
-    // kMulti: this workgroup's pairs are pair0, pair0 + gridDim.x, ...; the grid is a multiple of H, so
-    // they share the head and lie `bstep` batch rows apart
-    const int h = pair0 % H, bstep = kMulti ? (int)gridDim.x / H : 0;
-    const int npw = kMulti ? (a.npairs - pair0 + (int)gridDim.x - 1) / (int)gridDim.x : 1;
-    int b = pair0 / H;
-    int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
+    const int h = pair0 % H, b = pair0 / H;
+    const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
     const int nchunk = (T + CL - 1) / CL;
     auto mine = [](int p) { return (p & 1) == (GRP ^ 1); };   // group 0: tiles 3, 1; group 1: tiles 2, 0
     int item = 0;
@@ -114,22 +103,7 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     float gu_acc = 0.f;
     Tout *gr_h = reinterpret_cast<Tout *>(a.gr) + base, *gk_h = reinterpret_cast<Tout *>(a.gk) + base, *gw_h = reinterpret_cast<Tout *>(a.gw) + base;
     const uint32_t rowbytes = (uint32_t)C * (uint32_t)sizeof(Tout);
-    // kMulti, group 0: gu of the pair just finished, waiting for group 1's half (it is in LDS once the
-    // next barrier has been passed)
-    float gu_prev = 0.f;
-    float gu_wg = 0.f;   // kMulti, group 0: gu summed over the workgroup's pairs, as stored (for the fused batch sum)
-    int prev_slot = -1, prev_b = 0;
     float *gu_lds = reinterpret_cast<float *>(smem + BwdLds::kGu);
-    auto store_gu = [&](int b_, float total) {
-        Tout *dst = reinterpret_cast<Tout *>(a.gu) + (int64_t)b_ * C + h * kN + col;
-        store1(dst, total);
-        if (kMulti) gu_wg += sizeof(Tout) == 2 ? bf16_bits_to_float(pack_bf16x2(total, 0.f) & 0xffffu) : total;   // (as store1 rounds it)
-    };
-    auto deliver_gu = [&]() {
-        if (g == 0 && !s_wild[prev_slot])   // (the exact second pass writes gu itself)
-            store_gu(prev_b, gu_prev + gu_lds[(prev_slot & 1) * kN + col]);
-        prev_slot = -1;
-    };
     // Saved forward state of a chunk as packed bf16: Sraw[m] = S^T[i = 16m + 4g .. +3][j = col].  It
     // comes out of LDS, where the producer waves put the chunk's block from the workspace.  The
     // consumer waves issue no global load at all:
@@ -169,7 +143,6 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     };
     auto visit = [&](int c, uint2 (&Sraw)[4]) {
         __syncthreads();
-        if (kMulti && GRP == 0 && prev_slot >= 0) deliver_gu();
         {
             // the tile holds the state transposed (rows i, channels j): S^T[16m + 4g + e][col], e < 4, per read
             const unsigned char *stt = smem + BwdLds::kState + (item & 1) * kTileBytes;
@@ -345,23 +318,7 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
         }
         ++item;
     };
-    for (int pi = 0; pi < npw; ++pi) {
-        if (kMulti && pi > 0) {   // the next pair: its own rows, reverse state from zero
-            b += bstep;
-            base = (int64_t)b * T * C + (int64_t)h * kN;
-            gr_h = reinterpret_cast<Tout *>(a.gr) + base; gk_h = reinterpret_cast<Tout *>(a.gk) + base; gw_h = reinterpret_cast<Tout *>(a.gw) + base;
-#pragma unroll
-            for (int m = 0; m < 4; ++m) Gj[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        }
-        for (int c = nchunk - 1; c >= 0; --c) visit(c, Sraw);
-        if (kMulti && pi + 1 < npw) {   // hand this pair's gu over without a barrier of its own
-            gu_acc = sum_rows(gu_acc);
-            if (GRP == 1) { if (g == 0) gu_lds[(pi & 1) * kN + col] = gu_acc; }
-            else { gu_prev = gu_acc; prev_slot = pi; prev_b = b; }
-            gu_acc = 0.f;
-        }
-    }
-    const int last_slot = npw - 1;
+    for (int c = nchunk - 1; c >= 0; --c) visit(c, Sraw);
     if (a.gs0 && GRP == 0) {   // the reverse state has arrived at t = 0: dL/dS_0
 #pragma unroll
         for (int m = 0; m < 4; ++m)
@@ -369,13 +326,11 @@ __device__ __forceinline__ void bwd_consumer(const BwdArgs &a, unsigned char *sm
     }
     // gu: fold the four lane groups (different tokens, same channel), then the consumer groups
     gu_acc = sum_rows(gu_acc);
-    if (GRP == 1 && g == 0) gu_lds[(last_slot & 1) * kN + col] = gu_acc;
+    if (GRP == 1 && g == 0) gu_lds[col] = gu_acc;
     __threadfence_block();
     __syncthreads();
-    if (kMulti && GRP == 0 && prev_slot >= 0) deliver_gu();   // (a last pair of no chunks cannot happen: T >= 1)
-    if (GRP == 0 && g == 0 && !s_wild[last_slot])     // (the exact second pass writes gu itself)
-        store_gu(b, gu_acc + gu_lds[(last_slot & 1) * kN + col]);
-    if (kMulti && GRP == 0 && g == 0) reinterpret_cast<float *>(smem + BwdLds::kGuSum)[col] = gu_wg;
+    if (GRP == 0 && g == 0 && !*s_wild)     // (the exact second pass writes gu itself)
+        store1(reinterpret_cast<Tout *>(a.gu) + (int64_t)b * C + h * kN + col, gu_acc + gu_lds[col]);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -445,37 +400,28 @@ __device__ __forceinline__ void bwd_gv_chunk(GvState &st, const BwdArgs &a, cons
 // ------------------------------------------------------------------------------------------
 // Loader / producer: wave p <-> tile p of every chunk, lane = channel.
 // ------------------------------------------------------------------------------------------
-template <typename Tin, bool kRagged, bool kMulti>
+template <typename Tin, bool kRagged>
 __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *smem, int *s_wild, int pair0, int p, int lane)
 {
     const int T = a.T, H = a.H;
     const int ch = lane;
     const int64_t C = (int64_t)H * kN;
     const int nchunk = (T + CL - 1) / CL;
-    // kMulti: the workgroup's pairs (pair0, pair0 + gridDim.x, ...: same head, `bstep` batch rows apart)
-    // form one sequence of items; item = chunk visit: pair after pair, each from chunk n-1 down to 0
-    const int h = pair0 % H, b0 = pair0 / H, bstep = kMulti ? (int)gridDim.x / H : 0;
-    const int npw = kMulti ? (a.npairs - pair0 + (int)gridDim.x - 1) / (int)gridDim.x : 1;
-    const int nitem = nchunk * npw;
+    // item = chunk visit: from chunk n-1 down to 0
+    const int h = pair0 % H, b0 = pair0 / H;
+    const int nitem = nchunk;
     typedef typename OutOf<Tin>::type Tout;
     const float uc = load1(reinterpret_cast<const Tin *>(a.u) + h * kN + ch);
     const uint32_t rowbytes = (uint32_t)C * 2u;
     const uint32_t lds0 = lds_address(smem);
-    // Where an item is: which of the workgroup's pairs (slot) and which chunk of it.  Loads, operand
-    // preparation and the gv role each walk the item sequence with a cursor of their own.
-    // advance() says whether the cursor moved on to the next pair.
+    // Where an item is: which chunk.  Loads, operand preparation and the gv role each walk the item
+    // sequence with a cursor of their own.
     struct Cursor {
-        int c, slot;
-        __device__ __forceinline__ bool advance(int nchunk) {
-            if (kMulti && c == 0) { c = nchunk - 1; ++slot; return true; }
-            --c;
-            return false;
-        }
+        int c;
     };
-    // the rows of the pair a cursor is in (uniform pointers; moved by one pair's distance when it moves on)
-    const int64_t base0 = (int64_t)b0 * T * C + (int64_t)h * kN, pair_step = (int64_t)bstep * T * C;
+    // the rows of the pair
+    const int64_t base0 = (int64_t)b0 * T * C + (int64_t)h * kN;
     const bf16_t *rb = a.r + base0, *kb_ = a.k + base0, *vb = a.v + base0, *wb = a.w + base0, *gb = a.gy + base0;   // loads
-    const int64_t ck_step = (int64_t)bstep * H * nchunk * (kN * kN);
     const bf16_t *ckb = reinterpret_cast<const bf16_t *>(a.ckpt + (int64_t)(b0 * H + h) * nchunk * (kN * kN));      // state loads
     Tout *gvb = reinterpret_cast<Tout *>(a.gv) + base0;                                                            // gv role
     // this lane's part of an 8-row block load: row (lane >> 3), 16-byte piece swizzled with the row
@@ -571,7 +517,7 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
             pr[e] = fr[e] * uc * fk[e];
         }
         if (__builtin_amdgcn_ballot_w64(!(cs2 <= kWildLimit * kLog2e)) != 0ull) {
-            if (lane == 0) s_wild[cu.slot] = 1;
+            if (lane == 0) *s_wild = 1;
         }
 #pragma unroll
         for (int e = 0; e < 16; e += 2) {
@@ -601,13 +547,9 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
     // the ragged tail issues anything from 0 to 4 (a store whose lanes are all past the end is
     // skipped): counting none for it makes the waits behind it wait for everything older.
     auto gv_stores = [&](const Cursor &cu) { return (kRagged && cu.c == nchunk - 1) ? 0 : 4; };
-    Cursor cur_l = {nchunk - 1, 0}, cur_p = cur_l, cur_v = cur_l;   // items it+2 (loads), it+1 (state, preparation), it (gv)
-    auto next_load_item = [&]() {
-        if (cur_l.advance(nchunk)) { rb += pair_step; kb_ += pair_step; vb += pair_step; wb += pair_step; gb += pair_step; }
-    };
-    auto next_prepared_item = [&]() {
-        if (cur_p.advance(nchunk)) ckb += 2 * ck_step;   // (bf16 elements of a block counted in floats)
-    };
+    Cursor cur_l = {nchunk - 1}, cur_p = cur_l, cur_v = cur_l;   // items it+2 (loads), it+1 (state, preparation), it (gv)
+    auto next_load_item = [&]() { --cur_l.c; };
+    auto next_prepared_item = [&]() { --cur_p.c; };
     if (state_by_load(0)) issue_state(0, cur_p);
     issue_loads(0, cur_l);
     next_load_item();
@@ -635,7 +577,7 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
         gv_stores_before = gv_stores(cur_v);
         // the next item's state has to be in LDS when the consumers pass the barrier
         if (state_loads) wait_younger(younger + gv_stores_before);
-        if (cur_v.advance(nchunk)) { gvb += pair_step; gvst.init(nullptr, 0, 0); }   // a new pair: reverse state from zero
+        --cur_v.c;
     }
     wait_loads<0>();
     __threadfence_block();
@@ -646,32 +588,29 @@ __device__ __forceinline__ void bwd_producer(const BwdArgs &a, unsigned char *sm
 //   loader/producer + gv | consumer group 0 (tiles 3, 1) | consumer group 1 (tiles 2, 0)
 constexpr int kBwdWaves = 12;
 
-template <typename Tin, bool kRagged, bool kMulti>
+template <typename Tin, bool kRagged>
 __global__ __launch_bounds__(kBwdWaves * 64) void chunk_bwd_kernel(BwdArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
-    constexpr int kFlags = kMulti ? kBwdMaxPairs : 1;
-    __shared__ int s_wild[kFlags];   // per pair of this workgroup: a tile left the chunked form's range
+    __shared__ int s_wild[1];    // a tile of this workgroup's pair left the chunked form's range
     __shared__ float s_ft[kN];   // exact second pass with state gradients: the anchor of the gw sums
     static_assert(sizeof(ScanBwdALds) <= BwdLds::kBytes && sizeof(ScanBwdBLds) <= BwdLds::kBytes,
                   "the exact second pass reuses the LDS block");
-    if (threadIdx.x < kFlags) s_wild[threadIdx.x] = 0;
+    if (threadIdx.x == 0) s_wild[0] = 0;
     __syncthreads();
 
     const int pair0 = blockIdx.x;
-    const int npw = kMulti ? (a.npairs - pair0 + (int)gridDim.x - 1) / (int)gridDim.x : 1;   // pairs of this workgroup
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int role = wave >> 2, q = wave & 3;
     typedef typename OutOf<Tin>::type Tout;
-    if (role == 0) bwd_producer<Tin, kRagged, kMulti>(a, smem, s_wild, pair0, q, lane);
-    else if (role == 1) bwd_consumer<Tin, kRagged, kMulti, 0>(a, smem, s_wild, pair0, q, lane);
-    else bwd_consumer<Tin, kRagged, kMulti, 1>(a, smem, s_wild, pair0, q, lane);
+    if (role == 0) bwd_producer<Tin, kRagged>(a, smem, s_wild, pair0, q, lane);
+    else if (role == 1) bwd_consumer<Tin, kRagged, 0>(a, smem, s_wild, pair0, q, lane);
+    else bwd_consumer<Tin, kRagged, 1>(a, smem, s_wild, pair0, q, lane);
     // exact second pass for a (b, h) if any of its tiles left the representable range; the
     // pair's own slice of the state workspace (nchunk x 64 x 64 floats = T' x 64) holds P
-    for (int slot = 0; slot < npw; ++slot) {
-        if (!s_wild[slot]) continue;
-        const int pair = pair0 + slot * (int)gridDim.x, b = pair / a.H, h = pair % a.H;
+    if (s_wild[0]) {
+        const int b = pair0 / a.H, h = pair0 % a.H;
         const int nchunk = (a.T + CL - 1) / CL;
         float *ck = a.ckpt + (int64_t)(b * a.H + h) * nchunk * (kN * kN);
         const int64_t so = (int64_t)(b * a.H + h) * (kN * kN);
@@ -687,7 +626,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void chunk_bwd_kernel(BwdArgs a)
         __syncthreads();
         scan_bwd_b_body<Tin, Tout>(*reinterpret_cast<ScanBwdBLds *>(smem), b, h, a.T, a.H, in(a.r), in(a.k), in(a.v_orig), in(a.w), in(a.u), gyp, ck, kN,
                                    out(a.gk), out(a.gv), out(a.gw), gsTp, states ? s_ft : nullptr, a.gs0 ? a.gs0 + so : nullptr, a.s0 == nullptr);
-        __syncthreads();   // (the LDS block is free for the next pair's pass)
+        __syncthreads();
     }
     // Fused batch sum of gu (what the caller otherwise does with one more kernel): the workgroup that
     // is the last of its head to deliver adds up the B partials.  The partials travel as written-
@@ -695,23 +634,15 @@ __global__ __launch_bounds__(kBwdWaves * 64) void chunk_bwd_kernel(BwdArgs a)
     // completed before the arrival counter is bumped; no fence, which would write back the whole L2.
     if (a.gu_sum != nullptr) {
         __shared__ int s_last;
-        const int h = pair0 % a.H;   // (kMulti: the head of all pairs of this workgroup)
+        const int h = pair0 % a.H;
         const int nchunk = (a.T + CL - 1) / CL;
         const int64_t slice = (int64_t)nchunk * (kN * kN), C = (int64_t)a.H * kN;
-        // what adds up to the head's sum: one partial per batch row -- or, kMulti, one per workgroup of
-        // this head (its own pairs summed here first; it leaves the sum in the slice of its first pair)
-        // (workgroups h, h + H, h + 2H, ... below gridDim.x; their first pairs carry the same indices)
-        const int nparts = kMulti ? (int)gridDim.x / a.H : a.B;
+        const int nparts = a.B;   // what adds up to the head's sum: one partial per batch row
         __threadfence_block();   // this workgroup's gu rows (consumer group 0 or the second pass) are written
         __syncthreads();
         const int tid = threadIdx.x;
         if (tid < kN) {          // wave 0
-            // kMulti: the pairs done by the chunked code were summed by consumer group 0 as it stored them
-            // (LDS); only what an exact second pass wrote is read back
-            float part = kMulti ? reinterpret_cast<const float *>(smem + BwdLds::kGuSum)[tid] : 0.f;
-            for (int slot = 0; slot < npw; ++slot)
-                if (!kMulti || s_wild[slot])
-                    part += load1(reinterpret_cast<const Tout *>(a.gu) + (int64_t)((pair0 + slot * (int)gridDim.x) / a.H) * C + h * kN + tid);
+            const float part = load1(reinterpret_cast<const Tout *>(a.gu) + (int64_t)(pair0 / a.H) * C + h * kN + tid);
             __hip_atomic_store(a.ckpt + (int64_t)pair0 * slice + slice / 2 + tid, part, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             if (tid == 0)
@@ -769,34 +700,15 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
     a.gr = (bf16_t *)gr; a.gk = (bf16_t *)gk; a.gv = (bf16_t *)gv; a.gw = (bf16_t *)gw; a.gu = (bf16_t *)gu;
     a.ckpt = (float *)workspace;
     a.B = (int)B;
-    a.npairs = (int)(B * H);
     a.gu_sum = states_ready ? (bf16_t *)gu_sum : nullptr;
     a.arrivals = reinterpret_cast<int *>(reinterpret_cast<char *>(workspace) + chunk_backward_workspace_bytes(B, T, H));
-    // More pairs than compute units (and no gradients through the state): one workgroup per compute
-    // unit -- rounded down to a multiple of H, so that a workgroup's pairs share the head -- each
-    // taking its pairs back to back.
-    unsigned grid = (unsigned)(B * H);
-    bool multi = false;
-    {
-        const int64_t cus = compute_units(), pairs = B * H;
-        // (beyond 1024 tokens a pair's start-up no longer shows: B16 T2048 runs in the same time either way,
-        // B12 T4096 is 1 % faster with one workgroup per pair)
-        if (!s0 && !gsT && !gs0 && pairs > cus && H <= cus && T <= 16 * CL) {
-            // (more workgroups than that only where one would get more pairs than it keeps flags for)
-            const int64_t g = cus / H * H, per = (pairs + g - 1) / g;
-            multi = true;
-            grid = (unsigned)(g * ((per + kBwdMaxPairs - 1) / kBwdMaxPairs));
-        }
-    }
-    auto launch_as = [&](auto in_tag, auto ragged_tag, auto multi_tag) -> hipError_t {
-        constexpr auto kern = chunk_bwd_kernel<decltype(in_tag), decltype(ragged_tag)::value, decltype(multi_tag)::value>;
+    const unsigned grid = (unsigned)(B * H);
+    auto launch_in = [&](auto in_tag, auto ragged_tag) -> hipError_t {
+        constexpr auto kern = chunk_bwd_kernel<decltype(in_tag), decltype(ragged_tag)::value>;
         hipError_t e = allow_dynamic_lds<kern>((int)lds);
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3(grid), dim3(kBwdWaves * 64), lds, st, a);
         return hipGetLastError();
-    };
-    auto launch_in = [&](auto in_tag, auto ragged_tag) -> hipError_t {
-        return multi ? launch_as(in_tag, ragged_tag, std::true_type{}) : launch_as(in_tag, ragged_tag, std::false_type{});
     };
     auto launch = [&](auto ragged_tag) -> hipError_t {
         // fp16 tensors (fp32 gradients): only with saved states, v and gy as bf16 copies plus the originals
