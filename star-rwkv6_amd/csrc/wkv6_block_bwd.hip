@@ -537,7 +537,12 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
         ++cp.c;
         if (kMulti && cp.c == nchunk) { cp.c = 0; ++cp.slot; }
     };
-    constexpr int kRkwLoads = 6, kVgStateLoads = 6, kGvStores = 2;
+    constexpr int kRkwLoads = 6, kVgStateLoads = 6;
+    // gv stores a visit leaves in flight.  The chunk with the ragged end issues anything from 0 to 2 (a store
+    // whose lanes are all past the end is skipped): counting none for it makes the waits behind it wait for
+    // everything older, whereas counting one that was not issued would let them return early.
+    auto gv_stores = [&](int pos) { return (kRagged && pos == 0) ? 0 : 2; };   // pos: the visit's position in its pair
+    int gv_before = 0;   // of the visit before
     issue_vg_state();
     issue_rkw();
     if (nvisit > 1) issue_rkw();
@@ -549,12 +554,13 @@ __device__ __forceinline__ void block_bwd_producer(const BlockBwdArgs &a, unsign
         if (it + 1 < nvisit) issue_vg_state();
         if (it + 2 < nvisit) issue_rkw();
         // behind the r, k, w loads of visit it+1 (issued one visit ago): that visit's gv stores, and this visit's loads
-        if (it + 1 < nvisit) prepare((it > 0 ? kGvStores : 0) + vgs + rkw);
+        if (it + 1 < nvisit) prepare(gv_before + vgs + rkw);
         block_bwd_gv<kRagged>(smem, gvb, (uint32_t)C, T, nchunk - 1 - co.c, it, p, lane);
+        gv_before = gv_stores(co.c);
         ++co.c;
         if (kMulti && co.c == nchunk) { co.c = 0; ++co.slot; gvb = a.gv + pair_base(co.slot); }
         // v, gy and the state of the next visit have to be in LDS when the other waves pass the barrier
-        if (it + 1 < nvisit) wait_in_flight(rkw + kGvStores);
+        if (it + 1 < nvisit) wait_in_flight(rkw + gv_before);
     }
     wait_loads<0>();
     __threadfence_block();

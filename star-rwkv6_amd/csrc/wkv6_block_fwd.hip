@@ -255,7 +255,11 @@ __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsign
                 *reinterpret_cast<uint4 *>(ckb + ((uint32_t)co.c * (uint32_t)(kN * kN * 2) + (uint32_t)(row * kTileRow) + lpiece)) = s;
             }
         }
-        issued += kSave ? 4 : 2;
+        // (a store whose rows are all past the end is skipped: counting one that was not issued would let a later
+        // wait return early, so only those that certainly went out are counted)
+        issued += kSave ? 2 : 0;
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) issued += (!kRagged || co.c * kBlockTokens + 16 * p + 8 * blk < T) ? 1 : 0;
         ++co.it;
         if (++co.c == nchunk) {
             co.c = 0; ++co.slot;
