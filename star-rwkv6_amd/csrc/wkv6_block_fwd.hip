@@ -32,16 +32,21 @@
 
 namespace wkv6 {
 
-struct BlockFwdLds {
+// kFuse (the output stage in the kernel): the gate's rows come in like v, one visit before they are used, and v
+// is requested two visits ahead instead of three to make room for them.
+template <bool kFuse>
+struct BlockFwdLdsT {
+    static constexpr int kVAhead = kFuse ? 2 : 3;                        // visits between the request of v and its use
     static constexpr int kRaw = 0;                                       // [2 visit parities][r, k, w] raw tiles
-    static constexpr int kRawV = kRaw + 2 * 3 * kTileBytes;              // [visit & 3] raw v tiles
-    static constexpr int kOp = kRawV + 4 * kTileBytes;                   // [2][R~, K~]
+    static constexpr int kRawV = kRaw + 2 * 3 * kTileBytes;              // [visit % (kVAhead + 1)] raw v tiles
+    static constexpr int kOp = kRawV + (kVAhead + 1) * kTileBytes;       // [2][R~, K~]
     static constexpr int kVec = kOp + 2 * 2 * kTileBytes;                // [2] per-visit vectors
     static constexpr int kYStage = kVec + 2 * kBlockVecBytes;            // [2] y of one chunk, bf16 tile
     static constexpr int kSStage = kYStage + 2 * kTileBytes;             // [2] state at a chunk start, bf16 [i][j] tile
-    static constexpr int kBytes = kSStage + 2 * kTileBytes;
+    static constexpr int kGate = kSStage + 2 * kTileBytes;               // kFuse: [2] the gate's rows of one chunk
+    static constexpr int kBytes = kGate + (kFuse ? 2 * kTileBytes : 0);
 };
-static_assert(BlockFwdLds::kBytes <= 160 * 1024, "LDS block of the block-form forward kernel");
+static_assert(BlockFwdLdsT<false>::kBytes <= 160 * 1024 && BlockFwdLdsT<true>::kBytes <= 160 * 1024, "LDS block of the block-form forward kernel");
 
 struct BlockFwdArgs {
     int T, H, B;
@@ -53,13 +58,27 @@ struct BlockFwdArgs {
     void *sT;                // final state in Ts, or null
     float *ckpt;             // saved chunk states (bf16 [chunk][value][key] in the first half of each pair's slice), or null
     int *arrivals;           // with ckpt: per-head counters of the backward's fused gu sum, zeroed here
+    // fused output stage (kFuse): out = (layer_norm over the head's 64 channels of y * gn_scale + gn_offset) * gate
+    const bf16_t *gate;
+    const float *gn_scale, *gn_offset;   // (H, 64)
+    float gn_eps;
+    bf16_t *out;
+    float *stats;            // null, or (B, T, H, 2): mean and 1/sqrt(var + eps) per (token, head) for the backward
 };
+
+// sum over the 8 lanes that hold one 128-byte row (lanes 8k .. 8k+7), result in each of them
+__device__ __forceinline__ float sum_row8(float x) {
+    x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0xB1, 0xF, 0xF, true));    // quad_perm [1,0,3,2]
+    x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0x4E, 0xF, 0xF, true));    // quad_perm [2,3,0,1]
+    x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0x141, 0xF, 0xF, true));   // row_half_mirror
+    return x;
+}
 
 // ------------------------------------------------------------------------------------------
 // Consumer wave (q, HALF): value columns i = 16q + l16; y of block HALF (tokens 32 HALF .. +31).
 // State S[m]: rows j = block_row_channel(m, g) + rr, column i.
 // ------------------------------------------------------------------------------------------
-template <typename Ts, bool kSave, int HALF>
+template <typename Ts, bool kSave, bool kFuse, int HALF>
 __device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsigned char *smem, int pair0, int q, int lane)
 {
     const int T = a.T, H = a.H;
@@ -68,6 +87,7 @@ __device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsign
     const int b0 = pair0 / H, h = pair0 - b0 * H;
     const int npw = (a.B - b0 + a.bstep - 1) / a.bstep;   // pairs of this workgroup: batch rows b0, b0 + bstep, ...
     const int nvisit = npw * nchunk;
+    typedef BlockFwdLdsT<kFuse> BlockFwdLds;
     f32x4 S[4], Snext[4];
     // initial state of the workgroup's pair number `slot`, requested one visit before the pair begins
     auto request_state = [&](int slot) {
@@ -92,7 +112,7 @@ __device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsign
         const unsigned char *rt = smem + BlockFwdLds::kOp + (it & 1) * 2 * kTileBytes, *kt = rt + kTileBytes;
         const float *vec = reinterpret_cast<const float *>(smem + BlockFwdLds::kVec + (it & 1) * kBlockVecBytes);
         const float *ruk = vec + 4 * kN;
-        const unsigned char *vt = smem + BlockFwdLds::kRawV + (it & 3) * kTileBytes;
+        const unsigned char *vt = smem + BlockFwdLds::kRawV + (it % (BlockFwdLds::kVAhead + 1)) * kTileBytes;
         if (kSave && HALF == 0) {
             // the state at the chunk start, as the backward wants it: bf16, transposed ([i][j] rows of 128 bytes)
             unsigned char *ss = smem + BlockFwdLds::kSStage + (it & 1) * kTileBytes;
@@ -180,7 +200,7 @@ __device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsign
 // ------------------------------------------------------------------------------------------
 // Producer wave p: tokens 16p..16p+15 of every chunk.
 // ------------------------------------------------------------------------------------------
-template <bool kSave, bool kRagged>
+template <bool kSave, bool kRagged, bool kFuse>
 __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsigned char *smem, int *s_wild, int pair0, int p, int lane)
 {
     const int T = a.T, H = a.H;
@@ -192,6 +212,7 @@ __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsign
     const int nvisit = npw * nchunk;
     const uint32_t rowbytes = (uint32_t)C * 2u;
     const uint32_t lds0 = lds_address(smem);
+    typedef BlockFwdLdsT<kFuse> BlockFwdLds;
     // first element of the workgroup's pair number `slot` in a (B,T,C) tensor
     auto pair_base = [&](int slot) { return (int64_t)(b0 + slot * a.bstep) * T * C + (int64_t)h * kN; };
     // this lane's part of an 8-row block: row (lane >> 3), 16-byte piece swizzled with the row
@@ -206,14 +227,23 @@ __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsign
     };
     Cursor cv, cr, co, cp;   // v loads, r/k/w loads, stores of staged rows, operand preparation
     const bf16_t *vb = a.v + pair_base(0), *rb = a.r + pair_base(0), *kb_ = a.k + pair_base(0), *wb = a.w + pair_base(0);
-    bf16_t *yb = a.y + pair_base(0);
+    bf16_t *yb = (kFuse ? a.out : a.y) + pair_base(0);   // (kFuse: the rows that leave are those of `out`)
+    bf16_t *y2b = kFuse && a.y ? a.y + pair_base(0) : nullptr;   // kFuse, training: y as well
+    const bf16_t *gtb = kFuse ? a.gate + pair_base(0) : nullptr;
+    // kFuse: scale and offset of the eight channels this lane holds of a row (the row's piece (lane & 7) ^ lrow),
+    float gsc[8], gof[8];
+    if (kFuse) {
+        const float *sp = a.gn_scale + h * kN + (lpiece >> 1), *op_ = a.gn_offset + h * kN + (lpiece >> 1);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { gsc[i] = sp[i]; gof[i] = op_[i]; }
+    }
     char *ckb = kSave ? reinterpret_cast<char *>(a.ckpt + (int64_t)(b0 * H + h) * nchunk * (kN * kN)) : nullptr;
     // Vector-memory operations this wave has issued so far, and the count right after the r, k, w loads
     // of visit j went out: a wave's operations complete in program order, so "the loads of visit j have
     // landed" is "at most (issued - mark of j) operations are still in flight".
-    int issued = 0, mark_even = 0, mark_odd = 0;
+    int issued = 0, mark_even = 0, mark_odd = 0, mark_gate_even = 0, mark_gate_odd = 0;
     auto issue_v = [&]() {   // the next visit's v
-        const uint32_t vv = lds0 + BlockFwdLds::kRawV + (cv.it & 3) * kTileBytes + 16 * p * kTileRow;
+        const uint32_t vv = lds0 + BlockFwdLds::kRawV + (cv.it % (BlockFwdLds::kVAhead + 1)) * kTileBytes + 16 * p * kTileRow;
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk)
             load_rows8_to_lds(vb, row_offset(cv.c * kBlockTokens + 16 * p + 8 * blk + lrow), vv + 8 * blk * kTileRow);
@@ -241,15 +271,47 @@ __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsign
     };
     // what the consumers staged during the next visit in line, as whole rows: y rows of this wave's tokens
     // and rows 16p..16p+15 of the chunk's state
+    Cursor cg;   // kFuse: the gate's rows of a visit are requested when the visit begins and used one visit later
+    auto issue_gate = [&]() {
+        const uint32_t gg = lds0 + BlockFwdLds::kGate + (cg.it & 1) * kTileBytes + 16 * p * kTileRow;
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+            load_rows8_to_lds(gtb, row_offset(cg.c * kBlockTokens + 16 * p + 8 * blk + lrow), gg + 8 * blk * kTileRow);
+        issued += 2;
+        if (cg.it & 1) mark_gate_odd = issued; else mark_gate_even = issued;
+        ++cg.it;
+        if (++cg.c == nchunk) { cg.c = 0; ++cg.slot; gtb = a.gate + pair_base(cg.slot); }
+    };
     auto store_staged = [&]() {
         const unsigned char *ys = smem + BlockFwdLds::kYStage + (co.it & 1) * kTileBytes;
         const unsigned char *ss = smem + BlockFwdLds::kSStage + (co.it & 1) * kTileBytes;
+        const unsigned char *gs = smem + BlockFwdLds::kGate + (co.it & 1) * kTileBytes;
+        if (kFuse) wait_in_flight(issued - ((co.it & 1) ? mark_gate_odd : mark_gate_even));   // the visit's gate rows have landed
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
-            const int row = 16 * p + 8 * blk + lrow;
-            const uint4 x = *reinterpret_cast<const uint4 *>(ys + row * kTileRow + (lane & 7) * 16);
-            if (!kRagged || co.c * kBlockTokens + row < T)
-                *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(yb) + ((uint32_t)(co.c * kBlockTokens + row) * rowbytes + lpiece)) = x;
+            const int row = 16 * p + 8 * blk + lrow, tok = co.c * kBlockTokens + row;
+            const uint32_t o = (uint32_t)tok * rowbytes + lpiece;
+            uint4 x = *reinterpret_cast<const uint4 *>(ys + row * kTileRow + (lane & 7) * 16);
+            if (kFuse) {
+                // the head's 64 channels of a token sit in eight neighbouring lanes: mean, variance (two passes, as
+                // the unfused norm does it), scale, offset, gate
+                if (y2b && (!kRagged || tok < T)) *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(y2b) + o) = x;
+                float f[8], gt[8];
+                const uint4 gx = *reinterpret_cast<const uint4 *>(gs + row * kTileRow + (lane & 7) * 16);
+                unpack8(make_bf16x8(x.x, x.y, x.z, x.w), f);
+                unpack8(make_bf16x8(gx.x, gx.y, gx.z, gx.w), gt);
+                const float mean = sum_row8(((f[0] + f[1]) + (f[2] + f[3])) + ((f[4] + f[5]) + (f[6] + f[7]))) * (1.f / kN);
+                float sq = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) { f[i] -= mean; sq = fmaf(f[i], f[i], sq); }
+                const float rstd = __builtin_amdgcn_rsqf(sum_row8(sq) * (1.f / kN) + a.gn_eps);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) f[i] = fmaf(f[i] * rstd, gsc[i], gof[i]) * gt[i];
+                x = make_uint4(pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]), pack_bf16x2(f[6], f[7]));
+                if (a.stats && (lane & 7) == 0 && (!kRagged || tok < T))
+                    *reinterpret_cast<float2 *>(a.stats + (((int64_t)(b0 + co.slot * a.bstep) * T + tok) * H + h) * 2) = make_float2(mean, rstd);
+            }
+            if (!kRagged || tok < T) *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(yb) + o) = x;
             if (kSave) {
                 const uint4 s = *reinterpret_cast<const uint4 *>(ss + row * kTileRow + (lane & 7) * 16);
                 *reinterpret_cast<uint4 *>(ckb + ((uint32_t)co.c * (uint32_t)(kN * kN * 2) + (uint32_t)(row * kTileRow) + lpiece)) = s;
@@ -259,11 +321,15 @@ __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsign
         // wait return early, so only those that certainly went out are counted)
         issued += kSave ? 2 : 0;
 #pragma unroll
-        for (int blk = 0; blk < 2; ++blk) issued += (!kRagged || co.c * kBlockTokens + 16 * p + 8 * blk < T) ? 1 : 0;
+        for (int blk = 0; blk < 2; ++blk) {
+            const int rows_here = (!kRagged || co.c * kBlockTokens + 16 * p + 8 * blk < T) ? 1 : 0;
+            issued += rows_here * (1 + (kFuse && y2b ? 1 : 0) + (kFuse && a.stats ? 1 : 0));
+        }
         ++co.it;
         if (++co.c == nchunk) {
             co.c = 0; ++co.slot;
-            yb = a.y + pair_base(co.slot);
+            yb = (kFuse ? a.out : a.y) + pair_base(co.slot);
+            if (kFuse && y2b) y2b = a.y + pair_base(co.slot);
             if (kSave) ckb = reinterpret_cast<char *>(a.ckpt + (int64_t)((b0 + co.slot * a.bstep) * H + h) * nchunk * (kN * kN));
         }
     };
@@ -292,16 +358,18 @@ __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsign
         ++cp.it;
         if (++cp.c == nchunk) { cp.c = 0; ++cp.slot; }
     };
-    // r, k, w of visit j are requested three visits ahead (two in the prologue), v three visits ahead
+    // r, k, w of visit j are requested three visits ahead (two in the prologue), v kVAhead visits ahead
+    constexpr int kVAhead = BlockFwdLds::kVAhead;
     issue_v();
     issue_rkw();
     if (nvisit > 1) { issue_v(); issue_rkw(); }
-    if (nvisit > 2) issue_v();
+    if (kVAhead > 2 && nvisit > 2) issue_v();
     prepare(nvisit > 2);
     for (int it = 0; it < nvisit; ++it) {
         __syncthreads();
         // free again: the raw v block of visit it-1; the staging tiles of visit it-1 are complete
-        if (it + 3 < nvisit) issue_v();
+        if (it + kVAhead < nvisit) issue_v();
+        if (kFuse) issue_gate();
         if (it > 0) store_staged();
         if (it + 1 < nvisit) prepare(it + 3 < nvisit);
     }
@@ -312,21 +380,43 @@ __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsign
 
 constexpr int kBlockFwdThreads = 12 * 64;
 
-template <typename Ts, bool kSave, bool kRagged>
+// the exact second pass leaves y in `out`; this turns one pair's rows into the fused output in place (a wave per
+// token, lane = channel)
+__device__ __forceinline__ void block_output_stage_in_place(const BlockFwdArgs &a, int b, int h) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwave = blockDim.x >> 6;
+    const int64_t C = (int64_t)a.H * kN, first = (int64_t)b * a.T * C + (int64_t)h * kN + lane;
+    const float gsc = a.gn_scale[h * kN + lane], gof = a.gn_offset[h * kN + lane];
+    for (int t = wave; t < a.T; t += nwave) {
+        const float y = load1(a.out + first + (int64_t)t * C);
+        if (a.y) store1(a.y + first + (int64_t)t * C, y);
+        float sum = y;
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) sum += __shfl_xor(sum, m);
+        const float d = y - sum * (1.f / kN);
+        float sq = d * d;
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) sq += __shfl_xor(sq, m);
+        const float rstd = __builtin_amdgcn_rsqf(sq * (1.f / kN) + a.gn_eps);
+        if (a.stats && lane == 0) *reinterpret_cast<float2 *>(a.stats + (((int64_t)b * a.T + t) * a.H + h) * 2) = make_float2(sum * (1.f / kN), rstd);
+        store1(a.out + first + (int64_t)t * C, fmaf(d * rstd, gsc, gof) * load1(a.gate + first + (int64_t)t * C));
+    }
+}
+
+template <typename Ts, bool kSave, bool kRagged, bool kFuse>
 __global__ __launch_bounds__(kBlockFwdThreads) void block_fwd_kernel(BlockFwdArgs a)
 {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_wild[kBlockMaxSlots];   // per pair of the workgroup: 16 tokens left the scaled operands' range
-    static_assert(sizeof(ScanFwdLds) <= BlockFwdLds::kBytes, "the exact second pass reuses the LDS block");
+    static_assert(sizeof(ScanFwdLds) <= BlockFwdLdsT<kFuse>::kBytes, "the exact second pass reuses the LDS block");
     if (threadIdx.x < kBlockMaxSlots) s_wild[threadIdx.x] = 0;
     __syncthreads();
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int pair0 = (int)blockIdx.x;
-    if (wave < 4) block_fwd_producer<kSave, kRagged>(a, smem, s_wild, pair0, wave, lane);
-    else if (wave < 8) block_fwd_consumer<Ts, kSave, 0>(a, smem, pair0, wave - 4, lane);
-    else block_fwd_consumer<Ts, kSave, 1>(a, smem, pair0, wave - 8, lane);
+    if (wave < 4) block_fwd_producer<kSave, kRagged, kFuse>(a, smem, s_wild, pair0, wave, lane);
+    else if (wave < 8) block_fwd_consumer<Ts, kSave, kFuse, 0>(a, smem, pair0, wave - 4, lane);
+    else block_fwd_consumer<Ts, kSave, kFuse, 1>(a, smem, pair0, wave - 8, lane);
     // exact second pass for the pairs of which 16 tokens left the range the scaled operands can hold
     __threadfence_block();
     __syncthreads();
@@ -336,7 +426,12 @@ __global__ __launch_bounds__(kBlockFwdThreads) void block_fwd_kernel(BlockFwdArg
         if (!s_wild[slot]) continue;   // (uniform over the workgroup)
         __syncthreads();
         scan_fwd_body<bf16_t, bf16_t, Ts>(*reinterpret_cast<ScanFwdLds *>(smem), b0 + slot * a.bstep, h, a.T, a.H, a.r, a.k, a.v, a.w, a.u,
-                                          reinterpret_cast<const Ts *>(a.s0), a.map, a.y, reinterpret_cast<Ts *>(a.sT), false);
+                                          reinterpret_cast<const Ts *>(a.s0), a.map, kFuse ? a.out : a.y, reinterpret_cast<Ts *>(a.sT), false);
+        if (kFuse) {
+            __threadfence_block();
+            __syncthreads();
+            block_output_stage_in_place(a, b0 + slot * a.bstep, h);
+        }
     }
 }
 
@@ -358,9 +453,11 @@ bool block_forward_applies(int64_t B, int64_t T, int64_t H) {
     return 2 * pairs > cus && block_grid(B, H) > 0 && T * H * kN < (1LL << 31);
 }
 
-hipError_t block_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
-                         const void *r, const void *k, const void *v, const void *w, const void *u,
-                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states, bool counters)
+// gate != null: the fused output stage (out = (group norm of y) * gate; y and stats only where given)
+static hipError_t block_forward_launch(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
+                                       const void *r, const void *k, const void *v, const void *w, const void *u,
+                                       const void *s0, const int64_t *map, void *y, void *sT, void *saved_states, bool counters,
+                                       const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps, void *out, float *stats)
 {
     BlockFwdArgs a = {};
     a.T = (int)T; a.H = (int)H; a.B = (int)B;
@@ -369,19 +466,43 @@ hipError_t block_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
     a.s0 = s0; a.map = map; a.y = (bf16_t *)y; a.sT = sT; a.ckpt = (float *)saved_states;
     a.arrivals = saved_states && counters ? reinterpret_cast<int *>(reinterpret_cast<char *>(saved_states) + chunk_backward_workspace_bytes(B, T, H)) : nullptr;
-    auto launch = [&](auto ts_tag, auto save_tag, auto ragged_tag) -> hipError_t {
-        constexpr auto kern = block_fwd_kernel<decltype(ts_tag), decltype(save_tag)::value, decltype(ragged_tag)::value>;
-        hipError_t e = allow_dynamic_lds<kern>(BlockFwdLds::kBytes);
+    a.gate = (const bf16_t *)gate; a.gn_scale = gn_scale; a.gn_offset = gn_offset; a.gn_eps = gn_eps; a.out = (bf16_t *)out; a.stats = stats;
+    auto launch = [&](auto ts_tag, auto save_tag, auto ragged_tag, auto fuse_tag) -> hipError_t {
+        constexpr bool kFuse = decltype(fuse_tag)::value;
+        constexpr auto kern = block_fwd_kernel<decltype(ts_tag), decltype(save_tag)::value, decltype(ragged_tag)::value, kFuse>;
+        hipError_t e = allow_dynamic_lds<kern>(BlockFwdLdsT<kFuse>::kBytes);
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kBlockFwdThreads), BlockFwdLds::kBytes, st, a);
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(kBlockFwdThreads), BlockFwdLdsT<kFuse>::kBytes, st, a);
         return hipGetLastError();
     };
-    auto launch_ts = [&](auto ts_tag, auto save_tag) -> hipError_t {
-        return (T % kBlockTokens) != 0 ? launch(ts_tag, save_tag, std::true_type{}) : launch(ts_tag, save_tag, std::false_type{});
+    auto launch_ts = [&](auto ts_tag, auto save_tag, auto fuse_tag) -> hipError_t {
+        return (T % kBlockTokens) != 0 ? launch(ts_tag, save_tag, std::true_type{}, fuse_tag) : launch(ts_tag, save_tag, std::false_type{}, fuse_tag);
     };
     const bool save = saved_states != nullptr;
-    if (state_dtype == kF32) return save ? launch_ts(float{}, std::true_type{}) : launch_ts(float{}, std::false_type{});
-    return save ? launch_ts(bf16_t{}, std::true_type{}) : launch_ts(bf16_t{}, std::false_type{});
+    if (gate != nullptr) {
+        // (the saving variant is the training one: zero initial state, no final state; its state type is immaterial)
+        if (save) return launch_ts(float{}, std::true_type{}, std::true_type{});
+        return state_dtype == kF32 ? launch_ts(float{}, std::false_type{}, std::true_type{}) : launch_ts(bf16_t{}, std::false_type{}, std::true_type{});
+    }
+    if (state_dtype == kF32) return save ? launch_ts(float{}, std::true_type{}, std::false_type{}) : launch_ts(float{}, std::false_type{}, std::false_type{});
+    return save ? launch_ts(bf16_t{}, std::true_type{}, std::false_type{}) : launch_ts(bf16_t{}, std::false_type{}, std::false_type{});
+}
+
+hipError_t block_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
+                         const void *r, const void *k, const void *v, const void *w, const void *u,
+                         const void *s0, const int64_t *map, void *y, void *sT, void *saved_states, bool counters)
+{
+    return block_forward_launch(st, state_dtype, B, T, H, r, k, v, w, u, s0, map, y, sT, saved_states, counters,
+                                nullptr, nullptr, nullptr, 0.f, nullptr, nullptr);
+}
+
+hipError_t block_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
+                               const void *r, const void *k, const void *v, const void *w, const void *u,
+                               const void *s0, const int64_t *map, const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
+                               void *out, void *y, float *stats, void *sT, void *saved_states)
+{
+    return block_forward_launch(st, state_dtype, B, T, H, r, k, v, w, u, s0, map, y, sT, saved_states, saved_states != nullptr,
+                                gate, gn_scale, gn_offset, gn_eps, out, stats);
 }
 
 }  // namespace wkv6

@@ -671,6 +671,8 @@ hipError_t chunk_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64
                                const void *s0, const int64_t *map, const void *gate, const float *gn_scale,
                                const float *gn_offset, float gn_eps, void *out, void *sT)
 {
+    if (block_forward_applies(B, T, H))
+        return block_forward_fused(st, state_dtype, B, T, H, r, k, v, w, u, s0, map, gate, gn_scale, gn_offset, gn_eps, out, nullptr, nullptr, sT, nullptr);
     FwdArgs a = {};
     a.T = (int)T; a.H = (int)H; a.nitems = (int)(B * H);
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
@@ -692,6 +694,8 @@ hipError_t chunk_forward_fused_save(hipStream_t st, int64_t B, int64_t T, int64_
                                     const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
                                     void *out, void *y, float *stats, void *saved_states)
 {
+    if (block_forward_applies(B, T, H))
+        return block_forward_fused(st, kF32, B, T, H, r, k, v, w, u, nullptr, nullptr, gate, gn_scale, gn_offset, gn_eps, out, y, stats, nullptr, saved_states);
     FwdArgs a = {};
     a.T = (int)T; a.H = (int)H; a.nitems = (int)(B * H);
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;

@@ -69,6 +69,12 @@ hipError_t block_forward(hipStream_t st, int state_dtype, int64_t B, int64_t T, 
                          const void *r, const void *k, const void *v, const void *w, const void *u,
                          const void *s0, const int64_t *map, void *y, void *sT, void *saved_states, bool counters);
 
+// the block-form forward with the layer's output stage fused in (see chunk_forward_fused / chunk_forward_fused_save):
+// y and stats may be null (inference), saved_states null without a backward to follow
+hipError_t block_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64_t T, int64_t H,
+                               const void *r, const void *k, const void *v, const void *w, const void *u,
+                               const void *s0, const int64_t *map, const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
+                               void *out, void *y, float *stats, void *sT, void *saved_states);
 bool block_backward_applies(int64_t B, int64_t T, int64_t H);
 // workspace: the chunk-start states as a forward pass leaves them, followed by the per-head counters; gu_sum may be null
 hipError_t block_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,

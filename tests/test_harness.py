@@ -202,10 +202,10 @@ def test_config4_full_size_train_step(oracle):
     every gradient are finite, and what one mid-stack layer's fused output-stage call saw -- r, k, v,
     w, u, gate coming in, the gradient of its output arriving -- reproduces that call's output and
     its eight gradients against float64 (the oracle's operator, torch's layer_norm autograd), all
-    batch rows, at the tolerance of the fused stage's own parity test."""
+    batch rows, at the tolerance and with the conditioning of the fused stage's own parity test."""
     import collections
     import numpy as np
-    from _util import check_composite, fused_stage_reference, to_np
+    from _util import check_composite, flat_heads, fused_stage_reference, to_np
     from rwkv_kernel import RWKVKernelOperator
 
     dev = torch.device("cuda:0")
@@ -249,6 +249,14 @@ def test_config4_full_size_train_step(oracle):
             out, s = op.forward_gn_gate(r, k, v, w, u, gate, scale, offset, eps)
             if mine:
                 rec["out"] = out.detach()
+                # As in the fused stage's own parity test, the gradient arriving at this one call is zeroed on the
+                # (token, head) groups where the norm is ill-conditioned (a head's standard deviation below 5 % of
+                # the median: 1/std magnifies the bf16 rounding of y itself there, whatever computes the gradient);
+                # the step goes on with that gradient.
+                rec["y_ref"], _ = oracle.forward_c(*[to_np(x) for x in (r, k, v, w, u)], N)
+                keep = torch.tensor(~flat_heads(rec["y_ref"], N), device=out.device).view(B, T, H, 1).expand(B, T, H, N).reshape(B, T, H * N)
+                rec["flat"] = int((~keep).sum()) // N
+                out.register_hook(lambda g: g * keep.to(g.dtype))
                 out.register_hook(lambda g: rec.__setitem__("gout", g.detach().clone()))
             return out, s
 
@@ -269,7 +277,8 @@ def test_config4_full_size_train_step(oracle):
     assert rec["r"].dtype == torch.bfloat16 and tuple(rec["r"].shape) == (B, T, H * N) and "gout" in rec
 
     ins = [to_np(rec[n]) for n in "rkvw"] + [to_np(rec["u"])]
-    want = fused_stage_reference(oracle, ins, to_np(rec["gate"]), to_np(rec["gout"]), to_np(rec["scale"]), to_np(rec["offset"]), N, rec["eps"])
+    print("ill-conditioned (token, head) groups of the recorded call: %d of %d" % (rec["flat"], B * T * H), flush=True)
+    want = fused_stage_reference(oracle, ins, to_np(rec["gate"]), to_np(rec["gout"]), to_np(rec["scale"]), to_np(rec["offset"]), N, rec["eps"], rec["y_ref"])
     check_composite("out", rec["out"], want["out"])
     check_composite("ggate", rec["gate"].grad, want["ggate"])
     check_composite("gscale", rec["scale_param"].grad, want["gscale"])
