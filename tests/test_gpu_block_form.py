@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from _util import cast_inputs, check_close, to_np
+from _util import cast_inputs, check_close, check_composite, to_np
 
 pytestmark = pytest.mark.gpu
 BF16 = torch.bfloat16
@@ -167,6 +167,33 @@ def test_block_form_chunks_continue_each_other(op, oracle):
     y_ref, s_ref = oracle.forward_c(*ref, N)
     check_close("y", torch.cat([ya, yb], 1), y_ref, BF16)
     check_close("sT", sb, s_ref, BF16)
+
+
+# The output stage (group norm over a head's channels, scale, offset, gate) fused into the block-form forward.
+# (B, T, H, state): one pair per workgroup, a ragged end, several pairs per workgroup, one visit per pair
+@pytest.mark.parametrize("B,T,H,with_state", [(5, 256, 32, True), (5, 250, 32, False), (40, 128, 32, True), (300, 64, 1, False),
+                                              (13, 100, 40, True)])
+def test_block_form_fused_output_stage(op, oracle, B, T, H, with_state):
+    assert _pairs_in_range(B, H) or _several_pairs_per_workgroup(B, H)
+    ins = oracle.make_inputs(B, T, H, N, 170 + T, with_state=True)
+    if T >= 128:
+        ins[3][B - 1, 40:60, 0:64] = 6.0     # one pair is redone exactly and then normalised in place
+    dev, ref = cast_inputs(ins[:5], BF16)
+    g = torch.Generator().manual_seed(T)
+    gate_dev, gate_ref = cast_inputs([torch.randn(B, T, H * N, generator=g)], BF16)
+    scale = torch.rand(H, N, generator=g) + 0.5
+    offset = torch.randn(H, N, generator=g) * 0.3
+    s0 = ins[6].float() if with_state else None
+    op.algo = CHUNK
+    out, sT = op.forward_gn_gate(*dev, gate_dev[0], scale.cuda(), offset.cuda(), 64e-5, return_state=True,
+                                 init_state=s0.cuda() if with_state else None)
+    torch.cuda.synchronize()
+    y_ref, sT_ref = oracle.forward_c(*ref, N, to_np(s0) if with_state else None)
+    want = oracle.group_norm_gate_np(y_ref, gate_ref[0], scale.numpy(), offset.numpy(), N, 64e-5)
+    # (the norm divides by a head's standard deviation and so magnifies y's own rounding where that is small:
+    # the stage's output is held to the composite bound, 1e-2 in the l2 norm and 3e-2 element-wise)
+    check_composite("out", out, want)
+    check_close("sT", sT, sT_ref, BF16)
 
 
 def test_either_forward_feeds_either_backward(oracle):
