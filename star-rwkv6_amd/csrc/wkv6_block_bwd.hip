@@ -1,8 +1,9 @@
 // WKV6 backward in block form for gfx950 (bf16 MFMA, fp32 states).  Same cases as the block-form
-// forward (wkv6_block_fwd.hip: bf16 tensors, T a multiple of 64, between half a pair and one (batch,
-// head) pair per compute unit, no gradients through the state); the tile form in wkv6_chunk_bwd.hip
-// serves every other case.  The forward state at every chunk start comes from the workspace (bf16,
-// transposed: [chunk][i][j]).  Notation and the operand scaling are in wkv6_block.h.
+// forward (wkv6_block_fwd.hip: bf16 tensors, more than half a (batch, head) pair per compute unit;
+// kMulti: several pairs per workgroup, one after the other through one pipeline; kRagged: a sequence
+// length that is no multiple of 64), without gradients through the state; the tile form in
+// wkv6_chunk_bwd.hip serves every other case.  The forward state at every chunk start comes from the
+// workspace (bf16, transposed: [chunk][i][j]).  Notation and the operand scaling are in wkv6_block.h.
 //
 // Per block of 32 tokens (t, s local; G = reverse state arriving at the block's END from the future,
 // rows j; S = forward state at the block's start; alpha, g1, g2 of the block):
@@ -21,11 +22,13 @@
 //   Four producer waves (wave p <-> tokens 16p..16p+15): bring the raw r, k, w, v, gy rows of a chunk
 //       straight into LDS two visits ahead and the chunk's saved state one visit ahead; one visit
 //       ahead turn r, k, w into R~, K~ (over the raw r, k), exp(w) (over the raw w), alpha, g1, g2 and
-//       the diagonal; then run the gv role (wave q <-> value columns 16q..: its own copy of G, rows j).
+//       the diagonal; then run the gv role (wave q <-> value columns 16q..), which takes g2 o G of each
+//       block from LDS, where the other waves publish it as ready MFMA operands.
 //   Eight waves (q, half) <-> key channels 16q..16q+15, block `half` of the visit: X, W and the
 //       elementwise pass (gr, gk, gw, gu), products formed transposed (a lane holds four neighbouring
-//       channels of one token).  Each carries a copy of G with rows i through both blocks; the wave of
-//       the later block also steps the saved state over the earlier block to get its S.
+//       channels of one token; two 16-token row groups are paired through a lane-row swap so that every
+//       gradient leaves as 16-byte stores).  Each carries a copy of G with rows i through both blocks; the
+//       wave of the later block also steps the saved state over the earlier block to get its S.
 #include "wkv6_mfma.h"
 #include "wkv6_kernels.h"
 #include "wkv6_scan_body.h"
