@@ -61,6 +61,10 @@ struct BlockBwdArgs {
     bf16_t *gu_sum;   // null, or C elements: receives the sum of gu over the batch
     int *arrivals;    // per head: workgroups that have delivered their gu partial (zero on entry)
     float *ckpt;
+    // gradients through the state (all null for the stateless operator, and with several pairs per workgroup):
+    // fp32 (B,H,64,64) [key][value]
+    const float *s0, *gsT;   // initial state (the saved chunk states start from it); gradient arriving at the final state
+    float *gs0;              // receives dL/dS_0
 };
 
 // inclusive prefix over the 16 lanes of a row (tokens), per lane value
@@ -101,8 +105,18 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
     const int64_t base0 = (int64_t)b0 * T * C + (int64_t)h * kN;
     char *gr_h = reinterpret_cast<char *>(a.gr + base0), *gk_h = reinterpret_cast<char *>(a.gk + base0), *gw_h = reinterpret_cast<char *>(a.gw + base0);
     f32x4 Gj[4];
+    // the reverse state a pair starts from: zero, or the gradient arriving at its final state ([key j][value i])
+    const float *const gsT = kMulti ? nullptr : a.gsT;   // (state gradients: one pair per workgroup only)
+    float *const gs0 = kMulti ? nullptr : a.gs0;
+    const bool has_s0 = !kMulti && a.s0 != nullptr;
+    auto start_G = [&](int slot_) {
 #pragma unroll
-    for (int m = 0; m < 4; ++m) Gj[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int m = 0; m < 4; ++m) {
+            Gj[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            if (gsT) Gj[m] = *reinterpret_cast<const f32x4 *>(gsT + (int64_t)((b0 + slot_ * a.bstep) * H + h) * (kN * kN) + col * kN + block_row_channel(m, g));
+        }
+    };
+    start_G(0);
     float u4[4];
     load4(a.u + h * kN + 16 * q + 4 * g, u4);   // u of this lane's four channels 16q + 4g + rr
     float gu_acc[4] = {0.f, 0.f, 0.f, 0.f};
@@ -140,8 +154,7 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
         if (kMulti && cv == 0 && slot > 0) {   // a new pair: its rows, the reverse state from zero
             const int64_t base = (int64_t)(b0 + slot * a.bstep) * T * C + (int64_t)h * kN;
             gr_h = reinterpret_cast<char *>(a.gr + base); gk_h = reinterpret_cast<char *>(a.gk + base); gw_h = reinterpret_cast<char *>(a.gw + base);
-#pragma unroll
-            for (int m = 0; m < 4; ++m) Gj[m] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            start_G(slot);
             pend = 1.f;
             gu_acc[0] = gu_acc[1] = gu_acc[2] = gu_acc[3] = 0.f;
         }
@@ -340,8 +353,9 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
             }
             // the gradient of the first and the last decay of the sequence is zero by definition (the flow
             // balance leaves rounding residue there)
-            if ((HALF == 0 && n == 0 && c == 0 && l16 == 0) ||
-                (kRagged ? c * kBlockTokens + (n == 0 ? R0 : R1) + l16 == T - 1 : (HALF == 1 && n == 1 && c == nchunk - 1 && l16 == 15))) {
+            // (with an initial state / a gradient arriving at the final state they are not zero)
+            if ((HALF == 0 && n == 0 && c == 0 && l16 == 0 && !has_s0) ||
+                ((kRagged ? c * kBlockTokens + (n == 0 ? R0 : R1) + l16 == T - 1 : (HALF == 1 && n == 1 && c == nchunk - 1 && l16 == 15)) && !gsT)) {
                 gwo[0] = gwo[1] = gwo[2] = gwo[3] = 0.f;
             }
             packed[0][n][0] = pack_bf16x2(gro[0], gro[1]); packed[0][n][1] = pack_bf16x2(gro[2], gro[3]);
@@ -363,7 +377,14 @@ __device__ __forceinline__ void block_bwd_xw(const BlockBwdArgs &a, unsigned cha
         }
         __builtin_amdgcn_sched_barrier(0);
         if (++cv == nchunk) {
-            // the pair is done.  gu: fold the 16 tokens of a row; lanes l16 = 0 hold channels 16q + 4g + rr
+            // the pair is done.  The reverse state has arrived at t = 0: dL/dS_0 (both halves hold it)
+            if (gs0 && HALF == 0) {
+#pragma unroll
+                for (int m = 0; m < 4; ++m)
+                    *reinterpret_cast<f32x4 *>(gs0 + (int64_t)((b0 + slot * a.bstep) * H + h) * (kN * kN) + col * kN + block_row_channel(m, g)) =
+                        (f32x4){Gj[m][0] * pend, Gj[m][1] * pend, Gj[m][2] * pend, Gj[m][3] * pend};
+            }
+            // gu: fold the 16 tokens of a row; lanes l16 = 0 hold channels 16q + 4g + rr
 #pragma unroll
             for (int rr = 0; rr < 4; ++rr) gu_acc[rr] = sum_row16(gu_acc[rr]);
             if (l16 == 0) *reinterpret_cast<float4 *>(&gu_lds[((slot & 1) * 2 + HALF) * kN + 16 * q + 4 * g]) = make_float4(gu_acc[0], gu_acc[1], gu_acc[2], gu_acc[3]);
@@ -577,6 +598,7 @@ __global__ __launch_bounds__(kBlockBwdThreads) void block_bwd_kernel(BlockBwdArg
 {
     extern __shared__ __align__(16) unsigned char smem[];
     __shared__ int s_wild[kBlockMaxSlots];   // per pair of the workgroup: 16 tokens left the scaled operands' range
+    __shared__ float s_ft[kN];               // exact second pass with state gradients: the anchor of the gw sums
     static_assert(sizeof(ScanBwdALds) <= BlockBwdLds::kBytes && sizeof(ScanBwdBLds) <= BlockBwdLds::kBytes,
                   "the exact second pass reuses the LDS block");
     if (threadIdx.x < kBlockMaxSlots) s_wild[threadIdx.x] = 0;
@@ -609,14 +631,18 @@ __global__ __launch_bounds__(kBlockBwdThreads) void block_bwd_kernel(BlockBwdArg
         // computed ahead of the loop and kept in registers across the chunked code)
         const int z = fresh_s(0);
         float *ck = a.ckpt + (int64_t)(b * a.H + h) * slice + z;
+        const int64_t so = (int64_t)(b * a.H + h) * (kN * kN) + z;
+        const float *s0p = !kMulti && a.s0 ? a.s0 + so : nullptr, *gsTp = !kMulti && a.gsT ? a.gsT + so : nullptr;
+        float *gs0p = !kMulti && a.gs0 ? a.gs0 + so : nullptr;
+        const bool states = s0p || gsTp || gs0p;
         __syncthreads();
         scan_bwd_a_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdALds *>(smem), b, h, a.T, a.H, a.r + z, a.k + z, a.v + z, a.w + z, a.u + z, a.gy + z,
-                                        a.gr + z, a.gu + z, ck, kN, nullptr, nullptr, nullptr);
+                                        a.gr + z, a.gu + z, ck, kN, s0p, gsTp, states ? s_ft : nullptr);
         __threadfence_block();
         __syncthreads();
         const int z2 = fresh_s(0);
         scan_bwd_b_body<bf16_t, bf16_t>(*reinterpret_cast<ScanBwdBLds *>(smem), b, h, a.T, a.H, a.r + z2, a.k + z2, a.v + z2, a.w + z2, a.u + z2, a.gy + z2,
-                                        ck + z2, kN, a.gk + z2, a.gv + z2, a.gw + z2, nullptr, nullptr, nullptr, true);
+                                        ck + z2, kN, a.gk + z2, a.gv + z2, a.gw + z2, gsTp, states ? s_ft : nullptr, gs0p, s0p == nullptr);
         __threadfence_block();
         __syncthreads();
     }
@@ -657,7 +683,8 @@ bool block_backward_applies(int64_t B, int64_t T, int64_t H) { return block_forw
 
 hipError_t block_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
                           const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
-                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, void *gu_sum)
+                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, void *gu_sum,
+                          const float *s0, const float *gsT, float *gs0)
 {
     BlockBwdArgs a = {};
     a.T = (int)T; a.H = (int)H; a.B = (int)B;
@@ -667,6 +694,7 @@ hipError_t block_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
     a.u = (const bf16_t *)u; a.gy = (const bf16_t *)gy;
     a.gr = (bf16_t *)gr; a.gk = (bf16_t *)gk; a.gv = (bf16_t *)gv; a.gw = (bf16_t *)gw; a.gu = (bf16_t *)gu;
     a.gu_sum = (bf16_t *)gu_sum;
+    a.s0 = s0; a.gsT = gsT; a.gs0 = gs0;
     a.ckpt = (float *)workspace;
     a.arrivals = reinterpret_cast<int *>(reinterpret_cast<char *>(workspace) + chunk_backward_workspace_bytes(B, T, H));
     const bool multi = B * H > grid, ragged = (T % kBlockTokens) != 0;

@@ -716,14 +716,15 @@ hipError_t chunk_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
         return launch_in(bf16_t{}, ragged_tag);
     };
     const bool ragged = (T % CL) != 0;   // the last chunk has tokens past the end
-    const bool block_form = in_dtype == kBF16 && !s0 && !gsT && !gs0 && block_backward_applies(B, T, H);
+    // (gradients through the state: the block form takes them with one pair per workgroup)
+    const bool block_form = in_dtype == kBF16 && block_backward_applies(B, T, H) && ((!s0 && !gsT && !gs0) || B * H <= block_grid(B, H));
     if (!states_ready) {
         // No states from a saving forward: the forward kernel's state-only pass (no y) leaves them in
         // the workspace first.
         hipError_t e = chunk_forward(st, kF32, B, T, H, r, k, v, w, u, s0, nullptr, nullptr, nullptr, workspace, nullptr, false, false);
         if (e != hipSuccess) return e;
     }
-    if (block_form) return block_backward(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace, a.gu_sum);
+    if (block_form) return block_backward(st, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace, a.gu_sum, s0, gsT, gs0);
     return ragged ? launch(std::true_type{}) : launch(std::false_type{});
 }
 

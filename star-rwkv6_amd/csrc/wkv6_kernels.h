@@ -79,7 +79,8 @@ bool block_backward_applies(int64_t B, int64_t T, int64_t H);
 // workspace: the chunk-start states as a forward pass leaves them, followed by the per-head counters; gu_sum may be null
 hipError_t block_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
                           const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
-                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, void *gu_sum);
+                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, void *gu_sum,
+                          const float *s0 = nullptr, const float *gsT = nullptr, float *gs0 = nullptr);
 
 // fp16 tensors on the chunked kernels (training pair only: y and the gradients are fp32).  r, k, w stay
 // fp16 (the kernels unpack them exactly); v and gy are consumed as bf16 MFMA operands, so the caller

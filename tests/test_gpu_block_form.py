@@ -196,6 +196,17 @@ def test_block_form_fused_output_stage(op, oracle, B, T, H, with_state):
     check_close("sT", sT, sT_ref, BF16)
 
 
+# Gradients through the state (initial state in, gradient arriving at the final state, dL/dS_0 out) with one pair
+# per workgroup: both given, either one, a ragged end, a pair redone exactly
+@pytest.mark.parametrize("B,T,H,with_s0,with_gs,wild", [(5, 192, 32, True, True, False), (3, 128, 64, False, True, False),
+                                                        (5, 100, 32, True, False, False), (129, 64, 1, True, True, False),
+                                                        (5, 256, 32, True, True, True)])
+def test_block_form_state_gradients(op, oracle, B, T, H, with_s0, with_gs, wild):
+    from test_gpu_parity import _state_grad_case
+    assert _pairs_in_range(B, H)
+    _state_grad_case(op, oracle, B, T, H, 300 + T + H, BF16, CHUNK, with_s0=with_s0, with_gs=with_gs, wild=wild)
+
+
 def test_either_forward_feeds_either_backward(oracle):
     """The saved chunk states have one layout: the block-form backward on the states of the fused (tile-form)
     forward -- what a training layer runs -- and the plain backward, which rebuilds the states with the
