@@ -47,6 +47,13 @@ bool train_chunk(int dtype, int algo, int64_t T, int64_t C) {
     return algo == WKV6_ALGO_CHUNK || (algo == WKV6_ALGO_AUTO && dtype == WKV6_BF16 && T >= 32);
 }
 
+// fp32 tensors, and fp16 tensors unless their training pair asks for the bf16-operand kernels, train on the
+// full-precision chunk form; the per-timestep kernels on request (WKV6_ALGO_SCAN) and for short sequences.
+bool train_chunk32(int dtype, int algo, int64_t B, int64_t T, int64_t H) {
+    if (algo == WKV6_ALGO_SCAN || (dtype == WKV6_F16 && algo == WKV6_ALGO_CHUNK)) return false;
+    return wkv6::chunk32_forward_applies(dtype, B, T, H);
+}
+
 thread_local int g_last_status = WKV6_OK;
 thread_local int g_last_hip_error = 0;
 
@@ -111,6 +118,9 @@ static int forward_impl(void *stream, int dtype, int state_dtype, int algo,
     hipStream_t st = (hipStream_t)stream;
     const void *s_in = has_init_state ? s : nullptr;
     const int64_t *map_in = has_init_state ? state_map : nullptr;
+    // fp32 and fp16 tensors: the full-precision chunk form, unless the per-timestep kernels are asked for
+    if (algo != WKV6_ALGO_SCAN && wkv6::chunk32_forward_applies(dtype, B, T, H))
+        return finish(wkv6::chunk32_forward(st, dtype, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys, saved));
     if (algo == WKV6_ALGO_CHUNK && !chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;
     const bool chunk = algo == WKV6_ALGO_CHUNK ||
                        (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
@@ -297,6 +307,7 @@ static size_t f16_stage_offset(int algo, int64_t B, int64_t T, int64_t C, int64_
 
 size_t wkv6_saved_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
     if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
+    if (train_chunk32(dtype, algo, B, T, H)) return wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H);
     if (dtype == WKV6_F16)
         return train_chunk(dtype, algo, T, C) ? f16_stage_offset(algo, B, T, C, H) + 2 * (size_t)(B * T * C) * 2 : 0;
     const bool chunk = (algo == WKV6_ALGO_CHUNK && chunk_possible(dtype, T, C)) ||
@@ -314,7 +325,7 @@ int wkv6_forward_save(void *stream, int dtype, int algo, int64_t B, int64_t T, i
                       void *y, void *saved, size_t saved_bytes) {
     const size_t need = wkv6_saved_bytes(dtype, algo, B, T, C, H);
     if (need > 0 && (!saved || saved_bytes < need || !aligned16(saved))) return WKV6_ERR_WORKSPACE;
-    if (need > 0 && dtype == WKV6_F16) {
+    if (need > 0 && dtype == WKV6_F16 && !train_chunk32(dtype, algo, B, T, H)) {
         if (algo < WKV6_ALGO_AUTO || algo > WKV6_ALGO_CHUNK) return WKV6_ERR_ARG;
         if (!r || !k || !v || !w || !u || !y) return WKV6_ERR_ARG;
         if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(y)) return WKV6_ERR_ARG;
@@ -369,6 +380,10 @@ size_t wkv6_backward_workspace_bytes_ex(int dtype, int algo, int64_t B, int64_t 
     // The per-timestep path keeps one fp32 per element (P), the chunked path one fp32 state per
     // 64-token chunk (which a workgroup's exact second pass reuses for its own P).
     size_t need = wkv6::scan_backward_workspace_bytes(B, T, C);
+    if (train_chunk32(dtype, algo, B, T, H)) {   // one fp32 state per 32-token chunk
+        const size_t c = wkv6::chunk32_saved_bytes(B, T, H);
+        return c > need ? c : need;
+    }
     if (algo == WKV6_ALGO_CHUNK || (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C))) {
         const size_t c = wkv6::chunk_backward_workspace_bytes(B, T, H);
         if (c > need) need = c;
@@ -410,6 +425,16 @@ static int backward_impl(void *stream, int dtype, int algo, int64_t B, int64_t T
     const size_t need = wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H);
     if (need > 0 && (!workspace || workspace_bytes < need || !aligned16(workspace))) return WKV6_ERR_WORKSPACE;
     hipStream_t st = (hipStream_t)stream;
+    if (train_chunk32(dtype, algo, B, T, H)) {
+        // without saved states: a forward pass that only leaves the chunk states in the workspace
+        if (!states_ready) {
+            rc = finish(wkv6::chunk32_forward(st, dtype, WKV6_F32, B, T, H, r, k, v, w, u, nullptr, nullptr, nullptr, nullptr, workspace));
+            if (rc != WKV6_OK) return rc;
+        }
+        rc = finish(wkv6::chunk32_backward(st, dtype, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace));
+        if (rc == WKV6_OK && gu_sum) rc = finish(wkv6::sum_over_batch(st, out_type(dtype), B, C, gu, gu_sum));
+        return rc;
+    }
     if (algo == WKV6_ALGO_CHUNK && !chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;
     const bool chunk = algo == WKV6_ALGO_CHUNK ||
                        (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));

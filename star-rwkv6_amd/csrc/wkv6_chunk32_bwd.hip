@@ -1,0 +1,406 @@
+// Backward of the full-precision chunk form (see wkv6_chunk32.h): fp32 and fp16 tensors, gradients fp32-exact
+// to rounding, every product on v_mfma_f32_16x16x4_f32.
+//
+// Chunks of 32 tokens from the last to the first.  With S_0 the state at the chunk's start (saved by the
+// forward), G = dL/dS at its end, B[t][s] = sum_j gy_t[j] v_s[j] (s < t), vgy_t = B[t][t], A as in the forward:
+//   gv_s = K'_s G + sum_{t>=s} A[t][s] gy_t                       (A's diagonal holds sum_i r u k)
+//   gr_t = e^{c_t} o Z_t + u k_t vgy_t ,    Z_t = gy_t S_0^T + e^{-m} o sum_{s<t} B[t][s] K~_s
+//   gk_s = e^{c_32-c_{s+1}} o W_s + u r_s vgy_s ,  W_s = v_s G^T + e^{m-c_32} o sum_{t>s} B[t][s] R~_t
+//   gu  += r_t k_t vgy_t
+//   G   <- e^{c_32} o G + R'^T gy
+//   gw_t = d_t (E_{t+1} - K'_t W_t) ,  E_t = E_{t+1} + R'_t Z_t - K'_t W_t ,  E_T = 0
+// (E_t[i] = sum_j S_t[i][j] G_t[i][j]: what flows into channel i's decay at token t is the balance of what
+// the later tokens read from the state and what they wrote to it.)
+//
+// One workgroup of twelve waves per (batch, head) pair.  Waves 4..11 load, in two groups that take the
+// chunks in turn (as in the forward): tiles r, k, e^{c_t}, e^{c_32-c_{t+1}}, v, gy, d of the next chunk -> LDS.
+// Waves 0..3 compute: wave q owns value columns 16q.. of G (for K' G and the update), key rows 16q.. of
+// G^T (for v G^T) and of every per-channel output; S_0^T comes straight from the saved states.  Both G and
+// G^T are kept so that neither product needs a sum across waves.  Two workgroup barriers per chunk:
+//   phase 1  tiles of A and B (one or two per wave) -> LDS ; K' G ; gy S_0^T ; v G^T
+//   phase 2  the three products with A and B ; gradients out (16 lanes x 4 bytes per row piece) ; G, G^T updates
+#include "wkv6_chunk32.h"
+#include "wkv6_kernels.h"
+#include "wkv6_scan_body.h"
+
+#include <type_traits>
+
+#ifndef C32_GROUPS
+#define C32_GROUPS 2
+#endif
+
+namespace wkv6 {
+
+struct C32BwdLds {
+    float R[2][kC32][kLd], K[2][kC32][kLd], F1[2][kC32][kLd], F3[2][kC32][kLd];   // r, k, e^{c_t}, e^{c_32 - c_{t+1}}
+    float V[2][kC32][kLd], GY[2][kC32][kLd], D[2][kC32][kLd];                     // v, gy, log decay
+    float A[kC32][kLa], Bm[kC32][kLa];
+    float e_all[2][kN], e_mid[2][kN], e_rest[2][kN], inv0[2][kN], inv1[2][kN];    // e^{c_32}, e^{m}, e^{c_32-m}, e^{-m}, e^{m-c_32}
+    float ruk[2][4][kC32];
+    float vgy[kC32];
+    int wild[4 * 3];
+};
+union C32BwdSmem {
+    C32BwdLds chunk;
+    ScanBwdALds scan_a;
+    ScanBwdBLds scan_b;
+};
+
+struct C32BwdArgs {
+    int T, H;
+    const void *r, *k, *v, *w, *u, *gy;
+    void *gr, *gk, *gv, *gw, *gu;
+    float *saved;   // [pair][chunk][4096] chunk-start states as the forward leaves them (fragment order)
+};
+
+template <typename Tin, typename Tout, int kGroups>
+__global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_bwd_kernel(const C32BwdArgs a)
+{
+    extern __shared__ __align__(16) unsigned char c32_smem[];
+    C32BwdLds &L = reinterpret_cast<C32BwdSmem *>(c32_smem)->chunk;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int T = a.T, H = a.H;
+    const int pair = blockIdx.x, b = pair / H, h = pair - b * H;
+    const int64_t C = (int64_t)H * kN;
+    const int64_t base = (int64_t)b * T * C + (int64_t)h * kN;
+    const int nchunk = (T + kC32 - 1) / kC32;
+    const Tin *r = reinterpret_cast<const Tin *>(a.r), *k = reinterpret_cast<const Tin *>(a.k);
+    const Tin *v = reinterpret_cast<const Tin *>(a.v), *w = reinterpret_cast<const Tin *>(a.w);
+    const Tin *u = reinterpret_cast<const Tin *>(a.u);
+    const Tout *gy = reinterpret_cast<const Tout *>(a.gy);
+    float *const ck = a.saved + (int64_t)pair * nchunk * (kN * kN);
+    // step s handles chunk nchunk - 1 - s
+
+    if (wave >= 4) {
+        // ---------------- loading waves ----------------
+        const int grp = (wave - 4) >> 2, p = (wave - 4) & 3, t16 = lane & 15, ch = 16 * p + 4 * (lane >> 4);
+        float fu[4];
+        load4(u + h * kN + ch, fu);
+        float nr[2][4], nk[2][4], nv[2][4], nw[2][4], ng[2][4];   // the group's chunk as loaded (r, k, v, gy stay until handed on)
+        auto fetch = [&](int s) {
+            const int c = nchunk - 1 - s;
+#pragma unroll
+            for (int x = 0; x < 2; ++x) {
+                const int t = min(c * kC32 + 16 * x + t16, T - 1);
+                const int64_t o = base + (int64_t)t * C + ch;
+                load4(r + o, nr[x]); load4(k + o, nk[x]); load4(v + o, nv[x]); load4(w + o, nw[x]); load4(gy + o, ng[x]);
+            }
+        };
+        float f1[2][4], f3[2][4], dd[2][4], e_all[4], e_mid[4], e_rest[4], inv0[4], inv1[4], part[2];
+        bool wild = false;
+        // two channels of the lane's four at a time (a barrier in between)
+        auto form = [&](auto half, int s) {
+            constexpr int E0 = 2 * decltype(half)::value;
+            const int c = nchunk - 1 - s;
+            const bool valid[2] = {c * kC32 + t16 < T, c * kC32 + 16 + t16 < T};
+            C32Scale sc;
+            sc.wild = false;
+            c32_scale<E0, E0 + 2>(nw, valid, sc, dd);
+            wild |= sc.wild;
+#pragma unroll
+            for (int x = 0; x < 2; ++x) {
+                float acc = E0 == 0 ? 0.f : part[x];
+#pragma unroll
+                for (int e = E0; e < E0 + 2; ++e) {
+                    if (!valid[x]) { nr[x][e] = 0.f; nk[x][e] = 0.f; nv[x][e] = 0.f; ng[x][e] = 0.f; }
+                    f1[x][e] = sc.rp[x][e];
+                    f3[x][e] = sc.kp[x][e];
+                    e_all[e] = sc.all[e]; e_mid[e] = sc.mid[e]; e_rest[e] = sc.rest[e]; inv0[e] = sc.inv0[e]; inv1[e] = sc.inv1[e];
+                    acc = fmaf(nr[x][e] * nk[x][e], fu[e], acc);
+                }
+                part[x] = E0 == 0 ? acc : sum_rows4(acc);
+            }
+        };
+        auto as4 = [](const float (&f)[4]) { return (f32x4){f[0], f[1], f[2], f[3]}; };
+        auto publish = [&](int s) {
+            const int buf = s & 1;
+#pragma unroll
+            for (int x = 0; x < 2; ++x) {
+                const int t = 16 * x + t16;
+                *reinterpret_cast<f32x4 *>(&L.R[buf][t][ch]) = as4(nr[x]);
+                *reinterpret_cast<f32x4 *>(&L.K[buf][t][ch]) = as4(nk[x]);
+                *reinterpret_cast<f32x4 *>(&L.F1[buf][t][ch]) = as4(f1[x]);
+                *reinterpret_cast<f32x4 *>(&L.F3[buf][t][ch]) = as4(f3[x]);
+                *reinterpret_cast<f32x4 *>(&L.V[buf][t][ch]) = as4(nv[x]);
+                *reinterpret_cast<f32x4 *>(&L.GY[buf][t][ch]) = as4(ng[x]);
+                *reinterpret_cast<f32x4 *>(&L.D[buf][t][ch]) = as4(dd[x]);
+                if (lane < 16) L.ruk[buf][p][t] = part[x];
+            }
+            if (t16 == 0) {
+                *reinterpret_cast<f32x4 *>(&L.e_all[buf][ch]) = as4(e_all);
+                *reinterpret_cast<f32x4 *>(&L.e_mid[buf][ch]) = as4(e_mid);
+                *reinterpret_cast<f32x4 *>(&L.e_rest[buf][ch]) = as4(e_rest);
+                *reinterpret_cast<f32x4 *>(&L.inv0[buf][ch]) = as4(inv0);
+                *reinterpret_cast<f32x4 *>(&L.inv1[buf][ch]) = as4(inv1);
+            }
+        };
+        const std::integral_constant<int, 0> h0;
+        const std::integral_constant<int, 1> h1;
+        // Group s % kGroups brings step s: it forms the scale factors while step s - 2 is computed, hands the
+        // tiles to LDS while step s - 1 is computed and then sends for its next chunk (its loads are the only
+        // ones the wave has in flight, so the wait for them is exact).
+        if (grp < 2 && grp < nchunk) {
+            fetch(grp);
+            form(h0, grp);
+            form(h1, grp);
+            if (grp == 0) {
+                publish(0);
+                if (kGroups < nchunk) fetch(kGroups);
+            }
+        } else if (grp < nchunk) fetch(grp);
+        __syncthreads();
+        for (int s = 0; s < nchunk; ++s) {
+            const bool forming = (s + 2) % kGroups == grp && s + 2 < nchunk;
+            const bool handing = (s + 1) % kGroups == grp && s + 1 < nchunk;
+            if (forming) form(h0, s + 2);
+            if (handing) {
+                publish(s + 1);
+                if (s + 1 + kGroups < nchunk) fetch(s + 1 + kGroups);
+            }
+            __syncthreads();
+            if (forming) form(h1, s + 2);
+            __syncthreads();
+        }
+        const bool any = __any(wild);
+        if (lane == 0) L.wild[wave - 4] = any;
+    } else {
+        // ---------------- computing waves ----------------
+        const int q = wave, n = lane & 15, g = lane >> 4, col = 16 * q + n;
+        Tout *gr = reinterpret_cast<Tout *>(a.gr), *gk = reinterpret_cast<Tout *>(a.gk);
+        Tout *gv = reinterpret_cast<Tout *>(a.gv), *gw = reinterpret_cast<Tout *>(a.gw);
+        const f32x4 zero = (f32x4){0.f, 0.f, 0.f, 0.f};
+        f32x4 G[4], Gt[4], St[4];   // G[ib][e] = G[16ib+4g+e][col] ; Gt[jb][e] = G[col][16jb+4g+e] ; St likewise of S_0
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { G[i] = zero; Gt[i] = zero; }
+        float E = 0.f, gu_acc = 0.f;
+        const float u_lane = load1(u + h * kN + col);
+        // S_0^T from the forward's fragment order: S[i][j] sits in tile (j / 16, i / 16) at lane (j % 16) + 16 ((i % 16) / 4), element i % 4
+        auto load_state = [&](int c) {
+            const float *p0 = ck + (int64_t)c * (kN * kN) + (q * 64 + 4 * g + 16 * (n >> 2)) * 4 + (n & 3);
+#pragma unroll
+            for (int jb = 0; jb < 4; ++jb)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) St[jb][e] = p0[jb * 1024 + e * 4];
+        };
+        load_state(nchunk - 1);
+        __syncthreads();
+        for (int s = 0; s < nchunk; ++s) {
+            const int c = nchunk - 1 - s, buf = s & 1;
+            // ---- phase 1 ----
+            {   // tiles of A and B: wave 0 (0,0) of both, wave 1 (1,1) of both, wave 2 A(1,0), wave 3 B(1,0)
+                const int tb = q == 0 ? 0 : 1, sb = q == 1 ? 1 : 0;
+                if (q < 3) {
+                    f32x4 at = zero;
+#pragma unroll
+                    for (int ib = 0; ib < 4; ++ib) {
+                        const int i0 = 16 * ib + 4 * g;
+                        const f32x4 fk = *reinterpret_cast<const f32x4 *>(&L.K[buf][16 * sb + n][i0]) *
+                                         *reinterpret_cast<const f32x4 *>(&L.F3[buf][16 * sb + n][i0]) *
+                                         *reinterpret_cast<const f32x4 *>(&L.inv1[buf][i0]);
+                        const f32x4 fr = *reinterpret_cast<const f32x4 *>(&L.R[buf][16 * tb + n][i0]) *
+                                         *reinterpret_cast<const f32x4 *>(&L.F1[buf][16 * tb + n][i0]) *
+                                         *reinterpret_cast<const f32x4 *>(&L.inv0[buf][i0]);
+                        at = mfma16(fk, fr, at);
+                    }
+                    if (tb == sb) {
+                        const int t = 16 * tb + n;
+                        const float diag = (L.ruk[buf][0][t] + L.ruk[buf][1][t]) + (L.ruk[buf][2][t] + L.ruk[buf][3][t]);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) at[e] = (4 * g + e < n) ? at[e] : (4 * g + e == n ? diag : 0.f);
+                    }
+                    *reinterpret_cast<f32x4 *>(&L.A[16 * tb + n][16 * sb + 4 * g]) = at;
+                }
+                if (q != 2) {
+                    f32x4 bt = zero;
+#pragma unroll
+                    for (int jb = 0; jb < 4; ++jb) {
+                        const f32x4 fv = *reinterpret_cast<const f32x4 *>(&L.V[buf][16 * sb + n][16 * jb + 4 * g]);
+                        const f32x4 fg = *reinterpret_cast<const f32x4 *>(&L.GY[buf][16 * tb + n][16 * jb + 4 * g]);
+                        bt = mfma16(fv, fg, bt);
+                    }
+                    if (tb == sb) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            if (4 * g + e == n) L.vgy[16 * tb + n] = bt[e];
+                            bt[e] = (4 * g + e < n) ? bt[e] : 0.f;
+                        }
+                    }
+                    *reinterpret_cast<f32x4 *>(&L.Bm[16 * tb + n][16 * sb + 4 * g]) = bt;
+                }
+            }
+            f32x4 gvt[2] = {zero, zero}, Z[2] = {zero, zero}, W[2] = {zero, zero};
+#pragma unroll
+            for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+                for (int ib = 0; ib < 4; ++ib) {
+                    const f32x4 fk = *reinterpret_cast<const f32x4 *>(&L.K[buf][16 * sb + n][16 * ib + 4 * g]) *
+                                     *reinterpret_cast<const f32x4 *>(&L.F3[buf][16 * sb + n][16 * ib + 4 * g]);
+                    gvt[sb] = mfma16(fk, G[ib], gvt[sb]);
+                }
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+                for (int jb = 0; jb < 4; ++jb) {
+                    const f32x4 fg = *reinterpret_cast<const f32x4 *>(&L.GY[buf][16 * tb + n][16 * jb + 4 * g]);
+                    const f32x4 fv = *reinterpret_cast<const f32x4 *>(&L.V[buf][16 * tb + n][16 * jb + 4 * g]);
+                    Z[tb] = mfma16(fg, St[jb], Z[tb]);
+                    W[tb] = mfma16(fv, Gt[jb], W[tb]);
+                }
+            const float e_all = L.e_all[buf][col], e_mid = L.e_mid[buf][col], e_rest = L.e_rest[buf][col];
+            const float inv0 = L.inv0[buf][col], inv1 = L.inv1[buf][col];
+            // the products with B come scaled from the middle of the chunk: bring these to that scale, all back at the end
+#pragma unroll
+            for (int x = 0; x < 2; ++x) { Z[x] *= e_mid; W[x] *= e_rest; }
+            __syncthreads();
+            // ---- phase 2 ----
+            if (c > 0) load_state(c - 1);
+            f32x4 rc[2], kc[2], rp[2], kp[2], gyb[2];   // element e: token 16x + 4g + e, channel col
+#pragma unroll
+            for (int x = 0; x < 2; ++x)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int t = 16 * x + 4 * g + e;
+                    rc[x][e] = L.R[buf][t][col];
+                    kc[x][e] = L.K[buf][t][col];
+                    rp[x][e] = rc[x][e] * L.F1[buf][t][col];
+                    kp[x][e] = kc[x][e] * L.F3[buf][t][col];
+                    gyb[x][e] = L.GY[buf][t][col];
+                }
+#pragma unroll
+            for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+                for (int sb = 0; sb <= tb; ++sb) {
+                    const f32x4 fb = *reinterpret_cast<const f32x4 *>(&L.Bm[16 * tb + n][16 * sb + 4 * g]);
+                    Z[tb] = mfma16(fb, kp[sb] * inv1, Z[tb]);
+                }
+#pragma unroll
+            for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+                for (int tb = sb; tb < 2; ++tb) {
+                    f32x4 fbt, fat;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        fbt[e] = L.Bm[16 * tb + 4 * g + e][16 * sb + n];
+                        fat[e] = L.A[16 * tb + 4 * g + e][16 * sb + n];
+                    }
+                    W[sb] = mfma16(fbt, rp[tb] * inv0, W[sb]);
+                    gvt[sb] = mfma16(fat, gyb[tb], gvt[sb]);
+                }
+            // gradients out
+            float zt[2][4], kgk[2][4];
+#pragma unroll
+            for (int x = 0; x < 2; ++x) {
+                const f32x4 vg = *reinterpret_cast<const f32x4 *>(&L.vgy[16 * x + 4 * g]);
+                Z[x] *= inv0;
+                W[x] *= inv1;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int tl = 16 * x + 4 * g + e, t = c * kC32 + tl;
+                    const float f1 = L.F1[buf][tl][col], f3 = L.F3[buf][tl][col];
+                    const float o_r = fmaf(f1, Z[x][e], u_lane * kc[x][e] * vg[e]);
+                    const float o_k = fmaf(f3, W[x][e], u_lane * rc[x][e] * vg[e]);
+                    kgk[x][e] = kp[x][e] * W[x][e];
+                    zt[x][e] = fmaf(rp[x][e], Z[x][e], -kgk[x][e]);
+                    gu_acc = fmaf(rc[x][e] * kc[x][e], vg[e], gu_acc);
+                    if (t < T) {
+                        const int64_t o = base + (int64_t)t * C + col;
+                        store1(gr + o, o_r);
+                        store1(gk + o, o_k);
+                        store1(gv + o, gvt[x][e]);
+                    }
+                }
+            }
+            {   // E_{t+1} = E at the chunk's end + what the later tokens of the chunk add
+                float tot[2], other[2][4], later[2];
+#pragma unroll
+                for (int x = 0; x < 2; ++x) {
+                    tot[x] = (zt[x][0] + zt[x][1]) + (zt[x][2] + zt[x][3]);
+                    rows4(tot[x], other[x]);
+                    later[x] = (g < 1 ? other[x][1] : 0.f) + (g < 2 ? other[x][2] : 0.f) + (g < 3 ? other[x][3] : 0.f);
+                }
+                const float all1 = (other[1][0] + other[1][1]) + (other[1][2] + other[1][3]);
+                const float all0 = (other[0][0] + other[0][1]) + (other[0][2] + other[0][3]);
+                later[0] += all1;
+#pragma unroll
+                for (int x = 0; x < 2; ++x) {
+                    float run = E + later[x];
+#pragma unroll
+                    for (int e = 3; e >= 0; --e) {
+                        const int tl = 16 * x + 4 * g + e, t = c * kC32 + tl;
+                        const float o_w = (run - kgk[x][e]) * L.D[buf][tl][col];
+                        if (t < T) store1(gw + base + (int64_t)t * C + col, o_w);
+                        run += zt[x][e];
+                    }
+                }
+                E += all0 + all1;
+            }
+            // G <- e^{c_32} o G + R'^T gy, both copies
+#pragma unroll
+            for (int ib = 0; ib < 4; ++ib) {
+                G[ib] *= *reinterpret_cast<const f32x4 *>(&L.e_all[buf][16 * ib + 4 * g]);
+#pragma unroll
+                for (int tb = 0; tb < 2; ++tb) {
+                    f32x4 fra;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) fra[e] = L.R[buf][16 * tb + 4 * g + e][16 * ib + n] * L.F1[buf][16 * tb + 4 * g + e][16 * ib + n];
+                    G[ib] = mfma16(fra, gyb[tb], G[ib]);
+                }
+            }
+#pragma unroll
+            for (int jb = 0; jb < 4; ++jb) {
+                Gt[jb] *= e_all;
+#pragma unroll
+                for (int tb = 0; tb < 2; ++tb) {
+                    f32x4 fga;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) fga[e] = L.GY[buf][16 * tb + 4 * g + e][16 * jb + n];
+                    Gt[jb] = mfma16(fga, rp[tb], Gt[jb]);
+                }
+            }
+            __syncthreads();
+        }
+        // gu: the four row groups of the wave hold the tokens 4g .. 4g+3 (mod 16) of every chunk
+        gu_acc = sum_rows4(gu_acc);
+        if (g == 0) store1(reinterpret_cast<Tout *>(a.gu) + (int64_t)b * C + h * kN + col, gu_acc);
+    }
+    __syncthreads();
+    // a pair whose decay left the reach: once more, one timestep at a time (the pair's slice of the saved
+    // states, T/32 x 64 x 64 floats, is large enough for the T x 64 workspace of that pass)
+    int wild_any = 0;
+#pragma unroll
+    for (int i = 0; i < 4 * kGroups; ++i) wild_any |= L.wild[i];
+    if (wild_any) {
+        __syncthreads();
+        scan_bwd_a_body<Tin, Tout>(reinterpret_cast<C32BwdSmem *>(c32_smem)->scan_a, b, h, T, H, r, k, v, w, u, gy,
+                                   reinterpret_cast<Tout *>(a.gr), reinterpret_cast<Tout *>(a.gu), ck, kN);
+        __threadfence_block();
+        __syncthreads();
+        scan_bwd_b_body<Tin, Tout>(reinterpret_cast<C32BwdSmem *>(c32_smem)->scan_b, b, h, T, H, r, k, v, w, u, gy, ck, kN,
+                                   reinterpret_cast<Tout *>(a.gk), reinterpret_cast<Tout *>(a.gv), reinterpret_cast<Tout *>(a.gw));
+    }
+}
+
+template <typename Tin, typename Tout>
+static hipError_t launch(hipStream_t st, int64_t B, const C32BwdArgs &a) {
+    constexpr int kGroups = C32_GROUPS;
+    constexpr int lds = (int)sizeof(C32BwdSmem);
+    const hipError_t e = allow_dynamic_lds<chunk32_bwd_kernel<Tin, Tout, kGroups>>(lds);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL((chunk32_bwd_kernel<Tin, Tout, kGroups>), dim3((unsigned)(B * a.H)), dim3(256 + 256 * kGroups), lds, st, a);
+    return hipGetLastError();
+}
+
+hipError_t chunk32_backward(hipStream_t st, int dtype, int64_t B, int64_t T, int64_t H,
+                            const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                            void *gr, void *gk, void *gv, void *gw, void *gu, void *saved_states)
+{
+    C32BwdArgs a;
+    a.T = (int)T; a.H = (int)H;
+    a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.gy = gy;
+    a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu;
+    a.saved = reinterpret_cast<float *>(saved_states);
+    if (dtype == kF32) return launch<float, float>(st, B, a);
+    return launch<f16_t, float>(st, B, a);
+}
+
+}  // namespace wkv6

@@ -82,6 +82,21 @@ hipError_t block_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
                           void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, void *gu_sum,
                           const float *s0 = nullptr, const float *gsT = nullptr, float *gs0 = nullptr);
 
+// --- full-precision chunk form (wkv6_chunk32_fwd.hip, wkv6_chunk32_bwd.hip): fp32 and fp16 tensors on the
+// fp32 matrix instructions, chunks of 32 tokens, fp32 states; any T (the last chunk may be short).
+bool chunk32_forward_applies(int dtype, int64_t B, int64_t T, int64_t H);
+size_t chunk32_saved_bytes(int64_t B, int64_t T, int64_t H);   // one fp32 state per chunk and pair
+// saved_states (may be null): receives the chunk-start states for chunk32_backward; y may be null then
+hipError_t chunk32_forward(hipStream_t st, int dtype, int state_dtype, int64_t B, int64_t T, int64_t H,
+                           const void *r, const void *k, const void *v, const void *w, const void *u,
+                           const void *s0, const int64_t *map, void *y, void *sT, void *saved_states);
+
+// saved_states: what chunk32_forward left (the pair's slice also serves the per-timestep pass of a pair
+// whose decay left the chunk form's reach); gu (B, C)
+hipError_t chunk32_backward(hipStream_t st, int dtype, int64_t B, int64_t T, int64_t H,
+                            const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
+                            void *gr, void *gk, void *gv, void *gw, void *gu, void *saved_states);
+
 // fp16 tensors on the chunked kernels (training pair only: y and the gradients are fp32).  r, k, w stay
 // fp16 (the kernels unpack them exactly); v and gy are consumed as bf16 MFMA operands, so the caller
 // keeps bf16 copies of them (convert_to_bf16) next to the saved states.

@@ -389,13 +389,15 @@ def test_chunk_f16_falls_back_on_extreme_decay(op, oracle):
 
 
 def test_f16_chunked_training_pair_is_opt_in(op, oracle):
-    # AUTO keeps fp16 tensors on the exact per-timestep kernels (no saved states; fp32 tolerance, the same
-    # y with and without a gradient); the chunked pair -- bf16 operand precision -- runs on request only
+    # AUTO keeps fp16 tensors at fp32 accuracy (the full-precision chunk form, fp32 chunk states saved for the
+    # backward; the same y with and without a gradient); the bf16-operand pair runs on request only
     from rwkv_kernel import _native
     lib = _native.load()
-    assert lib.wkv6_saved_bytes(_native.F16, _native.ALGO_AUTO, 2, 256, 128, 2) == 0
+    full = 2 * 2 * (256 // 32) * 64 * 64 * 4
+    assert lib.wkv6_saved_bytes(_native.F16, _native.ALGO_AUTO, 2, 256, 128, 2) == full
+    assert lib.wkv6_saved_bytes(_native.F32, _native.ALGO_AUTO, 2, 256, 128, 2) == full
     assert lib.wkv6_saved_bytes(_native.F16, _native.ALGO_SCAN, 2, 256, 128, 2) == 0
-    assert lib.wkv6_saved_bytes(_native.F16, _native.ALGO_CHUNK, 2, 256, 128, 2) > 0
+    assert lib.wkv6_saved_bytes(_native.F16, _native.ALGO_CHUNK, 2, 256, 128, 2) > full
     assert lib.wkv6_saved_bytes(_native.BF16, _native.ALGO_AUTO, 2, 256, 128, 2) > 0
     y_train, _ = _case(op, oracle, 2, 256, 2, 77, torch.float16, 0)          # fp32 tolerance (1e-4 / 1e-3)
     ins = oracle.make_inputs(2, 256, 2, 64, 77)
