@@ -42,13 +42,21 @@ __device__ __forceinline__ f32x4 mfma16(const f32x4 a, const f32x4 b, f32x4 c) {
 template <int kCtrl> __device__ __forceinline__ float row_take(float x) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0x3f800000, __float_as_int(x), kCtrl, 0xF, 0xF, false));
 }
-// running products over the 16 lanes of a row: lane n gets x_0 .. x_n (up) or x_n .. x_15 (down)
+// running products over the 16 lanes of a row: lane n gets x_0 .. x_n (up) or x_n .. x_15 (down).  One DPP
+// multiply per step (a lane without a source keeps its value); the wait states a DPP read of a freshly written
+// register needs are spelled out, the compiler does not look inside.
 __device__ __forceinline__ float row_product_up(float x) {
-    x *= row_take<0x111>(x); x *= row_take<0x112>(x); x *= row_take<0x114>(x); x *= row_take<0x118>(x);
+    asm("s_nop 1\n\tv_mul_f32_dpp %0, %0, %0 row_shr:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_mul_f32_dpp %0, %0, %0 row_shr:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_mul_f32_dpp %0, %0, %0 row_shr:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_mul_f32_dpp %0, %0, %0 row_shr:8 row_mask:0xf bank_mask:0xf" : "+v"(x));
     return x;
 }
 __device__ __forceinline__ float row_product_down(float x) {
-    x *= row_take<0x101>(x); x *= row_take<0x102>(x); x *= row_take<0x104>(x); x *= row_take<0x108>(x);
+    asm("s_nop 1\n\tv_mul_f32_dpp %0, %0, %0 row_shl:1 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_mul_f32_dpp %0, %0, %0 row_shl:2 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_mul_f32_dpp %0, %0, %0 row_shl:4 row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\tv_mul_f32_dpp %0, %0, %0 row_shl:8 row_mask:0xf bank_mask:0xf" : "+v"(x));
     return x;
 }
 // x of the same lane-in-row in each of the wave's four rows (lanes n, 16 + n, 32 + n, 48 + n), in every lane

@@ -12,22 +12,21 @@
 // (E_t[i] = sum_j S_t[i][j] G_t[i][j]: what flows into channel i's decay at token t is the balance of what
 // the later tokens read from the state and what they wrote to it.)
 //
-// One workgroup of twelve waves per (batch, head) pair.  Waves 4..11 load, in two groups that take the
-// chunks in turn (as in the forward): tiles r, k, e^{c_t}, e^{c_32-c_{t+1}}, v, gy, d of the next chunk -> LDS.
-// Waves 0..3 compute: wave q owns value columns 16q.. of G (for K' G and the update), key rows 16q.. of
-// G^T (for v G^T) and of every per-channel output; S_0^T comes straight from the saved states.  Both G and
-// G^T are kept so that neither product needs a sum across waves.  Two workgroup barriers per chunk:
-//   phase 1  tiles of A and B (one or two per wave) -> LDS ; K' G ; gy S_0^T ; v G^T
+// One workgroup of twelve waves per (batch, head) pair, three roles of four waves (one wave of each role per SIMD,
+// so that one role's waits are another's issue slots):
+//   loading waves   tiles r, k, e^{c_t}, e^{c_32-c_{t+1}}, v, gy, d of the next chunk -> LDS (loads issued one phase
+//                   ahead of their use: the kernel is bound by arithmetic, not by memory)
+//   value waves     wave q owns value columns 16q.. of G: gv = K' G + A^T gy, the update of G, the tiles of A
+//   key waves       wave q owns key rows 16q.. of G^T and of every per-channel output: Z, W, gr, gk, gw, gu, the
+//                   update of G^T, the tiles of B; S_0^T comes straight from the saved states
+// Both G and G^T are kept so that neither K' G nor v G^T needs a sum across waves.  Two workgroup barriers per chunk:
+//   phase 1  tiles of A and B -> LDS ; K' G ; gy S_0^T ; v G^T
 //   phase 2  the three products with A and B ; gradients out (16 lanes x 4 bytes per row piece) ; G, G^T updates
 #include "wkv6_chunk32.h"
 #include "wkv6_kernels.h"
 #include "wkv6_scan_body.h"
 
 #include <type_traits>
-
-#ifndef C32_GROUPS
-#define C32_GROUPS 2
-#endif
 
 namespace wkv6 {
 
@@ -38,7 +37,7 @@ struct C32BwdLds {
     float e_all[2][kN], e_mid[2][kN], e_rest[2][kN], inv0[2][kN], inv1[2][kN];    // e^{c_32}, e^{m}, e^{c_32-m}, e^{-m}, e^{m-c_32}
     float ruk[2][4][kC32];
     float vgy[kC32];
-    int wild[4 * 3];
+    int wild[4];
 };
 union C32BwdSmem {
     C32BwdLds chunk;
@@ -53,8 +52,8 @@ struct C32BwdArgs {
     float *saved;   // [pair][chunk][4096] chunk-start states as the forward leaves them (fragment order)
 };
 
-template <typename Tin, typename Tout, int kGroups>
-__global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_bwd_kernel(const C32BwdArgs a)
+template <typename Tin, typename Tout>
+__global__ __launch_bounds__(768) void chunk32_bwd_kernel(const C32BwdArgs a)
 {
     extern __shared__ __align__(16) unsigned char c32_smem[];
     C32BwdLds &L = reinterpret_cast<C32BwdSmem *>(c32_smem)->chunk;
@@ -71,19 +70,20 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_bwd_kernel(const 
     float *const ck = a.saved + (int64_t)pair * nchunk * (kN * kN);
     // step s handles chunk nchunk - 1 - s
 
-    if (wave >= 4) {
+    if (wave >= 8) {
         // ---------------- loading waves ----------------
-        const int grp = (wave - 4) >> 2, p = (wave - 4) & 3, t16 = lane & 15, ch = 16 * p + 4 * (lane >> 4);
+        const int p = wave - 8, t16 = lane & 15, ch = 16 * p + 4 * (lane >> 4);
         float fu[4];
         load4(u + h * kN + ch, fu);
         float nr[2][4], nk[2][4], nv[2][4], nw[2][4], ng[2][4];   // the group's chunk as loaded (r, k, v, gy stay until handed on)
         auto fetch = [&](int s) {
             const int c = nchunk - 1 - s;
+            const int64_t row0 = base + (int64_t)c * kC32 * C;   // (uniform)
 #pragma unroll
             for (int x = 0; x < 2; ++x) {
-                const int t = min(c * kC32 + 16 * x + t16, T - 1);
-                const int64_t o = base + (int64_t)t * C + ch;
-                load4(r + o, nr[x]); load4(k + o, nk[x]); load4(v + o, nv[x]); load4(w + o, nw[x]); load4(gy + o, ng[x]);
+                const int o = min(16 * x + t16, T - 1 - c * kC32) * (int)C + ch;   // rows past the end read the last one
+                load4(r + row0 + o, nr[x]); load4(k + row0 + o, nk[x]); load4(v + row0 + o, nv[x]); load4(w + row0 + o, nw[x]);
+                load4(gy + row0 + o, ng[x]);
             }
         };
         float f1[2][4], f3[2][4], dd[2][4], e_all[4], e_mid[4], e_rest[4], inv0[4], inv1[4], part[2];
@@ -136,42 +136,122 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_bwd_kernel(const 
         };
         const std::integral_constant<int, 0> h0;
         const std::integral_constant<int, 1> h1;
-        // Group s % kGroups brings step s: it forms the scale factors while step s - 2 is computed, hands the
-        // tiles to LDS while step s - 1 is computed and then sends for its next chunk (its loads are the only
-        // ones the wave has in flight, so the wait for them is exact).
-        if (grp < 2 && grp < nchunk) {
-            fetch(grp);
-            form(h0, grp);
-            form(h1, grp);
-            if (grp == 0) {
-                publish(0);
-                if (kGroups < nchunk) fetch(kGroups);
-            }
-        } else if (grp < nchunk) fetch(grp);
+        // While step s is computed: the tiles of step s + 1 go to LDS and the loads of step s + 2 are issued
+        // (phase 1), the scale factors of step s + 2 are formed (phase 2).
+        fetch(0);
+        form(h0, 0);
+        form(h1, 0);
+        publish(0);
+        if (nchunk > 1) {
+            fetch(1);
+            form(h0, 1);
+            form(h1, 1);
+        }
         __syncthreads();
         for (int s = 0; s < nchunk; ++s) {
-            const bool forming = (s + 2) % kGroups == grp && s + 2 < nchunk;
-            const bool handing = (s + 1) % kGroups == grp && s + 1 < nchunk;
-            if (forming) form(h0, s + 2);
-            if (handing) {
-                publish(s + 1);
-                if (s + 1 + kGroups < nchunk) fetch(s + 1 + kGroups);
-            }
+            if (s + 1 < nchunk) publish(s + 1);
+            if (s + 2 < nchunk) fetch(s + 2);
             __syncthreads();
-            if (forming) form(h1, s + 2);
+            if (s + 2 < nchunk) {
+                form(h0, s + 2);
+                form(h1, s + 2);
+            }
             __syncthreads();
         }
         const bool any = __any(wild);
-        if (lane == 0) L.wild[wave - 4] = any;
-    } else {
-        // ---------------- computing waves ----------------
+        if (lane == 0) L.wild[p] = any;
+    } else if (wave < 4) {
+        // ---------------- value waves ----------------
         const int q = wave, n = lane & 15, g = lane >> 4, col = 16 * q + n;
-        Tout *gr = reinterpret_cast<Tout *>(a.gr), *gk = reinterpret_cast<Tout *>(a.gk);
-        Tout *gv = reinterpret_cast<Tout *>(a.gv), *gw = reinterpret_cast<Tout *>(a.gw);
+        Tout *gv = reinterpret_cast<Tout *>(a.gv);
         const f32x4 zero = (f32x4){0.f, 0.f, 0.f, 0.f};
-        f32x4 G[4], Gt[4], St[4];   // G[ib][e] = G[16ib+4g+e][col] ; Gt[jb][e] = G[col][16jb+4g+e] ; St likewise of S_0
+        const int lane_off = 4 * g * (int)C + col;
+        f32x4 G[4];   // G[ib][e] = G[16ib+4g+e][col]
 #pragma unroll
-        for (int i = 0; i < 4; ++i) { G[i] = zero; Gt[i] = zero; }
+        for (int i = 0; i < 4; ++i) G[i] = zero;
+        __syncthreads();
+        for (int s = 0; s < nchunk; ++s) {
+            const int c = nchunk - 1 - s, buf = s & 1;
+            const bool full = (c + 1) * kC32 <= T;
+            // ---- phase 1: a tile of A (wave 0: (0,0), 1: (1,1), 2: (1,0)), K' G ----
+            if (q < 3) {
+                const int tb = q == 0 ? 0 : 1, sb = q == 1 ? 1 : 0;
+                f32x4 at = zero;
+#pragma unroll
+                for (int ib = 0; ib < 4; ++ib) {
+                    const int i0 = 16 * ib + 4 * g;
+                    const f32x4 fk = *reinterpret_cast<const f32x4 *>(&L.K[buf][16 * sb + n][i0]) *
+                                     *reinterpret_cast<const f32x4 *>(&L.F3[buf][16 * sb + n][i0]) *
+                                     *reinterpret_cast<const f32x4 *>(&L.inv1[buf][i0]);
+                    const f32x4 fr = *reinterpret_cast<const f32x4 *>(&L.R[buf][16 * tb + n][i0]) *
+                                     *reinterpret_cast<const f32x4 *>(&L.F1[buf][16 * tb + n][i0]) *
+                                     *reinterpret_cast<const f32x4 *>(&L.inv0[buf][i0]);
+                    at = mfma16(fk, fr, at);
+                }
+                if (tb == sb) {
+                    const int t = 16 * tb + n;
+                    const float diag = (L.ruk[buf][0][t] + L.ruk[buf][1][t]) + (L.ruk[buf][2][t] + L.ruk[buf][3][t]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) at[e] = (4 * g + e < n) ? at[e] : (4 * g + e == n ? diag : 0.f);
+                }
+                *reinterpret_cast<f32x4 *>(&L.A[16 * tb + n][16 * sb + 4 * g]) = at;
+            }
+            f32x4 gvt[2] = {zero, zero};
+#pragma unroll
+            for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+                for (int ib = 0; ib < 4; ++ib) {
+                    const f32x4 fk = *reinterpret_cast<const f32x4 *>(&L.K[buf][16 * sb + n][16 * ib + 4 * g]) *
+                                     *reinterpret_cast<const f32x4 *>(&L.F3[buf][16 * sb + n][16 * ib + 4 * g]);
+                    gvt[sb] = mfma16(fk, G[ib], gvt[sb]);
+                }
+            __syncthreads();
+            // ---- phase 2: gv += A^T gy, out ; G <- e^{c_32} o G + R'^T gy ----
+            f32x4 gyb[2];   // element e: token 16x + 4g + e, channel col
+#pragma unroll
+            for (int x = 0; x < 2; ++x)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) gyb[x][e] = L.GY[buf][16 * x + 4 * g + e][col];
+#pragma unroll
+            for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+                for (int tb = sb; tb < 2; ++tb) {
+                    f32x4 fat;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) fat[e] = L.A[16 * tb + 4 * g + e][16 * sb + n];
+                    gvt[sb] = mfma16(fat, gyb[tb], gvt[sb]);
+                }
+            {
+                Tout *const out = gv + base + (int64_t)c * kC32 * C;   // (uniform; the lane's part of the address is lane_off)
+                const int left = T - c * kC32 - 4 * g;                 // rows of the lane's four-row groups that exist
+#pragma unroll
+                for (int x = 0; x < 2; ++x)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (full || 16 * x + e < left) store1(out + (16 * x + e) * C + lane_off, gvt[x][e]);
+            }
+#pragma unroll
+            for (int ib = 0; ib < 4; ++ib) {
+                G[ib] *= *reinterpret_cast<const f32x4 *>(&L.e_all[buf][16 * ib + 4 * g]);
+#pragma unroll
+                for (int tb = 0; tb < 2; ++tb) {
+                    f32x4 fra;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) fra[e] = L.R[buf][16 * tb + 4 * g + e][16 * ib + n] * L.F1[buf][16 * tb + 4 * g + e][16 * ib + n];
+                    G[ib] = mfma16(fra, gyb[tb], G[ib]);
+                }
+            }
+            __syncthreads();
+        }
+    } else {
+        // ---------------- key waves ----------------
+        const int q = wave - 4, n = lane & 15, g = lane >> 4, col = 16 * q + n;
+        Tout *gr = reinterpret_cast<Tout *>(a.gr), *gk = reinterpret_cast<Tout *>(a.gk), *gw = reinterpret_cast<Tout *>(a.gw);
+        const f32x4 zero = (f32x4){0.f, 0.f, 0.f, 0.f};
+        const int lane_off = 4 * g * (int)C + col;
+        f32x4 Gt[4], St[4];   // Gt[jb][e] = G[col][16jb+4g+e] ; St likewise of S_0
+#pragma unroll
+        for (int i = 0; i < 4; ++i) Gt[i] = zero;
         float E = 0.f, gu_acc = 0.f;
         const float u_lane = load1(u + h * kN + col);
         // S_0^T from the forward's fragment order: S[i][j] sits in tile (j / 16, i / 16) at lane (j % 16) + 16 ((i % 16) / 4), element i % 4
@@ -186,75 +266,45 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_bwd_kernel(const 
         __syncthreads();
         for (int s = 0; s < nchunk; ++s) {
             const int c = nchunk - 1 - s, buf = s & 1;
-            // ---- phase 1 ----
-            {   // tiles of A and B: wave 0 (0,0) of both, wave 1 (1,1) of both, wave 2 A(1,0), wave 3 B(1,0)
+            const bool full = (c + 1) * kC32 <= T;
+            // ---- phase 1: a tile of B (wave 0: (0,0), 1: (1,1), 3: (1,0)), gy S_0^T, v G^T ----
+            if (q != 2) {
                 const int tb = q == 0 ? 0 : 1, sb = q == 1 ? 1 : 0;
-                if (q < 3) {
-                    f32x4 at = zero;
-#pragma unroll
-                    for (int ib = 0; ib < 4; ++ib) {
-                        const int i0 = 16 * ib + 4 * g;
-                        const f32x4 fk = *reinterpret_cast<const f32x4 *>(&L.K[buf][16 * sb + n][i0]) *
-                                         *reinterpret_cast<const f32x4 *>(&L.F3[buf][16 * sb + n][i0]) *
-                                         *reinterpret_cast<const f32x4 *>(&L.inv1[buf][i0]);
-                        const f32x4 fr = *reinterpret_cast<const f32x4 *>(&L.R[buf][16 * tb + n][i0]) *
-                                         *reinterpret_cast<const f32x4 *>(&L.F1[buf][16 * tb + n][i0]) *
-                                         *reinterpret_cast<const f32x4 *>(&L.inv0[buf][i0]);
-                        at = mfma16(fk, fr, at);
-                    }
-                    if (tb == sb) {
-                        const int t = 16 * tb + n;
-                        const float diag = (L.ruk[buf][0][t] + L.ruk[buf][1][t]) + (L.ruk[buf][2][t] + L.ruk[buf][3][t]);
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) at[e] = (4 * g + e < n) ? at[e] : (4 * g + e == n ? diag : 0.f);
-                    }
-                    *reinterpret_cast<f32x4 *>(&L.A[16 * tb + n][16 * sb + 4 * g]) = at;
-                }
-                if (q != 2) {
-                    f32x4 bt = zero;
-#pragma unroll
-                    for (int jb = 0; jb < 4; ++jb) {
-                        const f32x4 fv = *reinterpret_cast<const f32x4 *>(&L.V[buf][16 * sb + n][16 * jb + 4 * g]);
-                        const f32x4 fg = *reinterpret_cast<const f32x4 *>(&L.GY[buf][16 * tb + n][16 * jb + 4 * g]);
-                        bt = mfma16(fv, fg, bt);
-                    }
-                    if (tb == sb) {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            if (4 * g + e == n) L.vgy[16 * tb + n] = bt[e];
-                            bt[e] = (4 * g + e < n) ? bt[e] : 0.f;
-                        }
-                    }
-                    *reinterpret_cast<f32x4 *>(&L.Bm[16 * tb + n][16 * sb + 4 * g]) = bt;
-                }
-            }
-            f32x4 gvt[2] = {zero, zero}, Z[2] = {zero, zero}, W[2] = {zero, zero};
-#pragma unroll
-            for (int sb = 0; sb < 2; ++sb)
-#pragma unroll
-                for (int ib = 0; ib < 4; ++ib) {
-                    const f32x4 fk = *reinterpret_cast<const f32x4 *>(&L.K[buf][16 * sb + n][16 * ib + 4 * g]) *
-                                     *reinterpret_cast<const f32x4 *>(&L.F3[buf][16 * sb + n][16 * ib + 4 * g]);
-                    gvt[sb] = mfma16(fk, G[ib], gvt[sb]);
-                }
-#pragma unroll
-            for (int tb = 0; tb < 2; ++tb)
+                f32x4 bt = zero;
 #pragma unroll
                 for (int jb = 0; jb < 4; ++jb) {
+                    const f32x4 fv = *reinterpret_cast<const f32x4 *>(&L.V[buf][16 * sb + n][16 * jb + 4 * g]);
                     const f32x4 fg = *reinterpret_cast<const f32x4 *>(&L.GY[buf][16 * tb + n][16 * jb + 4 * g]);
-                    const f32x4 fv = *reinterpret_cast<const f32x4 *>(&L.V[buf][16 * tb + n][16 * jb + 4 * g]);
-                    Z[tb] = mfma16(fg, St[jb], Z[tb]);
-                    W[tb] = mfma16(fv, Gt[jb], W[tb]);
+                    bt = mfma16(fv, fg, bt);
+                }
+                if (tb == sb) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        if (4 * g + e == n) L.vgy[16 * tb + n] = bt[e];
+                        bt[e] = (4 * g + e < n) ? bt[e] : 0.f;
+                    }
+                }
+                *reinterpret_cast<f32x4 *>(&L.Bm[16 * tb + n][16 * sb + 4 * g]) = bt;
+            }
+            f32x4 Z[2] = {zero, zero}, W[2] = {zero, zero};
+#pragma unroll
+            for (int x = 0; x < 2; ++x)
+#pragma unroll
+                for (int jb = 0; jb < 4; ++jb) {
+                    const f32x4 fg = *reinterpret_cast<const f32x4 *>(&L.GY[buf][16 * x + n][16 * jb + 4 * g]);
+                    const f32x4 fv = *reinterpret_cast<const f32x4 *>(&L.V[buf][16 * x + n][16 * jb + 4 * g]);
+                    Z[x] = mfma16(fg, St[jb], Z[x]);
+                    W[x] = mfma16(fv, Gt[jb], W[x]);
                 }
             const float e_all = L.e_all[buf][col], e_mid = L.e_mid[buf][col], e_rest = L.e_rest[buf][col];
             const float inv0 = L.inv0[buf][col], inv1 = L.inv1[buf][col];
             // the products with B come scaled from the middle of the chunk: bring these to that scale, all back at the end
 #pragma unroll
             for (int x = 0; x < 2; ++x) { Z[x] *= e_mid; W[x] *= e_rest; }
+            if (c > 0) load_state(c - 1);
             __syncthreads();
             // ---- phase 2 ----
-            if (c > 0) load_state(c - 1);
-            f32x4 rc[2], kc[2], rp[2], kp[2], gyb[2];   // element e: token 16x + 4g + e, channel col
+            f32x4 rc[2], kc[2], rp[2], kp[2];   // element e: token 16x + 4g + e, channel col
 #pragma unroll
             for (int x = 0; x < 2; ++x)
 #pragma unroll
@@ -264,7 +314,6 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_bwd_kernel(const 
                     kc[x][e] = L.K[buf][t][col];
                     rp[x][e] = rc[x][e] * L.F1[buf][t][col];
                     kp[x][e] = kc[x][e] * L.F3[buf][t][col];
-                    gyb[x][e] = L.GY[buf][t][col];
                 }
 #pragma unroll
             for (int tb = 0; tb < 2; ++tb)
@@ -277,17 +326,27 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_bwd_kernel(const 
             for (int sb = 0; sb < 2; ++sb)
 #pragma unroll
                 for (int tb = sb; tb < 2; ++tb) {
-                    f32x4 fbt, fat;
+                    f32x4 fbt;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        fbt[e] = L.Bm[16 * tb + 4 * g + e][16 * sb + n];
-                        fat[e] = L.A[16 * tb + 4 * g + e][16 * sb + n];
-                    }
+                    for (int e = 0; e < 4; ++e) fbt[e] = L.Bm[16 * tb + 4 * g + e][16 * sb + n];
                     W[sb] = mfma16(fbt, rp[tb] * inv0, W[sb]);
-                    gvt[sb] = mfma16(fat, gyb[tb], gvt[sb]);
                 }
+            // G^T <- e^{c_32} o G^T + gy^T R' (before the outputs: they need no matrix unit)
+#pragma unroll
+            for (int jb = 0; jb < 4; ++jb) {
+                Gt[jb] *= e_all;
+#pragma unroll
+                for (int tb = 0; tb < 2; ++tb) {
+                    f32x4 fga;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) fga[e] = L.GY[buf][16 * tb + 4 * g + e][16 * jb + n];
+                    Gt[jb] = mfma16(fga, rp[tb], Gt[jb]);
+                }
+            }
             // gradients out
             float zt[2][4], kgk[2][4];
+            const int64_t out0 = base + (int64_t)c * kC32 * C;   // (uniform; the lane's part of the address is lane_off)
+            const int left = T - c * kC32 - 4 * g;               // rows of the lane's four-row groups that exist
 #pragma unroll
             for (int x = 0; x < 2; ++x) {
                 const f32x4 vg = *reinterpret_cast<const f32x4 *>(&L.vgy[16 * x + 4 * g]);
@@ -295,18 +354,16 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_bwd_kernel(const 
                 W[x] *= inv1;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const int tl = 16 * x + 4 * g + e, t = c * kC32 + tl;
+                    const int tl = 16 * x + 4 * g + e;
                     const float f1 = L.F1[buf][tl][col], f3 = L.F3[buf][tl][col];
                     const float o_r = fmaf(f1, Z[x][e], u_lane * kc[x][e] * vg[e]);
                     const float o_k = fmaf(f3, W[x][e], u_lane * rc[x][e] * vg[e]);
                     kgk[x][e] = kp[x][e] * W[x][e];
                     zt[x][e] = fmaf(rp[x][e], Z[x][e], -kgk[x][e]);
                     gu_acc = fmaf(rc[x][e] * kc[x][e], vg[e], gu_acc);
-                    if (t < T) {
-                        const int64_t o = base + (int64_t)t * C + col;
-                        store1(gr + o, o_r);
-                        store1(gk + o, o_k);
-                        store1(gv + o, gvt[x][e]);
+                    if (full || 16 * x + e < left) {
+                        store1(gr + out0 + (16 * x + e) * C + lane_off, o_r);
+                        store1(gk + out0 + (16 * x + e) * C + lane_off, o_k);
                     }
                 }
             }
@@ -326,36 +383,13 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_bwd_kernel(const 
                     float run = E + later[x];
 #pragma unroll
                     for (int e = 3; e >= 0; --e) {
-                        const int tl = 16 * x + 4 * g + e, t = c * kC32 + tl;
+                        const int tl = 16 * x + 4 * g + e;
                         const float o_w = (run - kgk[x][e]) * L.D[buf][tl][col];
-                        if (t < T) store1(gw + base + (int64_t)t * C + col, o_w);
+                        if (full || 16 * x + e < left) store1(gw + out0 + (16 * x + e) * C + lane_off, o_w);
                         run += zt[x][e];
                     }
                 }
                 E += all0 + all1;
-            }
-            // G <- e^{c_32} o G + R'^T gy, both copies
-#pragma unroll
-            for (int ib = 0; ib < 4; ++ib) {
-                G[ib] *= *reinterpret_cast<const f32x4 *>(&L.e_all[buf][16 * ib + 4 * g]);
-#pragma unroll
-                for (int tb = 0; tb < 2; ++tb) {
-                    f32x4 fra;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) fra[e] = L.R[buf][16 * tb + 4 * g + e][16 * ib + n] * L.F1[buf][16 * tb + 4 * g + e][16 * ib + n];
-                    G[ib] = mfma16(fra, gyb[tb], G[ib]);
-                }
-            }
-#pragma unroll
-            for (int jb = 0; jb < 4; ++jb) {
-                Gt[jb] *= e_all;
-#pragma unroll
-                for (int tb = 0; tb < 2; ++tb) {
-                    f32x4 fga;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) fga[e] = L.GY[buf][16 * tb + 4 * g + e][16 * jb + n];
-                    Gt[jb] = mfma16(fga, rp[tb], Gt[jb]);
-                }
             }
             __syncthreads();
         }
@@ -366,10 +400,7 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_bwd_kernel(const 
     __syncthreads();
     // a pair whose decay left the reach: once more, one timestep at a time (the pair's slice of the saved
     // states, T/32 x 64 x 64 floats, is large enough for the T x 64 workspace of that pass)
-    int wild_any = 0;
-#pragma unroll
-    for (int i = 0; i < 4 * kGroups; ++i) wild_any |= L.wild[i];
-    if (wild_any) {
+    if (L.wild[0] | L.wild[1] | L.wild[2] | L.wild[3]) {
         __syncthreads();
         scan_bwd_a_body<Tin, Tout>(reinterpret_cast<C32BwdSmem *>(c32_smem)->scan_a, b, h, T, H, r, k, v, w, u, gy,
                                    reinterpret_cast<Tout *>(a.gr), reinterpret_cast<Tout *>(a.gu), ck, kN);
@@ -382,11 +413,10 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_bwd_kernel(const 
 
 template <typename Tin, typename Tout>
 static hipError_t launch(hipStream_t st, int64_t B, const C32BwdArgs &a) {
-    constexpr int kGroups = C32_GROUPS;
     constexpr int lds = (int)sizeof(C32BwdSmem);
-    const hipError_t e = allow_dynamic_lds<chunk32_bwd_kernel<Tin, Tout, kGroups>>(lds);
+    const hipError_t e = allow_dynamic_lds<chunk32_bwd_kernel<Tin, Tout>>(lds);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((chunk32_bwd_kernel<Tin, Tout, kGroups>), dim3((unsigned)(B * a.H)), dim3(256 + 256 * kGroups), lds, st, a);
+    hipLaunchKernelGGL((chunk32_bwd_kernel<Tin, Tout>), dim3((unsigned)(B * a.H)), dim3(768), lds, st, a);
     return hipGetLastError();
 }
 

@@ -47,7 +47,8 @@ struct C32FwdArgs {
     float *saved;   // [pair][chunk][4096] chunk-start states in fragment order (null: not kept)
 };
 
-template <typename Tin, typename Tout, typename Ts, int kGroups>
+// kOut = false: only the states (chunk states and / or the final one): no y, no R-side operands
+template <typename Tin, typename Tout, typename Ts, int kGroups, bool kOut>
 __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_fwd_kernel(const C32FwdArgs a)
 {
     extern __shared__ __align__(16) unsigned char c32_smem[];
@@ -70,11 +71,11 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_fwd_kernel(const 
         load4(u + h * kN + ch, fu);
         float nr[2][4], nk[2][4], nv[2][4], nw[2][4];   // the group's next chunk on its way in
         auto fetch = [&](int c) {
+            const int64_t row0 = base + (int64_t)c * kC32 * C;   // (uniform)
 #pragma unroll
             for (int x = 0; x < 2; ++x) {
-                const int t = min(c * kC32 + 16 * x + t16, T - 1);
-                const int64_t o = base + (int64_t)t * C + ch;
-                load4(r + o, nr[x]); load4(k + o, nk[x]); load4(v + o, nv[x]); load4(w + o, nw[x]);
+                const int o = min(16 * x + t16, T - 1 - c * kC32) * (int)C + ch;   // rows past the end read the last one
+                load4(r + row0 + o, nr[x]); load4(k + row0 + o, nk[x]); load4(v + row0 + o, nv[x]); load4(w + row0 + o, nw[x]);
             }
         };
         // the chunk whose operands are formed: two channels of the lane's four at a time (a barrier in between)
@@ -94,15 +95,17 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_fwd_kernel(const 
 #pragma unroll
                 for (int e = E0; e < E0 + 2; ++e) {
                     const float fr = valid[x] ? nr[x][e] : 0.f, fk = valid[x] ? nk[x][e] : 0.f;
-                    op_r[x][e] = fr * sc.rp[x][e];
                     op_k[x][e] = fk * sc.kp[x][e];
-                    hm_r[x][e] = fr * sc.rm[x][e];
-                    hm_k[x][e] = fk * sc.km[x][e];
+                    if (kOut) {
+                        op_r[x][e] = fr * sc.rp[x][e];
+                        hm_r[x][e] = fr * sc.rm[x][e];
+                        hm_k[x][e] = fk * sc.km[x][e];
+                    }
                     op_v[x][e] = valid[x] ? nv[x][e] : 0.f;
                     e_all[e] = sc.all[e];
                     s = fmaf(fr * fk, fu[e], s);
                 }
-                part[x] = E0 == 0 ? s : sum_rows4(s);
+                if (kOut) part[x] = E0 == 0 ? s : sum_rows4(s);
             }
         };
         const std::integral_constant<int, 0> h0;
@@ -112,13 +115,14 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_fwd_kernel(const 
 #pragma unroll
             for (int x = 0; x < 2; ++x) {
                 const int t = 16 * x + t16;
-                *reinterpret_cast<f32x4 *>(&L.Rp[buf][t][ch]) = (f32x4){op_r[x][0], op_r[x][1], op_r[x][2], op_r[x][3]};
+                if (kOut) *reinterpret_cast<f32x4 *>(&L.Rp[buf][t][ch]) = (f32x4){op_r[x][0], op_r[x][1], op_r[x][2], op_r[x][3]};
                 *reinterpret_cast<f32x4 *>(&L.Kp[buf][t][ch]) = (f32x4){op_k[x][0], op_k[x][1], op_k[x][2], op_k[x][3]};
                 *reinterpret_cast<f32x4 *>(&L.V[buf][t][ch]) = (f32x4){op_v[x][0], op_v[x][1], op_v[x][2], op_v[x][3]};
             }
             if (t16 == 0) *reinterpret_cast<f32x4 *>(&L.e_all[buf][ch]) = (f32x4){e_all[0], e_all[1], e_all[2], e_all[3]};
         };
         auto finish = [&]() {
+            if (!kOut) return;
 #pragma unroll
             for (int x = 0; x < 2; ++x) {
                 const int t = 16 * x + t16;
@@ -185,7 +189,7 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_fwd_kernel(const 
         __syncthreads();
         for (int c = 0; c < nchunk; ++c) {
             const int buf = c & 1;
-            if (c > 0 && y) store_y(c - 1);
+            if (kOut && c > 0 && y) store_y(c - 1);
             if (saved) {
 #pragma unroll
                 for (int ib = 0; ib < 4; ++ib) *reinterpret_cast<f32x4 *>(saved + (int64_t)c * (kN * kN) + ib * 256) = S[ib];
@@ -193,13 +197,13 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_fwd_kernel(const 
             // phase 1: y = R' S, one tile of A
             f32x4 yt[2] = {(f32x4){0.f, 0.f, 0.f, 0.f}, (f32x4){0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-            for (int tb = 0; tb < 2; ++tb)
+            for (int tb = 0; kOut && tb < 2; ++tb)
 #pragma unroll
                 for (int ib = 0; ib < 4; ++ib) {
                     const f32x4 fr = *reinterpret_cast<const f32x4 *>(&L.Rp[buf][16 * tb + n][16 * ib + 4 * g]);
                     yt[tb] = mfma16(fr, S[ib], yt[tb]);
                 }
-            if (q < 3) {
+            if (kOut && q < 3) {
                 // tile (tb, sb) of A, computed transposed: lane (n, g) ends with A[16 tb + n][16 sb + 4g + v]
                 const int tb = q == 0 ? 0 : 1, sb = q == 1 ? 1 : 0;
                 f32x4 at = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -225,14 +229,14 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_fwd_kernel(const 
 #pragma unroll
                 for (int e = 0; e < 4; ++e) fv[sb][e] = L.V[buf][16 * sb + 4 * g + e][16 * q + n];
 #pragma unroll
-            for (int tb = 0; tb < 2; ++tb)
+            for (int tb = 0; kOut && tb < 2; ++tb)
 #pragma unroll
                 for (int sb = 0; sb <= tb; ++sb) {
                     const f32x4 fa = *reinterpret_cast<const f32x4 *>(&L.A[16 * tb + n][16 * sb + 4 * g]);
                     yt[tb] = mfma16(fa, fv[sb], yt[tb]);
                 }
 #pragma unroll
-            for (int tb = 0; tb < 2; ++tb)
+            for (int tb = 0; kOut && tb < 2; ++tb)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) L.Y[16 * tb + 4 * g + e][16 * q + n] = yt[tb][e];
 #pragma unroll
@@ -249,7 +253,7 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_fwd_kernel(const 
             }
             __syncthreads();
         }
-        if (y) store_y(nchunk - 1);
+        if (kOut && y) store_y(nchunk - 1);
         if (a.sT) {
             StateT *p0 = reinterpret_cast<StateT *>(a.sT) + (int64_t)pair * (kN * kN) + 16 * q + n;
 #pragma unroll
@@ -263,7 +267,7 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_fwd_kernel(const 
     int wild_any = 0;
 #pragma unroll
     for (int i = 0; i < 4 * kGroups; ++i) wild_any |= L.wild[i];
-    if (wild_any) {
+    if (wild_any && (kOut || a.sT)) {   // (its chunk states are not used: the backward takes the same way out)
         __syncthreads();
         scan_fwd_body<Tin, Tout, Ts, 8>(reinterpret_cast<C32FwdSmem *>(c32_smem)->scan, b, h, T, H, r, k, v, w, u,
                                         reinterpret_cast<const Ts *>(a.s0), a.map, y, reinterpret_cast<Ts *>(a.sT));
@@ -277,13 +281,13 @@ size_t chunk32_saved_bytes(int64_t B, int64_t T, int64_t H) {
     return (size_t)(B * H) * (size_t)((T + kC32 - 1) / kC32) * (kN * kN) * sizeof(float);
 }
 
-template <typename Tin, typename Tout, typename Ts>
+template <typename Tin, typename Tout, typename Ts, bool kOut>
 static hipError_t launch(hipStream_t st, int64_t B, const C32FwdArgs &a) {
     constexpr int lds = (int)sizeof(C32FwdSmem);
     constexpr int kGroups = C32_GROUPS;
-    const hipError_t e = allow_dynamic_lds<chunk32_fwd_kernel<Tin, Tout, Ts, kGroups>>(lds);
+    const hipError_t e = allow_dynamic_lds<chunk32_fwd_kernel<Tin, Tout, Ts, kGroups, kOut>>(lds);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL((chunk32_fwd_kernel<Tin, Tout, Ts, kGroups>), dim3((unsigned)(B * a.H)), dim3(256 + 256 * kGroups), lds, st, a);
+    hipLaunchKernelGGL((chunk32_fwd_kernel<Tin, Tout, Ts, kGroups, kOut>), dim3((unsigned)(B * a.H)), dim3(256 + 256 * kGroups), lds, st, a);
     return hipGetLastError();
 }
 
@@ -296,8 +300,9 @@ hipError_t chunk32_forward(hipStream_t st, int dtype, int state_dtype, int64_t B
     a.T = (int)T; a.H = (int)H;
     a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.s0 = s0; a.map = map; a.y = y; a.sT = sT;
     a.saved = reinterpret_cast<float *>(saved_states);
-    if (dtype == kF32) return launch<float, float, float>(st, B, a);
-    return launch<f16_t, float, float>(st, B, a);
+    if (y == nullptr)
+        return dtype == kF32 ? launch<float, float, float, false>(st, B, a) : launch<f16_t, float, float, false>(st, B, a);
+    return dtype == kF32 ? launch<float, float, float, true>(st, B, a) : launch<f16_t, float, float, true>(st, B, a);
 }
 
 }  // namespace wkv6
