@@ -1,0 +1,217 @@
+"""GPU parity tests of the full-precision chunk form (fp32 and fp16 tensors on the fp32 matrix instructions,
+what WKV6_ALGO_AUTO runs for them from T = 64 on): called through the operator class and the C ABI, against
+the float64 CPU oracle on the same seeded (and identically rounded) inputs, at the fp32 tolerances:
+max|y - y_ref| <= 1e-4 (scaled by max|y_ref| / 64 above 64), gradients max|g - g_ref| / max|g_ref| <= 1e-3."""
+import numpy as np
+import pytest
+import torch
+
+from _util import cast_inputs, check_close, to_np
+
+pytestmark = pytest.mark.gpu
+
+AUTO, SCAN, CHUNK = 0, 1, 2
+N = 64
+DTYPES = {"f32": torch.float32, "f16": torch.float16}
+
+
+@pytest.fixture(scope="module")
+def op():
+    assert torch.cuda.is_available(), "these tests need the GPU"
+    import rwkv_kernel
+
+    return rwkv_kernel.RWKVKernelOperator(64, 1 << 16)
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from rwkv_kernel import _native
+
+    return _native.load()
+
+
+def _fwd_bwd(op, dev, gy, algo):
+    op.algo = algo
+    leaves = [x.clone().requires_grad_(True) for x in dev]
+    y, none = op(*leaves)
+    assert none is None
+    y.backward(gy)
+    torch.cuda.synchronize()
+    return y, [x.grad for x in leaves]
+
+
+def _check_grads(grads, g_ref, dtype, what=""):
+    # fp16 gradients come back rounded to fp16 by the operator class: held to the 16-bit bound then
+    tol = torch.float32 if dtype == torch.float32 else torch.float16
+    for name, g, gr in zip("gr gk gv gw gu".split(), grads, g_ref):
+        check_close(what + name, to_np(g).reshape(gr.shape), gr, tol, is_grad=True)
+
+
+def _case(op, oracle, B, T, H, seed, dtype, edit=None, strict=False):
+    print("case B=%d T=%d H=%d seed=%d dtype=%s" % (B, T, H, seed, dtype), flush=True)
+    ins = oracle.make_inputs(B, T, H, N, seed)
+    if edit:
+        edit(ins)
+    dev, ref = cast_inputs(ins[:5], dtype)
+    gyd, gyr = cast_inputs(ins[5:6], torch.float32)
+    y, grads = _fwd_bwd(op, dev, gyd[0], AUTO)
+    assert y.dtype == torch.float32 and all(g.dtype == dtype for g in grads)
+    y_ref, _ = oracle.forward_c(*ref, N)
+    if strict:
+        assert np.abs(to_np(y) - y_ref).max() <= 1e-4
+    check_close("y", y, y_ref, torch.float32)
+    _check_grads(grads, oracle.backward_c(*ref, gyr[0], N), dtype)
+    return y, grads
+
+
+def test_selected_from_64_tokens_on(lib):
+    from rwkv_kernel import _native
+
+    per_pair_chunk = 64 * 64 * 4
+    for dt in (_native.F32, _native.F16):
+        assert lib.wkv6_saved_bytes(dt, _native.ALGO_AUTO, 2, 64, 128, 2) == 2 * 2 * 2 * per_pair_chunk
+        assert lib.wkv6_saved_bytes(dt, _native.ALGO_AUTO, 2, 100, 128, 2) == 2 * 2 * 4 * per_pair_chunk   # the last chunk is short
+        assert lib.wkv6_saved_bytes(dt, _native.ALGO_AUTO, 2, 63, 128, 2) == 0      # short sequences: per-timestep kernels
+        assert lib.wkv6_saved_bytes(dt, _native.ALGO_SCAN, 2, 256, 128, 2) == 0
+    assert lib.wkv6_saved_bytes(_native.F32, _native.ALGO_CHUNK, 2, 256, 128, 2) == 2 * 2 * 8 * per_pair_chunk
+    # the workspace of a backward without saved states holds the same chunk states (or the per-timestep pass's rows)
+    assert lib.wkv6_backward_workspace_bytes_ex(_native.F32, _native.ALGO_AUTO, 2, 256, 128, 2) == 2 * 2 * 8 * per_pair_chunk
+    assert lib.wkv6_backward_workspace_bytes_ex(_native.F32, _native.ALGO_SCAN, 2, 256, 128, 2) == 2 * 256 * 128 * 4
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_config1_forward_backward_fp32_strict(op, oracle, seed):
+    # the fp32 correctness shape: B=2 T=128 H=4 N=64; max-abs(y) <= 1e-4
+    _case(op, oracle, 2, 128, 4, seed, torch.float32, strict=True)
+
+
+@pytest.mark.parametrize("dt", ["f32", "f16"])
+@pytest.mark.parametrize("B,T,H", [(1, 64, 1), (2, 65, 2), (2, 95, 3), (2, 100, 2), (1, 333, 3), (3, 1024, 2), (1, 2080, 1)])
+def test_shapes_and_ragged_ends(op, oracle, dt, B, T, H):
+    _case(op, oracle, B, T, H, 100 + T, DTYPES[dt])
+
+
+def test_more_pairs_than_compute_units(op, oracle):
+    _case(op, oracle, 40, 96, 8, 7, torch.float32)
+
+
+@pytest.mark.parametrize("dt", ["f32", "f16"])
+def test_state_in_and_out(op, oracle, dt):
+    B, T, H = 5, 170, 3
+    ins = oracle.make_inputs(B, T, H, N, 21, with_state=True)
+    dev, ref = cast_inputs(ins[:5], DTYPES[dt])
+    s_dev, s_ref = cast_inputs([ins[6][:3]], torch.float32)
+    smap = [2, 0, 1, 1, 2]
+    op.algo = AUTO
+    with torch.no_grad():
+        y, sT = op(*dev, return_state=True, init_state=s_dev[0], state_map=smap)
+        y0, sT0 = op(*dev, return_state=True)
+    torch.cuda.synchronize()
+    y_ref, sT_ref = oracle.forward_c(*ref, N, s_ref[0], smap)
+    check_close("y", y, y_ref, torch.float32)
+    check_close("sT", sT, sT_ref, torch.float32, is_grad=True)
+    y_ref0, sT_ref0 = oracle.forward_c(*ref, N)
+    check_close("y from zero", y0, y_ref0, torch.float32)
+    check_close("sT from zero", sT0, sT_ref0, torch.float32, is_grad=True)
+
+
+def test_decay_outside_the_reach_is_redone_exactly(op, oracle):
+    # one pair decays by e^-4.5 per token over 40 tokens (a half-chunk sum of 72 > 40), another carries the
+    # model's padding values (w = -1e9: decay exactly 1, with k = 0) and a decay of exactly 0 (w = 20): those
+    # pairs take the per-timestep pass inside the same launches, the others stay on the chunk form
+    def edit(ins):
+        ins[3][0, 40:80, :64] = 1.5
+        ins[3][1, 10:30, 64:128] = -1e9
+        ins[1][1, 10:30, 64:128] = 0
+        ins[3][1, 50, 64:128] = 20.0
+
+    y, grads = _case(op, oracle, 2, 256, 3, 9, torch.float32, edit=edit)
+    assert all(torch.isfinite(t).all() for t in [y] + grads)
+
+
+def test_small_decay_sums_and_constant_inputs(op):
+    # reference test_jax.py:12-16: r=k=v=u=1, w=-4 -> y_t = 64*(1 + (1-d^t)/(1-d)), d = exp(-exp(-4))
+    B, T, C = 2, 512, 256
+    one = torch.ones(B, T, C, device="cuda")
+    op.algo = AUTO
+    with torch.no_grad():
+        y, _ = op(one, one, one, one * 0 - 4, torch.ones(C, device="cuda"))
+    d = np.exp(-np.exp(-4.0))
+    expect = 64 * (1 + (1 - d ** np.arange(T)) / (1 - d))
+    got = to_np(y)
+    assert got[0, 0, 0] == 64.0
+    np.testing.assert_allclose(got[1, :, 77], expect, rtol=2e-5)
+
+
+@pytest.mark.parametrize("dt", ["f32", "f16"])
+def test_saved_and_recomputed_states_give_the_same_gradients(lib, oracle, dt):
+    # wkv6_forward / wkv6_backward (the reference-shaped pair: a forward pass that only leaves the chunk states
+    # comes first) against wkv6_forward_save / wkv6_backward_saved_sum: the same kernels on the same states,
+    # bit for bit; y does not depend on whether the states are kept
+    from rwkv_kernel import _native
+
+    B, T, H = 3, 200, 2
+    C = H * N
+    code = _native.F32 if dt == "f32" else _native.F16
+    ins = oracle.make_inputs(B, T, H, N, 33)
+    dev, ref = cast_inputs(ins[:5], DTYPES[dt])
+    gyd, gyr = cast_inputs(ins[5:6], torch.float32)
+    r, k, v, w, u = dev
+    gy = gyd[0]
+    st = torch.cuda.current_stream().cuda_stream
+    P = lambda t: t.data_ptr()
+    n = lib.wkv6_saved_bytes(code, AUTO, B, T, C, H)
+    assert n == lib.wkv6_backward_workspace_bytes_ex(code, AUTO, B, T, C, H) > 0
+    res = []
+    for mode in ("plain", "saved"):
+        y = torch.empty(B, T, C, dtype=torch.float32, device="cuda")
+        outs = [torch.empty(B, T, C, dtype=torch.float32, device="cuda") for _ in range(4)]
+        gu = torch.empty(B, C, dtype=torch.float32, device="cuda")
+        gus = torch.zeros(C, dtype=torch.float32, device="cuda")
+        buf = torch.empty(n, dtype=torch.uint8, device="cuda")
+        if mode == "plain":
+            _native.check(lib.wkv6_forward(st, code, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(y)))
+            _native.check(lib.wkv6_backward(st, code, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy),
+                                            *[P(o) for o in outs], P(gu), P(buf), n))
+        else:
+            _native.check(lib.wkv6_forward_save(st, code, AUTO, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(y), P(buf), n))
+            _native.check(lib.wkv6_backward_saved_sum(st, code, AUTO, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy),
+                                                      *[P(o) for o in outs], P(gu), P(gus), P(buf), n))
+        torch.cuda.synchronize()
+        res.append([y] + outs + [gu, gus])
+    for a, b in zip(res[0][:6], res[1][:6]):
+        assert torch.equal(a, b)
+    g_ref = oracle.backward_c(*ref, gyr[0], N)
+    check_close("y", res[1][0], oracle.forward_c(*ref, N)[0], torch.float32)
+    for name, g, gr in zip("gr gk gv gw".split(), res[1][1:5], g_ref):
+        check_close(name, g, gr, torch.float32, is_grad=True)
+    check_close("gu summed", to_np(res[1][6]).reshape(H, N), g_ref[4], torch.float32, is_grad=True)
+    check_close("gu rows", to_np(res[1][5]).sum(0).reshape(H, N), g_ref[4], torch.float32, is_grad=True)
+
+
+def test_fp16_inference_on_request_too(op, oracle):
+    # a forward of fp16 tensors asked for as WKV6_ALGO_CHUNK has no bf16-operand form: it runs at full precision
+    ins = oracle.make_inputs(2, 256, 2, N, 5)
+    dev, ref = cast_inputs(ins[:5], torch.float16)
+    outs = []
+    for algo in (AUTO, CHUNK, SCAN):
+        op.algo = algo
+        with torch.no_grad():
+            outs.append(op(*dev)[0])
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1])
+    y_ref, _ = oracle.forward_c(*ref, N)
+    for y in outs:
+        check_close("y", y, y_ref, torch.float32)
+
+
+def test_c2_shape_fp32_vs_oracle(op, oracle):
+    # B=8 T=1024 C=2048 H=32 with fp32 tensors: every output against the float64 oracle
+    B, T, H = 8, 1024, 32
+    print("C2 shape, fp32", flush=True)
+    ins = oracle.make_inputs(B, T, H, N, 0)
+    dev, ref = cast_inputs(ins[:5], torch.float32)
+    gyd, gyr = cast_inputs(ins[5:6], torch.float32)
+    y, grads = _fwd_bwd(op, dev, gyd[0], AUTO)
+    check_close("y", y, oracle.forward_c(*ref, N)[0], torch.float32)
+    _check_grads(grads, oracle.backward_c(*ref, gyr[0], N), torch.float32)
