@@ -27,7 +27,8 @@ WORKLOADS = {
     "c2": (8, 1024, 32, "bf16"),   # RWKV6-1.6B layer shape: the configuration the metric is quoted on
     "c3": (4, 4096, 64, "bf16"),   # RWKV6-7B layer shape
     "c1": (2, 128, 4, "f32"),
-    "c2_f16": (8, 1024, 32, "f16"),   # the c2 shape with fp16 tensors: y, gy and the gradients are fp32 (chunked pair: --algo chunk)
+    "c2_f32": (8, 1024, 32, "f32"),   # the c2 shape with fp32 tensors (the full-precision chunk form; --algo scan: per-timestep kernels)
+    "c2_f16": (8, 1024, 32, "f16"),   # ... with fp16 tensors: y, gy and the gradients are fp32 (--algo chunk: the bf16-operand pair)
     "long1": (1, 8192, 32, "bf16"),   # one long sequence per GPU (fine-tuning): 32 pairs, runs as time segments
     "short": (128, 256, 32, "bf16"),  # many short sequences: 4096 pairs, every workgroup takes 16 of them back to back
 }
