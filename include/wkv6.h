@@ -44,22 +44,27 @@ enum {
 
 /* Algorithm selector for the *_ex entry points. */
 enum {
-    WKV6_ALGO_AUTO = 0,  /* library picks: chunked MFMA path for bf16 tensors with T >= 32, else scan.
-                            fp16 and fp32 tensors always take the scan: their results are fp32-exact
-                            (1e-4 class), the same with and without a gradient                   */
+    WKV6_ALGO_AUTO = 0,  /* library picks.  bf16 tensors with T >= 32: chunked bf16-MFMA path.  fp32 and
+                            fp16 tensors with T >= 64: the full-precision chunk form (every product on
+                            the fp32 matrix instructions, chunks of 32 tokens, fp32 accuracy: y within
+                            1e-4, gradients within 1e-3 relative, the same y with and without a
+                            gradient; its training pair saves one fp32 state per chunk).  Everything
+                            else, and every call that takes gradients through the state of fp32 /
+                            fp16 tensors: the per-timestep kernels                              */
     WKV6_ALGO_SCAN = 1,  /* per-timestep fp32 recurrence, state in VGPRs                       */
-    WKV6_ALGO_CHUNK = 2  /* chunk-parallel form, bf16 MFMA for the dense intra-chunk products: bf16
-                            tensors in every call; fp16 tensors (fp32 outputs) in the training pair
-                            wkv6_forward_save / wkv6_backward_saved* only, where r, k, w are
-                            unpacked exactly and v, gy reach the MFMAs as bf16 copies kept in the
-                            saved block.  ACCURACY: for fp16 tensors this is an explicit trade --
+    WKV6_ALGO_CHUNK = 2  /* chunk-parallel form.  bf16 tensors: bf16 MFMA for the dense intra-chunk
+                            products in every call.  fp32 tensors: the full-precision chunk form, as
+                            under AUTO.  fp16 tensors (fp32 outputs): the training pair
+                            wkv6_forward_save / wkv6_backward_saved* runs on the bf16-MFMA kernels
+                            (r, k, w unpacked exactly; v, gy reach the MFMAs as bf16 copies kept in
+                            the saved block); calls without a gradient run the full-precision chunk
+                            form.  ACCURACY: for the fp16 training pair this is an explicit trade --
                             the fp32-typed y and gradients then carry bf16 operand precision
-                            (relative error up to 1e-2, against 1e-4 of the scan), and differ by
-                            that much from what wkv6_forward returns for the same inputs (calls
-                            without a gradient always take the scan for fp16).  A workgroup whose
-                            (batch, head) pair has a 16-token tile with decay beyond what the
-                            operand scaling can hold redoes that pair with the exact per-timestep
-                            code inside the same launch                                        */
+                            (relative error up to 1e-2, against 1e-4 under AUTO), and differ by
+                            that much from what wkv6_forward returns for the same inputs.  In
+                            either chunk form a (batch, head) pair whose decay goes beyond what the
+                            operand scaling can hold is redone with the exact per-timestep code
+                            inside the same launch                                             */
 };
 
 const char *wkv6_status_string(int status);
@@ -210,8 +215,10 @@ size_t wkv6_backward_workspace_bytes(int dtype, int64_t B, int64_t T, int64_t C,
  * point of the call -- code under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc -- and neither the library nor anything it calls allocates or frees memory here (the
  * first call on a device looks the array's address up once).  Shapes whose
- * wkv6_backward_workspace_bytes() exceeds WKV6_STATIC_SCRATCH_BYTES are refused with
- * WKV6_ERR_WORKSPACE (the benchmark shape B=8 T=1024 C=2048 needs exactly that much).  All calls
+ * wkv6_backward_workspace_bytes() exceeds WKV6_STATIC_SCRATCH_BYTES run on the per-timestep kernels
+ * if their workspace (4 bytes per element of r) fits, and are refused with WKV6_ERR_WORKSPACE
+ * otherwise (the benchmark shape B=8 T=1024 C=2048 needs exactly the array's size, as bf16 on the
+ * chunked kernels and as fp32 on the per-timestep ones).  All calls
  * on one GPU share the one array: two calls whose kernels overlap in time on the same GPU
  * (different streams, different host threads) race -- serialise them.  Same results as
  * wkv6_backward. */
@@ -232,8 +239,9 @@ int wkv6_backward_ex(void *stream, int dtype, int algo, int64_t B, int64_t T, in
                      void *workspace, size_t workspace_bytes);
 size_t wkv6_backward_workspace_bytes_ex(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H);
 
-/* Training pair: a forward that also saves what the backward can reuse (with the chunked kernels:
- * the state at every 64-token chunk start, as bf16), and the backward that consumes it and therefore
+/* Training pair: a forward that also saves what the backward can reuse (bf16 tensors on the chunked
+ * kernels: the state at every 64-token chunk start, as bf16; fp32 and fp16 tensors on the full-precision
+ * chunk form: the fp32 state at every 32-token chunk start), and the backward that consumes it and therefore
  * skips its own forward state sweep.  `saved` is caller-owned device memory of wkv6_saved_bytes()
  * bytes (0 = this path saves nothing; pass NULL), must be left untouched between the two calls,
  * and serves the backward as its workspace too.  A long sequence (T >= 1024) of so few (batch, head)

@@ -558,13 +558,18 @@ int wkv6_backward_static(void *stream, int dtype, int64_t B, int64_t T, int64_t 
                          void *gr, void *gk, void *gv, void *gw, void *gu) {
     const int rc = check_shape(dtype, B, T, C, H);
     if (rc != WKV6_OK) return rc;
-    const size_t need = wkv6_backward_workspace_bytes(dtype, B, T, C, H);
+    int algo = WKV6_ALGO_AUTO;
+    size_t need = wkv6_backward_workspace_bytes(dtype, B, T, C, H);
+    if (need > WKV6_STATIC_SCRATCH_BYTES) {   // the per-timestep kernels keep less
+        algo = WKV6_ALGO_SCAN;
+        need = wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H);
+    }
     if (need > WKV6_STATIC_SCRATCH_BYTES) return WKV6_ERR_WORKSPACE;   // larger than the library's own array
     hipError_t e = hipSuccess;
     void *ws = static_scratch(&e);
     if (ws == nullptr) return finish(e);
     // (the workspace needs no initial contents; what the last call left in it is overwritten)
-    return wkv6_backward(stream, dtype, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, ws, WKV6_STATIC_SCRATCH_BYTES);
+    return wkv6_backward_ex(stream, dtype, algo, B, T, C, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, ws, WKV6_STATIC_SCRATCH_BYTES);
 }
 
 // ---- XLA custom-call surface ------------------------------------------------------------

@@ -67,11 +67,13 @@ def test_argument_validation_returns_status_codes(native):
     assert lib.wkv6_forward(None, native.BF16, 2, 16, 64, 2, *args) == 2                   # head size 32
     assert lib.wkv6_forward(None, native.BF16, 0, 16, 128, 2, *args) == 1                  # empty batch
     assert lib.wkv6_forward(None, native.BF16, 2, 16, 128, 2, fake + 2, *args[1:]) == 1    # misaligned
-    assert lib.wkv6_forward_ex(None, native.F32, native.ALGO_CHUNK, 2, 64, 128, 2, *args, None, 0) == 2
+    assert lib.wkv6_forward_ex(None, native.F32, native.ALGO_CHUNK, 2, 63, 128, 2, *args, None, 0) == 2   # no chunk form below 64 tokens
     assert lib.wkv6_forward_ex(None, native.BF16, 3, 2, 64, 128, 2, *args, None, 0) == 1   # unknown algo
     need = lib.wkv6_backward_workspace_bytes(native.BF16, 8, 1024, 2048, 32)
     assert need == 8 * 1024 * 2048 * 4
     assert lib.wkv6_backward_workspace_bytes_ex(native.F32, native.ALGO_SCAN, 2, 100, 128, 2) == 2 * 100 * 128 * 4
+    assert lib.wkv6_backward_workspace_bytes_ex(native.F32, native.ALGO_AUTO, 2, 100, 128, 2) == 2 * 2 * 4 * 64 * 64 * 4   # fp32 chunk states
+    assert lib.wkv6_backward_workspace_bytes_ex(native.F16, native.ALGO_AUTO, 2, 40, 128, 2) == 2 * 40 * 128 * 4
     assert lib.wkv6_backward_workspace_bytes_ex(native.BF16, native.ALGO_CHUNK, 2, 100, 128, 2) == 2 * 128 * 128 * 4
     assert lib.wkv6_backward_workspace_bytes(native.BF16, 2, 16, 130, 2) == 0
     gargs = [fake] * 11

@@ -49,8 +49,9 @@ def test_static_scratch_backward_equals_workspace_backward():
 
     lib = _native.load()
     torch.cuda.set_device(0)
-    # first the largest shape the array holds (the benchmark's), then smaller ones on both kernel families
-    for B, T, H, dtype, seed in ((8, 1024, 32, torch.bfloat16, 0), (3, 200, 2, torch.bfloat16, 1), (2, 77, 3, torch.float32, 2)):
+    # first the largest shape the array holds (the benchmark's), then smaller ones on every kernel family
+    for B, T, H, dtype, seed in ((8, 1024, 32, torch.bfloat16, 0), (3, 200, 2, torch.bfloat16, 1), (2, 200, 3, torch.float32, 3),
+                                 (2, 77, 3, torch.float32, 2)):   # (fp32: the full-precision chunk form, then the per-timestep kernels)
         print("static scratch backward B%d T%d H%d %s" % (B, T, H, dtype), flush=True)
         assert lib.wkv6_backward_workspace_bytes(
             _native.BF16 if dtype == torch.bfloat16 else _native.F32, B, T, H * 64, H) <= _native.STATIC_SCRATCH_BYTES
@@ -58,6 +59,35 @@ def test_static_scratch_backward_equals_workspace_backward():
         for name, a, b in zip("gr gk gv gw gu".split(), got, want):
             assert bool(torch.isfinite(a.float()).all()), name
             assert torch.equal(a, b), "%s differs (max %g)" % (name, float((a.float() - b.float()).abs().max()))
+
+
+def test_static_scratch_backward_takes_the_smaller_workspace_when_only_that_fits():
+    # fp32 tensors at the benchmark's shape: the chunk states of the full-precision chunk form (128 MiB) do not
+    # fit the array, the rows of the per-timestep kernels (64 MiB) do: the call runs those, bit for bit
+    from rwkv_kernel import _native
+
+    lib = _native.load()
+    torch.cuda.set_device(0)
+    B, T, H = 8, 1024, 32
+    C = H * 64
+    assert lib.wkv6_backward_workspace_bytes(_native.F32, B, T, C, H) > _native.STATIC_SCRATCH_BYTES
+    n = lib.wkv6_backward_workspace_bytes_ex(_native.F32, _native.ALGO_SCAN, B, T, C, H)
+    assert n <= _native.STATIC_SCRATCH_BYTES
+    g = torch.Generator().manual_seed(5)
+    r, k, v, gy = (torch.randn(B, T, C, generator=g).cuda() for _ in range(4))
+    w = (torch.rand(B, T, C, generator=g) * 7.0 - 6.0).cuda()
+    u = (torch.randn(H, 64, generator=g) * 0.5).cuda()
+    st = torch.cuda.current_stream().cuda_stream
+    P = lambda t: t.data_ptr()
+    outs = lambda: [torch.empty(B, T, C, device="cuda") for _ in range(4)] + [torch.empty(B, C, device="cuda")]
+    want, got = outs(), outs()
+    ws = torch.empty(n, dtype=torch.uint8, device="cuda")
+    _native.check(lib.wkv6_backward_ex(st, _native.F32, _native.ALGO_SCAN, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy),
+                                       *[P(x) for x in want], P(ws), n))
+    _native.check(lib.wkv6_backward_static(st, _native.F32, B, T, C, H, P(r), P(k), P(v), P(w), P(u), P(gy), *[P(x) for x in got]))
+    torch.cuda.synchronize()
+    for name, a, b in zip("gr gk gv gw gu".split(), got, want):
+        assert torch.equal(a, b), name
 
 
 def test_static_scratch_backward_refuses_what_does_not_fit():
