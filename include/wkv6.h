@@ -37,7 +37,7 @@ enum { WKV6_BF16 = 0, WKV6_F16 = 1, WKV6_F32 = 2 };
 enum {
     WKV6_OK = 0,
     WKV6_ERR_ARG = 1,         /* null pointer, non-positive size, C != H*N, unknown dtype   */
-    WKV6_ERR_UNSUPPORTED = 2, /* head size the kernels are not built for                     */
+    WKV6_ERR_UNSUPPORTED = 2, /* head size (or path for this head size / dtype) without a kernel   */
     WKV6_ERR_WORKSPACE = 3,   /* workspace missing or smaller than the query function says   */
     WKV6_ERR_LAUNCH = 4       /* the HIP runtime refused a launch (see wkv6_last_hip_error)   */
 };
@@ -69,7 +69,12 @@ enum {
 
 const char *wkv6_status_string(int status);
 int wkv6_version(void);
-/* Head sizes compiled into the library: returns 1 if N is supported. */
+/* Head sizes compiled into the library: returns 1 if N is supported.  64: every entry point.  8, 16, 32 (the
+ * reference builds for any multiple of 4, rwkv_kernel/torch_rwkv_kernel.py:13; its scripts run 8 and 32): the
+ * plain calls -- wkv6_forward*, wkv6_forward_with_state*, wkv6_backward*, wkv6_backward_with_state, the
+ * training pair (which then saves nothing: wkv6_saved_bytes = 0) and the XLA targets -- on per-timestep fp32
+ * kernels with one thread per channel, states (B, H, N, N); WKV6_ALGO_CHUNK, the fused stages and
+ * wkv6_backward_static answer WKV6_ERR_UNSUPPORTED for them. */
 int wkv6_supports_head_size(int64_t N);
 
 /* Stateless forward.

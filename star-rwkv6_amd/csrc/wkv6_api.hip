@@ -59,12 +59,21 @@ thread_local int g_last_hip_error = 0;
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-int check_shape(int dtype, int64_t B, int64_t T, int64_t C, int64_t H) {
+// WKV6_OK: head size 64, every entry point.  kSmallHead: head size 8, 16 or 32 (otherwise valid), which the plain
+// calls (forward, forward with state, backward, backward with state, the training pair without saved states)
+// serve with the kernels of wkv6_generic.hip and every other entry point refuses as unsupported.
+constexpr int kSmallHead = -1;
+int check_shape_any(int dtype, int64_t B, int64_t T, int64_t C, int64_t H) {
     if (dtype != WKV6_BF16 && dtype != WKV6_F16 && dtype != WKV6_F32) return WKV6_ERR_ARG;
     if (B <= 0 || T <= 0 || C <= 0 || H <= 0 || C % H != 0) return WKV6_ERR_ARG;
     if (B * H > 0x7fffffffLL || T > 0x7fffffffLL) return WKV6_ERR_ARG;
-    if (!wkv6_supports_head_size(C / H)) return WKV6_ERR_UNSUPPORTED;
-    return WKV6_OK;
+    if (C / H == 64) return WKV6_OK;
+    if (wkv6::generic_head_size(C / H)) return B <= 65535 && B * T * C < (1LL << 40) ? kSmallHead : WKV6_ERR_UNSUPPORTED;
+    return WKV6_ERR_UNSUPPORTED;
+}
+int check_shape(int dtype, int64_t B, int64_t T, int64_t C, int64_t H) {
+    const int rc = check_shape_any(dtype, B, T, C, H);
+    return rc == kSmallHead ? WKV6_ERR_UNSUPPORTED : rc;
 }
 
 int out_type(int dtype) { return dtype == WKV6_BF16 ? WKV6_BF16 : WKV6_F32; }
@@ -82,7 +91,7 @@ const char *wkv6_status_string(int s) {
     switch (s) {
     case WKV6_OK: return "ok";
     case WKV6_ERR_ARG: return "invalid argument (null/misaligned pointer, bad size or dtype)";
-    case WKV6_ERR_UNSUPPORTED: return "unsupported head size (library is built for N = 64)";
+    case WKV6_ERR_UNSUPPORTED: return "unsupported: head size (64 everywhere; 8, 16, 32 in the plain calls) or a path this dtype / shape has no kernel for";
     case WKV6_ERR_WORKSPACE: return "workspace missing or too small";
     case WKV6_ERR_LAUNCH: return "HIP launch failed";
     default: return "unknown status";
@@ -90,7 +99,7 @@ const char *wkv6_status_string(int s) {
 }
 
 int wkv6_version(void) { return 100; }
-int wkv6_supports_head_size(int64_t N) { return N == 64; }
+int wkv6_supports_head_size(int64_t N) { return N == 64 || wkv6::generic_head_size(N); }
 int wkv6_last_status(void) { return g_last_status; }
 int wkv6_last_hip_error(void) { return g_last_hip_error; }
 
@@ -108,8 +117,8 @@ static int forward_impl(void *stream, int dtype, int state_dtype, int algo,
                         const void *r, const void *k, const void *v, const void *w, const void *u,
                         const void *s, void *y, void *ys, void *saved,
                         void *workspace = nullptr, size_t workspace_bytes = 0) {
-    int rc = check_shape(dtype, B, T, C, H);
-    if (rc != WKV6_OK) return rc;
+    int rc = check_shape_any(dtype, B, T, C, H);
+    if (rc != WKV6_OK && rc != kSmallHead) return rc;
     if (!r || !k || !v || !w || !u || !y) return WKV6_ERR_ARG;
     if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(y)) return WKV6_ERR_ARG;
     if (has_init_state && !s) return WKV6_ERR_ARG;
@@ -118,6 +127,10 @@ static int forward_impl(void *stream, int dtype, int state_dtype, int algo,
     hipStream_t st = (hipStream_t)stream;
     const void *s_in = has_init_state ? s : nullptr;
     const int64_t *map_in = has_init_state ? state_map : nullptr;
+    if (rc == kSmallHead) {
+        if (algo == WKV6_ALGO_CHUNK) return WKV6_ERR_UNSUPPORTED;
+        return finish(wkv6::generic_forward(st, dtype, state_dtype, B, T, H, C / H, r, k, v, w, u, s_in, map_in, y, ys));
+    }
     // fp32 and fp16 tensors: the full-precision chunk form, unless the per-timestep kernels are asked for
     if (algo != WKV6_ALGO_SCAN && wkv6::chunk32_forward_applies(dtype, B, T, H))
         return finish(wkv6::chunk32_forward(st, dtype, state_dtype, B, T, H, r, k, v, w, u, s_in, map_in, y, ys, saved));
@@ -376,6 +389,7 @@ static size_t segments_workspace_bytes(int dtype, int algo, int64_t B, int64_t T
 }
 
 size_t wkv6_backward_workspace_bytes_ex(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
+    if (check_shape_any(dtype, B, T, C, H) == kSmallHead) return wkv6::generic_backward_workspace_bytes(B, T, C);
     if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
     // The per-timestep path keeps one fp32 per element (P), the chunked path one fp32 state per
     // 64-token chunk (which a workgroup's exact second pass reuses for its own P).
@@ -416,8 +430,8 @@ static int backward_impl(void *stream, int dtype, int algo, int64_t B, int64_t T
                          const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace, size_t workspace_bytes,
                          bool states_ready, void *gu_sum = nullptr) {
-    int rc = check_shape(dtype, B, T, C, H);
-    if (rc != WKV6_OK) return rc;
+    int rc = check_shape_any(dtype, B, T, C, H);
+    if (rc != WKV6_OK && rc != kSmallHead) return rc;
     if (!r || !k || !v || !w || !u || !gy || !gr || !gk || !gv || !gw || !gu) return WKV6_ERR_ARG;
     if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(gy) || !aligned16(gr) ||
         !aligned16(gk) || !aligned16(gv) || !aligned16(gw)) return WKV6_ERR_ARG;
@@ -425,6 +439,12 @@ static int backward_impl(void *stream, int dtype, int algo, int64_t B, int64_t T
     const size_t need = wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H);
     if (need > 0 && (!workspace || workspace_bytes < need || !aligned16(workspace))) return WKV6_ERR_WORKSPACE;
     hipStream_t st = (hipStream_t)stream;
+    if (rc == kSmallHead) {
+        if (algo == WKV6_ALGO_CHUNK) return WKV6_ERR_UNSUPPORTED;
+        rc = finish(wkv6::generic_backward(st, dtype, B, T, H, C / H, r, k, v, w, u, nullptr, gy, nullptr, gr, gk, gv, gw, gu, nullptr, workspace));
+        if (rc == WKV6_OK && gu_sum) rc = finish(wkv6::sum_over_batch(st, out_type(dtype), B, C, gu, gu_sum));
+        return rc;
+    }
     if (train_chunk32(dtype, algo, B, T, H)) {
         // without saved states: a forward pass that only leaves the chunk states in the workspace
         if (!states_ready) {
@@ -510,6 +530,7 @@ int wkv6_backward_saved_sum(void *stream, int dtype, int algo, int64_t B, int64_
 }
 
 size_t wkv6_backward_with_state_workspace_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
+    if (check_shape_any(dtype, B, T, C, H) == kSmallHead) return wkv6::generic_backward_workspace_bytes(B, T, C);
     if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
     size_t need = wkv6::scan_backward_state_workspace_bytes(B, T, C);
     const size_t c = wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H);
@@ -522,8 +543,8 @@ int wkv6_backward_with_state(void *stream, int dtype, int algo, int64_t B, int64
                              const float *s0, const void *gy, const float *gsT,
                              void *gr, void *gk, void *gv, void *gw, void *gu, float *gs0,
                              void *workspace, size_t workspace_bytes) {
-    int rc = check_shape(dtype, B, T, C, H);
-    if (rc != WKV6_OK) return rc;
+    int rc = check_shape_any(dtype, B, T, C, H);
+    if (rc != WKV6_OK && rc != kSmallHead) return rc;
     if (!r || !k || !v || !w || !u || !gy || !gr || !gk || !gv || !gw || !gu) return WKV6_ERR_ARG;
     if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(gy) || !aligned16(gr) ||
         !aligned16(gk) || !aligned16(gv) || !aligned16(gw)) return WKV6_ERR_ARG;
@@ -531,6 +552,10 @@ int wkv6_backward_with_state(void *stream, int dtype, int algo, int64_t B, int64
     if (algo < WKV6_ALGO_AUTO || algo > WKV6_ALGO_CHUNK) return WKV6_ERR_ARG;
     const size_t need = wkv6_backward_with_state_workspace_bytes(dtype, algo, B, T, C, H);
     if (!workspace || workspace_bytes < need || !aligned16(workspace)) return WKV6_ERR_WORKSPACE;
+    if (rc == kSmallHead) {
+        if (algo == WKV6_ALGO_CHUNK) return WKV6_ERR_UNSUPPORTED;
+        return finish(wkv6::generic_backward((hipStream_t)stream, dtype, B, T, H, C / H, r, k, v, w, u, s0, gy, gsT, gr, gk, gv, gw, gu, gs0, workspace));
+    }
     if (algo == WKV6_ALGO_CHUNK && !chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
     const bool chunk = algo == WKV6_ALGO_CHUNK || (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));

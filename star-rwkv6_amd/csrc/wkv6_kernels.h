@@ -37,6 +37,18 @@ hipError_t scan_backward(hipStream_t st, int dtype, int64_t B, int64_t T, int64_
                          const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace);
 
+// --- head sizes 8, 16, 32 (wkv6_generic.hip): the per-timestep recurrence, one thread per channel; every
+// dtype, states (B,H,N,N), state_map, gradients through the state (s0 / gsT / gs0 fp32, may be null)
+bool generic_head_size(int64_t N);
+hipError_t generic_forward(hipStream_t st, int dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N,
+                           const void *r, const void *k, const void *v, const void *w, const void *u,
+                           const void *s0, const int64_t *map, void *y, void *sT);
+size_t generic_backward_workspace_bytes(int64_t B, int64_t T, int64_t C);
+hipError_t generic_backward(hipStream_t st, int dtype, int64_t B, int64_t T, int64_t H, int64_t N,
+                            const void *r, const void *k, const void *v, const void *w, const void *u,
+                            const float *s0, const void *gy, const float *gsT,
+                            void *gr, void *gk, void *gv, void *gw, void *gu, float *gs0, void *workspace);
+
 // one timestep (T = 1) with the layer's output stage fused in (bf16 tensors), see chunk_forward_fused
 hipError_t step_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64_t H,
                               const void *r, const void *k, const void *v, const void *w, const void *u,
