@@ -19,9 +19,8 @@
 
 #include <type_traits>
 
-#ifndef C32_GROUPS
-#define C32_GROUPS 2
-#endif
+// groups of loading waves that take the chunks in turn (three measured no faster than two)
+constexpr int kC32FwdGroups = 2;
 
 namespace wkv6 {
 
@@ -284,7 +283,7 @@ size_t chunk32_saved_bytes(int64_t B, int64_t T, int64_t H) {
 template <typename Tin, typename Tout, typename Ts, bool kOut>
 static hipError_t launch(hipStream_t st, int64_t B, const C32FwdArgs &a) {
     constexpr int lds = (int)sizeof(C32FwdSmem);
-    constexpr int kGroups = C32_GROUPS;
+    constexpr int kGroups = kC32FwdGroups;
     const hipError_t e = allow_dynamic_lds<chunk32_fwd_kernel<Tin, Tout, Ts, kGroups, kOut>>(lds);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL((chunk32_fwd_kernel<Tin, Tout, Ts, kGroups, kOut>), dim3((unsigned)(B * a.H)), dim3(256 + 256 * kGroups), lds, st, a);

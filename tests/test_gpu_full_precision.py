@@ -215,3 +215,55 @@ def test_c2_shape_fp32_vs_oracle(op, oracle):
     y, grads = _fwd_bwd(op, dev, gyd[0], AUTO)
     check_close("y", y, oracle.forward_c(*ref, N)[0], torch.float32)
     _check_grads(grads, oracle.backward_c(*ref, gyr[0], N), torch.float32)
+
+
+def test_random_shapes_agree_with_the_per_timestep_kernels(op):
+    # a property test, not parity evidence: 40 random (B, T, H, dtype, kind) cases, some with a stretch of strong
+    # decay in one pair, through WKV6_ALGO_AUTO and WKV6_ALGO_SCAN: the two kernel families agree to fp32 rounding
+    import random
+
+    rng = random.Random(2024)
+
+    def rel(a, b):
+        return float((a.double() - b.double()).abs().max() / max(float(b.double().abs().max()), 1e-30))
+
+    for case in range(40):
+        B, H = rng.choice([1, 2, 3, 5, 9, 33]), rng.choice([1, 2, 3, 5, 8])
+        T = rng.choice([64, 65, 95, 96, 97, 127, 128, 160, 333, 511, 1000])
+        if B * H * T > 300000:
+            T = 128
+        dt = rng.choice([torch.float32, torch.float16])
+        kind = rng.choice(["train", "train", "state", "infer"])
+        g = torch.Generator().manual_seed(7000 + case)
+        C = H * N
+        r, k, v = [torch.randn(B, T, C, generator=g) for _ in range(3)]
+        w = torch.rand(B, T, C, generator=g) * 7 - 6
+        u = torch.randn(H, N, generator=g) * 0.5
+        gy = torch.randn(B, T, C, generator=g).cuda()
+        if rng.random() < 0.3:
+            b0, h0, t0 = rng.randrange(B), rng.randrange(H), rng.randrange(T - 20)
+            w[b0, t0:t0 + rng.choice([12, 20]), N * h0:N * h0 + N] = rng.choice([1.2, 2.0, 20.0])
+        dev = [x.to(dt).cuda() for x in (r, k, v, w, u)]
+        nrow = rng.choice([1, B])
+        s0 = (torch.randn(nrow, H, N, N, generator=g) * 0.1).cuda()
+        smap = [rng.randrange(nrow) for _ in range(B)]
+        print("case %d B%d T%d H%d %s %s" % (case, B, T, H, dt, kind), flush=True)
+        outs = {}
+        for algo in (AUTO, SCAN):
+            op.algo = algo
+            if kind == "train":
+                leaves = [x.clone().requires_grad_(True) for x in dev]
+                y, _ = op(*leaves)
+                y.backward(gy)
+                outs[algo] = [y.detach()] + [x.grad for x in leaves]
+            elif kind == "state":
+                with torch.no_grad():
+                    outs[algo] = list(op(*dev, return_state=True, init_state=s0, state_map=smap))
+            else:
+                with torch.no_grad():
+                    outs[algo] = [op(*dev)[0]]
+        torch.cuda.synchronize()
+        tol = 2e-3 if dt == torch.float16 and kind == "train" else 2e-5   # (fp16 gradients come back rounded to fp16)
+        for a, b in zip(outs[AUTO], outs[SCAN]):
+            assert torch.isfinite(a.float()).all()
+            assert rel(a, b) <= tol, (case, rel(a, b))
