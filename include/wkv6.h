@@ -205,7 +205,10 @@ int wkv6_shift_mix_x_backward(void *stream, int dtype, int64_t B, int64_t T, int
  * rwkv_kernel/torch_kernel/wkv6_op.cpp:33-41 (kernel_backward_101/102/103/201,
  * rwkv_kernel/jax_kernel/rwkv_kernels.cu:205-407, launched by HostApplyGradient :436-444).
  * `workspace` is device memory of at least wkv6_backward_workspace_bytes(...) bytes owned by the
- * caller; its contents on entry and exit are meaningless. */
+ * caller; its contents on entry and exit are meaningless.  (What it holds depends on the kernels the
+ * shape takes -- 4 bytes per element of r on the per-timestep kernels and the bf16 chunk forms, one
+ * fp32 64x64 state per 32 tokens and head = 8 bytes per element of r on the full-precision chunk form of
+ * fp32 / fp16 tensors -- so size it with the query, not by hand.) */
 int wkv6_backward(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
                   const void *r, const void *k, const void *v, const void *w, const void *u,
                   const void *gy,
