@@ -45,6 +45,49 @@ def _staggered(count, shape, dtype, device, first=1):
     return [block[first * _STAGGER + i * step: first * _STAGGER + i * step + n * es].view(dtype).view(shape) for i in range(count)]
 
 
+def _carve(device, specs):
+    """Tensors of different shapes and dtypes out of ONE allocation: specs = [(shape, dtype, slot), ...]; each tensor
+    starts `slot` * 256 bytes past a 4 KiB boundary of the block (see _staggered for why)."""
+    offs, total = [], 0
+    for shape, dtype, slot in specs:
+        n = 1
+        for d in shape:
+            n *= d
+        nb = n * _ELEMENT_SIZE[dtype]
+        offs.append((total + slot * _STAGGER, nb))
+        total += (slot * _STAGGER + nb + 4095) // 4096 * 4096
+    block = torch.empty(total, dtype=torch.uint8, device=device)
+    return [block[o:o + nb].view(dtype).view(shape) for (o, nb), (shape, dtype, _) in zip(offs, specs)]
+
+
+_ELEMENT_SIZE = {torch.bfloat16: 2, torch.float16: 2, torch.float32: 4, torch.uint8: 1}
+_saved_bytes_cache = {}
+
+
+def _saved_bytes(lib, code, algo, B, T, C, H):
+    key = (code, algo, B, T, C, H)
+    n = _saved_bytes_cache.get(key)
+    if n is None:
+        n = _saved_bytes_cache[key] = int(lib.wkv6_saved_bytes(code, algo, B, T, C, H))
+    return n
+
+
+class _on_device:
+    """torch.cuda.device(dev) only where dev is not already the current device (the context manager costs as much
+    host time as a kernel launch)."""
+
+    def __init__(self, dev):
+        self.ctx = None if dev.index is None or dev.index == torch.cuda.current_device() else torch.cuda.device(dev)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+
+
 def _ptr(t):
     return None if t is None else t.data_ptr()
 
@@ -67,13 +110,15 @@ class _WKV6(torch.autograd.Function):
             ctx.dims = (B, T, C, H)
             ctx.algo = algo
             code = _DTYPE_CODE[r.dtype]
-            (y,) = _staggered(1, (B, T, C), _out_dtype(r.dtype), r.device, first=5)
+            need_grad = any(ctx.needs_input_grad[4:9])
+            nsave = _saved_bytes(lib, code, algo, B, T, C, H) if need_grad else 0
             saved = None
-            with torch.cuda.device(r.device):
-                need_grad = any(ctx.needs_input_grad[4:9])
-                nsave = lib.wkv6_saved_bytes(code, algo, B, T, C, H) if need_grad else 0
+            if nsave:
+                y, saved = _carve(r.device, [((B, T, C), _out_dtype(r.dtype), 5), ((nsave,), torch.uint8, 6)])
+            else:
+                (y,) = _staggered(1, (B, T, C), _out_dtype(r.dtype), r.device, first=5)
+            with _on_device(r.device):
                 if nsave:
-                    (saved,) = _staggered(1, (nsave,), torch.uint8, r.device, first=6)
                     _native.check(lib.wkv6_forward_save(_stream(), code, algo, B, T, C, H,
                                                         _ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(y),
                                                         _ptr(saved), nsave))
@@ -97,16 +142,16 @@ class _WKV6(torch.autograd.Function):
             odt = _out_dtype(r.dtype)
             assert gy.dtype in (torch.bfloat16, torch.float32) and gy.dtype == odt
             gy = gy.contiguous()
-            gr, gk, gv, gw = _staggered(4, (B, T, C), odt, gy.device, first=7)
-            gu = torch.empty((B, C), device=gy.device, dtype=odt)
+            big = ((B, T, C), odt)
+            gr, gk, gv, gw, gu, gu_sum = _carve(gy.device, [big + (7,), big + (8,), big + (9,), big + (10,),
+                                                            ((B, C), odt, 0), ((C,), odt, 0)])
             code = _DTYPE_CODE[r.dtype]
             args = (_ptr(r), _ptr(k), _ptr(v), _ptr(w), _ptr(u), _ptr(gy), _ptr(gr), _ptr(gk), _ptr(gv), _ptr(gw), _ptr(gu))
-            with torch.cuda.device(gy.device):
+            with _on_device(gy.device):
                 saved = ctx.saved_states
                 if saved is not None:
                     # the batch sum of gu (rwkv_kernel/torch_rwkv_kernel.py:73) comes out of the same launch
                     ctx.saved_states = None
-                    gu_sum = torch.empty(C, device=gy.device, dtype=odt)
                     _native.check(lib.wkv6_backward_saved_sum(_stream(), code, ctx.algo, B, T, C, H, *args, _ptr(gu_sum),
                                                               _ptr(saved), saved.numel()))
                     return (None, None, None, None, gr, gk, gv, gw, gu_sum.reshape(u.shape), None)
