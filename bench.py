@@ -41,6 +41,8 @@ MEASURED_TRAFFIC_BYTES = {
     # forward_save 134.5 MB read + 67.1 MB written
     ("c2", "auto", "bwd"): 337.5e6, ("c2", "chunk", "bwd"): 337.5e6,
     ("c2", "auto", "fwd"): 201.6e6, ("c2", "chunk", "fwd"): 201.6e6,
+    # profiles/c2_f32_fwd_bwd_kernel_trace.md: backward 470.3 MB read + 268.5 MB written, forward 268.8 + 201.3 MB
+    ("c2_f32", "auto", "bwd"): 738.8e6, ("c2_f32", "auto", "fwd"): 470.1e6,
 }
 
 
