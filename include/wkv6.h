@@ -69,8 +69,9 @@ enum {
 
 const char *wkv6_status_string(int status);
 int wkv6_version(void);
-/* Head sizes compiled into the library: returns 1 if N is supported.  64: every entry point.  8, 16, 32 (the
- * reference builds for any multiple of 4, rwkv_kernel/torch_rwkv_kernel.py:13; its scripts run 8 and 32): the
+/* Head sizes compiled into the library: returns 1 if N is supported.  64: every entry point.  Every other multiple of
+ * 4 up to 128 (the reference builds for any multiple of 4, rwkv_kernel/torch_rwkv_kernel.py:13; its scripts run 8
+ * and 32): the
  * plain calls -- wkv6_forward*, wkv6_forward_with_state*, wkv6_backward*, wkv6_backward_with_state, the
  * training pair (which then saves nothing: wkv6_saved_bytes = 0) and the XLA targets -- on per-timestep fp32
  * kernels with one thread per channel, states (B, H, N, N); WKV6_ALGO_CHUNK, the fused stages and

@@ -59,7 +59,7 @@ thread_local int g_last_hip_error = 0;
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// WKV6_OK: head size 64, every entry point.  kSmallHead: head size 8, 16 or 32 (otherwise valid), which the plain
+// WKV6_OK: head size 64, every entry point.  kSmallHead: another head size that is a multiple of 4, up to 128 (otherwise valid), which the plain
 // calls (forward, forward with state, backward, backward with state, the training pair without saved states)
 // serve with the kernels of wkv6_generic.hip and every other entry point refuses as unsupported.
 constexpr int kSmallHead = -1;
@@ -91,7 +91,7 @@ const char *wkv6_status_string(int s) {
     switch (s) {
     case WKV6_OK: return "ok";
     case WKV6_ERR_ARG: return "invalid argument (null/misaligned pointer, bad size or dtype)";
-    case WKV6_ERR_UNSUPPORTED: return "unsupported: head size (64 everywhere; 8, 16, 32 in the plain calls) or a path this dtype / shape has no kernel for";
+    case WKV6_ERR_UNSUPPORTED: return "unsupported: head size (64 everywhere; other multiples of 4 up to 128 in the plain calls) or a path this dtype / shape has no kernel for";
     case WKV6_ERR_WORKSPACE: return "workspace missing or too small";
     case WKV6_ERR_LAUNCH: return "HIP launch failed";
     default: return "unknown status";

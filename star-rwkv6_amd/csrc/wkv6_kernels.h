@@ -37,7 +37,7 @@ hipError_t scan_backward(hipStream_t st, int dtype, int64_t B, int64_t T, int64_
                          const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
                          void *gr, void *gk, void *gv, void *gw, void *gu, void *workspace);
 
-// --- head sizes 8, 16, 32 (wkv6_generic.hip): the per-timestep recurrence, one thread per channel; every
+// --- head sizes other than 64, multiples of 4 up to 128 (wkv6_generic.hip): the per-timestep recurrence, one thread per channel; every
 // dtype, states (B,H,N,N), state_map, gradients through the state (s0 / gsT / gs0 fp32, may be null)
 bool generic_head_size(int64_t N);
 hipError_t generic_forward(hipStream_t st, int dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N,

@@ -61,7 +61,7 @@ class RWKVKernelOperator:
         assert head_size % 4 == 0, "head_size must be a multiple of 4"
         lib = _native.load()
         if not lib.wkv6_supports_head_size(head_size):
-            raise _native.WKV6Error("libwkv6_gfx950 is built for head sizes 64 (all paths) and 8, 16, 32 (plain calls), got %d" % head_size)
+            raise _native.WKV6Error("libwkv6_gfx950 is built for head sizes 64 (all paths) and the other multiples of 4 up to 128 (plain calls), got %d" % head_size)
         _register()
         self.head_size = head_size
         self.max_sequence_length = max_sequence_length

@@ -403,7 +403,7 @@ class RWKVKernelOperator:
         assert head_size > 0 and max_sequence_length > 0
         assert head_size % 4 == 0, "head_size must be a multiple of 4"
         if not lib.wkv6_supports_head_size(head_size):
-            raise _native.WKV6Error("libwkv6_gfx950 is built for head sizes 64 (all paths) and 8, 16, 32 (plain calls), got %d" % head_size)
+            raise _native.WKV6Error("libwkv6_gfx950 is built for head sizes 64 (all paths) and the other multiples of 4 up to 128 (plain calls), got %d" % head_size)
         self.head_size = head_size
         # the reference bakes this into a per-thread array bound (-D_T_); nothing here is sized by
         # it, so longer sequences simply work

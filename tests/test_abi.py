@@ -43,7 +43,8 @@ def test_version_and_head_size(native):
     assert lib.wkv6_version() >= 100
     assert lib.wkv6_supports_head_size(64) == 1
     assert lib.wkv6_supports_head_size(32) == 1 and lib.wkv6_supports_head_size(8) == 1   # the plain calls
-    assert lib.wkv6_supports_head_size(12) == 0 and lib.wkv6_supports_head_size(128) == 0
+    assert lib.wkv6_supports_head_size(12) == 1 and lib.wkv6_supports_head_size(128) == 1   # any multiple of 4 up to 128
+    assert lib.wkv6_supports_head_size(6) == 0 and lib.wkv6_supports_head_size(132) == 0 and lib.wkv6_supports_head_size(0) == 0
     assert lib.wkv6_status_string(0) == b"ok"
     assert b"workspace" in lib.wkv6_status_string(3)
 
@@ -65,7 +66,8 @@ def test_argument_validation_returns_status_codes(native):
     assert lib.wkv6_forward(None, native.BF16, 2, 16, 128, 2, None, *args[1:]) == 1        # null pointer
     assert lib.wkv6_forward(None, 7, 2, 16, 128, 2, *args) == 1                            # unknown dtype
     assert lib.wkv6_forward(None, native.BF16, 2, 16, 130, 2, *args) == 2                  # head size 65
-    assert lib.wkv6_forward(None, native.BF16, 2, 16, 24, 2, *args) == 2                   # head size 12
+    assert lib.wkv6_forward(None, native.BF16, 2, 16, 20, 2, *args) == 2                   # head size 10
+    assert lib.wkv6_forward(None, native.BF16, 2, 16, 264, 2, *args) == 2                  # head size 132
     assert lib.wkv6_forward_gn_gate(None, native.BF16, native.BF16, 2, 16, 64, 2, 0, None, *([fake] * 6), fake, fake, fake, 1e-5, fake, None) == 2   # head size 32: plain calls only
     assert lib.wkv6_forward(None, native.BF16, 0, 16, 128, 2, *args) == 1                  # empty batch
     assert lib.wkv6_forward(None, native.BF16, 2, 16, 128, 2, fake + 2, *args[1:]) == 1    # misaligned

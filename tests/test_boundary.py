@@ -79,8 +79,8 @@ def test_ops_flavour_matches_oracle(oracle, restore_backend):
 def test_torch_flavour_argument_checks(restore_backend):
     pkg = _fresh_import("torch")
     with pytest.raises(Exception):
-        pkg.RWKVKernelOperator(128, 64)         # the library has kernels for head sizes 8, 16, 32 and 64
-    assert pkg.RWKVKernelOperator(32, 64).head_size == 32
+        pkg.RWKVKernelOperator(132, 64)         # the library has kernels for the multiples of 4 up to 128
+    assert pkg.RWKVKernelOperator(32, 64).head_size == 32 and pkg.RWKVKernelOperator(12, 64).head_size == 12
     with pytest.raises(AssertionError):
         pkg.RWKVKernelOperator(6, 64)           # head size must be a multiple of 4 (rwkv_kernels.cu:101)
     op = pkg.RWKVKernelOperator(64, 1024)

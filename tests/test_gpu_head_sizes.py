@@ -1,4 +1,4 @@
-"""Head sizes 8, 16 and 32 (the reference builds for any multiple of 4, rwkv_kernel/torch_rwkv_kernel.py:13; its own
+"""Head sizes other than 64 (the reference builds for any multiple of 4, rwkv_kernel/torch_rwkv_kernel.py:13; its own
 scripts run 8 -- rwkv_kernel/jax_rwkv_kernel.py:513-518 -- and 32 -- deprecated_code/test_rwkv_torch.py:62-99):
 the plain calls of the operator class through the C ABI against the float64 oracle."""
 import numpy as np
@@ -20,7 +20,10 @@ def _op(N):
 
 
 @pytest.mark.parametrize("dt", ["f32", "bf16", "f16"])
-@pytest.mark.parametrize("N,B,T,H", [(8, 2, 37, 3), (8, 1, 16, 9), (16, 3, 50, 2), (32, 2, 64, 4), (32, 1, 129, 1), (32, 2, 5, 3)])
+@pytest.mark.parametrize("N,B,T,H", [(8, 2, 37, 3), (8, 1, 16, 9), (16, 3, 50, 2), (32, 2, 64, 4), (32, 1, 129, 1), (32, 2, 5, 3),
+                                     # head sizes that do not divide the workgroup: 5 heads of 12 per workgroup, 3 of 20, 2 of 24, one of 40 ...
+                                     (4, 2, 19, 35), (12, 2, 33, 7), (20, 1, 40, 4), (24, 2, 21, 3), (40, 2, 18, 2), (48, 1, 35, 3),
+                                     (60, 1, 17, 2), (96, 1, 34, 2), (128, 2, 20, 1)])
 def test_forward_backward(oracle, dt, N, B, T, H):
     dtype = DTYPES[dt]
     odt = out_dtype(dtype)
@@ -53,7 +56,7 @@ def test_reference_script_shape_head_size_8(oracle):
 
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
-@pytest.mark.parametrize("N", [8, 32])
+@pytest.mark.parametrize("N", [8, 32, 12, 48, 128])
 def test_state_in_and_out_with_map(oracle, dt, N):
     B, T, H = 4, 45, 3
     dtype = DTYPES[dt]
@@ -70,7 +73,7 @@ def test_state_in_and_out_with_map(oracle, dt, N):
     check_close("sT", sT, sT_ref, out_dtype(dtype), is_grad=True)
 
 
-@pytest.mark.parametrize("N", [8, 16, 32])
+@pytest.mark.parametrize("N", [8, 16, 32, 4, 20, 56, 100])
 def test_gradients_through_the_state(oracle, N):
     B, T, H = 2, 41, 2
     op = _op(N)
@@ -95,7 +98,8 @@ def test_what_small_heads_do_not_have():
 
     lib = _native.load()
     assert lib.wkv6_supports_head_size(8) and lib.wkv6_supports_head_size(16) and lib.wkv6_supports_head_size(32) and lib.wkv6_supports_head_size(64)
-    assert not lib.wkv6_supports_head_size(12) and not lib.wkv6_supports_head_size(128)
+    assert lib.wkv6_supports_head_size(12) and lib.wkv6_supports_head_size(128)
+    assert not lib.wkv6_supports_head_size(10) and not lib.wkv6_supports_head_size(132)
     # no saved states, no chunk form, no fused stage
     assert lib.wkv6_saved_bytes(_native.BF16, _native.ALGO_AUTO, 2, 256, 64, 2) == 0
     assert lib.wkv6_backward_workspace_bytes(_native.F32, 2, 100, 64, 2) == (2 * 100 * 64 + 2 * 64) * 4
