@@ -145,8 +145,8 @@ int wkv6_forward_gn_gate_ex(void *stream, int dtype, int state_dtype,
  * wkv6_forward_gn_gate_save: zero initial state; writes `out` as above and, for the backward, y
  * (B,T,C) bf16, the norm's statistics `stats` (B,T,H,2) fp32 = (mean, 1/sqrt(var + gn_eps)) of y over
  * each head's channels, and the chunk states into `saved` (wkv6_saved_bytes(dtype, WKV6_ALGO_CHUNK, ...)
- * bytes, as for wkv6_forward_save).  bf16 tensors only; shapes whose training pair runs in time segments
- * (few pairs, long sequence) return WKV6_ERR_UNSUPPORTED: use the unfused calls there.
+ * bytes, as for wkv6_forward_save).  bf16 tensors only.  Where the training pair runs in time segments (few
+ * pairs, long sequence) the output stage is part of the segments' second pass.
  *
  * wkv6_gn_gate_backward: given gout = dL/dout, writes gy = dL/dy (feed it to wkv6_backward_saved* with
  * the same `saved`), ggate = dL/dgate (both (B,T,C) bf16) and gscale, goffset = dL/dgn_scale,

@@ -201,10 +201,10 @@ int wkv6_forward_gn_gate_ex(void *stream, int dtype, int state_dtype,
 }
 
 static int train_segments(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H);
+static size_t saved_base_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H);
 
 int wkv6_forward_gn_gate_save_supported(int dtype, int64_t B, int64_t T, int64_t C, int64_t H) {
-    return check_shape(dtype, B, T, C, H) == WKV6_OK && dtype == WKV6_BF16 && chunk_possible(dtype, T, C) &&
-           train_segments(dtype, WKV6_ALGO_CHUNK, B, T, C, H) <= 1;
+    return check_shape(dtype, B, T, C, H) == WKV6_OK && dtype == WKV6_BF16 && chunk_possible(dtype, T, C);
 }
 
 int wkv6_forward_gn_gate_save(void *stream, int dtype, int64_t B, int64_t T, int64_t C, int64_t H,
@@ -214,13 +214,18 @@ int wkv6_forward_gn_gate_save(void *stream, int dtype, int64_t B, int64_t T, int
     int rc = check_shape(dtype, B, T, C, H);
     if (rc != WKV6_OK) return rc;
     if (dtype != WKV6_BF16 || !chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;
-    if (train_segments(dtype, WKV6_ALGO_CHUNK, B, T, C, H) > 1) return WKV6_ERR_UNSUPPORTED;   // (time segments: unfused calls)
     if (!r || !k || !v || !w || !u || !gate || !gn_scale || !gn_offset || !out || !y || !stats) return WKV6_ERR_ARG;
     if (!aligned16(r) || !aligned16(k) || !aligned16(v) || !aligned16(w) || !aligned16(gate) || !aligned16(out) || !aligned16(y) ||
         !aligned16(stats) || !aligned16(gn_scale) || !aligned16(gn_offset)) return WKV6_ERR_ARG;
     if (!(gn_eps >= 0.f)) return WKV6_ERR_ARG;
     const size_t need = wkv6_saved_bytes(dtype, WKV6_ALGO_CHUNK, B, T, C, H);
     if (!saved || saved_bytes < need || !aligned16(saved)) return WKV6_ERR_WORKSPACE;
+    const int P = train_segments(dtype, WKV6_ALGO_CHUNK, B, T, C, H);
+    if (P > 1) {   // few pairs, long sequence: time segments side by side, the output stage in their second pass
+        char *extra = reinterpret_cast<char *>(saved) + saved_base_bytes(dtype, WKV6_ALGO_CHUNK, B * P, T / P, C, H);
+        return finish(wkv6::chunk_forward_fused_save_segments((hipStream_t)stream, B, T, H, r, k, v, w, u, gate, gn_scale, gn_offset,
+                                                              gn_eps, out, y, stats, saved, extra));
+    }
     return finish(wkv6::chunk_forward_fused_save((hipStream_t)stream, B, T, H, r, k, v, w, u, gate, gn_scale, gn_offset, gn_eps,
                                                  out, y, stats, saved));
 }

@@ -688,15 +688,17 @@ hipError_t chunk_forward_fused(hipStream_t st, int state_dtype, int64_t B, int64
 }
 
 // Training with the fused output stage: out = (group_norm_head(y) * gn_scale + gn_offset) * gate, and for
-// the backward y itself (bf16), the norm's statistics and the chunk states.  Zero initial state.
-hipError_t chunk_forward_fused_save(hipStream_t st, int64_t B, int64_t T, int64_t H,
-                                    const void *r, const void *k, const void *v, const void *w, const void *u,
-                                    const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
-                                    void *out, void *y, float *stats, void *saved_states)
+// the backward y itself (bf16), the norm's statistics and the chunk states.  s0: null (zero initial state: what
+// the caller sees), or one fp32 state per pair (a segment's incoming state).
+static hipError_t fused_save_from(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                                  const void *r, const void *k, const void *v, const void *w, const void *u, const float *s0,
+                                  const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
+                                  void *out, void *y, float *stats, void *saved_states)
 {
     if (block_forward_applies(B, T, H))
-        return block_forward_fused(st, kF32, B, T, H, r, k, v, w, u, nullptr, nullptr, gate, gn_scale, gn_offset, gn_eps, out, y, stats, nullptr, saved_states);
+        return block_forward_fused(st, kF32, B, T, H, r, k, v, w, u, s0, nullptr, gate, gn_scale, gn_offset, gn_eps, out, y, stats, nullptr, saved_states);
     FwdArgs a = {};
+    a.s0 = s0;
     a.T = (int)T; a.H = (int)H; a.nitems = (int)(B * H);
     a.r = (const bf16_t *)r; a.k = (const bf16_t *)k; a.v = (const bf16_t *)v; a.w = (const bf16_t *)w; a.u = (const bf16_t *)u;
     a.v_orig = v;
@@ -708,6 +710,13 @@ hipError_t chunk_forward_fused_save(hipStream_t st, int64_t B, int64_t T, int64_
     a.split = 1;
     return (T % CL) != 0 ? launch_fwd<bf16_t, float, true, true, true>(st, a, multi, grid)
                          : launch_fwd<bf16_t, float, true, false, true>(st, a, multi, grid);
+}
+hipError_t chunk_forward_fused_save(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                                    const void *r, const void *k, const void *v, const void *w, const void *u,
+                                    const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
+                                    void *out, void *y, float *stats, void *saved_states)
+{
+    return fused_save_from(st, B, T, H, r, k, v, w, u, nullptr, gate, gn_scale, gn_offset, gn_eps, out, y, stats, saved_states);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -883,6 +892,21 @@ hipError_t chunk_forward_save_segments(hipStream_t st, int64_t B, int64_t T, int
     if (e != hipSuccess) return e;
     if ((e = launch_chain<float, false>(st, s.P, B, H, nullptr, nullptr, s.dsum, s.states, nullptr)) != hipSuccess) return e;
     return chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, s.states, nullptr, y, nullptr, saved);
+}
+
+// The same with the fused output stage in the second pass.  out, y, gate and the statistics are indexed by
+// token, and the tokens of the (B*P, T/P) rows are those of the (B, T) rows in the same order.
+hipError_t chunk_forward_fused_save_segments(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                                             const void *r, const void *k, const void *v, const void *w, const void *u,
+                                             const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
+                                             void *out, void *y, float *stats, void *saved, void *extra)
+{
+    const TrainSegments s = train_segments_layout(B, T, H, extra);
+    const int64_t L = T / s.P, rows = B * s.P;
+    hipError_t e = chunk_forward(st, kF32, rows, L, H, r, k, v, w, u, nullptr, nullptr, nullptr, s.states, nullptr, s.dsum);
+    if (e != hipSuccess) return e;
+    if ((e = launch_chain<float, false>(st, s.P, B, H, nullptr, nullptr, s.dsum, s.states, nullptr)) != hipSuccess) return e;
+    return fused_save_from(st, rows, L, H, r, k, v, w, u, s.states, gate, gn_scale, gn_offset, gn_eps, out, y, stats, saved);
 }
 
 }  // namespace wkv6

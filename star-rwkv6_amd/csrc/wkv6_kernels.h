@@ -171,6 +171,11 @@ hipError_t chunk_forward_fused_save(hipStream_t st, int64_t B, int64_t T, int64_
                                     const void *r, const void *k, const void *v, const void *w, const void *u,
                                     const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
                                     void *out, void *y, float *stats, void *saved_states);
+// ... of a shape whose training pair runs in time segments (saved / extra as in chunk_forward_save_segments)
+hipError_t chunk_forward_fused_save_segments(hipStream_t st, int64_t B, int64_t T, int64_t H,
+                                             const void *r, const void *k, const void *v, const void *w, const void *u,
+                                             const void *gate, const float *gn_scale, const float *gn_offset, float gn_eps,
+                                             void *out, void *y, float *stats, void *saved, void *extra);
 // backward of the output stage (wkv6_gn.hip): bf16 tensors, gscale / goffset fp32 (C), zeroed inside
 hipError_t gn_gate_backward(hipStream_t st, int64_t B, int64_t T, int64_t H,
                             const void *gout, const void *y, const float *stats, const void *gate,

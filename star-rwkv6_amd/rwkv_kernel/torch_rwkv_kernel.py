@@ -537,7 +537,7 @@ class RWKVKernelOperator:
             lib = _native.load()
             if lib.wkv6_forward_gn_gate_save_supported(_DTYPE_CODE[r.dtype], B, T, C, H):
                 return _WKV6GnGate.apply(B, T, C, H, r, k, v, w, u, gate, gn_scale.to(r.device), gn_offset.to(r.device), epsilon), None
-            # (few pairs and a long sequence: the operator runs in time segments; unfused calls)
+            # (a shape the fused training kernels do not take, e.g. a sequence too long for the chunk form: unfused calls)
             y, _ = self(r, k, v, w, u)
             z = torch.nn.functional.layer_norm(y.float().view(B, T, H, N), (N,), eps=epsilon).view(B, T, C)
             out = (z * gn_scale.reshape(1, 1, C).float() + gn_offset.reshape(1, 1, C).float()) * gate.float()

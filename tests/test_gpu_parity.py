@@ -584,12 +584,15 @@ def test_fused_group_norm_gate_training_on_a_fallback_pair(op, oracle):
     _fused_training_case(op, oracle, 2, 128, 2, 333, wild=True)
 
 
-def test_fused_group_norm_gate_training_in_time_segments_uses_the_unfused_calls(op, oracle):
-    # few pairs and a long sequence: the operator's training pair runs in time segments, which the fused
-    # kernels do not take; the call stays differentiable
+@pytest.mark.parametrize("B,T,H,wild", [(1, 2048, 2, False), (2, 1024, 3, False), (1, 2048, 32, False), (1, 4096, 4, True)])
+def test_fused_group_norm_gate_training_in_time_segments(op, oracle, B, T, H, wild):
+    # few pairs and a long sequence: the operator's training pair runs in time segments, and the output stage
+    # is part of their second pass (tile form; with 32 heads the segments fill the chip and run on the block
+    # form; the last case has pairs that fall back to the per-timestep pass inside their segment)
     from rwkv_kernel import _native
-    assert _native.load().wkv6_forward_gn_gate_save_supported(_native.BF16, 1, 2048, 128, 2) == 0
-    _fused_training_case(op, oracle, 1, 2048, 2, 340)
+    lib = _native.load()
+    assert lib.wkv6_forward_gn_gate_save_supported(_native.BF16, B, T, H * 64, H) == 1
+    _fused_training_case(op, oracle, B, T, H, 340 + H, wild=wild)
 
 
 def test_fused_group_norm_gate_on_a_fallback_pair(op, oracle):
