@@ -321,6 +321,18 @@ size_t wkv6_create_descriptor(int B, int T, int C, int H, int S, int x_type, int
 void wkv_forward(void *stream, void **buffers, const char *opaque, size_t opaque_len);
 void wkv_backward(void *stream, void **buffers, const char *opaque, size_t opaque_len);
 void wkv_forward_with_state(void *stream, void **buffers, const char *opaque, size_t opaque_len);
+/* Two more targets, for the forward and backward rules of the custom_vjp (rwkv_kernel/jax_rwkv_kernel.py:148-170
+ * registers wkv_forward and wkv_backward there): the training pair wkv6_forward_save / wkv6_backward_saved_sum
+ * under WKV6_ALGO_AUTO, for shapes with wkv6_saved_bytes(x_type, WKV6_ALGO_AUTO, ...) = n > 0 (otherwise
+ * WKV6_ERR_UNSUPPORTED is recorded and nothing runs).  No counterpart in the reference, whose backward
+ * recomputes everything from the inputs.
+ *   wkv_forward_save    [r,k,v,w,u | y, saved(n bytes)]
+ *   wkv_backward_saved  [r,k,v,w,u,gy,saved | gr,gk,gv,gw,gu(B,C), saved_out(n bytes), gu_sum(C)]
+ * The backward uses parts of the block as scratch, so the caller declares saved_out as an alias of the
+ * operand saved (output_operand_aliases / input_output_aliases={6: 5}); given two different buffers the
+ * target copies the operand into the result first and leaves the operand alone. */
+void wkv_forward_save(void *stream, void **buffers, const char *opaque, size_t opaque_len);
+void wkv_backward_saved(void *stream, void **buffers, const char *opaque, size_t opaque_len);
 /* Status of the calling thread's most recent custom-call target invocation. */
 int wkv6_last_status(void);
 /* hipError_t value of the calling thread's most recent failed launch (0 if none). */

@@ -650,4 +650,29 @@ void wkv_forward_with_state(void *stream, void **buffers, const char *opaque, si
     }
 }
 
+void wkv_forward_save(void *stream, void **buffers, const char *opaque, size_t opaque_len) {
+    wkv6_descriptor d;
+    if (!unpack(opaque, opaque_len, &d) || !buffers) { g_last_status = WKV6_ERR_ARG; return; }
+    const size_t n = wkv6_saved_bytes(d.x_type, WKV6_ALGO_AUTO, d.B, d.T, d.C, d.H);
+    if (n == 0) { g_last_status = WKV6_ERR_UNSUPPORTED; return; }   // (nothing to save: the caller uses wkv_forward)
+    g_last_status = wkv6_forward_save(stream, d.x_type, WKV6_ALGO_AUTO, d.B, d.T, d.C, d.H, buffers[0], buffers[1], buffers[2],
+                                      buffers[3], buffers[4], buffers[5], buffers[6], n);
+}
+
+void wkv_backward_saved(void *stream, void **buffers, const char *opaque, size_t opaque_len) {
+    wkv6_descriptor d;
+    if (!unpack(opaque, opaque_len, &d) || !buffers) { g_last_status = WKV6_ERR_ARG; return; }
+    const size_t n = wkv6_saved_bytes(d.x_type, WKV6_ALGO_AUTO, d.B, d.T, d.C, d.H);
+    if (n == 0) { g_last_status = WKV6_ERR_UNSUPPORTED; return; }
+    // the block the call works on is the result that the caller aliases to the operand `saved`; if the two
+    // are different buffers after all, the operand stays as it is and the result starts as its copy
+    if (buffers[12] != buffers[6]) {
+        const hipError_t e = hipMemcpyAsync(buffers[12], buffers[6], n, hipMemcpyDeviceToDevice, (hipStream_t)stream);
+        if (e != hipSuccess) { g_last_status = finish(e); return; }
+    }
+    g_last_status = wkv6_backward_saved_sum(stream, d.x_type, WKV6_ALGO_AUTO, d.B, d.T, d.C, d.H, buffers[0], buffers[1], buffers[2],
+                                            buffers[3], buffers[4], buffers[5], buffers[7], buffers[8], buffers[9],
+                                            buffers[10], buffers[11], buffers[13], buffers[12], n);
+}
+
 }  // extern "C"

@@ -50,6 +50,8 @@ SIGNATURES = {
     "wkv_forward": (None, [_p, ctypes.POINTER(_p), ctypes.c_char_p, _sz]),
     "wkv_backward": (None, [_p, ctypes.POINTER(_p), ctypes.c_char_p, _sz]),
     "wkv_forward_with_state": (None, [_p, ctypes.POINTER(_p), ctypes.c_char_p, _sz]),
+    "wkv_forward_save": (None, [_p, ctypes.POINTER(_p), ctypes.c_char_p, _sz]),
+    "wkv_backward_saved": (None, [_p, ctypes.POINTER(_p), ctypes.c_char_p, _sz]),
     "wkv6_last_status": (_int, []),
     "wkv6_last_hip_error": (_int, []),
 }

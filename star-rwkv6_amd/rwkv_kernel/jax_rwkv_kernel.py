@@ -12,6 +12,12 @@ jax.ffi.ffi_call(custom_call_api_version=2, legacy_backend_config=<28-byte descr
 the same opaque descriptor and buffer orders as the reference's lowering (:75-111, :172-218,
 :358-376).  The backward call declares one extra result that XLA allocates as scratch.
 
+Where the library has something worth keeping for the backward (the chunked kernels' per-chunk
+states), the custom_vjp's forward rule runs the target wkv_forward_save, whose second result -- a
+block of bytes -- joins the residuals, and the backward rule runs wkv_backward_saved, which skips the
+forward state sweep and returns gu already summed over the batch.  The primal call outside of
+differentiation stays wkv_forward.
+
 jax is not installed in the image this library is developed in, so this module is exercised only
 where jax (ROCm build) exists; importing it without jax raises ImportError.
 """
@@ -25,7 +31,7 @@ import numpy as np
 from . import _native
 
 _REGISTERED = False
-_TARGETS = ("wkv_forward", "wkv_backward", "wkv_forward_with_state")
+_TARGETS = ("wkv_forward", "wkv_backward", "wkv_forward_with_state", "wkv_forward_save", "wkv_backward_saved")
 
 
 def _register():
@@ -95,16 +101,48 @@ class RWKVKernelOperator:
             gr, gk, gv, gw, gu, _ = outs
             return gr, gk, gv, gw, jnp.sum(gu, axis=0)
 
+        def saved_bytes(r, k, v, w, u):
+            B, T, C, H, code, odt = check(r, k, v, w, u)
+            return int(lib.wkv6_saved_bytes(code, _native.ALGO_AUTO, B, T, C, H))
+
+        def fwd_save_call(r, k, v, w, u, nsave):
+            B, T, C, H, code, odt = check(r, k, v, w, u)
+            desc = _native.create_descriptor(B, T, C, H, False, code, _code(odt))
+            return jax.ffi.ffi_call("wkv_forward_save",
+                                    (jax.ShapeDtypeStruct(r.shape, odt), jax.ShapeDtypeStruct((nsave,), jnp.uint8)),
+                                    custom_call_api_version=2, legacy_backend_config=desc)(r, k, v, w, u)
+
+        def bwd_saved_call(r, k, v, w, u, gy, saved):
+            B, T, C, H, code, odt = check(r, k, v, w, u)
+            desc = _native.create_descriptor(B, T, C, H, False, code, _code(odt))
+            big = jax.ShapeDtypeStruct(r.shape, odt)
+            # the call works inside the saved block: it is handed on as a result that aliases the operand
+            outs = jax.ffi.ffi_call(
+                "wkv_backward_saved",
+                (big, big, big, big, jax.ShapeDtypeStruct((B,) + tuple(u.shape), odt),
+                 jax.ShapeDtypeStruct(saved.shape, jnp.uint8), jax.ShapeDtypeStruct(tuple(u.shape), odt)),
+                custom_call_api_version=2, legacy_backend_config=desc,
+                input_output_aliases={6: 5})(r, k, v, w, u, gy.astype(odt), saved)
+            gr, gk, gv, gw, _, _, gu_sum = outs
+            return gr, gk, gv, gw, gu_sum
+
         @jax.custom_vjp
         def rwkv_normal_operator(r, k, v, w, u):
             return fwd_call(r, k, v, w, u)
 
         def vjp_fwd(r, k, v, w, u):
-            return fwd_call(r, k, v, w, u), (r, k, v, w, u)
+            nsave = saved_bytes(r, k, v, w, u)
+            if nsave > 0:
+                y, saved = fwd_save_call(r, k, v, w, u, nsave)
+                return y, (r, k, v, w, u, saved)
+            return fwd_call(r, k, v, w, u), (r, k, v, w, u, None)
 
         def vjp_bwd(res, gy):
-            r, k, v, w, u = res
-            gr, gk, gv, gw, gu = bwd_call(r, k, v, w, u, gy)
+            r, k, v, w, u, saved = res
+            if saved is not None:
+                gr, gk, gv, gw, gu = bwd_saved_call(r, k, v, w, u, gy, saved)
+            else:
+                gr, gk, gv, gw, gu = bwd_call(r, k, v, w, u, gy)
             dt = r.dtype
             return gr.astype(dt), gk.astype(dt), gv.astype(dt), gw.astype(dt), gu.astype(dt).reshape(u.shape)
 

@@ -18,7 +18,7 @@ def register_ffi_target(name, capsule, platform, api_version):
     _TARGETS[name] = capsule
 
 
-def ffi_call(name, result_shape_dtypes, custom_call_api_version, legacy_backend_config):
+def ffi_call(name, result_shape_dtypes, custom_call_api_version, legacy_backend_config, input_output_aliases=None):
     """Returns the callable that runs target `name` the way XLA's legacy custom call does."""
     from . import ShapeDtypeStruct, _wrap
     assert custom_call_api_version == 2, "API_VERSION_STATUS_RETURNING_UNIFIED carries the opaque string"
@@ -30,6 +30,12 @@ def ffi_call(name, result_shape_dtypes, custom_call_api_version, legacy_backend_
         ops = [o.contiguous() for o in operands]
         assert all(o.is_cuda for o in ops)
         results = [torch.empty(s.shape, dtype=s.dtype, device=ops[0].device) for s in specs]
+        # a result that aliases an operand is the operand's buffer; the operand itself must look untouched to the
+        # rest of the program, so (as XLA does when the value is still needed) the call gets a copy of it
+        for operand, result in (input_output_aliases or {}).items():
+            assert tuple(ops[operand].shape) == tuple(specs[result].shape) and ops[operand].dtype == specs[result].dtype
+            ops[operand] = ops[operand].clone()
+            results[result] = ops[operand]
         bufs = ops + results
         arr = (ctypes.c_void_p * len(bufs))(*[b.data_ptr() for b in bufs])
         _TARGETS[name](torch.cuda.current_stream().cuda_stream, arr, opaque, len(opaque))

@@ -120,6 +120,10 @@ def test_custom_call_rejects_bad_opaque_without_throwing(native):
     assert lib.wkv6_last_status() == 1
     lib.wkv_backward(None, arr, None, 0)
     assert lib.wkv6_last_status() == 1
+    lib.wkv_forward_save(None, arr, b"x" * 29, 29)
+    assert lib.wkv6_last_status() == 1
+    lib.wkv_backward_saved(None, None, b"x" * 28, 28)
+    assert lib.wkv6_last_status() == 1
     # output type that contradicts the dtype rule (bf16 in -> f32 out) is refused
     bad = native.create_descriptor(1, 16, 64, 1, False, native.BF16, native.F32)
     lib.wkv_forward_with_state(None, arr, bad, len(bad))

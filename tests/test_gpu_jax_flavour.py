@@ -44,7 +44,9 @@ def flavour():
 
 
 @pytest.mark.parametrize("B,T,H,dtype", [(2, 256, 2, torch.bfloat16), (3, 100, 1, torch.bfloat16),
-                                         (2, 40, 2, torch.float32), (2, 40, 1, torch.float16)])
+                                         (2, 40, 2, torch.float32), (2, 40, 1, torch.float16),
+                                         # (the differentiated call of the first two runs the saving pair's targets; so do these)
+                                         (2, 128, 2, torch.float32), (1, 100, 2, torch.float16), (1, 2048, 2, torch.bfloat16)])
 def test_stateless_call_and_its_vjp(flavour, oracle, B, T, H, dtype):
     mod, jax = flavour
     jnp = jax.numpy
@@ -72,6 +74,10 @@ def test_stateless_call_and_its_vjp(flavour, oracle, B, T, H, dtype):
     gu = grads[4]
     assert tuple(gu.shape) == tuple(dev[4].shape) and gu.dtype == dtype       # summed over the batch, u's shape
     check_close("gu", to_np(gu).reshape(H, N), g_ref[4], dtype, is_grad=True)
+    again = pull(jnp.asarray(gyd[0]))                                          # the residuals serve a second pull
+    torch.cuda.synchronize()
+    for a, b in zip(grads, again):
+        assert torch.equal(a, b)
 
 
 def test_stateful_call_packs_the_state_map(flavour, oracle):

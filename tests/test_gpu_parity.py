@@ -278,6 +278,76 @@ def test_xla_custom_call_targets_bf16(op, oracle, B, T, H):
     check_close("ys from zero", ys, oracle.forward_c(*ref, N)[1], torch.bfloat16)
 
 
+@pytest.mark.parametrize("B,T,H,dt", [(2, 256, 2, "bf16"), (8, 1024, 32, "bf16"), (1, 2048, 2, "bf16"), (2, 128, 2, "f32"), (2, 100, 1, "f16")])
+def test_xla_custom_call_targets_of_the_saving_pair(op, oracle, B, T, H, dt):
+    # The targets behind the jax flavour's custom_vjp rules: wkv_forward_save leaves y and the saved block,
+    # wkv_backward_saved works inside the result that aliases the block and returns gu summed over the batch.
+    # Run twice from one forward (the second time on a separate result buffer, which the target fills from the
+    # operand first) and with the operand checked for being left alone.  (1, 2048, 2): the pair runs in time segments.
+    from rwkv_kernel import _native
+
+    lib = _native.load()
+    N = 64
+    C = H * N
+    dtype = {"bf16": torch.bfloat16, "f32": torch.float32, "f16": torch.float16}[dt]
+    code = {"bf16": _native.BF16, "f32": _native.F32, "f16": _native.F16}[dt]
+    odt = out_dtype(dtype)
+    ocode = _native.BF16 if dt == "bf16" else _native.F32
+    print("custom-call targets of the saving pair %s B%d T%d H%d" % (dt, B, T, H), flush=True)
+    ins = oracle.make_inputs(B, T, H, N, 78)
+    dev, ref = cast_inputs(ins[:5], dtype)
+    gyd, gyr = cast_inputs(ins[5:6], odt)
+    stream = torch.cuda.current_stream().cuda_stream
+    desc = _native.create_descriptor(B, T, C, H, False, code, ocode)
+    nsave = lib.wkv6_saved_bytes(code, _native.ALGO_AUTO, B, T, C, H)
+    assert nsave > 0
+
+    def call(fn, bufs):
+        arr = (ctypes.c_void_p * len(bufs))(*[b.data_ptr() for b in bufs])
+        fn(stream, arr, desc, len(desc))
+        torch.cuda.synchronize()
+        assert lib.wkv6_last_status() == 0
+
+    y = torch.empty(B, T, C, dtype=odt, device="cuda")
+    saved = torch.empty(nsave, dtype=torch.uint8, device="cuda")
+    call(lib.wkv_forward_save, dev + [y, saved])
+    check_close("y", y, oracle.forward_c(*ref, N)[0], odt)
+    g_ref = oracle.backward_c(*ref, gyr[0], N)
+    kept = saved.clone()
+    first = None
+    for aliased in (False, True):
+        outs = [torch.full((B, T, C), 7.0, dtype=odt, device="cuda") for _ in range(4)] + [torch.empty(B, C, dtype=odt, device="cuda")]
+        gu_sum = torch.empty(C, dtype=odt, device="cuda")
+        block = saved if aliased else torch.empty_like(saved)
+        call(lib.wkv_backward_saved, dev + gyd + [saved] + outs + [block, gu_sum])
+        if not aliased:
+            assert torch.equal(saved, kept)          # two buffers: the operand is left alone
+        for name, g, want in zip("gr gk gv gw".split(), outs, g_ref):
+            check_close(name, g, want, odt, is_grad=True)
+        check_close("gu", to_np(gu_sum).reshape(H, N), g_ref[4], odt, is_grad=True)
+        if first is None:
+            first = [g.clone() for g in outs[:4]] + [gu_sum.clone()]
+        else:
+            for a, b in zip(first, outs[:4] + [gu_sum]):
+                assert torch.equal(a, b)             # the same block, the same result
+
+
+def test_xla_saving_pair_refuses_shapes_that_save_nothing(op):
+    from rwkv_kernel import _native
+
+    lib = _native.load()
+    B, T, C, H = 2, 16, 64, 1                        # too short for a chunk form: nothing to save
+    assert lib.wkv6_saved_bytes(_native.F32, _native.ALGO_AUTO, B, T, C, H) == 0
+    desc = _native.create_descriptor(B, T, C, H, False, _native.F32, _native.F32)
+    x = torch.zeros(B, T, C, device="cuda")
+    arr = (ctypes.c_void_p * 14)(*([x.data_ptr()] * 14))
+    lib.wkv_forward_save(None, arr, desc, len(desc))
+    assert lib.wkv6_last_status() == 2
+    lib.wkv_backward_saved(None, arr, desc, len(desc))
+    assert lib.wkv6_last_status() == 2
+    torch.cuda.synchronize()
+
+
 # ---------------------------------------------------------------------------------------------
 # chunk-parallel MFMA path (bf16 tensors)
 # ---------------------------------------------------------------------------------------------
