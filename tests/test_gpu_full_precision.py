@@ -217,9 +217,10 @@ def test_c2_shape_fp32_vs_oracle(op, oracle):
     _check_grads(grads, oracle.backward_c(*ref, gyr[0], N), torch.float32)
 
 
-def test_random_shapes_agree_with_the_per_timestep_kernels(op):
-    # a property test, not parity evidence: 40 random (B, T, H, dtype, kind) cases, some with a stretch of strong
-    # decay in one pair, through WKV6_ALGO_AUTO and WKV6_ALGO_SCAN: the two kernel families agree to fp32 rounding
+def test_random_shapes_against_the_oracle_and_the_per_timestep_kernels(op, oracle):
+    # 40 random (B, T, H, dtype, kind) cases, some with a stretch of strong decay in one pair, through
+    # WKV6_ALGO_AUTO and WKV6_ALGO_SCAN: each against the float64 oracle at the fp32 tolerances, and the two kernel
+    # families against each other to fp32 rounding
     import random
 
     rng = random.Random(2024)
@@ -263,6 +264,18 @@ def test_random_shapes_agree_with_the_per_timestep_kernels(op):
                 with torch.no_grad():
                     outs[algo] = [op(*dev)[0]]
         torch.cuda.synchronize()
+        ref = [to_np(x) for x in dev]
+        if kind == "train":
+            want = [oracle.forward_c(*ref, N)[0]] + list(oracle.backward_c(*ref, to_np(gy), N))
+        elif kind == "state":
+            want = list(oracle.forward_c(*ref, N, to_np(s0), smap))
+        else:
+            want = [oracle.forward_c(*ref, N)[0]]
+        for algo in (AUTO, SCAN):
+            for i, (got, w_) in enumerate(zip(outs[algo], want)):
+                # (y is fp32 whatever the tensors are; fp16 gradients come back rounded to fp16)
+                tol_dt = torch.float16 if (dt == torch.float16 and kind == "train" and i > 0) else torch.float32
+                check_close("case %d algo %d output %d" % (case, algo, i), to_np(got).reshape(w_.shape), w_, tol_dt, is_grad=i > 0)
         tol = 2e-3 if dt == torch.float16 and kind == "train" else 2e-5   # (fp16 gradients come back rounded to fp16)
         for a, b in zip(outs[AUTO], outs[SCAN]):
             assert torch.isfinite(a.float()).all()

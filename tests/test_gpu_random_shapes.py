@@ -1,12 +1,14 @@
-"""Seeded random shapes: the chunk-parallel MFMA path against the exact per-timestep kernels, both
-on the GPU through the package surface (the exact kernels are checked against the float64 oracle in
-test_gpu_parity.py).  Covers what the fixed cases leave open: odd batch and head counts, lengths
-around chunk and segment boundaries, long sequences of few pairs (time segments with and without a
-remainder), training, state gradients and inference on the same inputs."""
+"""Seeded random shapes: the chunk-parallel MFMA path and the exact per-timestep kernels, both on the GPU
+through the package surface, each against the float64 oracle on the same (bf16-rounded) inputs and against each
+other.  Covers what the fixed cases leave open: odd batch and head counts, lengths around chunk and segment
+boundaries, long sequences of few pairs (time segments with and without a remainder), training, state
+gradients and inference on the same inputs."""
 import random
 
 import pytest
 import torch
+
+from _util import check_close, to_np
 
 pytestmark = pytest.mark.gpu
 SCAN, CHUNK = 1, 2
@@ -66,6 +68,26 @@ def test_chunk_path_equals_exact_path(oracle, B, T, H, mode, wild):
                 y, _ = op(r, k, v, w, u)
             res[algo] = [y]
     torch.cuda.synchronize()
+    # the float64 oracle on exactly these rounded inputs
+    ref = [to_np(x) for x in (r, k, v, w, u)]
+    bf = torch.bfloat16
+    if mode == 0:
+        names = "y gr gk gv gw gu".split()
+        want = [oracle.forward_c(*ref, N)[0]] + list(oracle.backward_c(*ref, to_np(gy), N))
+    elif mode == 1:
+        names = "y sT gr gk gv gw gu gs0".split()
+        want = list(oracle.forward_c(*ref, N, to_np(s0))) + list(oracle.backward_state_c(*ref, to_np(gy), N, to_np(s0), to_np(gS)))
+    elif mode == 2:
+        names = "y sT".split()
+        want = list(oracle.forward_c(*ref, N, to_np(s0)))
+    else:
+        names = ["y"]
+        want = [oracle.forward_c(*ref, N)[0]]
+    for algo in (SCAN, CHUNK):
+        assert len(res[algo]) == len(want)
+        for name, got, w_ in zip(names, res[algo], want):
+            # (states and their gradients are fp32 tensors computed from bf16 products: held to the bf16 bound)
+            check_close("%s (%s)" % (name, "scan" if algo == SCAN else "chunk"), to_np(got).reshape(w_.shape), w_, bf, is_grad=name != "y")
     # both paths round their outputs to bf16 (1e-2 relative each against the oracle)
     for i, (a, b) in enumerate(zip(res[CHUNK], res[SCAN])):
         assert _rel(a, b) <= 2e-2, (i, _rel(a, b))
