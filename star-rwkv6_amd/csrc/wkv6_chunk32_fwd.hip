@@ -24,6 +24,9 @@ constexpr int kC32FwdGroups = 2;
 
 namespace wkv6 {
 
+// The value is final here: what computes it stays in front of this point and what reads it behind it.
+__device__ __forceinline__ void pin_value(float &x) { asm volatile("" : "+v"(x)); }
+
 struct C32FwdLds {
     float Rp[2][kC32][kLd], Kp[2][kC32][kLd], V[2][kC32][kLd];   // R', K', v of the chunk in hand and the next
     float Rm[kC32][kLd], Km[kC32][kLd];                          // R~, K~
@@ -107,6 +110,21 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_fwd_kernel(const 
                 if (kOut) part[x] = E0 == 0 ? s : sum_rows4(s);
             }
         };
+        auto settle = [&](auto half) {
+            constexpr int E0 = 2 * decltype(half)::value;
+#pragma unroll
+            for (int x = 0; x < 2; ++x) {
+#pragma unroll
+                for (int e = E0; e < E0 + 2; ++e) {
+                    pin_value(op_k[x][e]);
+                    pin_value(op_v[x][e]);
+                    if (kOut) { pin_value(op_r[x][e]); pin_value(hm_r[x][e]); pin_value(hm_k[x][e]); }
+                }
+                if (kOut) pin_value(part[x]);
+            }
+#pragma unroll
+            for (int e = E0; e < E0 + 2; ++e) pin_value(e_all[e]);
+        };
         const std::integral_constant<int, 0> h0;
         const std::integral_constant<int, 1> h1;
         auto publish = [&](int c) {
@@ -149,6 +167,10 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_fwd_kernel(const 
             __syncthreads();
             if (forming) {
                 form(h1, c + 2);
+                // (every value of this chunk is final before the next loads are issued: left to itself the compiler
+                // moves the last products behind the loads, whose destinations are then other registers than the
+                // ones still being read, and the copy back at the end of the iteration waits for the loads)
+                settle(h1);
                 if (c + 2 + kGroups < nchunk) fetch(c + 2 + kGroups);
             }
             if (handing) finish();

@@ -32,14 +32,19 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 // prefetch held across a compute phase costs 4 VGPRs for 16-bit types.
 template <typename T> struct Raw8;
 template <> struct Raw8<float> {
-    float4 a, b;
+    // (one native vector: as a struct of two of the runtime's float4 the eight values are kept in scratch memory, and a
+    // prefetch then waits for its loads at once to store them there)
+    typedef float v4 __attribute__((ext_vector_type(4)));
+    typedef float v8 __attribute__((ext_vector_type(8)));
+    v8 a;
     __device__ __forceinline__ void load(const float *p) {
-        a = *reinterpret_cast<const float4 *>(p);
-        b = *reinterpret_cast<const float4 *>(p + 4);
+        const v4 lo = *reinterpret_cast<const v4 *>(p), hi = *reinterpret_cast<const v4 *>(p + 4);
+        a = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     }
-    __device__ __forceinline__ void zero() { a = make_float4(0, 0, 0, 0); b = a; }
+    __device__ __forceinline__ void zero() { a = (v8)(0.f); }
     __device__ __forceinline__ void to_float(float (&o)[8]) const {
-        o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w; o[4] = b.x; o[5] = b.y; o[6] = b.z; o[7] = b.w;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = a[i];
     }
 };
 template <> struct Raw8<bf16_t> {
