@@ -21,6 +21,21 @@ namespace wkv6 {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// Four consecutive elements as they sit in memory, converted when they are used: a 16-bit load whose conversion
+// stood next to it would make the wave wait for the load where it is issued.
+template <typename T> struct Raw4;
+template <> struct Raw4<float> {
+    f32x4 x;
+    __device__ __forceinline__ void load(const float *p) { x = *reinterpret_cast<const f32x4 *>(p); }
+    __device__ __forceinline__ float at(int i) const { return x[i]; }
+};
+template <> struct Raw4<f16_t> {
+    typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+    h4 x;
+    __device__ __forceinline__ void load(const f16_t *p) { x = *reinterpret_cast<const h4 *>(p); }
+    __device__ __forceinline__ float at(int i) const { return (float)x[i]; }
+};
+
 constexpr int kC32 = 32;            // tokens per chunk
 constexpr int kLd = 68;             // floats per row of a [token][channel] LDS tile (64 + 4: 16-byte fragment reads without bank conflicts)
 constexpr int kLa = 36;             // floats per row of a [token][token] LDS tile

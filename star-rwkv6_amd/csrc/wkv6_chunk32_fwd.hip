@@ -71,13 +71,13 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_fwd_kernel(const 
         const int grp = (wave - 4) >> 2, p = (wave - 4) & 3, t16 = lane & 15, ch = 16 * p + 4 * (lane >> 4);
         float fu[4];
         load4(u + h * kN + ch, fu);
-        float nr[2][4], nk[2][4], nv[2][4], nw[2][4];   // the group's next chunk on its way in
+        Raw4<Tin> nr[2], nk[2], nv[2], nw[2];   // the group's next chunk on its way in, as loaded
         auto fetch = [&](int c) {
             const int64_t row0 = base + (int64_t)c * kC32 * C;   // (uniform)
 #pragma unroll
             for (int x = 0; x < 2; ++x) {
                 const int o = min(16 * x + t16, T - 1 - c * kC32) * (int)C + ch;   // rows past the end read the last one
-                load4(r + row0 + o, nr[x]); load4(k + row0 + o, nk[x]); load4(v + row0 + o, nv[x]); load4(w + row0 + o, nw[x]);
+                nr[x].load(r + row0 + o); nk[x].load(k + row0 + o); nv[x].load(v + row0 + o); nw[x].load(w + row0 + o);
             }
         };
         // the chunk whose operands are formed: two channels of the lane's four at a time (a barrier in between)
@@ -88,22 +88,26 @@ __global__ __launch_bounds__(256 + 256 * kGroups) void chunk32_fwd_kernel(const 
             const bool valid[2] = {c * kC32 + t16 < T, c * kC32 + 16 + t16 < T};
             C32Scale sc;
             sc.wild = false;
-            float d[2][4];
-            c32_scale<E0, E0 + 2>(nw, valid, sc, d);
+            float d[2][4], fw[2][4];
+#pragma unroll
+            for (int x = 0; x < 2; ++x)
+#pragma unroll
+                for (int e = E0; e < E0 + 2; ++e) fw[x][e] = nw[x].at(e);
+            c32_scale<E0, E0 + 2>(fw, valid, sc, d);
             wild |= sc.wild;
 #pragma unroll
             for (int x = 0; x < 2; ++x) {
                 float s = E0 == 0 ? 0.f : part[x];
 #pragma unroll
                 for (int e = E0; e < E0 + 2; ++e) {
-                    const float fr = valid[x] ? nr[x][e] : 0.f, fk = valid[x] ? nk[x][e] : 0.f;
+                    const float fr = valid[x] ? nr[x].at(e) : 0.f, fk = valid[x] ? nk[x].at(e) : 0.f;
                     op_k[x][e] = fk * sc.kp[x][e];
                     if (kOut) {
                         op_r[x][e] = fr * sc.rp[x][e];
                         hm_r[x][e] = fr * sc.rm[x][e];
                         hm_k[x][e] = fk * sc.km[x][e];
                     }
-                    op_v[x][e] = valid[x] ? nv[x][e] : 0.f;
+                    op_v[x][e] = valid[x] ? nv[x].at(e) : 0.f;
                     e_all[e] = sc.all[e];
                     s = fmaf(fr * fk, fu[e], s);
                 }
