@@ -124,10 +124,12 @@ __device__ __forceinline__ void c32_scale(const float (&raw)[2][4], const bool (
     for (int e = kFrom; e < kTo; ++e) {
         d[0][e] = valid[0] ? -fast_exp(raw[0][e]) : 0.f;
         d[1][e] = valid[1] ? -fast_exp(raw[1][e]) : 0.f;
-        const float w0 = fast_exp(d[0][e]), w1 = fast_exp(d[1][e]), i0 = fast_exp(-d[0][e]), i1 = fast_exp(-d[1][e]);
+        const float w0 = fast_exp(d[0][e]), w1 = fast_exp(d[1][e]);
         const float up0 = row_product_up(w0), up1 = row_product_up(w1);
         const float dn0 = row_product_down(w0), dn1 = row_product_down(w1);
-        const float to_mid0 = row_product_down(i0), to_mid1 = row_product_up(i1);
+        // the way back to the chunk's middle: the reciprocal of the product from there (1 ulp, as good as a product
+        // of sixteen rounded factors; outside the reach, where it overflows, the pair is redone anyway)
+        const float to_mid0 = __builtin_amdgcn_rcpf(dn0), to_mid1 = __builtin_amdgcn_rcpf(up1);
         const float before0 = row_take<0x111>(up0), before1 = row_take<0x111>(up1);   // products of the tokens before this one
         const float after0 = row_take<0x101>(dn0), after1 = row_take<0x101>(dn1);     // ... behind this one
         const float all0 = up0 * after0, all1 = up1 * after1;                         // the whole row (each lane's own rounding of it)
@@ -138,8 +140,8 @@ __device__ __forceinline__ void c32_scale(const float (&raw)[2][4], const bool (
         o.all[e] = all0 * all1;
         o.mid[e] = all0;
         o.rest[e] = all1;
-        o.inv0[e] = to_mid0 * row_take<0x111>(row_product_up(i0));
-        o.inv1[e] = to_mid1 * row_take<0x101>(row_product_down(i1));
+        o.inv0[e] = __builtin_amdgcn_rcpf(all0);
+        o.inv1[e] = __builtin_amdgcn_rcpf(all1);
         o.wild |= !(all0 >= reach) || !(all1 >= reach);   // (NaN counts as outside)
     }
 }
