@@ -48,9 +48,9 @@ enum {
                             fp16 tensors with T >= 64: the full-precision chunk form (every product on
                             the fp32 matrix instructions, chunks of 32 tokens, fp32 accuracy: y within
                             1e-4, gradients within 1e-3 relative, the same y with and without a
-                            gradient; its training pair saves one fp32 state per chunk).  Everything
-                            else, and every call that takes gradients through the state of fp32 /
-                            fp16 tensors: the per-timestep kernels                              */
+                            gradient; its training pair saves one fp32 state per chunk; gradients
+                            through the state included).  Everything else: the per-timestep
+                            kernels                                                             */
     WKV6_ALGO_SCAN = 1,  /* per-timestep fp32 recurrence, state in VGPRs                       */
     WKV6_ALGO_CHUNK = 2  /* chunk-parallel form.  bf16 tensors: bf16 MFMA for the dense intra-chunk
                             products in every call.  fp32 tensors: the full-precision chunk form, as

@@ -534,12 +534,19 @@ int wkv6_backward_saved_sum(void *stream, int dtype, int algo, int64_t B, int64_
                          need > 0, gu_sum);
 }
 
+// where the pairs' final states sit in the workspace of a full-precision backward with state gradients
+static size_t state32_offset(int64_t B, int64_t T, int64_t H) { return (wkv6::chunk32_saved_bytes(B, T, H) + 255) & ~(size_t)255; }
+
 size_t wkv6_backward_with_state_workspace_bytes(int dtype, int algo, int64_t B, int64_t T, int64_t C, int64_t H) {
     if (check_shape_any(dtype, B, T, C, H) == kSmallHead) return wkv6::generic_backward_workspace_bytes(B, T, C);
     if (check_shape(dtype, B, T, C, H) != WKV6_OK) return 0;
     size_t need = wkv6::scan_backward_state_workspace_bytes(B, T, C);
     const size_t c = wkv6_backward_workspace_bytes_ex(dtype, algo, B, T, C, H);
     if (c > need) need = c;
+    if (train_chunk32(dtype, algo, B, T, H)) {   // the chunk states, then the final state of every pair
+        const size_t s = state32_offset(B, T, H) + (size_t)(B * H) * 64 * 64 * sizeof(float);
+        if (s > need) need = s;
+    }
     return need;   // (includes the segments' states where the backward runs in time segments)
 }
 
@@ -563,6 +570,14 @@ int wkv6_backward_with_state(void *stream, int dtype, int algo, int64_t B, int64
     }
     if (algo == WKV6_ALGO_CHUNK && !chunk_possible(dtype, T, C)) return WKV6_ERR_UNSUPPORTED;
     hipStream_t st = (hipStream_t)stream;
+    if (train_chunk32(dtype, algo, B, T, H)) {
+        // full-precision chunk form: the chunk states (and the final one, which anchors the decay gradient's sums
+        // where a gradient arrives at it) from a states-only forward that starts from s0, then the backward
+        float *sT = gsT ? reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + state32_offset(B, T, H)) : nullptr;
+        const hipError_t e = wkv6::chunk32_forward(st, dtype, WKV6_F32, B, T, H, r, k, v, w, u, s0, nullptr, nullptr, sT, workspace);
+        if (e != hipSuccess) return finish(e);
+        return finish(wkv6::chunk32_backward(st, dtype, B, T, H, r, k, v, w, u, gy, gr, gk, gv, gw, gu, workspace, s0, gsT, sT, gs0));
+    }
     const bool chunk = algo == WKV6_ALGO_CHUNK || (algo == WKV6_ALGO_AUTO && chunk_eligible(dtype, T, C));
     if (!chunk)
         return finish(wkv6::scan_backward_state(st, dtype, B, T, H, r, k, v, w, u, s0, gy, gsT, gr, gk, gv, gw, gu, gs0, workspace));

@@ -50,6 +50,11 @@ struct C32BwdArgs {
     const void *r, *k, *v, *w, *u, *gy;
     void *gr, *gk, *gv, *gw, *gu;
     float *saved;   // [pair][chunk][4096] chunk-start states as the forward leaves them (fragment order)
+    // gradients through the state, [pair][key][value] fp32, all null for the stateless operator: the initial state
+    // (only the per-timestep second pass reads it: the chunk states already contain it), the gradient arriving at
+    // the final state, the final state itself (read where gsT is given: E_T = sum_j S_T o gsT), dL/dS_0 (out)
+    const float *s0, *gsT, *sT;
+    float *gs0;
 };
 
 template <typename Tin, typename Tout>
@@ -169,6 +174,13 @@ __global__ __launch_bounds__(768) void chunk32_bwd_kernel(const C32BwdArgs a)
         f32x4 G[4];   // G[ib][e] = G[16ib+4g+e][col]
 #pragma unroll
         for (int i = 0; i < 4; ++i) G[i] = zero;
+        if (a.gsT) {
+            const float *p = a.gsT + (int64_t)pair * (kN * kN) + col;
+#pragma unroll
+            for (int ib = 0; ib < 4; ++ib)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) G[ib][e] = p[(16 * ib + 4 * g + e) * kN];
+        }
         __syncthreads();
         for (int s = 0; s < nchunk; ++s) {
             const int c = nchunk - 1 - s, buf = s & 1;
@@ -243,6 +255,13 @@ __global__ __launch_bounds__(768) void chunk32_bwd_kernel(const C32BwdArgs a)
             }
             __syncthreads();
         }
+        if (a.gs0) {   // what is left after the first chunk is dL/dS_0
+            float *p = a.gs0 + (int64_t)pair * (kN * kN) + col;
+#pragma unroll
+            for (int ib = 0; ib < 4; ++ib)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) p[(16 * ib + 4 * g + e) * kN] = G[ib][e];
+        }
     } else {
         // ---------------- key waves ----------------
         const int q = wave - 4, n = lane & 15, g = lane >> 4, col = 16 * q + n;
@@ -253,6 +272,18 @@ __global__ __launch_bounds__(768) void chunk32_bwd_kernel(const C32BwdArgs a)
 #pragma unroll
         for (int i = 0; i < 4; ++i) Gt[i] = zero;
         float E = 0.f, gu_acc = 0.f;
+        if (a.gsT) {   // G_T^T, and the anchor of the decay gradient's sums: E_T = sum_j S_T o G_T over the row
+            const float *pg = a.gsT + (int64_t)pair * (kN * kN) + col * kN + 4 * g;
+            const float *ps = a.sT + (int64_t)pair * (kN * kN) + col * kN + 4 * g;
+            float part = 0.f;
+#pragma unroll
+            for (int jb = 0; jb < 4; ++jb) {
+                Gt[jb] = *reinterpret_cast<const f32x4 *>(pg + 16 * jb);
+                const f32x4 sv = *reinterpret_cast<const f32x4 *>(ps + 16 * jb);
+                part += (sv[0] * Gt[jb][0] + sv[1] * Gt[jb][1]) + (sv[2] * Gt[jb][2] + sv[3] * Gt[jb][3]);
+            }
+            E = sum_rows4(part);
+        }
         const float u_lane = load1(u + h * kN + col);
         // S_0^T from the forward's fragment order: S[i][j] sits in tile (j / 16, i / 16) at lane (j % 16) + 16 ((i % 16) / 4), element i % 4
         auto load_state = [&](int c) {
@@ -384,7 +415,10 @@ __global__ __launch_bounds__(768) void chunk32_bwd_kernel(const C32BwdArgs a)
 #pragma unroll
                     for (int e = 3; e >= 0; --e) {
                         const int tl = 16 * x + 4 * g + e;
-                        const float o_w = (run - kgk[x][e]) * L.D[buf][tl][col];
+                        float o_w = (run - kgk[x][e]) * L.D[buf][tl][col];
+                        // (a zero initial state: the first decay reaches no output, its gradient is zero and not
+                        // what rounding leaves of two equal sums)
+                        if (x == 0 && e == 0 && a.s0 == nullptr && c == 0 && g == 0) o_w = 0.f;
                         if (full || 16 * x + e < left) store1(gw + out0 + (16 * x + e) * C + lane_off, o_w);
                         run += zt[x][e];
                     }
@@ -400,14 +434,21 @@ __global__ __launch_bounds__(768) void chunk32_bwd_kernel(const C32BwdArgs a)
     __syncthreads();
     // a pair whose decay left the reach: once more, one timestep at a time (the pair's slice of the saved
     // states, T/32 x 64 x 64 floats, is large enough for the T x 64 workspace of that pass)
+    __shared__ float s_ft[kN];
     if (L.wild[0] | L.wild[1] | L.wild[2] | L.wild[3]) {
+        const int64_t so = (int64_t)pair * (kN * kN);
+        const float *s0p = a.s0 ? a.s0 + so : nullptr, *gsTp = a.gsT ? a.gsT + so : nullptr;
+        float *gs0p = a.gs0 ? a.gs0 + so : nullptr;
+        const bool states = s0p || gsTp || gs0p;
         __syncthreads();
         scan_bwd_a_body<Tin, Tout>(reinterpret_cast<C32BwdSmem *>(c32_smem)->scan_a, b, h, T, H, r, k, v, w, u, gy,
-                                   reinterpret_cast<Tout *>(a.gr), reinterpret_cast<Tout *>(a.gu), ck, kN);
+                                   reinterpret_cast<Tout *>(a.gr), reinterpret_cast<Tout *>(a.gu), ck, kN,
+                                   s0p, gsTp, states ? s_ft : nullptr);
         __threadfence_block();
         __syncthreads();
         scan_bwd_b_body<Tin, Tout>(reinterpret_cast<C32BwdSmem *>(c32_smem)->scan_b, b, h, T, H, r, k, v, w, u, gy, ck, kN,
-                                   reinterpret_cast<Tout *>(a.gk), reinterpret_cast<Tout *>(a.gv), reinterpret_cast<Tout *>(a.gw));
+                                   reinterpret_cast<Tout *>(a.gk), reinterpret_cast<Tout *>(a.gv), reinterpret_cast<Tout *>(a.gw),
+                                   gsTp, states ? s_ft : nullptr, gs0p, s0p == nullptr);
     }
 }
 
@@ -422,9 +463,12 @@ static hipError_t launch(hipStream_t st, int64_t B, const C32BwdArgs &a) {
 
 hipError_t chunk32_backward(hipStream_t st, int dtype, int64_t B, int64_t T, int64_t H,
                             const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
-                            void *gr, void *gk, void *gv, void *gw, void *gu, void *saved_states)
+                            void *gr, void *gk, void *gv, void *gw, void *gu, void *saved_states,
+                            const float *s0, const float *gsT, const float *sT, float *gs0)
 {
+    if (gsT != nullptr && sT == nullptr) return hipErrorInvalidValue;   // (the anchor of the decay gradient needs S_T)
     C32BwdArgs a;
+    a.s0 = s0; a.gsT = gsT; a.sT = sT; a.gs0 = gs0;
     a.T = (int)T; a.H = (int)H;
     a.r = r; a.k = k; a.v = v; a.w = w; a.u = u; a.gy = gy;
     a.gr = gr; a.gk = gk; a.gv = gv; a.gw = gw; a.gu = gu;

@@ -107,7 +107,10 @@ hipError_t chunk32_forward(hipStream_t st, int dtype, int state_dtype, int64_t B
 // whose decay left the chunk form's reach); gu (B, C)
 hipError_t chunk32_backward(hipStream_t st, int dtype, int64_t B, int64_t T, int64_t H,
                             const void *r, const void *k, const void *v, const void *w, const void *u, const void *gy,
-                            void *gr, void *gk, void *gv, void *gw, void *gu, void *saved_states);
+                            void *gr, void *gk, void *gv, void *gw, void *gu, void *saved_states,
+                            // gradients through the state ((B,H,64,64) fp32 [key][value]; sT = the forward's final state,
+                            // needed with gsT); the saved states come from a forward that started from s0
+                            const float *s0 = nullptr, const float *gsT = nullptr, const float *sT = nullptr, float *gs0 = nullptr);
 
 // fp16 tensors on the chunked kernels (training pair only: y and the gradients are fp32).  r, k, w stay
 // fp16 (the kernels unpack them exactly); v and gy are consumed as bf16 MFMA operands, so the caller

@@ -115,6 +115,56 @@ def test_state_in_and_out(op, oracle, dt):
     check_close("sT from zero", sT0, sT_ref0, torch.float32, is_grad=True)
 
 
+@pytest.mark.parametrize("dt", ["f32", "f16"])
+@pytest.mark.parametrize("B,T,H,with_s0,with_gs,wild", [(2, 64, 2, True, True, False), (2, 150, 1, True, True, False), (1, 512, 3, True, True, False),
+                                                     (2, 96, 2, False, True, False), (2, 97, 2, True, False, False), (3, 128, 2, False, False, False),
+                                                     (2, 160, 2, True, True, True), (260, 64, 1, True, True, False)])
+def test_gradients_through_the_state(op, oracle, dt, B, T, H, with_s0, with_gs, wild):
+    # loss = sum(y * gy) + sum(S_T * gS) with S_0 given: wkv6_backward_with_state on the full-precision chunk form (a
+    # states-only forward from S_0, the backward with the reverse state started from gS), against the float64
+    # adjoint-form oracle; one-sided cases, a pair redone per timestep, more pairs than compute units
+    dtype = DTYPES[dt]
+    print("state gradients B=%d T=%d H=%d %s s0=%d gS=%d wild=%d" % (B, T, H, dt, with_s0, with_gs, wild), flush=True)
+    ins = oracle.make_inputs(B, T, H, N, 500 + T, with_state=True)
+    if wild:
+        ins[3][B - 1, T // 3:T // 3 + 20, 5:25] = 6.0
+    dev, ref = cast_inputs(ins[:5], dtype)
+    gyd, gyr = cast_inputs(ins[5:6], torch.float32)
+    s0 = ins[6].float() * 3 if with_s0 else None
+    gS = torch.randn(B, H, N, N, generator=torch.Generator().manual_seed(T)) if with_gs else None
+    leaves = [x.clone().requires_grad_(True) for x in dev]
+    s0_dev = s0.cuda().requires_grad_(True) if with_s0 else None
+    op.algo = AUTO
+    y, sT = op(*leaves, return_state=True, init_state=s0_dev)
+    loss = (y * gyd[0]).sum()
+    if with_gs:
+        loss = loss + (sT * gS.cuda()).sum()
+    got = torch.autograd.grad(loss, leaves + ([s0_dev] if with_s0 else []))
+    torch.cuda.synchronize()
+    want = oracle.backward_state_c(*ref, gyr[0], N, None if s0 is None else to_np(s0), None if gS is None else to_np(gS))
+    y_ref, sT_ref = oracle.forward_c(*ref, N, None if s0 is None else to_np(s0))
+    check_close("y", y.detach(), y_ref, torch.float32)
+    check_close("sT", sT.detach(), sT_ref, torch.float32, is_grad=True)
+    _check_grads(got[:5], want[:5], dtype)
+    if with_s0:
+        check_close("gs0", to_np(got[5]), want[5], torch.float32, is_grad=True)
+    else:
+        assert float(got[3][:, 0].abs().max()) == 0.0      # zero initial state: the first decay reaches nothing
+    if not with_gs:
+        assert float(got[3][:, -1].abs().max()) == 0.0
+    # the same call on the per-timestep kernels agrees to fp32 rounding
+    op.algo = SCAN
+    leaves2 = [x.clone().requires_grad_(True) for x in dev]
+    s0_2 = s0.cuda().requires_grad_(True) if with_s0 else None
+    y2, sT2 = op(*leaves2, return_state=True, init_state=s0_2)
+    loss2 = (y2 * gyd[0]).sum() + ((sT2 * gS.cuda()).sum() if with_gs else 0.0)
+    got2 = torch.autograd.grad(loss2, leaves2 + ([s0_2] if with_s0 else []))
+    torch.cuda.synchronize()
+    tol = 2e-3 if dtype == torch.float16 else 5e-5
+    for a_, b_ in zip(got, got2):
+        assert float((a_.double() - b_.double()).abs().max()) <= tol * max(float(b_.double().abs().max()), 1e-30)
+
+
 def test_decay_outside_the_reach_is_redone_exactly(op, oracle):
     # one pair decays by e^-4.5 per token over 40 tokens (a half-chunk sum of 72 > 40), another carries the
     # model's padding values (w = -1e9: decay exactly 1, with k = 0) and a decay of exactly 0 (w = 20): those
