@@ -16,13 +16,16 @@
 // instead of once per 16-token tile; A is three 16x16 blocks; nothing but the scalings and the masks
 // of the diagonal blocks is VALU work in the consumer waves.
 //
-// Workgroup: 12 waves.  Four producer waves (wave p <-> tokens 16p..16p+15 of every chunk) bring the
-// raw rows from global memory straight into LDS three chunk visits ahead, turn r, k, w of the next
-// chunk into R~, K~, g1, g2 and the diagonal, and write out what the consumers staged during the
-// previous visit.  Eight consumer waves (q, half): value columns 16q..16q+15; both halves carry the
-// state through both blocks of a visit, half h produces y of block h.  y and the saved chunk states
-// never leave a consumer wave as partial rows: they are staged in LDS as [token][channel] tiles and
-// stored one visit later by the producer waves as whole 128-byte rows.
+// Workgroup: 12 waves in three roles, one wave of each per SIMD.  Four loading waves (wave p <-> tokens
+// 16p..16p+15 of every chunk) bring the raw rows from global memory straight into LDS three chunk visits
+// ahead and turn r, k, w of the next chunk into R~, K~, g1, g2 and the diagonal.  Four consumer waves
+// (q): value columns 16q..16q+15 of the state and of y, both blocks of a visit.  Four storing waves
+// write out what the consumers staged during the previous visit (kFuse: with the output stage, whose
+// gate rows they fetch themselves): y and the saved chunk states never leave a consumer wave as partial
+// rows, they are staged in LDS as [token][channel] tiles and leave one visit later as whole 128-byte rows.
+// (Loads and stores in different waves: a wave's vector-memory operations complete in order, and a
+// loading wave that also stored waited for its stores with every load; two sets of consumer waves that
+// both carried the state took as long as one.)
 #include "wkv6_mfma.h"
 #include "wkv6_kernels.h"
 #include "wkv6_scan_body.h"
@@ -75,10 +78,10 @@ __device__ __forceinline__ float sum_row8(float x) {
 }
 
 // ------------------------------------------------------------------------------------------
-// Consumer wave (q, HALF): value columns i = 16q + l16; y of block HALF (tokens 32 HALF .. +31).
+// Consumer wave q: value columns i = 16q + l16.
 // State S[m]: rows j = block_row_channel(m, g) + rr, column i.
 // ------------------------------------------------------------------------------------------
-template <typename Ts, bool kSave, bool kFuse, int HALF>
+template <typename Ts, bool kSave, bool kFuse>
 __device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsigned char *smem, int pair0, int q, int lane)
 {
     const int T = a.T, H = a.H;
@@ -100,7 +103,7 @@ __device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsign
             for (int rr = 0; rr < 4; ++rr) Snext[m][rr] = load1(p + (block_row_channel(m, g) + rr) * kN);
     };
     if (a.s0 != nullptr) request_state(0);
-    if (kSave && HALF == 0 && b0 == 0 && q == 0 && lane == 0 && a.arrivals) a.arrivals[h] = 0;
+    if (kSave && b0 == 0 && q == 0 && lane == 0 && a.arrivals) a.arrivals[h] = 0;
     int c = 0, slot = 0;   // visit `it` is chunk c of pair number `slot`
     for (int it = 0; it < nvisit; ++it) {
         __syncthreads();
@@ -113,7 +116,7 @@ __device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsign
         const float *vec = reinterpret_cast<const float *>(smem + BlockFwdLds::kVec + (it & 1) * kBlockVecBytes);
         const float *ruk = vec + 4 * kN;
         const unsigned char *vt = smem + BlockFwdLds::kRawV + (it % (BlockFwdLds::kVAhead + 1)) * kTileBytes;
-        if (kSave && HALF == 0) {
+        if (kSave) {
             // the state at the chunk start, as the backward wants it: bf16, transposed ([i][j] rows of 128 bytes)
             unsigned char *ss = smem + BlockFwdLds::kSStage + (it & 1) * kTileBytes;
 #pragma unroll
@@ -132,7 +135,7 @@ __device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsign
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
             scale(vec + 2 * blk * kN);   // g1 of the block
-            if (blk == HALF) {
+            {
                 // y of this block's two 16-token row groups; products transposed (accumulator rows i = 4g + rr,
                 // column t = l16: a lane holds four neighbouring channels of one token).  Every fragment is
                 // fetched first, then the MFMAs run as independent chains.
@@ -183,7 +186,7 @@ __device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsign
         }
         __builtin_amdgcn_sched_barrier(0);
         if (++c == nchunk) {
-            if (a.sT != nullptr && HALF == 0) {   // the pair's final state
+            if (a.sT != nullptr) {   // the pair's final state
                 Ts *p = reinterpret_cast<Ts *>(a.sT) + ((int64_t)(b0 + slot * a.bstep) * H + h) * (kN * kN) + 16 * q + l16;
 #pragma unroll
                 for (int m = 0; m < 4; ++m)
@@ -198,9 +201,12 @@ __device__ __forceinline__ void block_fwd_consumer(const BlockFwdArgs &a, unsign
 }
 
 // ------------------------------------------------------------------------------------------
-// Producer wave p: tokens 16p..16p+15 of every chunk.
+// Loading wave p (kRole = kBlockFwdLoads): tokens 16p..16p+15 of every chunk in, operands prepared.
+// Storing wave p (kRole = kBlockFwdStores): the same rows of what the consumers staged, out.
+// One function: both walk the same visits with the same cursors and lane mapping.
 // ------------------------------------------------------------------------------------------
-template <bool kSave, bool kRagged, bool kFuse>
+constexpr int kBlockFwdLoads = 1, kBlockFwdStores = 2;
+template <bool kSave, bool kRagged, bool kFuse, int kRole>
 __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsigned char *smem, int *s_wild, int pair0, int p, int lane)
 {
     const int T = a.T, H = a.H;
@@ -360,21 +366,23 @@ __device__ __forceinline__ void block_fwd_producer(const BlockFwdArgs &a, unsign
     };
     // r, k, w of visit j are requested three visits ahead (two in the prologue), v kVAhead visits ahead
     constexpr int kVAhead = BlockFwdLds::kVAhead;
-    issue_v();
-    issue_rkw();
-    if (nvisit > 1) { issue_v(); issue_rkw(); }
-    if (kVAhead > 2 && nvisit > 2) issue_v();
-    prepare(nvisit > 2);
+    if (kRole == kBlockFwdLoads) {
+        issue_v();
+        issue_rkw();
+        if (nvisit > 1) { issue_v(); issue_rkw(); }
+        if (kVAhead > 2 && nvisit > 2) issue_v();
+        prepare(nvisit > 2);
+    }
     for (int it = 0; it < nvisit; ++it) {
         __syncthreads();
         // free again: the raw v block of visit it-1; the staging tiles of visit it-1 are complete
-        if (it + kVAhead < nvisit) issue_v();
-        if (kFuse) issue_gate();
-        if (it > 0) store_staged();
-        if (it + 1 < nvisit) prepare(it + 3 < nvisit);
+        if (kRole == kBlockFwdLoads && it + kVAhead < nvisit) issue_v();
+        if (kRole == kBlockFwdStores && kFuse) issue_gate();
+        if (kRole == kBlockFwdStores && it > 0) store_staged();
+        if (kRole == kBlockFwdLoads && it + 1 < nvisit) prepare(it + 3 < nvisit);
     }
     __syncthreads();
-    store_staged();
+    if (kRole == kBlockFwdStores) store_staged();
     wait_loads<0>();
 }
 
@@ -414,9 +422,9 @@ __global__ __launch_bounds__(kBlockFwdThreads) void block_fwd_kernel(BlockFwdArg
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int pair0 = (int)blockIdx.x;
-    if (wave < 4) block_fwd_producer<kSave, kRagged, kFuse>(a, smem, s_wild, pair0, wave, lane);
-    else if (wave < 8) block_fwd_consumer<Ts, kSave, kFuse, 0>(a, smem, pair0, wave - 4, lane);
-    else block_fwd_consumer<Ts, kSave, kFuse, 1>(a, smem, pair0, wave - 8, lane);
+    if (wave < 4) block_fwd_producer<kSave, kRagged, kFuse, kBlockFwdLoads>(a, smem, s_wild, pair0, wave, lane);
+    else if (wave < 8) block_fwd_consumer<Ts, kSave, kFuse>(a, smem, pair0, wave - 4, lane);
+    else block_fwd_producer<kSave, kRagged, kFuse, kBlockFwdStores>(a, smem, s_wild, pair0, wave - 8, lane);
     // exact second pass for the pairs of which 16 tokens left the range the scaled operands can hold
     __threadfence_block();
     __syncthreads();
